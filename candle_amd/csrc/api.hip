@@ -1,0 +1,401 @@
+// C ABI of libcandle_qhip (declarations and reference citations: include/candle_qhip.h).
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <new>
+
+#include "qhip_internal.h"
+
+// ------------------------------------------------------------------ errors ----
+static thread_local char g_err[512] = "";
+
+int cq_set_error(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+extern "C" const char *cq_last_error(void) { return g_err; }
+extern "C" const char *cq_version(void) { return "candle_qhip 0.1 (gfx950)"; }
+
+extern "C" int cq_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return n;
+}
+
+// ------------------------------------------------------------ dtype tables ----
+extern "C" int64_t cq_block_size(int dt) {
+    switch (dt) {
+    case CQ_DTYPE_Q4_0: case CQ_DTYPE_Q8_0: case CQ_DTYPE_Q8_1: return 32;
+    case CQ_DTYPE_Q4K: case CQ_DTYPE_Q6K: case CQ_DTYPE_Q8K: return 256;
+    default: return 0;
+    }
+}
+extern "C" int64_t cq_type_size(int dt) {
+    switch (dt) {
+    case CQ_DTYPE_Q4_0: return 18;
+    case CQ_DTYPE_Q8_0: return 34;
+    case CQ_DTYPE_Q8_1: return 36;
+    case CQ_DTYPE_Q4K: return 144;
+    case CQ_DTYPE_Q6K: return 210;
+    case CQ_DTYPE_Q8K: return 292;
+    default: return 0;
+    }
+}
+extern "C" int cq_vec_dot_type(int dt) {
+    switch (dt) {
+    case CQ_DTYPE_Q4_0: case CQ_DTYPE_Q8_0: return CQ_DTYPE_Q8_0;
+    case CQ_DTYPE_Q4K: case CQ_DTYPE_Q6K: return CQ_DTYPE_Q8K;
+    default: return -1;
+    }
+}
+
+static bool is_weight_dtype(int dt) {
+    return dt == CQ_DTYPE_Q4_0 || dt == CQ_DTYPE_Q8_0 || dt == CQ_DTYPE_Q4K || dt == CQ_DTYPE_Q6K;
+}
+
+// --------------------------------------------------------------- weights ----
+static int weight_alloc(int dev, int dt, int64_t n, int64_t k, cq_weight **out) {
+    if (!out) return cq_set_error(CQ_ERR_INVALID, "out is null");
+    *out = nullptr;
+    if (!is_weight_dtype(dt)) return cq_set_error(CQ_ERR_UNSUPPORTED, "unsupported weight dtype %d", dt);
+    if (n < 0 || k < 0) return cq_set_error(CQ_ERR_INVALID, "negative shape [%lld, %lld]", (long long)n, (long long)k);
+    const int64_t bs = cq_block_size(dt);
+    // check_shape, candle-core/src/quantized/mod.rs:304-316
+    if (k % bs != 0)
+        return cq_set_error(CQ_ERR_INVALID,
+                            "quantized tensor must have their last dim divisible by block size [%lld, %lld] %lld",
+                            (long long)n, (long long)k, (long long)bs);
+    int ndev = cq_device_count();
+    if (dev < 0 || dev >= ndev) return cq_set_error(CQ_ERR_INVALID, "device %d out of range (%d visible)", dev, ndev);
+    CQ_HIP_CHECK(hipSetDevice(dev));
+    cq_weight *w = new (std::nothrow) cq_weight();
+    if (!w) return cq_set_error(CQ_ERR_INVALID, "out of host memory");
+    w->dev = dev; w->dtype = dt; w->n = n; w->k = k;
+    const int64_t nb = n * (k / bs);
+    w->ggml_bytes = (size_t)nb * (size_t)cq_type_size(dt);
+    size_t s0 = 0, s1 = 0, s2 = 0, s3 = 0;
+    switch (dt) {
+    case CQ_DTYPE_Q4_0: s0 = (size_t)nb * 16; s1 = (size_t)nb * 2; break;
+    case CQ_DTYPE_Q8_0: s0 = (size_t)nb * 32; s1 = (size_t)nb * 2; break;
+    case CQ_DTYPE_Q4K: s0 = (size_t)nb * 128; s1 = (size_t)nb * 16; break;
+    case CQ_DTYPE_Q6K: s0 = (size_t)nb * 128; s1 = (size_t)nb * 64; s2 = (size_t)nb * 16; s3 = (size_t)nb * 2; break;
+    }
+    const size_t o1 = cq_align_up(s0 + CQ_TAIL_PAD, 256);
+    const size_t o2 = cq_align_up(o1 + s1 + CQ_TAIL_PAD, 256);
+    const size_t o3 = cq_align_up(o2 + s2 + CQ_TAIL_PAD, 256);
+    w->alloc_bytes = cq_align_up(o3 + s3 + CQ_TAIL_PAD, 256);
+    hipError_t e = hipMalloc(&w->base, w->alloc_bytes);
+    if (e != hipSuccess) {
+        const size_t bytes = w->alloc_bytes;
+        delete w;
+        return cq_set_error(CQ_ERR_HIP, "hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+    }
+    w->p0 = (uint8_t *)w->base;
+    w->p1 = (uint8_t *)w->base + o1;
+    w->p2 = (uint8_t *)w->base + o2;
+    w->p3 = (uint8_t *)w->base + o3;
+    *out = w;
+    return CQ_OK;
+}
+
+extern "C" int cq_weight_zeros(int dev, int dt, int64_t n, int64_t k, cq_weight **out) {
+    int rc = weight_alloc(dev, dt, n, k, out);
+    if (rc) return rc;
+    hipError_t e = hipMemset((*out)->base, 0, (*out)->alloc_bytes);
+    if (e != hipSuccess) {
+        cq_weight_destroy(*out);
+        *out = nullptr;
+        return cq_set_error(CQ_ERR_HIP, "hipMemset failed: %s", hipGetErrorString(e));
+    }
+    return CQ_OK;
+}
+
+extern "C" int cq_weight_create(int dev, int dt, const void *host_blocks, size_t nbytes, int64_t n, int64_t k,
+                                cq_weight **out) {
+    if (!host_blocks && nbytes) return cq_set_error(CQ_ERR_INVALID, "host_ggml_blocks is null");
+    int rc = cq_weight_zeros(dev, dt, n, k, out);
+    if (rc) return rc;
+    cq_weight *w = *out;
+    if (nbytes != w->ggml_bytes) {
+        cq_weight_destroy(w);
+        *out = nullptr;
+        return cq_set_error(CQ_ERR_INVALID, "expected %zu bytes of GGML blocks for [%lld, %lld] dtype %d, got %zu",
+                            w->ggml_bytes, (long long)n, (long long)k, dt, nbytes);
+    }
+    if (nbytes == 0) return CQ_OK;
+    void *tmp = nullptr;
+    hipError_t e = hipMalloc(&tmp, nbytes + 256);
+    if (e == hipSuccess) e = hipMemcpy(tmp, host_blocks, nbytes, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = cq_launch_repack(w, (const uint8_t *)tmp, nullptr);
+    if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
+    if (tmp) (void)hipFree(tmp);
+    if (e != hipSuccess) {
+        cq_weight_destroy(w);
+        *out = nullptr;
+        return cq_set_error(CQ_ERR_HIP, "weight upload failed: %s", hipGetErrorString(e));
+    }
+    return CQ_OK;
+}
+
+extern "C" int cq_weight_quantize(cq_weight *w, const float *src_dev, void *stream) {
+    if (!w || !src_dev) return cq_set_error(CQ_ERR_INVALID, "null argument");
+    if (w->ggml_bytes == 0) return CQ_OK;
+    CQ_HIP_CHECK(hipSetDevice(w->dev));
+    hipStream_t s = (hipStream_t)stream;
+    void *tmp = nullptr;
+    CQ_HIP_CHECK(hipMalloc(&tmp, w->ggml_bytes + 256));
+    const int64_t nb = w->n * (w->k / cq_block_size(w->dtype));
+    hipError_t e = cq_launch_quantize_weight(w->dtype, src_dev, nb, (uint8_t *)tmp, s);
+    if (e == hipSuccess) e = cq_launch_repack(w, (const uint8_t *)tmp, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);  // the temporary is freed below
+    (void)hipFree(tmp);
+    if (e != hipSuccess) return cq_set_error(CQ_ERR_HIP, "weight quantize failed: %s", hipGetErrorString(e));
+    return CQ_OK;
+}
+
+extern "C" int cq_weight_dequantize(const cq_weight *w, float *dst_dev, void *stream) {
+    if (!w || !dst_dev) return cq_set_error(CQ_ERR_INVALID, "null argument");
+    CQ_HIP_CHECK(hipSetDevice(w->dev));
+    CQ_HIP_CHECK(cq_launch_dequantize(w, dst_dev, nullptr, (hipStream_t)stream));
+    return CQ_OK;
+}
+
+extern "C" int cq_weight_dequantize_f16(const cq_weight *w, uint16_t *dst_dev, void *stream) {
+    if (!w || !dst_dev) return cq_set_error(CQ_ERR_INVALID, "null argument");
+    CQ_HIP_CHECK(hipSetDevice(w->dev));
+    CQ_HIP_CHECK(cq_launch_dequantize(w, nullptr, dst_dev, (hipStream_t)stream));
+    return CQ_OK;
+}
+
+extern "C" int cq_weight_to_ggml(const cq_weight *w, void *host_dst, size_t nbytes) {
+    if (!w || (!host_dst && nbytes)) return cq_set_error(CQ_ERR_INVALID, "null argument");
+    if (nbytes != w->ggml_bytes)
+        return cq_set_error(CQ_ERR_INVALID, "expected a %zu-byte destination, got %zu", w->ggml_bytes, nbytes);
+    if (nbytes == 0) return CQ_OK;
+    CQ_HIP_CHECK(hipSetDevice(w->dev));
+    void *tmp = nullptr;
+    CQ_HIP_CHECK(hipMalloc(&tmp, nbytes + 256));
+    hipError_t e = hipDeviceSynchronize();
+    if (e == hipSuccess) e = cq_launch_unpack(w, (uint8_t *)tmp, nullptr);
+    if (e == hipSuccess) e = hipMemcpy(host_dst, tmp, nbytes, hipMemcpyDeviceToHost);
+    (void)hipFree(tmp);
+    if (e != hipSuccess) return cq_set_error(CQ_ERR_HIP, "weight download failed: %s", hipGetErrorString(e));
+    return CQ_OK;
+}
+
+extern "C" size_t cq_weight_size_in_bytes(const cq_weight *w) { return w ? w->ggml_bytes : 0; }
+extern "C" int cq_weight_dtype(const cq_weight *w) { return w ? w->dtype : -1; }
+extern "C" int cq_weight_device(const cq_weight *w) { return w ? w->dev : -1; }
+extern "C" int cq_weight_shape(const cq_weight *w, int64_t *n, int64_t *k) {
+    if (!w) return cq_set_error(CQ_ERR_INVALID, "null weight");
+    if (n) *n = w->n;
+    if (k) *k = w->k;
+    return CQ_OK;
+}
+
+extern "C" void cq_weight_destroy(cq_weight *w) {
+    if (!w) return;
+    if (w->base) {
+        (void)hipSetDevice(w->dev);
+        (void)hipFree(w->base);
+    }
+    delete w;
+}
+
+// ----------------------------------------------------------- activations ----
+static bool is_act_dtype(int dt) { return dt == CQ_DTYPE_Q8_0 || dt == CQ_DTYPE_Q8_1 || dt == CQ_DTYPE_Q8K; }
+
+extern "C" size_t cq_act_bytes(int act_dtype, int64_t m, int64_t k) {
+    if (!is_act_dtype(act_dtype) || m < 0 || k < 0 || k % cq_block_size(act_dtype) != 0) return 0;
+    return (size_t)(m * (k / cq_block_size(act_dtype))) * (size_t)cq_type_size(act_dtype);
+}
+
+extern "C" int cq_quantize_act(int dev, int act_dtype, const float *x_dev, int64_t m, int64_t k, void *dst,
+                               void *stream) {
+    if (!is_act_dtype(act_dtype)) return cq_set_error(CQ_ERR_UNSUPPORTED, "unsupported activation dtype %d", act_dtype);
+    if (m < 0 || k < 0) return cq_set_error(CQ_ERR_INVALID, "negative shape");
+    if (k % cq_block_size(act_dtype) != 0)
+        return cq_set_error(CQ_ERR_INVALID, "%lld is not divisible by %lld", (long long)k,
+                            (long long)cq_block_size(act_dtype));
+    if (m == 0 || k == 0) return CQ_OK;
+    if (!x_dev || !dst) return cq_set_error(CQ_ERR_INVALID, "null argument");
+    if (((uintptr_t)x_dev & 15) || ((uintptr_t)dst & 3))
+        return cq_set_error(CQ_ERR_INVALID, "x must be 16-byte aligned and dst 4-byte aligned");
+    CQ_HIP_CHECK(hipSetDevice(dev));
+    CQ_HIP_CHECK(cq_launch_quantize_act_aos(act_dtype, x_dev, m, k, dst, (hipStream_t)stream));
+    return CQ_OK;
+}
+
+// Workspace layout for m rows of K elements (see cq_act_view).
+static size_t act_ws_layout(int act_dtype, int64_t m, int64_t k, uint8_t *base, cq_act_view *v) {
+    size_t off = 0;
+    auto take = [&](size_t bytes) { size_t o = off; off = cq_align_up(off + bytes, 256); return o; };
+    const size_t o_qs = take((size_t)(m * k));
+    cq_act_view view{};
+    if (act_dtype == CQ_DTYPE_Q8K) {
+        const size_t o_d = take((size_t)(m * (k / 256)) * 4);
+        const size_t o_bs = take((size_t)(m * (k / 256)) * 32);
+        if (base) { view.qs = (int8_t *)(base + o_qs); view.d = (float *)(base + o_d); view.bsums = (int16_t *)(base + o_bs); }
+    } else {
+        const size_t o_d = take((size_t)(m * (k / 32)) * 4);
+        const size_t o_s = take((size_t)(m * (k / 32)) * 4);
+        const size_t o_h = take((size_t)(m * (k / 32)) * 2);
+        if (base) {
+            view.qs = (int8_t *)(base + o_qs); view.d = (float *)(base + o_d);
+            view.bsum32 = (int32_t *)(base + o_s); view.s16 = (uint16_t *)(base + o_h);
+        }
+    }
+    if (v) *v = view;
+    return off;
+}
+
+static int act_dtype_for(const cq_weight *w, int flags) {
+    int a = cq_vec_dot_type(w->dtype);
+    if ((flags & CQ_FLAG_ACT_Q8_1) && (w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q6K)) a = CQ_DTYPE_Q8_1;
+    return a;
+}
+
+extern "C" size_t cq_workspace_bytes(const cq_weight *w, int64_t m, int flags) {
+    if (!w || m <= 0) return 0;
+    return act_ws_layout(act_dtype_for(w, flags), m, w->k, nullptr, nullptr);
+}
+
+static int check_matmul_args(const cq_weight *w, const float *x, int64_t m, const void *y, void *ws, size_t ws_bytes,
+                             size_t need) {
+    if (!w) return cq_set_error(CQ_ERR_INVALID, "null weight");
+    if (m < 0) return cq_set_error(CQ_ERR_INVALID, "negative row count");
+    if (m == 0 || w->n == 0) return CQ_OK;
+    if (!x || !y) return cq_set_error(CQ_ERR_INVALID, "null argument");
+    if ((uintptr_t)x & 15) return cq_set_error(CQ_ERR_INVALID, "x must be 16-byte aligned");
+    if (!ws || ws_bytes < need)
+        return cq_set_error(CQ_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, ws ? ws_bytes : (size_t)0);
+    if ((uintptr_t)ws & 255) return cq_set_error(CQ_ERR_INVALID, "workspace must be 256-byte aligned");
+    return CQ_OK;
+}
+
+extern "C" int cq_qmatmul(const cq_weight *w, const float *x_dev, int64_t m, float *y_dev, int flags, void *ws,
+                          size_t ws_bytes, void *stream) {
+    const size_t need = cq_workspace_bytes(w, m, flags);
+    int rc = check_matmul_args(w, x_dev, m, y_dev, ws, ws_bytes, need);
+    if (rc || m == 0 || w->n == 0) return rc;
+    if (w->k == 0) {
+        CQ_HIP_CHECK(hipSetDevice(w->dev));
+        CQ_HIP_CHECK(cq_launch_fill_zero(y_dev, m * w->n, (hipStream_t)stream));
+        return CQ_OK;
+    }
+    const int act = act_dtype_for(w, flags);
+    CQ_HIP_CHECK(hipSetDevice(w->dev));
+    hipStream_t s = (hipStream_t)stream;
+    cq_act_view v;
+    act_ws_layout(act, m, w->k, (uint8_t *)ws, &v);
+    CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, nullptr, m, w->k, v, s));
+    bool use_gemm = false;
+    if (flags & CQ_FLAG_FORCE_GEMM) {
+        if (!cq_gemm_supported(w, m, act))
+            return cq_set_error(CQ_ERR_UNSUPPORTED, "no MFMA GEMM for dtype %d with activation dtype %d", w->dtype, act);
+        use_gemm = true;
+    } else if (!(flags & CQ_FLAG_FORCE_MATVEC)) {
+        use_gemm = m > 8 && cq_gemm_supported(w, m, act);  // the reference switches kernels at 8 rows (cuda.rs:484-498)
+    }
+    if (act == CQ_DTYPE_Q8_1 && !use_gemm)
+        return cq_set_error(CQ_ERR_UNSUPPORTED, "Q8_1 activations are only handled by the GEMM kernel");
+    if (use_gemm) CQ_HIP_CHECK(cq_launch_gemm(w, v, act, m, y_dev, s));
+    else CQ_HIP_CHECK(cq_launch_matvec(w, v, act, m, y_dev, s));
+    return CQ_OK;
+}
+
+extern "C" int cq_qmatmul_int_dots(const cq_weight *w, const float *x_dev, int64_t m, int32_t *out_i, int32_t *out_mn,
+                                   void *ws, size_t ws_bytes, void *stream) {
+    const size_t need = cq_workspace_bytes(w, m, 0);
+    int rc = check_matmul_args(w, x_dev, m, out_i, ws, ws_bytes, need);
+    if (rc || m == 0 || w->n == 0 || w->k == 0) return rc;
+    const int act = cq_vec_dot_type(w->dtype);
+    CQ_HIP_CHECK(hipSetDevice(w->dev));
+    hipStream_t s = (hipStream_t)stream;
+    cq_act_view v;
+    act_ws_layout(act, m, w->k, (uint8_t *)ws, &v);
+    CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, nullptr, m, w->k, v, s));
+    CQ_HIP_CHECK(cq_launch_int_dots(w, v, m, out_i, w->dtype == CQ_DTYPE_Q4K ? out_mn : nullptr, s));
+    return CQ_OK;
+}
+
+// ------------------------------------------------------------------- MoE ----
+extern "C" size_t cq_grouped_workspace_bytes(const cq_weight *const *experts, int n_experts, int64_t total_rows,
+                                             int flags) {
+    if (!experts || n_experts <= 0 || !experts[0] || total_rows <= 0) return 0;
+    return act_ws_layout(act_dtype_for(experts[0], flags), total_rows, experts[0]->k, nullptr, nullptr);
+}
+
+extern "C" int cq_qmatmul_grouped(const cq_weight *const *experts, int n_experts, const float *x_dev,
+                                  const int32_t *row_ids_dev, const int32_t *offsets, float *y_dev, int flags,
+                                  void *ws, size_t ws_bytes, void *stream) {
+    if (!experts || n_experts <= 0 || !offsets) return cq_set_error(CQ_ERR_INVALID, "null argument");
+    const cq_weight *w0 = experts[0];
+    if (!w0) return cq_set_error(CQ_ERR_INVALID, "null expert");
+    for (int e = 0; e < n_experts; e++) {
+        if (!experts[e]) return cq_set_error(CQ_ERR_INVALID, "null expert %d", e);
+        if (experts[e]->dtype != w0->dtype || experts[e]->n != w0->n || experts[e]->k != w0->k || experts[e]->dev != w0->dev)
+            return cq_set_error(CQ_ERR_INVALID, "expert %d differs in dtype, shape or device from expert 0", e);
+        if (offsets[e + 1] < offsets[e]) return cq_set_error(CQ_ERR_INVALID, "offsets must be non-decreasing");
+    }
+    if (offsets[0] != 0) return cq_set_error(CQ_ERR_INVALID, "offsets[0] must be 0");
+    const int64_t total = offsets[n_experts];
+    const size_t need = cq_grouped_workspace_bytes(experts, n_experts, total, flags);
+    int rc = check_matmul_args(w0, x_dev, total, y_dev, ws, ws_bytes, need);
+    if (rc || total == 0 || w0->n == 0 || w0->k == 0) return rc;
+    const int act = act_dtype_for(w0, flags);
+    if (act == CQ_DTYPE_Q8_1) return cq_set_error(CQ_ERR_UNSUPPORTED, "grouped matmul takes the CPU formulation only");
+    CQ_HIP_CHECK(hipSetDevice(w0->dev));
+    hipStream_t s = (hipStream_t)stream;
+    cq_act_view v;
+    act_ws_layout(act, total, w0->k, (uint8_t *)ws, &v);
+    // gather + quantize every routed row once, then one matmul per non-empty expert over its slice
+    CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, row_ids_dev, total, w0->k, v, s));
+    for (int e = 0; e < n_experts; e++) {
+        const int64_t r0 = offsets[e], te = offsets[e + 1] - offsets[e];
+        if (te == 0) continue;
+        cq_act_view ve = v;
+        ve.qs += r0 * w0->k;
+        if (act == CQ_DTYPE_Q8K) {
+            ve.d += r0 * (w0->k / 256);
+            ve.bsums += r0 * (w0->k / 256) * 16;
+        } else {
+            ve.d += r0 * (w0->k / 32);
+            ve.bsum32 += r0 * (w0->k / 32);
+        }
+        float *ye = y_dev + r0 * w0->n;
+        const bool use_gemm = (flags & CQ_FLAG_FORCE_GEMM) ? true
+                              : (flags & CQ_FLAG_FORCE_MATVEC) ? false
+                                                               : (te > 8 && cq_gemm_supported(experts[e], te, act));
+        if (use_gemm) CQ_HIP_CHECK(cq_launch_gemm(experts[e], ve, act, te, ye, s));
+        else CQ_HIP_CHECK(cq_launch_matvec(experts[e], ve, act, te, ye, s));
+    }
+    return CQ_OK;
+}
+
+extern "C" int cq_silu_mul(int dev, const float *a, const float *b, float *h, int64_t count, void *stream) {
+    if (count < 0) return cq_set_error(CQ_ERR_INVALID, "negative count");
+    if (count == 0) return CQ_OK;
+    if (!a || !b || !h) return cq_set_error(CQ_ERR_INVALID, "null argument");
+    CQ_HIP_CHECK(hipSetDevice(dev));
+    CQ_HIP_CHECK(cq_launch_silu_mul(a, b, h, count, (hipStream_t)stream));
+    return CQ_OK;
+}
+
+extern "C" int cq_moe_scatter_add(int dev, const float *y, const int32_t *row_ids, const float *weights,
+                                  int64_t total_rows, int64_t hidden, float *ys, int64_t tokens, void *stream) {
+    if (total_rows < 0 || hidden < 0 || tokens < 0) return cq_set_error(CQ_ERR_INVALID, "negative size");
+    if (tokens == 0 || hidden == 0) return CQ_OK;
+    if (!ys || (total_rows && (!y || !row_ids || !weights))) return cq_set_error(CQ_ERR_INVALID, "null argument");
+    CQ_HIP_CHECK(hipSetDevice(dev));
+    CQ_HIP_CHECK(cq_launch_scatter_add(y, row_ids, weights, total_rows, hidden, ys, tokens, (hipStream_t)stream));
+    return CQ_OK;
+}

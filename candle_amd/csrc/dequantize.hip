@@ -1,0 +1,133 @@
+// Device planes -> f32 / f16 (QTensor::dequantize, dequantize_f16;
+// candle-core/src/quantized/mod.rs:361-382, CUDA precedent cuda.rs:69-181).
+// The f32 values are those of T::to_float (k_quants.rs:163-183, :568-584, :1313-1341,
+// :1716-1746): same products in the same order, no contraction.  The f16 output is the
+// f32 output rounded to nearest-even, as the reference's tests require
+// (candle-core/tests/quantized_tests.rs:229-234).
+// One thread per 16-byte lane of the main plane; a wave covers 1 KiB of it.
+#include "qhip_internal.h"
+
+namespace {
+
+template <bool F16>
+__device__ __forceinline__ void put(float *d32, uint16_t *d16, int64_t i, float v) {
+    if (F16) d16[i] = cq_f2h(v); else d32[i] = v;
+}
+
+template <bool F16>
+__global__ void dequant_q4_0(const uint8_t *__restrict__ qs, const uint16_t *__restrict__ dpl, int64_t nblocks,
+                             float *d32, uint16_t *d16) {
+    const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    const uint4 q = *(const uint4 *)(qs + b * 16);
+    const float d = cq_h2f(dpl[b]);
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        const uint32_t byte = (w[j >> 2] >> (8 * (j & 3))) & 0xff;
+        const int x0 = (int)(byte & 0xF) - 8, x1 = (int)(byte >> 4) - 8;
+        put<F16>(d32, d16, b * 32 + j, (float)x0 * d);
+        put<F16>(d32, d16, b * 32 + j + 16, (float)x1 * d);
+    }
+}
+
+template <bool F16>
+__global__ void dequant_q8_0(const uint8_t *__restrict__ qs, const uint16_t *__restrict__ dpl, int64_t nunits,
+                             float *d32, uint16_t *d16) {
+    const int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // 16 elements each
+    if (u >= nunits) return;
+    const uint4 q = *(const uint4 *)(qs + u * 16);
+    const float d = cq_h2f(dpl[u >> 1]);
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        const int8_t v = (int8_t)((w[j >> 2] >> (8 * (j & 3))) & 0xff);
+        put<F16>(d32, d16, u * 16 + j, (float)v * d);
+    }
+}
+
+template <bool F16>
+__global__ void dequant_q4k(const uint8_t *__restrict__ qs, const uint8_t *__restrict__ hd, int64_t nunits,
+                            float *d32, uint16_t *d16) {
+    const int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // 16 bytes of qs = 32 elements
+    if (u >= nunits) return;
+    const int64_t b = u >> 3;
+    const int p = (int)(u & 7), g = p >> 1, half = p & 1;
+    const uint4 q = *(const uint4 *)(qs + u * 16);
+    const uint4 h = *(const uint4 *)(hd + b * 16);
+    const float d = cq_h2f((uint16_t)(h.x & 0xffff)), dmin = cq_h2f((uint16_t)(h.x >> 16));
+    int sc1, m1, sc2, m2;
+    cq_scale_min_k4(2 * g, h.y, h.z, h.w, sc1, m1);
+    cq_scale_min_k4(2 * g + 1, h.y, h.z, h.w, sc2, m2);
+    const float d1 = d * (float)sc1, mm1 = dmin * (float)m1;
+    const float d2 = d * (float)sc2, mm2 = dmin * (float)m2;
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+    const int64_t base = b * 256 + 64 * g + 16 * half;
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        const uint32_t byte = (w[j >> 2] >> (8 * (j & 3))) & 0xff;
+        put<F16>(d32, d16, base + j, d1 * (float)(byte & 0xF) - mm1);
+        put<F16>(d32, d16, base + 32 + j, d2 * (float)(byte >> 4) - mm2);
+    }
+}
+
+template <bool F16>
+__global__ void dequant_q6k(const uint8_t *__restrict__ ql, const uint8_t *__restrict__ qh,
+                            const int8_t *__restrict__ sc, const uint16_t *__restrict__ dpl, int64_t nunits,
+                            float *d32, uint16_t *d16) {
+    const int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // 16 bytes of ql = 32 elements
+    if (u >= nunits) return;
+    const int64_t b = u >> 3;
+    const int p = (int)(u & 7), h = p >> 2, t = (p >> 1) & 1, i0 = (p & 1) * 16;
+    const uint4 q = *(const uint4 *)(ql + u * 16);
+    const uint2 hh = *(const uint2 *)(qh + u * 8);
+    const float d = cq_h2f(dpl[b]);
+    // low nibbles: elements 128h + 32t + i0 + e, one 16-element scale group; high nibbles: +64
+    const int js = 8 * h + 2 * t + (i0 >> 4);
+    const float s_lo = (float)sc[b * 16 + js], s_hi = (float)sc[b * 16 + js + 4];
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+    const uint32_t hw[2] = {hh.x, hh.y};
+    const int64_t base = b * 256 + 128 * h + 32 * t + i0;
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+        const int wi = e >> 2, c = e & 3;
+        const uint32_t byte = (w[wi] >> (8 * c)) & 0xff;
+        const uint32_t hb = (hw[wi >> 1] >> (8 * c)) & 0xff;
+        const int sh = (wi & 1) * 4;
+        const int q_lo = (int)((byte & 0xF) | (((hb >> sh) & 3) << 4)) - 32;
+        const int q_hi = (int)((byte >> 4) | (((hb >> (sh + 2)) & 3) << 4)) - 32;
+        put<F16>(d32, d16, base + e, d * s_lo * (float)q_lo);
+        put<F16>(d32, d16, base + 64 + e, d * s_hi * (float)q_hi);
+    }
+}
+
+template <bool F16>
+hipError_t launch(const cq_weight *w, float *d32, uint16_t *d16, hipStream_t s) {
+    const int threads = 256;
+    const int64_t total = w->n * w->k;
+    if (total == 0) return hipSuccess;
+    auto grid = [&](int64_t n) { return (unsigned)((n + threads - 1) / threads); };
+    switch (w->dtype) {
+    case CQ_DTYPE_Q4_0:
+        dequant_q4_0<F16><<<grid(total / 32), threads, 0, s>>>(w->p0, (const uint16_t *)w->p1, total / 32, d32, d16);
+        break;
+    case CQ_DTYPE_Q8_0:
+        dequant_q8_0<F16><<<grid(total / 16), threads, 0, s>>>(w->p0, (const uint16_t *)w->p1, total / 16, d32, d16);
+        break;
+    case CQ_DTYPE_Q4K:
+        dequant_q4k<F16><<<grid(total / 32), threads, 0, s>>>(w->p0, w->p1, total / 32, d32, d16);
+        break;
+    case CQ_DTYPE_Q6K:
+        dequant_q6k<F16><<<grid(total / 32), threads, 0, s>>>(w->p0, w->p1, (const int8_t *)w->p2,
+                                                              (const uint16_t *)w->p3, total / 32, d32, d16);
+        break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t cq_launch_dequantize(const cq_weight *w, float *dst32, uint16_t *dst16, hipStream_t s) {
+    return dst16 ? launch<true>(w, nullptr, dst16, s) : launch<false>(w, dst32, nullptr, s);
+}

@@ -1,0 +1,147 @@
+// Internal declarations shared by the HIP sources of libcandle_qhip.
+// Device layouts here are private to the library (see include/candle_qhip.h).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/candle_qhip.h"
+
+#define QK_K 256
+
+// ---------------------------------------------------------------------------
+// Device weight storage: GGML blocks split into planes so that every wave-wide
+// load is a run of 16-byte lanes over whole 128-byte lines.
+//
+//   Q4_0 : qs [n][k/32][16]  u8   (nibbles, element j low / j+16 high)
+//          d  [n][k/32]      f16
+//   Q8_0 : qs [n][k/32][32]  i8
+//          d  [n][k/32]      f16
+//   Q4K  : qs [n][k/256][128] u8  (GGML order: byte 32g+l = elem 64g+l | elem 64g+32+l << 4)
+//          hd [n][k/256][16]      (d f16, dmin f16, scales[12]: the first 16 bytes of the GGML block)
+//   Q6K  : ql [n][k/256][128] u8  (GGML order)
+//          qh [n][k/256][64]  u8  (re-ordered, see repack.hip: 8 bytes per 16-byte ql lane)
+//          sc [n][k/256][16]  i8
+//          d  [n][k/256]      f16
+// All planes live in one allocation; each plane starts 256-byte aligned and the
+// allocation carries CQ_TAIL_PAD spare bytes so that a partial tail tile can be
+// read with full-width loads.
+// ---------------------------------------------------------------------------
+#define CQ_TAIL_PAD 4096
+
+struct cq_weight {
+    int dev;
+    int dtype;
+    int64_t n, k;
+    size_t ggml_bytes;   // n * k/block * type_size
+    void *base;          // the single device allocation
+    size_t alloc_bytes;
+    uint8_t *p0;         // qs / ql
+    uint8_t *p1;         // d (Q4_0,Q8_0) / hd (Q4K) / qh (Q6K)
+    uint8_t *p2;         // sc (Q6K)
+    uint8_t *p3;         // d  (Q6K)
+};
+
+// ---------------------------------------------------------------------------
+// Device activation storage used between the quantizer and the matmul kernels
+// (workspace layout).  Same numbers as the GGML activation blocks, split so
+// that int8 values are 16-byte aligned:
+//   Q8K : qs [m][k] i8 ; d [m][k/256] f32 ; bsums [m][k/256][16] i16
+//   Q8_0: qs [m][k] i8 ; d [m][k/32]  f32 (the f16-rounded scale widened) ;
+//         bsum [m][k/32] i32 (sum of the 32 quants, for the Q4_0 "-8" term)
+// ---------------------------------------------------------------------------
+struct cq_act_view {
+    int8_t *qs;
+    float *d;
+    int16_t *bsums;  // Q8K
+    int32_t *bsum32; // Q8_0 / Q8_1
+    uint16_t *s16;   // Q8_1: the block's `s` field (f16 bits)
+};
+
+static inline size_t cq_align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// error plumbing (api.cpp)
+int cq_set_error(int code, const char *fmt, ...);
+#define CQ_HIP_CHECK(expr)                                                                       \
+    do {                                                                                         \
+        hipError_t _e = (expr);                                                                  \
+        if (_e != hipSuccess)                                                                    \
+            return cq_set_error(CQ_ERR_HIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), \
+                                __FILE__, __LINE__);                                             \
+    } while (0)
+
+// ---- launchers implemented in the .hip files -------------------------------
+// repack.hip
+hipError_t cq_launch_repack(const cq_weight *w, const uint8_t *aos_dev, hipStream_t s);   // GGML AoS -> planes
+hipError_t cq_launch_unpack(const cq_weight *w, uint8_t *aos_dev, hipStream_t s);         // planes -> GGML AoS
+// quantize_act.hip
+hipError_t cq_launch_quantize_act_aos(int act_dtype, const float *x, int64_t m, int64_t k, void *dst, hipStream_t s);
+hipError_t cq_launch_quantize_act_ws(int act_dtype, const float *x, const int32_t *row_ids, int64_t m, int64_t k,
+                                     cq_act_view v, hipStream_t s);
+// quantize_weight.hip
+hipError_t cq_launch_quantize_weight(int dtype, const float *src, int64_t nblocks, uint8_t *aos_dev, hipStream_t s);
+// dequantize.hip
+hipError_t cq_launch_dequantize(const cq_weight *w, float *dst32, uint16_t *dst16, hipStream_t s);
+// matvec.hip
+hipError_t cq_launch_matvec(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s);
+hipError_t cq_launch_int_dots(const cq_weight *w, cq_act_view a, int64_t m, int32_t *out_i, int32_t *out_mn,
+                              hipStream_t s);
+// gemm.hip
+bool cq_gemm_supported(const cq_weight *w, int64_t m, int act_dtype);
+hipError_t cq_launch_gemm(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s);
+// moe.hip
+hipError_t cq_launch_silu_mul(const float *a, const float *b, float *h, int64_t count, hipStream_t s);
+hipError_t cq_launch_scatter_add(const float *y, const int32_t *row_ids, const float *weights, int64_t total_rows,
+                                 int64_t hidden, float *ys, int64_t tokens, hipStream_t s);
+
+hipError_t cq_launch_fill_zero(float *p, int64_t count, hipStream_t s);
+
+// ---- small device helpers ---------------------------------------------------
+#if defined(__HIPCC__)
+__device__ __forceinline__ float cq_h2f(uint16_t h) {
+    _Float16 v;
+    __builtin_memcpy(&v, &h, 2);
+    return (float)v;
+}
+__device__ __forceinline__ uint16_t cq_f2h(float f) {  // round-to-nearest-even
+    _Float16 v = (_Float16)f;
+    uint16_t h;
+    __builtin_memcpy(&h, &v, 2);
+    return h;
+}
+// Rust `as i8` / `as u8` / `as i32` on f32: truncate toward zero, saturate, NaN -> 0.
+__device__ __forceinline__ int8_t cq_as_i8(float v) {
+    if (!(v == v)) return 0;
+    if (v <= -128.0f) return -128;
+    if (v >= 127.0f) return 127;
+    return (int8_t)(int)v;
+}
+__device__ __forceinline__ uint8_t cq_as_u8(float v) {
+    if (!(v == v)) return 0;
+    if (v <= 0.0f) return 0;
+    if (v >= 255.0f) return 255;
+    return (uint8_t)(int)v;
+}
+__device__ __forceinline__ int32_t cq_as_i32(float v) {
+    if (!(v == v)) return 0;
+    if (v >= 2147483648.0f) return 2147483647;
+    if (v <= -2147483648.0f) return (-2147483647 - 1);
+    return (int32_t)v;
+}
+// utils.rs:3-5 nearest_int = v.round() as i32 (round half away from zero)
+__device__ __forceinline__ int32_t cq_nearest_int(float v) { return cq_as_i32(roundf(v)); }
+__device__ __forceinline__ int32_t cq_clampi(int32_t v, int32_t lo, int32_t hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+// utils.rs:49-59 on the 12 scale bytes held as three little-endian words
+__device__ __forceinline__ void cq_scale_min_k4(int j, uint32_t u0, uint32_t u1, uint32_t u2, int &sc, int &mn) {
+    const int sh = 8 * (j & 3);
+    if (j < 4) {
+        sc = (u0 >> sh) & 63;
+        mn = (u1 >> sh) & 63;
+    } else {
+        sc = ((u2 >> sh) & 0xF) | (((u0 >> (sh + 6)) & 3) << 4);
+        mn = ((u2 >> (sh + 4)) & 0xF) | (((u1 >> (sh + 6)) & 3) << 4);
+    }
+}
+#endif

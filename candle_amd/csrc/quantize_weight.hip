@@ -1,0 +1,281 @@
+// Weight quantizers on the device: f32 -> GGML blocks (array-of-blocks bytes), the
+// arithmetic of T::from_float in candle-core/src/quantized/k_quants.rs and utils.rs,
+// one thread per block, every f32 operation a single IEEE operation in the reference's
+// order (compiled with -ffp-contract=off).  The reference's CUDA arm copies the tensor to
+// the host and quantizes there (cuda.rs:448-472); the bytes produced here are the same.
+//   Q4_0 k_quants.rs:185-220      Q8_0 :586-615
+//   Q4K  :1252-1311 + utils.rs:201-258 (make_qkx1_quants) + :49-59 (get_scale_min_k4)
+//   Q6K  :1643-1713 + utils.rs:61-198  (make_qx_quants, n=16, nmax=32, rmse_type=1)
+#include "qhip_internal.h"
+
+namespace {
+
+__device__ void store_u16(uint8_t *p, uint16_t v) { p[0] = (uint8_t)(v & 0xff); p[1] = (uint8_t)(v >> 8); }
+
+__global__ void quantize_q4_0(const float *__restrict__ src, int64_t nblocks, uint8_t *__restrict__ out) {
+    const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    const float *x = src + b * 32;
+    float amax = 0.0f, max = 0.0f;
+    for (int j = 0; j < 32; j++) {
+        const float v = x[j];
+        if (amax < fabsf(v)) { amax = fabsf(v); max = v; }
+    }
+    const float d = max / -8.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    uint8_t *y = out + b * 18;
+    store_u16(y, cq_f2h(d));
+    for (int j = 0; j < 16; j++) {
+        const float x0 = x[j] * id;
+        const float x1 = x[16 + j] * id;
+        uint8_t xi0 = cq_as_u8(x0 + 8.5f);
+        uint8_t xi1 = cq_as_u8(x1 + 8.5f);
+        if (xi0 > 15) xi0 = 15;
+        if (xi1 > 15) xi1 = 15;
+        y[2 + j] = (uint8_t)(xi0 | (xi1 << 4));
+    }
+}
+
+__global__ void quantize_q8_0(const float *__restrict__ src, int64_t nblocks, uint8_t *__restrict__ out) {
+    const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    const float *x = src + b * 32;
+    float amax = 0.0f;
+    for (int j = 0; j < 32; j++) amax = fmaxf(amax, fabsf(x[j]));
+    const float d = amax / 127.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    uint8_t *y = out + b * 34;
+    store_u16(y, cq_f2h(d));
+    for (int j = 0; j < 32; j++) y[2 + j] = (uint8_t)cq_as_i8(roundf(x[j] * id));
+}
+
+// utils.rs:201-258
+__device__ void make_qkx1_quants(const float *x, float &out_scale, float &out_min) {
+    const int n = 32, nmax = 15, ntry = 5;
+    uint8_t l[32];
+    for (int i = 0; i < n; i++) l[i] = 0;
+    float min = x[0], max = x[0];
+    for (int i = 1; i < n; i++) {
+        if (x[i] < min) min = x[i];
+        if (x[i] > max) max = x[i];
+    }
+    if (max == min) { out_scale = 0.0f; out_min = 0.0f; return; }
+    min = fminf(min, 0.0f);
+    float iscale = (float)nmax / (max - min);
+    float scale = 1.0f / iscale;
+    for (int t = 0; t < ntry; t++) {
+        float sumlx = 0.0f;
+        int32_t suml2 = 0;
+        bool did_change = false;
+        for (int i = 0; i < n; i++) {
+            const int32_t li = cq_clampi(cq_nearest_int(iscale * (x[i] - min)), 0, nmax);
+            if ((uint8_t)li != l[i]) { l[i] = (uint8_t)li; did_change = true; }
+            sumlx += (x[i] - min) * (float)li;
+            suml2 += li * li;
+        }
+        scale = sumlx / (float)suml2;
+        float sum = 0.0f;
+        for (int i = 0; i < n; i++) sum += x[i] - scale * (float)l[i];
+        min = sum / (float)n;
+        if (min > 0.0f) min = 0.0f;
+        iscale = 1.0f / scale;
+        if (!did_change) break;
+    }
+    out_scale = scale;
+    out_min = -min;
+}
+
+__global__ void quantize_q4k(const float *__restrict__ src, int64_t nblocks, uint8_t *__restrict__ out) {
+    const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    const float *x = src + b * QK_K;
+    uint8_t *y = out + b * 144;
+    float mins[8], scales[8];
+    for (int j = 0; j < 8; j++) make_qkx1_quants(x + 32 * j, scales[j], mins[j]);
+    float max_scale = 0.0f, max_min = 0.0f;
+    for (int j = 0; j < 8; j++) max_scale = fmaxf(scales[j], max_scale);
+    for (int j = 0; j < 8; j++) max_min = fmaxf(mins[j], max_min);
+    const float inv_scale = max_scale > 0.0f ? 63.0f / max_scale : 0.0f;
+    const float inv_min = max_min > 0.0f ? 63.0f / max_min : 0.0f;
+    uint8_t sc12[12];
+    for (int j = 0; j < 12; j++) sc12[j] = 0;
+    for (int j = 0; j < 8; j++) {
+        int32_t lsi = cq_nearest_int(inv_scale * scales[j]);
+        int32_t lmi = cq_nearest_int(inv_min * mins[j]);
+        if (lsi > 63) lsi = 63;
+        if (lmi > 63) lmi = 63;
+        const uint8_t ls = (uint8_t)lsi, lm = (uint8_t)lmi;
+        if (j < 4) {
+            sc12[j] = ls;
+            sc12[j + 4] = lm;
+        } else {
+            sc12[j + 4] = (uint8_t)((ls & 0xF) | ((lm & 0xF) << 4));
+            sc12[j - 4] |= (uint8_t)((ls >> 4) << 6);
+            sc12[j] |= (uint8_t)((lm >> 4) << 6);
+        }
+    }
+    const uint16_t dh = cq_f2h(max_scale / 63.0f);
+    const uint16_t dminh = cq_f2h(max_min / 63.0f);
+    store_u16(y, dh);
+    store_u16(y + 2, dminh);
+    for (int j = 0; j < 12; j++) y[4 + j] = sc12[j];
+    const uint32_t u0 = sc12[0] | (sc12[1] << 8) | (sc12[2] << 16) | ((uint32_t)sc12[3] << 24);
+    const uint32_t u1 = sc12[4] | (sc12[5] << 8) | (sc12[6] << 16) | ((uint32_t)sc12[7] << 24);
+    const uint32_t u2 = sc12[8] | (sc12[9] << 8) | (sc12[10] << 16) | ((uint32_t)sc12[11] << 24);
+    // two 32-element sub-blocks share the 32 output bytes of their 64-element group
+    for (int g = 0; g < 4; g++) {
+        uint8_t lo[32], hi[32];
+        for (int half = 0; half < 2; half++) {
+            const int j = 2 * g + half;
+            int sc, m;
+            cq_scale_min_k4(j, u0, u1, u2, sc, m);
+            const float d = cq_h2f(dh) * (float)sc;
+            uint8_t *dst = half ? hi : lo;
+            if (d != 0.0f) {
+                const float dm = cq_h2f(dminh) * (float)m;
+                for (int ii = 0; ii < 32; ii++)
+                    dst[ii] = (uint8_t)cq_clampi(cq_nearest_int((x[32 * j + ii] + dm) / d), 0, 15);
+            } else {
+                for (int ii = 0; ii < 32; ii++) dst[ii] = 0;
+            }
+        }
+        for (int l = 0; l < 32; l++) y[16 + 32 * g + l] = (uint8_t)(lo[l] | (hi[l] << 4));
+    }
+}
+
+// utils.rs:61-198 specialised to n = 16, nmax = 32, rmse_type = 1 (weights w = x*x; returns after
+// the five refinement passes, utils.rs:168-170).
+__device__ float make_qx_quants_16_32(const float *x, int8_t *ls) {
+    const int n = 16, nmax = 32;
+    float max = 0.0f, amax = 0.0f;
+    for (int i = 0; i < n; i++) {
+        const float ax = fabsf(x[i]);
+        if (ax > amax) { amax = ax; max = x[i]; }
+    }
+    if (amax == 0.0f) {
+        for (int i = 0; i < n; i++) ls[i] = 0;
+        return 0.0f;
+    }
+    const float iscale = -(float)nmax / max;
+    float sumlx = 0.0f, suml2 = 0.0f;
+    for (int i = 0; i < n; i++) {
+        const int32_t l = cq_clampi(cq_nearest_int(iscale * x[i]), -nmax, nmax - 1);
+        ls[i] = (int8_t)(l + nmax);
+        const float w = x[i] * x[i];
+        const float lf = (float)l;
+        sumlx += w * x[i] * lf;
+        suml2 += w * lf * lf;
+    }
+    float scale = sumlx / suml2;
+    float best = scale * sumlx;
+    for (int itry = 0; itry < 3; itry++) {
+        const float is2 = 1.0f / scale;
+        float slx = 0.0f, sl2 = 0.0f;
+        bool changed = false;
+        for (int i = 0; i < n; i++) {
+            const int32_t l = cq_clampi(cq_nearest_int(is2 * x[i]), -nmax, nmax - 1);
+            if (l + nmax != (int32_t)ls[i]) changed = true;
+            const float w = x[i] * x[i];
+            const float lf = (float)l;
+            slx += w * x[i] * lf;
+            sl2 += w * lf * lf;
+        }
+        if (!changed || sl2 == 0.0f || slx * slx <= best * sl2) break;
+        for (int i = 0; i < n; i++) {
+            const int32_t l = cq_nearest_int(is2 * x[i]);
+            ls[i] = (int8_t)(nmax + cq_clampi(l, -nmax, nmax - 1));
+        }
+        sumlx = slx;
+        suml2 = sl2;
+        scale = sumlx / suml2;
+        best = scale * sumlx;
+    }
+    for (int itry = 0; itry < 5; itry++) {
+        int n_changed = 0;
+        for (int i = 0; i < n; i++) {
+            const float w = x[i] * x[i];
+            const int32_t l = (int32_t)ls[i] - nmax;
+            float slx = sumlx - w * x[i] * (float)l;
+            if (slx > 0.0f) {
+                float sl2 = suml2 - w * (float)l * (float)l;
+                const int32_t new_l = cq_clampi(cq_nearest_int(x[i] * sl2 / slx), -nmax, nmax - 1);
+                if (new_l != l) {
+                    slx += w * x[i] * (float)new_l;
+                    sl2 += w * (float)new_l * (float)new_l;
+                    if (sl2 > 0.0f && slx * slx * suml2 > sumlx * sumlx * sl2) {
+                        ls[i] = (int8_t)(nmax + new_l);
+                        sumlx = slx;
+                        suml2 = sl2;
+                        scale = sumlx / suml2;
+                        best = scale * sumlx;
+                        n_changed++;
+                    }
+                }
+            }
+        }
+        if (n_changed == 0) break;
+    }
+    (void)best;
+    return scale;
+}
+
+__global__ void quantize_q6k(const float *__restrict__ src, int64_t nblocks, uint8_t *__restrict__ out) {
+    const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    const float *x = src + b * QK_K;
+    uint8_t *y = out + b * 210;
+    int8_t l[QK_K];
+    float scales[16];
+    float max_scale = 0.0f, max_abs_scale = 0.0f;
+    for (int j = 0; j < 16; j++) {
+        const float scale = make_qx_quants_16_32(x + 16 * j, l + 16 * j);
+        scales[j] = scale;
+        const float a = fabsf(scale);
+        if (a > max_abs_scale) { max_abs_scale = a; max_scale = scale; }
+    }
+    const float iscale = -128.0f / max_scale;
+    const uint16_t dh = cq_f2h(1.0f / iscale);
+    int8_t sc8[16];
+    for (int j = 0; j < 16; j++) {
+        int32_t v = cq_nearest_int(iscale * scales[j]);
+        if (v > 127) v = 127;
+        sc8[j] = (int8_t)v;
+    }
+    for (int j = 0; j < 16; j++) {
+        const float d = cq_h2f(dh) * (float)sc8[j];
+        if (d == 0.0f) continue;
+        for (int ii = 0; ii < 16; ii++) {
+            const int32_t ll = cq_clampi(cq_nearest_int(x[16 * j + ii] / d), -32, 31);
+            l[16 * j + ii] = (int8_t)(ll + 32);
+        }
+    }
+    for (int h = 0; h < 2; h++) {
+        const int j = 128 * h;
+        for (int li = 0; li < 32; li++) {
+            const int8_t q1 = l[j + li] & 0xF, q2 = l[j + li + 32] & 0xF, q3 = l[j + li + 64] & 0xF,
+                         q4 = l[j + li + 96] & 0xF;
+            y[64 * h + li] = (uint8_t)(q1 | (q3 << 4));
+            y[64 * h + li + 32] = (uint8_t)(q2 | (q4 << 4));
+            y[128 + 32 * h + li] = (uint8_t)((l[j + li] >> 4) | ((l[j + li + 32] >> 4) << 2) |
+                                             ((l[j + li + 64] >> 4) << 4) | ((l[j + li + 96] >> 4) << 6));
+        }
+    }
+    for (int j = 0; j < 16; j++) y[192 + j] = (uint8_t)sc8[j];
+    store_u16(y + 208, dh);
+}
+
+}  // namespace
+
+hipError_t cq_launch_quantize_weight(int dtype, const float *src, int64_t nblocks, uint8_t *aos_dev, hipStream_t s) {
+    if (nblocks == 0) return hipSuccess;
+    const int threads = 64;
+    const unsigned grid = (unsigned)((nblocks + threads - 1) / threads);
+    switch (dtype) {
+    case CQ_DTYPE_Q4_0: quantize_q4_0<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
+    case CQ_DTYPE_Q8_0: quantize_q8_0<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
+    case CQ_DTYPE_Q4K: quantize_q4k<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
+    case CQ_DTYPE_Q6K: quantize_q6k<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}

@@ -1,0 +1,155 @@
+// GGML array-of-blocks <-> device planes (and back).  Pure byte permutations:
+// cq_launch_unpack(cq_launch_repack(x)) == x for every input.
+//
+// Replaces the plain host->device copy of cuda::load_quantized
+// (candle-core/src/quantized/cuda.rs:591-612); the inverse serves QStorage::data
+// (mod.rs:118-130).
+#include "qhip_internal.h"
+
+namespace {
+
+// ---- Q4_0: 18-byte blocks {f16 d; u8 qs[16]} --------------------------------
+__global__ void repack_q4_0(const uint8_t *__restrict__ aos, uint8_t *__restrict__ qs, uint16_t *__restrict__ d,
+                            int64_t nblocks, bool inverse) {
+    int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    uint16_t *a16 = (uint16_t *)(aos + b * 18);   // 18*b is even
+    uint16_t *q16 = (uint16_t *)(qs + b * 16);
+    if (!inverse) {
+        d[b] = a16[0];
+        for (int i = 0; i < 8; i++) q16[i] = a16[1 + i];
+    } else {
+        a16[0] = d[b];
+        for (int i = 0; i < 8; i++) a16[1 + i] = q16[i];
+    }
+}
+
+// ---- Q8_0: 34-byte blocks {f16 d; i8 qs[32]} --------------------------------
+__global__ void repack_q8_0(const uint8_t *__restrict__ aos, uint8_t *__restrict__ qs, uint16_t *__restrict__ d,
+                            int64_t nblocks, bool inverse) {
+    int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    uint16_t *a16 = (uint16_t *)(aos + b * 34);
+    uint16_t *q16 = (uint16_t *)(qs + b * 32);
+    if (!inverse) {
+        d[b] = a16[0];
+        for (int i = 0; i < 16; i++) q16[i] = a16[1 + i];
+    } else {
+        a16[0] = d[b];
+        for (int i = 0; i < 16; i++) a16[1 + i] = q16[i];
+    }
+}
+
+// ---- Q4K: 144-byte blocks {f16 d; f16 dmin; u8 scales[12]; u8 qs[128]} ------
+// One thread per 16-byte unit: unit 0 is the header, units 1..8 the nibbles.
+__global__ void repack_q4k(const uint8_t *__restrict__ aos, uint8_t *__restrict__ qs, uint8_t *__restrict__ hd,
+                           int64_t nblocks, bool inverse) {
+    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t b = t / 9;
+    int u = (int)(t - b * 9);
+    if (b >= nblocks) return;
+    uint4 *a = (uint4 *)(aos + b * 144) + u;      // 144 = 9 * 16, base is 256-byte aligned
+    uint4 *p = (u == 0) ? (uint4 *)(hd + b * 16) : (uint4 *)(qs + b * 128) + (u - 1);
+    if (!inverse) *p = *a; else *a = *p;
+}
+
+// ---- Q6K: 210-byte blocks {u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d} -----
+// qh is re-ordered so that the thread that owns ql bytes [16u, 16u+16) of a block
+// finds the high bits of exactly those 32 elements in qh' bytes [8u, 8u+8):
+//   u = 4h + 2t + i  ->  ql byte 64h + 32t + 16i + e  (e < 16)
+//   low  nibble: element 128h + 32t + 16i + e        hi bits = qh[32h + 16i + e] >> 2t
+//   high nibble: element 128h + 64 + 32t + 16i + e   hi bits = qh[32h + 16i + e] >> (2t + 4)
+//   qh'[8u + 4x + c] (x < 2, c < 4) =   lo2(8x + c)       | hi2(8x + c) << 2
+//                                      | lo2(8x + 4 + c) << 4 | hi2(8x + 4 + c) << 6
+// i.e. for the two ql words 2x and 2x+1 of the lane, (H >> {0,2,4,6}) & 0x03030303 lines the
+// two high bits up with each byte of {word 2x low, word 2x high, word 2x+1 low, word 2x+1 high}.
+__global__ void repack_q6k(const uint8_t *__restrict__ aos, uint8_t *__restrict__ ql, uint8_t *__restrict__ qh,
+                           uint8_t *__restrict__ sc, uint16_t *__restrict__ d, int64_t nblocks, bool inverse) {
+    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t b = t / 8;
+    int u = (int)(t & 7);
+    if (b >= nblocks) return;
+    uint8_t *a = (uint8_t *)aos + b * 210;
+    uint8_t *a_ql = a, *a_qh = a + 128, *a_sc = a + 192, *a_d = a + 208;
+    const int h = u >> 2, tt = (u >> 1) & 1, i0 = (u & 1) * 16;
+    uint8_t *pql = ql + b * 128 + 16 * u;
+    uint8_t *pqh = qh + b * 64 + 8 * u;
+    if (!inverse) {
+        for (int e = 0; e < 16; e++) pql[e] = a_ql[16 * u + e];
+        for (int x = 0; x < 2; x++)
+            for (int c = 0; c < 4; c++) {
+                uint8_t s0 = a_qh[32 * h + i0 + 8 * x + c];
+                uint8_t s1 = a_qh[32 * h + i0 + 8 * x + 4 + c];
+                uint8_t v = (uint8_t)(((s0 >> (2 * tt)) & 3) | (((s0 >> (2 * tt + 4)) & 3) << 2) |
+                                      (((s1 >> (2 * tt)) & 3) << 4) | (((s1 >> (2 * tt + 4)) & 3) << 6));
+                pqh[4 * x + c] = v;
+            }
+        if (u == 0) {
+            for (int e = 0; e < 16; e++) sc[b * 16 + e] = a_sc[e];
+            d[b] = (uint16_t)(a_d[0] | (a_d[1] << 8));
+        }
+    } else {
+        for (int e = 0; e < 16; e++) a_ql[16 * u + e] = pql[e];
+        if (u == 0) {
+            for (int e = 0; e < 16; e++) a_sc[e] = sc[b * 16 + e];
+            a_d[0] = (uint8_t)(d[b] & 0xff);
+            a_d[1] = (uint8_t)(d[b] >> 8);
+        }
+        // Each GGML qh byte 32h + j collects 2-bit fields from the two lanes t = 0, 1 that share
+        // (h, i); lane (h, t = 0, i) rebuilds the 16 bytes 32h + 16i + e from both lanes' qh'.
+        if (tt == 0) {
+            const uint8_t *p0 = qh + b * 64 + 8 * u;        // t = 0
+            const uint8_t *p1 = qh + b * 64 + 8 * (u + 2);  // t = 1
+            for (int x = 0; x < 2; x++)
+                for (int c = 0; c < 4; c++) {
+                    uint8_t v0 = p0[4 * x + c], v1 = p1[4 * x + c];
+                    // element e = 8x + c : fields lo2 (bits 0-1) and hi2 (bits 2-3)
+                    a_qh[32 * h + i0 + 8 * x + c] =
+                        (uint8_t)((v0 & 3) | ((v1 & 3) << 2) | (((v0 >> 2) & 3) << 4) | (((v1 >> 2) & 3) << 6));
+                    // element e = 8x + 4 + c : fields at bits 4-5 and 6-7
+                    a_qh[32 * h + i0 + 8 * x + 4 + c] = (uint8_t)(((v0 >> 4) & 3) | (((v1 >> 4) & 3) << 2) |
+                                                                  (((v0 >> 6) & 3) << 4) | (((v1 >> 6) & 3) << 6));
+                }
+        }
+    }
+}
+
+hipError_t launch(const cq_weight *w, uint8_t *aos, bool inverse, hipStream_t s) {
+    const int64_t bs = cq_block_size(w->dtype);
+    const int64_t nblocks = w->n * (w->k / bs);
+    if (nblocks == 0) return hipSuccess;
+    const int threads = 256;
+    switch (w->dtype) {
+    case CQ_DTYPE_Q4_0: {
+        unsigned grid = (unsigned)((nblocks + threads - 1) / threads);
+        repack_q4_0<<<grid, threads, 0, s>>>(aos, w->p0, (uint16_t *)w->p1, nblocks, inverse);
+        break;
+    }
+    case CQ_DTYPE_Q8_0: {
+        unsigned grid = (unsigned)((nblocks + threads - 1) / threads);
+        repack_q8_0<<<grid, threads, 0, s>>>(aos, w->p0, (uint16_t *)w->p1, nblocks, inverse);
+        break;
+    }
+    case CQ_DTYPE_Q4K: {
+        unsigned grid = (unsigned)((nblocks * 9 + threads - 1) / threads);
+        repack_q4k<<<grid, threads, 0, s>>>(aos, w->p0, w->p1, nblocks, inverse);
+        break;
+    }
+    case CQ_DTYPE_Q6K: {
+        unsigned grid = (unsigned)((nblocks * 8 + threads - 1) / threads);
+        repack_q6k<<<grid, threads, 0, s>>>(aos, w->p0, w->p1, w->p2, (uint16_t *)w->p3, nblocks, inverse);
+        break;
+    }
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t cq_launch_repack(const cq_weight *w, const uint8_t *aos_dev, hipStream_t s) {
+    return launch(w, (uint8_t *)aos_dev, false, s);
+}
+hipError_t cq_launch_unpack(const cq_weight *w, uint8_t *aos_dev, hipStream_t s) {
+    return launch(w, aos_dev, true, s);
+}

@@ -1,0 +1,144 @@
+/*
+ * candle_qhip.h - C ABI of the MI355X (gfx950) quantized-matmul library.
+ *
+ * This is the boundary a `Hip` arm of candle's `QStorage` enum binds to: each
+ * entry point names the reference interface it replaces (paths relative to the
+ * candle repository).  Plain pointers and sizes only; every function returns 0
+ * on success or a negative code and leaves a message for cq_last_error().
+ *
+ * Conventions
+ *  - dtype ids are GgmlDType::to_u32 (candle-core/src/quantized/mod.rs:173-190).
+ *  - weights are logical [n, k] row-major, row = k/block consecutive blocks
+ *    (k_quants.rs:1875); activations [m, k] contiguous f32; outputs [m, n] f32.
+ *  - pointers named *_dev are device pointers on the weight's device; work is
+ *    enqueued on `stream` (a hipStream_t, NULL = default stream) with no host
+ *    synchronisation, like the reference's CUDA arm (cuda.rs:478-499).
+ *  - the device layout of a cq_weight is private (re-packed planes), as
+ *    QStorage::data() is "not implemented" for device arms (mod.rs:126-128).
+ *  - no C++ exception or abort crosses this boundary.
+ */
+#ifndef CANDLE_QHIP_H
+#define CANDLE_QHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* GgmlDType ids handled by this library (mod.rs:133-190). */
+enum {
+    CQ_DTYPE_Q4_0 = 2,
+    CQ_DTYPE_Q8_0 = 8,
+    CQ_DTYPE_Q8_1 = 9,  /* activation format only */
+    CQ_DTYPE_Q4K = 12,
+    CQ_DTYPE_Q6K = 14,
+    CQ_DTYPE_Q8K = 15   /* activation format only */
+};
+
+/* error codes */
+enum {
+    CQ_OK = 0,
+    CQ_ERR_INVALID = -1,     /* bad argument (shape, dtype, null pointer)      */
+    CQ_ERR_UNSUPPORTED = -2, /* dtype / combination not handled by this build  */
+    CQ_ERR_HIP = -3,         /* a HIP runtime call failed                      */
+    CQ_ERR_WORKSPACE = -4    /* workspace missing or too small                 */
+};
+
+/* flags of cq_qmatmul / cq_workspace_bytes */
+enum {
+    CQ_FLAG_AUTO = 0,
+    CQ_FLAG_FORCE_MATVEC = 1, /* row-streaming kernel whatever m is (A/B runs; replaces cuda.rs:22-26 set_force_dmmv) */
+    CQ_FLAG_FORCE_GEMM = 2,   /* int8-MFMA tile kernel whatever m is                                                  */
+    CQ_FLAG_ACT_Q8_1 = 4      /* K-quant weights x Q8_1 activations (the reference CUDA formulation, cuda.rs:322-326)
+                                 instead of the CPU formulation's Q8K; not bit-comparable with the CPU QMatMul        */
+};
+
+typedef struct cq_weight cq_weight;
+
+/* ---- library / device ---------------------------------------------------- */
+/* Number of usable HIP devices; 0 when no GPU is visible (Device::new_cuda's role, device.rs). */
+int cq_device_count(void);
+/* Thread-local message of the last failing call on this thread (candle_core::Error's role). */
+const char *cq_last_error(void);
+const char *cq_version(void);
+
+/* ---- GgmlDType helpers (mod.rs:211-246) ---------------------------------- */
+int64_t cq_block_size(int ggml_dtype); /* GgmlDType::block_size, 0 if unknown */
+int64_t cq_type_size(int ggml_dtype);  /* GgmlDType::type_size,  0 if unknown */
+/* The activation block type a weight type is contracted with on the CPU path
+ * (GgmlType::VecDotType, k_quants.rs:160,565,1155,1569); -1 if unknown. */
+int cq_vec_dot_type(int ggml_dtype);
+
+/* ---- weight storage ------------------------------------------------------ */
+/* cuda::load_quantized (cuda.rs:591-612; funnel ggml_file.rs:120-135): host GGML blocks of a
+ * [n, k] matrix -> device storage.  Uploads and re-packs; k % block_size must be 0. */
+int cq_weight_create(int dev, int ggml_dtype, const void *host_ggml_blocks, size_t nbytes,
+                     int64_t n, int64_t k, cq_weight **out);
+/* QCudaStorage::zeros (cuda.rs:368-381): zero-filled storage for n*k elements. */
+int cq_weight_zeros(int dev, int ggml_dtype, int64_t n, int64_t k, cq_weight **out);
+/* QCudaStorage::quantize (cuda.rs:448-472): f32 [n*k] on the device -> this storage.  The
+ * reference copies to the host and runs T::from_float there; here the same arithmetic runs in
+ * a HIP kernel and yields the same bytes. */
+int cq_weight_quantize(cq_weight *w, const float *src_dev, void *stream);
+/* QCudaStorage::dequantize / dequantize_f16 (cuda.rs:391-446): dst has n*k elements. */
+int cq_weight_dequantize(const cq_weight *w, float *dst_dev, void *stream);
+int cq_weight_dequantize_f16(const cq_weight *w, uint16_t *dst_dev, void *stream);
+/* Inverse re-pack: the exact GGML bytes back on the host (QStorage::data, mod.rs:118-130; what
+ * gguf_file::write needs).  Synchronises the device. */
+int cq_weight_to_ggml(const cq_weight *w, void *host_dst, size_t nbytes);
+/* QCudaStorage::storage_size_in_bytes (cuda.rs:474-476): unpadded GGML byte size. */
+size_t cq_weight_size_in_bytes(const cq_weight *w);
+int cq_weight_dtype(const cq_weight *w);                        /* QCudaStorage::dtype  (cuda.rs:383) */
+int cq_weight_device(const cq_weight *w);                       /* QCudaStorage::device (cuda.rs:387) */
+int cq_weight_shape(const cq_weight *w, int64_t *n, int64_t *k); /* QTensor::shape (mod.rs:357)       */
+void cq_weight_destroy(cq_weight *w);                           /* Drop of the storage                */
+
+/* ---- activation quantizer ------------------------------------------------ */
+/* T::VecDotType::from_float over m rows (k_quants.rs:1857-1862; launch precedent cuda.rs:46-67).
+ * act_dtype in {Q8_0, Q8_1, Q8K}.  dst receives m * k/block GGML blocks in the reference's
+ * struct layout (k_quants.rs:78-93, 148-155), byte-comparable with the CPU path. */
+size_t cq_act_bytes(int act_dtype, int64_t m, int64_t k);
+int cq_quantize_act(int dev, int act_dtype, const float *x_dev, int64_t m, int64_t k,
+                    void *dst_blocks_dev, void *stream);
+
+/* ---- matmul -------------------------------------------------------------- */
+/* Scratch the caller must provide to cq_qmatmul for m activation rows (the reference allocates
+ * its quantized-activation buffer per call, cuda.rs:249-252, 322-325). */
+size_t cq_workspace_bytes(const cq_weight *w, int64_t m, int flags);
+/* QCudaStorage::fwd (cuda.rs:478-499) = <QTensor as CustomOp1>::cuda_fwd (mod.rs:514-524):
+ * y[m, n] = x[m, k] . W[n, k]^T with x quantized to W's VecDotType first (k_quants.rs:1842-1883).
+ * x contiguous f32; m = product of the leading dims of the input tensor. */
+int cq_qmatmul(const cq_weight *w, const float *x_dev, int64_t m, float *y_dev, int flags,
+               void *workspace_dev, size_t workspace_bytes, void *stream);
+/* Debug/verification: the per-block integer dot products the f32 result is combined from
+ * (k_quants.rs:1221-1241 for Q4K, :1615-1633 for Q6K, :245-250 / :640-645 for Q4_0/Q8_0).
+ * out_i[(r*n + c)*kb + b] = I_b; out_mn likewise = sum_j bsums_j*min_j (Q4K only, else NULL). */
+int cq_qmatmul_int_dots(const cq_weight *w, const float *x_dev, int64_t m, int32_t *out_i_dev,
+                        int32_t *out_mn_dev, void *workspace_dev, size_t workspace_bytes,
+                        void *stream);
+
+/* ---- grouped experts (MoE FFN) ------------------------------------------- */
+/* One QMatMul per expert over gathered rows, as MlpOrMoe::forward does sequentially
+ * (candle-transformers/src/models/quantized_llama.rs:117-135): for expert e and p in
+ * [offsets[e], offsets[e+1]):  y[p, :] = x[row_ids[p], :] . W_e^T   (row_ids == NULL: x[p, :]).
+ * All experts share dtype and shape.  y has offsets[n_experts] rows. */
+size_t cq_grouped_workspace_bytes(const cq_weight *const *experts, int n_experts, int64_t total_rows,
+                                  int flags);
+int cq_qmatmul_grouped(const cq_weight *const *experts, int n_experts, const float *x_dev,
+                       const int32_t *row_ids_dev, const int32_t *offsets_host, float *y_dev,
+                       int flags, void *workspace_dev, size_t workspace_bytes, void *stream);
+/* h[i] = silu(a[i]) * b[i], silu(v) = v / (1 + exp(-v))  (Mlp::forward, quantized_llama.rs:56-63;
+ * candle-core/src/op.rs:607-609). */
+int cq_silu_mul(int dev, const float *a_dev, const float *b_dev, float *h_dev, int64_t count, void *stream);
+/* ys[row_ids[p], :] += weights[p] * y[p, :] for p in expert order (broadcast_mul + index_add,
+ * quantized_llama.rs:132-134; cpu_backend/mod.rs:619-653).  Each destination element is summed in
+ * increasing p, which is increasing expert index, like the reference's sequential loop. */
+int cq_moe_scatter_add(int dev, const float *y_dev, const int32_t *row_ids_dev, const float *weights_dev,
+                       int64_t total_rows, int64_t hidden, float *ys_dev, int64_t tokens, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CANDLE_QHIP_H */

@@ -1,0 +1,277 @@
+"""Parity of the HIP path (through the C ABI) against the CPU oracle on identical seeded inputs.
+
+Bars (BASELINE north star): quantized activation blocks and per-block integer dot products
+bit-exact; f32 outputs within relative L2 1e-4 and max-abs <= 1e-3 * ||row||_2.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+from oracle import cpu_oracle as orc  # noqa: E402  (checker only)
+
+REL_L2_TOL = 1e-4       # north star: relative L2 error of the f32 output
+MAX_ABS_FACTOR = 1e-3   # north star: max-abs <= 1e-3 * ||row||_2
+
+
+@pytest.fixture(scope="module")
+def qh():
+    from candle_amd import qhip
+    qhip.load()
+    assert qhip.load().cq_device_count() >= 1, "no HIP device visible"
+    return qhip
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def check_f32(got: np.ndarray, want: np.ndarray):
+    got = got.astype(np.float64).reshape(want.shape)
+    want64 = want.astype(np.float64)
+    for r in range(want.shape[0]):
+        nrm = np.linalg.norm(want64[r])
+        err = np.linalg.norm(got[r] - want64[r])
+        assert err <= REL_L2_TOL * max(nrm, 1e-30), (r, err / max(nrm, 1e-30))
+        assert np.abs(got[r] - want64[r]).max() <= MAX_ABS_FACTOR * max(nrm, 1e-30), r
+
+
+def make_inputs(seed, m, k, n, wscale=0.02, outliers=False):
+    rng = np.random.default_rng(seed)
+    w = (rng.standard_normal((n, k)) * wscale).astype(np.float32)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    if outliers:  # 1% of positions at +-8 sigma (BASELINE config 3)
+        idx = rng.choice(x.size, size=max(1, x.size // 100), replace=False)
+        x.ravel()[idx] = np.where(rng.random(idx.size) < 0.5, -8.0, 8.0).astype(np.float32)
+    return w, x
+
+
+WEIGHT_DTYPES = [orc.Q4_0, orc.Q8_0, orc.Q4K, orc.Q6K]
+
+
+# ------------------------------------------------------------ activation quantizers ----
+def _act_cases(k):
+    rng = np.random.default_rng(k)
+    x = rng.standard_normal((5, k)).astype(np.float32)
+    x[1] *= 1e-3
+    x[2] = 0.0                                    # all-zero blocks
+    x[3, ::7] = 8.0; x[3, 3::11] = -8.0           # ties on |x| with both signs, outliers
+    x[4] = (np.arange(k, dtype=np.float32) - k / 2) / 64.0  # ramp with exact .5 rounding cases
+    return x
+
+
+@pytest.mark.parametrize("act", [orc.Q8_0, orc.Q8_1, orc.Q8K])
+@pytest.mark.parametrize("k", [256, 4096, 11008])
+def test_quantize_act_bit_exact(qh, act, k):
+    x = _act_cases(k)
+    got = qh.quantize_act(act, dev(x)).cpu().numpy()
+    want = np.concatenate([orc.quantize(act, x[r]) for r in range(x.shape[0])])
+    assert got.size == want.size
+    assert np.array_equal(got, want), np.flatnonzero(got != want)[:10]
+
+
+def test_quantize_act_tie_first_index(qh):
+    x = np.zeros((2, 256), np.float32)
+    x[0, 200] = -3.0; x[0, 13] = 3.0      # first max is +3 at 13 -> iscale < 0
+    x[1, 200] = 3.0; x[1, 13] = -3.0
+    got = qh.quantize_act(orc.Q8K, dev(x)).cpu().numpy()
+    want = np.concatenate([orc.quantize(orc.Q8K, x[r]) for r in range(2)])
+    assert np.array_equal(got, want)
+
+
+def test_quantize_act_rejects_bad_k(qh):
+    with pytest.raises(qh.QHipError):
+        qh.quantize_act(orc.Q8K, torch.zeros((1, 128), device="cuda"))
+
+
+# ---------------------------------------------------------------- storage round trips ----
+@pytest.mark.parametrize("dt", WEIGHT_DTYPES)
+@pytest.mark.parametrize("n,k", [(3, 512), (37, 1024), (5, 11008)])
+def test_repack_roundtrip_and_dequantize(qh, dt, n, k):
+    w, _ = make_inputs(n * k + dt, 1, k, n)
+    blocks = orc.quantize(dt, w)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    assert qw.dtype == dt and qw.shape == (n, k) and qw.size_in_bytes == blocks.size
+    assert np.array_equal(qw.to_ggml(), blocks)
+    want = orc.dequantize(dt, blocks).reshape(n, k)
+    got = qw.dequantize().cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    got16 = qw.dequantize_f16().cpu().numpy()
+    assert np.array_equal(got16.view(np.uint16), want.astype(np.float16).view(np.uint16))
+
+
+def test_repack_roundtrip_random_bytes(qh):
+    # the re-pack is a byte permutation: any byte pattern must survive, not only valid quantizations
+    rng = np.random.default_rng(3)
+    for dt in WEIGHT_DTYPES:
+        n, k = 4, 768
+        blocks = rng.integers(0, 256, size=n * k // orc.BLOCK_SIZE[dt] * orc.TYPE_SIZE[dt], dtype=np.uint8)
+        qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+        assert np.array_equal(qw.to_ggml(), blocks)
+
+
+@pytest.mark.parametrize("dt", WEIGHT_DTYPES)
+def test_weight_quantize_on_device_bit_exact(qh, dt):
+    rng = np.random.default_rng(dt)
+    n, k = 24, 1024
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    w[0] = 0.0                          # all-zero blocks
+    w[1, :256] = 0.5                    # constant sub-blocks (max == min)
+    w[2] = np.linspace(-1, 1, k)        # ramp
+    w[3, ::2] = -w[3, 1::2]             # |x| ties
+    qw = qh.QWeight.zeros(dt, n, k)
+    qw.quantize_(dev(w))
+    assert np.array_equal(qw.to_ggml(), orc.quantize(dt, w))
+
+
+def test_weight_create_rejects_bad_shapes(qh):
+    with pytest.raises(qh.QHipError):
+        qh.QWeight.from_ggml(orc.Q4K, np.zeros(144, np.uint8), 1, 128)      # k not a block multiple
+    with pytest.raises(qh.QHipError):
+        qh.QWeight.from_ggml(orc.Q4K, np.zeros(100, np.uint8), 1, 256)      # byte size mismatch
+    with pytest.raises(qh.QHipError):
+        qh.QWeight.from_ggml(5, np.zeros(144, np.uint8), 1, 256)            # unknown dtype
+
+
+# ------------------------------------------------------------- integer block dots ----
+@pytest.mark.parametrize("dt", WEIGHT_DTYPES)
+@pytest.mark.parametrize("m,k,n", [(3, 512, 37), (1, 11008, 9), (2, 4096, 16)])
+def test_int_dots_bit_exact(qh, dt, m, k, n):
+    w, x = make_inputs(1000 + dt + k, m, k, n, outliers=True)
+    blocks = orc.quantize(dt, w)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    oi, om = qh.qmatmul_int_dots(qw, dev(x))
+    acts = np.concatenate([orc.quantize(orc.VEC_DOT_TYPE[dt], x[r]) for r in range(m)])
+    wi, wm = orc.block_int_dots(dt, acts, m, blocks, n, k)
+    assert np.array_equal(oi.cpu().numpy(), wi)
+    if dt == orc.Q4K:
+        assert np.array_equal(om.cpu().numpy(), wm)
+
+
+# ----------------------------------------------------------------- f32 results ----
+@pytest.mark.parametrize("dt,m,k,n", [
+    (orc.Q4_0, 1, 4096, 4096),     # config 0
+    (orc.Q4K, 1, 4096, 4096),      # config 1: q/k/v/o
+    (orc.Q4K, 1, 4096, 11008),     # config 1: gate/up (headline matvec)
+    (orc.Q6K, 1, 11008, 4096),     # config 1: down
+    (orc.Q6K, 1, 4096, 2048),      # config 1: lm_head rows (a 2048-row slice of the 32000)
+    (orc.Q8_0, 1, 4096, 4096),
+    (orc.Q4_0, 3, 64, 4),          # smallest shapes of the reference's tests
+    (orc.Q4K, 5, 256, 3),
+])
+def test_matvec_matches_oracle(qh, dt, m, k, n):
+    w, x = make_inputs(7 * dt + k + n, m, k, n)
+    blocks = orc.quantize(dt, w)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    got = qh.qmatmul(qw, dev(x), qh.FLAG_FORCE_MATVEC).cpu().numpy()
+    check_f32(got, orc.matmul(dt, x, blocks, n))
+
+
+@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q8_0])
+@pytest.mark.parametrize("m", [2, 4, 8, 16])
+@pytest.mark.parametrize("k,n", [(4096, 4096), (4096, 11008)])
+def test_small_batch_matches_oracle(qh, dt, m, k, n):
+    """BASELINE config 2: M in {2,4,8,16} on the decode shapes."""
+    w, x = make_inputs(dt + m + n, m, k, n)
+    blocks = orc.quantize(dt, w)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    got = qh.qmatmul(qw, dev(x)).cpu().numpy()
+    check_f32(got, orc.matmul(dt, x, blocks, n))
+
+
+def test_reference_goldens_through_hip(qh, goldens, seeded_inputs):
+    # quantized_tests.rs:49-64 and :109-129 (Q4_0, m=3, k=64, n=4)
+    m, k, n = 3, 64, 4
+    lhs = np.arange(m * k, dtype=np.float32).reshape(m, k)
+    rhs = np.arange(k * n, dtype=np.float32).reshape(n, k)
+    qw = qh.QWeight.from_ggml(orc.Q4_0, orc.quantize(orc.Q4_0, rhs), n, k)
+    got = qh.qmatmul(qw, dev(lhs)).cpu().numpy()
+    assert np.round(got).ravel().tolist() == goldens["q4_0_matmul_m3_k64_n4"]["rounded"]
+    lhs = (np.arange(m * k, dtype=np.float32) - np.float32(m * k) / 2).reshape(m, k)
+    rhs = (np.arange(k * n, dtype=np.float32) - np.float32(k * n) / np.float32(3.0)).reshape(n, k)
+    qw = qh.QWeight.from_ggml(orc.Q4_0, orc.quantize(orc.Q4_0, rhs), n, k)
+    got = qh.qmatmul(qw, dev(lhs)).cpu().numpy()
+    assert np.round(got).ravel().tolist() == goldens["q4_0_matmul_neg_m3_k64_n4"]["rounded"]
+    # quantized_tests.rs:1051-1151 (seeded m=11, k=512, n=21), weights quantized on the device
+    g = goldens["seeded_matmul_m11_k512_n21"]
+    lhs, rhs = seeded_inputs
+    for name, dt in (("q4k", orc.Q4K), ("q6k", orc.Q6K)):
+        qw = qh.QWeight.zeros(dt, 21, 512).quantize_(dev(rhs))
+        out = qh.qmatmul(qw, dev(lhs)).cpu().numpy().ravel()
+        spot = [float(np.round(np.float32(1000.0) * out[i]) / np.float32(1000.0)) for i in g["flat_indices"]]
+        assert spot == [float(np.float32(v)) for v in g[name]], (name, spot)
+
+
+@pytest.mark.parametrize("dt", WEIGHT_DTYPES)
+def test_batch_invariance(qh, dt, seeded_inputs):
+    """quantized_tests.rs:181-216: a row's result does not depend on how many rows are stacked."""
+    lhs, rhs = seeded_inputs
+    lhs, rhs = lhs[:2, :256], rhs[:6, :256]
+    qw = qh.QWeight.from_ggml(dt, orc.quantize(dt, rhs), 6, 256)
+    mm = qh.qmatmul(qw, dev(lhs), qh.FLAG_FORCE_MATVEC).cpu().numpy()
+    for reps in (2, 3, 6):
+        mmr = qh.qmatmul(qw, dev(np.concatenate([lhs] * reps)), qh.FLAG_FORCE_MATVEC).cpu().numpy()
+        for r in range(reps):
+            assert np.array_equal(mmr[2 * r:2 * r + 2], mm)
+
+
+def test_forward_shape_and_errors(qh):
+    w, x = make_inputs(5, 6, 256, 8)
+    qw = qh.QWeight.from_ggml(orc.Q4K, orc.quantize(orc.Q4K, w), 8, 256)
+    x3 = dev(x.reshape(2, 3, 256))
+    y = qh.qmatmul(qw, x3)
+    assert tuple(y.shape) == (2, 3, 8)                       # last dim replaced by n (mod.rs:483-489)
+    assert torch.equal(y.reshape(6, 8), qh.qmatmul(qw, dev(x)))
+    with pytest.raises(qh.QHipError):                        # mod.rs:485-487
+        qh.qmatmul(qw, torch.zeros((2, 512), device="cuda"))
+    with pytest.raises(qh.QHipError):                        # mod.rs:480-482
+        qh.qmatmul(qw, torch.zeros((256,), device="cuda"))
+    with pytest.raises(qh.QHipError):                        # mod.rs:474-476
+        qh.qmatmul(qw, torch.zeros((256, 4), device="cuda").t())
+    assert tuple(qh.qmatmul(qw, torch.zeros((0, 256), device="cuda")).shape) == (0, 8)
+
+
+# ------------------------------------------------------------------------- MoE ----
+def test_moe_ffn_matches_oracle(qh):
+    """Mixtral-shaped expert FFN at reduced width: routed top-2, per-expert gathered QMatMul,
+    silu(w1 x) * w3 x, w2, scaled scatter-add (quantized_llama.rs:75-143)."""
+    rng = np.random.default_rng(23)
+    tokens, hidden, ffn, n_e, top_k = 24, 512, 1024, 8, 2
+    xs = rng.standard_normal((tokens, hidden)).astype(np.float32)
+    logits = rng.standard_normal((tokens, n_e)).astype(np.float32)
+    offsets, row_ids, weights = orc.moe_route(orc.softmax_last_dim(logits), top_k)
+    w1 = [orc.quantize(orc.Q4K, (rng.standard_normal((ffn, hidden)) * 0.05).astype(np.float32)) for _ in range(n_e)]
+    w3 = [orc.quantize(orc.Q4K, (rng.standard_normal((ffn, hidden)) * 0.05).astype(np.float32)) for _ in range(n_e)]
+    w2 = [orc.quantize(orc.Q6K, (rng.standard_normal((hidden, ffn)) * 0.05).astype(np.float32)) for _ in range(n_e)]
+    want = orc.moe_ffn(orc.Q4K, orc.Q6K, w1, w2, w3, hidden, ffn, xs, offsets, row_ids, weights)
+    q1 = [qh.QWeight.from_ggml(orc.Q4K, b, ffn, hidden) for b in w1]
+    q3 = [qh.QWeight.from_ggml(orc.Q4K, b, ffn, hidden) for b in w3]
+    q2 = [qh.QWeight.from_ggml(orc.Q6K, b, hidden, ffn) for b in w2]
+    x_d, rid_d, wt_d = dev(xs), dev(row_ids), dev(weights)
+    h1 = qh.qmatmul_grouped(q1, x_d, rid_d, offsets)
+    h3 = qh.qmatmul_grouped(q3, x_d, rid_d, offsets)
+    h = qh.silu_mul(h1, h3)
+    y = qh.qmatmul_grouped(q2, h, None, offsets)
+    ys = qh.moe_scatter_add(y, rid_d, wt_d, tokens).cpu().numpy()
+    # Stage by stage against the oracle.  The second matmul re-quantizes h; a 1-ulp difference
+    # between the device expf and libm's can move one int8 activation across a rounding boundary
+    # (an error of ~1e-3 of that row), so stage 3 feeds the oracle the device's own h.
+    h1n, h3n, hn, yn = (t.cpu().numpy() for t in (h1, h3, h, y))
+    for e in range(n_e):
+        sl = slice(offsets[e], offsets[e + 1])
+        if sl.start == sl.stop:
+            continue
+        cur = xs[row_ids[sl]]
+        check_f32(h1n[sl], orc.matmul(orc.Q4K, cur, w1[e], ffn))
+        check_f32(h3n[sl], orc.matmul(orc.Q4K, cur, w3[e], ffn))
+        check_f32(yn[sl], orc.matmul(orc.Q6K, hn[sl], w2[e], hidden))
+    silu = h1n.astype(np.float64) / (1.0 + np.exp(-h1n.astype(np.float64))) * h3n
+    assert np.abs(hn - silu).max() <= 1e-6 * np.abs(silu).max()
+    acc = np.zeros((tokens, hidden), np.float32)
+    for p in range(offsets[-1]):               # sequential index_add in expert order
+        acc[row_ids[p]] += yn[p] * weights[p]
+    assert np.array_equal(ys, acc)
+    # end to end: only as loose as the re-quantization effect described above
+    assert np.linalg.norm(ys - want) / np.linalg.norm(want) < 5e-3
