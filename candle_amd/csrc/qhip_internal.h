@@ -105,6 +105,10 @@ __device__ __forceinline__ float cq_h2f(uint16_t h) {
     return (float)v;
 }
 __device__ __forceinline__ uint16_t cq_f2h(float f) {  // round-to-nearest-even
+    // Keep the f32 value in a register of its own: otherwise the compiler folds a preceding
+    // multiply into one mixed-precision fma (x*c + 0 -> f16), which skips the f32 rounding step
+    // and turns a -0.0 product into +0.0.
+    asm volatile("" : "+v"(f));
     _Float16 v = (_Float16)f;
     uint16_t h;
     __builtin_memcpy(&h, &v, 2);
