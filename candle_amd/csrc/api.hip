@@ -1,6 +1,7 @@
 // C ABI of libcandle_qhip (declarations and reference citations: include/candle_qhip.h).
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <new>
@@ -22,6 +23,12 @@ extern "C" const char *cq_last_error(void) { return g_err; }
 extern "C" const char *cq_version(void) { return "candle_qhip 0.1 (gfx950)"; }
 
 extern "C" int cq_device_count(void) {
+    static bool env_read = false;
+    if (!env_read) {  // A/B switch for tuning runs: waves per workgroup of the fused decode kernel
+        env_read = true;
+        const char *e = getenv("CQ_MATVEC_WAVES");
+        if (e && *e) cq_matvec_set_waves(atoi(e));
+    }
     int n = 0;
     if (hipGetDeviceCount(&n) != hipSuccess) {
         (void)hipGetLastError();
@@ -294,9 +301,15 @@ extern "C" int cq_qmatmul(const cq_weight *w, const float *x_dev, int64_t m, flo
     const int act = act_dtype_for(w, flags);
     CQ_HIP_CHECK(hipSetDevice(w->dev));
     hipStream_t s = (hipStream_t)stream;
+    // decode (one activation row): a single launch that quantizes x in its prologue
+    if (m == 1 && !(flags & (CQ_FLAG_REUSE_ACT | CQ_FLAG_FORCE_GEMM | CQ_FLAG_STAGED_ACT | CQ_FLAG_ACT_Q8_1)) &&
+        cq_matvec_fused_supported(w)) {
+        CQ_HIP_CHECK(cq_launch_matvec_fused(w, x_dev, y_dev, s));
+        return CQ_OK;
+    }
     cq_act_view v;
     act_ws_layout(act, m, w->k, (uint8_t *)ws, &v);
-    CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, nullptr, m, w->k, v, s));
+    if (!(flags & CQ_FLAG_REUSE_ACT)) CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, nullptr, m, w->k, v, s));
     bool use_gemm = false;
     if (flags & CQ_FLAG_FORCE_GEMM) {
         if (!cq_gemm_supported(w, m, act))

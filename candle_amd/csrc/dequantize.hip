@@ -83,8 +83,7 @@ __global__ void dequant_q6k(const uint8_t *__restrict__ ql, const uint8_t *__res
     const uint2 hh = *(const uint2 *)(qh + u * 8);
     const float d = cq_h2f(dpl[b]);
     // low nibbles: elements 128h + 32t + i0 + e, one 16-element scale group; high nibbles: +64
-    const int js = 8 * h + 2 * t + (i0 >> 4);
-    const float s_lo = (float)sc[b * 16 + js], s_hi = (float)sc[b * 16 + js + 4];
+    const float s_lo = (float)sc[u * 2], s_hi = (float)sc[u * 2 + 1];  // re-packed: the lane's two scales
     const uint32_t w[4] = {q.x, q.y, q.z, q.w};
     const uint32_t hw[2] = {hh.x, hh.y};
     const int64_t base = b * 256 + 128 * h + 32 * t + i0;

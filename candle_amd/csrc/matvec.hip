@@ -1,51 +1,62 @@
-// Decode matvec: y[m, n] = sum_k W[n, k] * x[m, k] for a few activation rows (m <= 4 per
-// launch), weights streamed once from HBM.  Replaces the reference's MMVQ kernels
-// (candle-kernels/src/quantized.cu:2626-2698, launched from quantized/cuda.rs:227-295) with the
-// CPU formulation's arithmetic (k_quants.rs:237-254, :631-649, :1171-1250, :1585-1641):
-// integer block dots against Q8_0 / Q8K activations, then f32 scales.
+// Decode matvec: y[m, n] = sum_k W[n, k] * x[m, k] for a few activation rows, weights streamed
+// once from HBM.  Replaces the reference's MMVQ kernels (candle-kernels/src/quantized.cu:2626-2698,
+// launched from quantized/cuda.rs:227-295) with the CPU formulation's arithmetic
+// (k_quants.rs:237-254, :631-649, :1171-1250, :1585-1641): integer block dots against Q8_0 / Q8K
+// activations, then f32 scales.
 //
 // Work split: a "unit" is one 16-byte lane of a row's main plane (32 elements for Q4_0, Q4K and
 // Q6K, 16 for Q8_0).  A wave walks one row 64 units (1 KiB, eight 128-byte lines) at a time;
 // nibbles are split in registers and contracted with v_dot4_i32_i8; the lane sums are reduced
-// with DPP.  Activations are staged once per workgroup in LDS, permuted so that lane l of a
-// chunk reads its operands at l * 16 bytes (no bank conflicts).
+// with DPP.  Quantized activations sit in LDS, permuted so that lane l of a chunk reads its
+// operands at l * 16 bytes (no bank conflicts).
+//
+// Two kernels:
+//   fused_kernel  (m == 1): one launch per QMatMul call.  Each wave first issues the loads of its
+//       first weight row, then the workgroup quantizes the f32 activation row into LDS
+//       (BlockQ8K / BlockQ8_0::from_float, bit-identical to quantize_act.hip), then rows are
+//       processed with the next row's loads in flight (register double buffering).
+//   staged_kernel (m <= 4 rows per launch): activations come from the workspace written by the
+//       stand-alone quantizer.
 #include "qhip_internal.h"
 
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kWaves = kThreads / 64;
-
 template <int DT> struct Geo;
-template <> struct Geo<CQ_DTYPE_Q4_0> { static constexpr int kElems = 32; static constexpr bool kHi = true;  static constexpr int kAux = 1; };
-template <> struct Geo<CQ_DTYPE_Q8_0> { static constexpr int kElems = 16; static constexpr bool kHi = false; static constexpr int kAux = 0; };
-template <> struct Geo<CQ_DTYPE_Q4K>  { static constexpr int kElems = 32; static constexpr bool kHi = true;  static constexpr int kAux = 1; };
-template <> struct Geo<CQ_DTYPE_Q6K>  { static constexpr int kElems = 32; static constexpr bool kHi = true;  static constexpr int kAux = 2; };
+template <> struct Geo<CQ_DTYPE_Q4_0> { static constexpr int kElems = 32; static constexpr bool kHi = true;  static constexpr int kUnitsPerBlock = 1; static constexpr bool kActK = false; };
+template <> struct Geo<CQ_DTYPE_Q8_0> { static constexpr int kElems = 16; static constexpr bool kHi = false; static constexpr int kUnitsPerBlock = 2; static constexpr bool kActK = false; };
+template <> struct Geo<CQ_DTYPE_Q4K>  { static constexpr int kElems = 32; static constexpr bool kHi = true;  static constexpr int kUnitsPerBlock = 8; static constexpr bool kActK = true; };
+template <> struct Geo<CQ_DTYPE_Q6K>  { static constexpr int kElems = 32; static constexpr bool kHi = true;  static constexpr int kUnitsPerBlock = 8; static constexpr bool kActK = true; };
 
-// LDS bytes of one staged activation row with `units` units.
-template <int DT> __host__ __device__ constexpr size_t lds_row_bytes(int64_t units) {
-    return (size_t)units * (16 + (Geo<DT>::kHi ? 16 : 0) + 4 + 4 * Geo<DT>::kAux);
+// ---------------------------------------------------------------------------------------------
+// LDS image of one quantized activation row:
+//   lo [units] int4, hi [units] int4 (nibble types), d [blocks] f32,
+//   bs: Q8K activations: bsums [blocks][16] i16 ; Q8_0 activations: sum of the 32 quants [blocks] i32
+// ---------------------------------------------------------------------------------------------
+template <int DT> __host__ __device__ constexpr int64_t act_blocks(int64_t k) { return Geo<DT>::kActK ? k / 256 : k / 32; }
+template <int DT> __host__ __device__ constexpr size_t lds_row_bytes(int64_t k) {
+    const int64_t units = k / Geo<DT>::kElems;
+    return (size_t)units * (Geo<DT>::kHi ? 32 : 16) + (size_t)act_blocks<DT>(k) * (Geo<DT>::kActK ? 4 + 32 : 4 + 4);
 }
 
+// Byte offsets from the start of dynamic LDS (plain integers: every access below is then a
+// ds_read / ds_write on the one LDS base pointer, never a generic-address access).
 struct LdsRow {
-    const int4 *lo;   // [units]
-    const int4 *hi;   // [units]   (types with two nibble planes)
-    const float *ad;  // [units]   activation scale of the unit's block
-    const int *s0;    // [units]   Q4_0: sum of the block's quants; Q4K: bsums of the lane's sub-block pair;
-                      //           Q6K: bsums of the low-nibble group
-    const int *s1;    // [units]   Q6K: bsums of the high-nibble group
+    uint32_t lo, hi, d, bs;
 };
 
-template <int DT> __device__ __forceinline__ LdsRow lds_row(uint8_t *smem, int64_t units, int m) {
-    uint8_t *p = smem + (size_t)m * lds_row_bytes<DT>(units);
+template <int DT> __device__ __forceinline__ LdsRow lds_row(int64_t k, int m) {
+    const uint32_t units = (uint32_t)(k / Geo<DT>::kElems);
+    uint32_t p = (uint32_t)m * (uint32_t)lds_row_bytes<DT>(k);
     LdsRow r;
-    r.lo = (const int4 *)p; p += units * 16;
-    r.hi = (const int4 *)p; if (Geo<DT>::kHi) p += units * 16;
-    r.ad = (const float *)p; p += units * 4;
-    r.s0 = (const int *)p; if (Geo<DT>::kAux >= 1) p += units * 4;
-    r.s1 = (const int *)p;
+    r.lo = p; p += units * 16;
+    r.hi = p; if (Geo<DT>::kHi) p += units * 16;
+    r.d = p; p += (uint32_t)act_blocks<DT>(k) * 4;
+    r.bs = p;
     return r;
 }
+
+template <typename T> __device__ __forceinline__ T lds_get(const uint8_t *smem, uint32_t off) { return *(const T *)(smem + off); }
+template <typename T> __device__ __forceinline__ void lds_put(uint8_t *smem, uint32_t off, T v) { *(T *)(smem + off) = v; }
 
 // Where the 16 consecutive activation elements [16*piece, 16*piece+16) of a row go.
 template <int DT> __device__ __forceinline__ void piece_slot(int64_t piece, int64_t &unit, bool &hi) {
@@ -66,34 +77,188 @@ template <int DT> __device__ __forceinline__ void piece_slot(int64_t piece, int6
     }
 }
 
+// ------------------------------------------------------------------ wave reductions (DPP) ----
+template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+template <int CTRL> __device__ __forceinline__ int dpp_i(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
+}
+constexpr int kQuadSwap1 = 0xB1;   // quad_perm [1,0,3,2]
+constexpr int kQuadSwap2 = 0x4E;   // quad_perm [2,3,0,1]
+constexpr int kHalfMirror = 0x141; // lanes i <-> 7-i inside each 8
+constexpr int kRowMirror = 0x140;  // lanes i <-> 15-i inside each 16
+
+__device__ __forceinline__ float readlane_f(float v, int l) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+}
+// Sum over the 64 lanes, valid in every lane.
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_f<kQuadSwap1>(v);
+    v += dpp_f<kQuadSwap2>(v);
+    v += dpp_f<kHalfMirror>(v);
+    v += dpp_f<kRowMirror>(v);
+    return readlane_f(v, 0) + readlane_f(v, 16) + readlane_f(v, 32) + readlane_f(v, 48);
+}
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, dpp_f<kQuadSwap1>(v));
+    v = fmaxf(v, dpp_f<kQuadSwap2>(v));
+    v = fmaxf(v, dpp_f<kHalfMirror>(v));
+    v = fmaxf(v, dpp_f<kRowMirror>(v));
+    return fmaxf(fmaxf(readlane_f(v, 0), readlane_f(v, 16)), fmaxf(readlane_f(v, 32), readlane_f(v, 48)));
+}
+__device__ __forceinline__ int wave_min_i(int v) {
+    v = min(v, dpp_i<kQuadSwap1>(v));
+    v = min(v, dpp_i<kQuadSwap2>(v));
+    v = min(v, dpp_i<kHalfMirror>(v));
+    v = min(v, dpp_i<kRowMirror>(v));
+    return min(min(__builtin_amdgcn_readlane(v, 0), __builtin_amdgcn_readlane(v, 16)),
+               min(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
+}
+
+// ------------------------------------------------ activation quantizer inside the matvec ----
+__device__ __forceinline__ uint32_t pack4(int8_t a, int8_t b, int8_t c, int8_t d) {
+    return (uint32_t)(uint8_t)a | ((uint32_t)(uint8_t)b << 8) | ((uint32_t)(uint8_t)c << 16) | ((uint32_t)(uint8_t)d << 24);
+}
+
+// The workgroup's waves quantize x[0, k) into the LDS image of row 0.  Same arithmetic, operation
+// for operation, as quantize_act.hip (BlockQ8K::from_float k_quants.rs:1788-1825,
+// BlockQ8_0::from_float :586-615).
+// One 256-element chunk (chunk index c, this lane's four elements f at e0 = 256c + 4*lane).
 template <int DT>
-__device__ void stage_row(uint8_t *smem, int64_t units, int m, const cq_act_view &a, int64_t row, int64_t k) {
-    LdsRow r = lds_row<DT>(smem, units, m);
-    const int4 *src = (const int4 *)(a.qs + row * k);
-    for (int64_t piece = threadIdx.x; piece < k / 16; piece += kThreads) {
-        int64_t unit; bool hi;
-        piece_slot<DT>(piece, unit, hi);
-        ((int4 *)(hi ? r.hi : r.lo))[unit] = src[piece];
-    }
-    for (int64_t u = threadIdx.x; u < units; u += kThreads) {
-        if (DT == CQ_DTYPE_Q4_0) {
-            ((float *)r.ad)[u] = a.d[row * units + u];
-            ((int *)r.s0)[u] = a.bsum32[row * units + u];
-        } else if (DT == CQ_DTYPE_Q8_0) {
-            ((float *)r.ad)[u] = a.d[row * (units >> 1) + (u >> 1)];
+__device__ __forceinline__ void quantize_chunk_to_lds(uint8_t *smem, const float4 fin, int c, int e0, bool active,
+                                                      bool chunk_ok, const LdsRow r) {
+    const int lane = threadIdx.x & 63;
+    const float4 f = active ? fin : make_float4(0.f, 0.f, 0.f, 0.f);
+    {
+        uint32_t packed = 0;
+        int sum4 = 0;
+        if (Geo<DT>::kActK) {
+            const float a0 = fabsf(f.x), a1 = fabsf(f.y), a2 = fabsf(f.z), a3 = fabsf(f.w);
+            const float amax = wave_max(fmaxf(fmaxf(fmaxf(fmaxf(0.0f, a0), a1), a2), a3));
+            // the first element whose |x| equals the block maximum decides the sign of the scale
+            int idx = 0x7fffffff;
+            if (a3 == amax) idx = 4 * lane + 3;
+            if (a2 == amax) idx = 4 * lane + 2;
+            if (a1 == amax) idx = 4 * lane + 1;
+            if (a0 == amax) idx = 4 * lane;
+            idx = wave_min_i(idx);
+            const int sel = idx & 3;
+            const float cand = sel == 0 ? f.x : (sel == 1 ? f.y : (sel == 2 ? f.z : f.w));
+            const float max = readlane_f(cand, __builtin_amdgcn_readfirstlane(idx >> 2));
+            float d = 0.0f;
+            if (amax != 0.0f) {
+                const float iscale = -128.0f / max;
+                const int8_t q0 = cq_as_i8(fminf(roundf(iscale * f.x), 127.0f));
+                const int8_t q1 = cq_as_i8(fminf(roundf(iscale * f.y), 127.0f));
+                const int8_t q2 = cq_as_i8(fminf(roundf(iscale * f.z), 127.0f));
+                const int8_t q3 = cq_as_i8(fminf(roundf(iscale * f.w), 127.0f));
+                packed = pack4(q0, q1, q2, q3);
+                sum4 = (int)q0 + (int)q1 + (int)q2 + (int)q3;
+                d = 1.0f / iscale;
+            }
+            sum4 += dpp_i<kQuadSwap1>(sum4);
+            sum4 += dpp_i<kQuadSwap2>(sum4);  // the four lanes of a 16-element group hold its sum
+            if (chunk_ok && lane == 0) lds_put<float>(smem, r.d + 4 * c, d);
+            if (chunk_ok && (lane & 3) == 0) lds_put<int16_t>(smem, r.bs + 2 * (c * 16 + (lane >> 2)), (int16_t)sum4);
         } else {
-            const int64_t blk = row * (units >> 3) + (u >> 3);
-            const int p = (int)(u & 7);
-            ((float *)r.ad)[u] = a.d[blk];
-            const int16_t *bs = a.bsums + blk * 16;
-            if (DT == CQ_DTYPE_Q4K) {
-                ((int *)r.s0)[u] = (int)bs[2 * p] + (int)bs[2 * p + 1];
-            } else {
-                const int js = 8 * (p >> 2) + 2 * ((p >> 1) & 1) + (p & 1);
-                ((int *)r.s0)[u] = bs[js];
-                ((int *)r.s1)[u] = bs[js + 4];
+            float amax = fmaxf(fmaxf(fmaxf(fmaxf(0.0f, fabsf(f.x)), fabsf(f.y)), fabsf(f.z)), fabsf(f.w));
+            amax = fmaxf(amax, dpp_f<kQuadSwap1>(amax));
+            amax = fmaxf(amax, dpp_f<kQuadSwap2>(amax));
+            amax = fmaxf(amax, dpp_f<kHalfMirror>(amax));  // 8 lanes = one 32-element block
+            const float d = amax / 127.0f;
+            const float id = d != 0.0f ? 1.0f / d : 0.0f;
+            const int8_t q0 = cq_as_i8(roundf(f.x * id)), q1 = cq_as_i8(roundf(f.y * id)),
+                         q2 = cq_as_i8(roundf(f.z * id)), q3 = cq_as_i8(roundf(f.w * id));
+            packed = pack4(q0, q1, q2, q3);
+            sum4 = (int)q0 + (int)q1 + (int)q2 + (int)q3;
+            sum4 += dpp_i<kQuadSwap1>(sum4);
+            sum4 += dpp_i<kQuadSwap2>(sum4);
+            sum4 += dpp_i<kHalfMirror>(sum4);
+            if (active && (lane & 7) == 0) {
+                lds_put<float>(smem, r.d + 4 * (e0 >> 5), cq_h2f(cq_f2h(d)));
+                lds_put<int32_t>(smem, r.bs + 4 * (e0 >> 5), sum4);
             }
         }
+        if (active) {
+            int64_t unit; bool hi;
+            piece_slot<DT>(e0 >> 4, unit, hi);
+            lds_put<uint32_t>(smem, (hi ? r.hi : r.lo) + (uint32_t)unit * 16 + 4 * (lane & 3), packed);
+        }
+    }
+}
+
+__device__ __forceinline__ float4 load_x_chunk(const float *x, int64_t k, int c, int chunks) {
+    // Unconditional load from a clamped address (a masked load would make the compiler wait for it
+    // at once); lanes past the end of the row are zeroed where the values are used.
+    const int e0 = c * 256 + 4 * (int)(threadIdx.x & 63);
+    (void)chunks;
+    return *(const float4 *)(x + (e0 < k ? e0 : 0));
+}
+
+// A wave of an NW-wave workgroup owns chunks wave, wave + NW, ...: at most XCH of them.  All are
+// loaded up front (before the weight rows) and quantized in straight-line code, so every wait is
+// an exact count and the weight loads behind them stay in flight.
+template <int XCH, int NW>
+__device__ __forceinline__ void load_x_chunks(const float *x, int64_t k, int wave, float4 (&fx)[XCH]) {
+#pragma unroll
+    for (int i = 0; i < XCH; i++) fx[i] = load_x_chunk(x, k, wave + i * NW, 0);
+}
+
+template <int DT, int XCH, int NW>
+__device__ __forceinline__ void quantize_row_to_lds(uint8_t *smem, int64_t k, int wave, const LdsRow r,
+                                                    const float4 (&fx)[XCH]) {
+    const int lane = threadIdx.x & 63;
+    const int chunks = (int)((k + 255) / 256);
+#pragma unroll
+    for (int i = 0; i < XCH; i++) {
+        const int c = wave + i * NW;
+        const int e0 = c * 256 + 4 * lane;
+        quantize_chunk_to_lds<DT>(smem, fx[i], c, e0, c < chunks && e0 < k, c < chunks, r);
+    }
+}
+
+// Copy an already-quantized activation row from the workspace into its LDS image.
+template <int DT, int NT>
+__device__ __forceinline__ void stage_row(uint8_t *smem, const LdsRow r, const cq_act_view &a, int64_t row, int64_t k) {
+    const int4 *src = (const int4 *)(a.qs + row * k);
+    for (int piece = threadIdx.x; piece < (int)(k / 16); piece += NT) {
+        int64_t unit; bool hi;
+        piece_slot<DT>(piece, unit, hi);
+        lds_put<int4>(smem, (hi ? r.hi : r.lo) + (uint32_t)unit * 16, src[piece]);
+    }
+    const int nb = (int)act_blocks<DT>(k);
+    for (int b = threadIdx.x; b < nb; b += NT) {
+        lds_put<float>(smem, r.d + 4 * b, a.d[row * nb + b]);
+        if (!Geo<DT>::kActK) lds_put<int32_t>(smem, r.bs + 4 * b, a.bsum32[row * nb + b]);
+    }
+    if (Geo<DT>::kActK) {
+        const int32_t *bs = (const int32_t *)(a.bsums + row * nb * 16);  // 8 words per block
+        for (int i = threadIdx.x; i < nb * 8; i += NT) lds_put<int32_t>(smem, r.bs + 4 * i, bs[i]);
+    }
+}
+
+// ------------------------------------------------------------------------ weight units ----
+// Raw bytes of one unit as loaded from the planes (decoded later, so loads can run ahead).
+template <int DT> struct UnitRaw {
+    uint4 q;       // main plane lane
+    uint4 h;       // Q4K: block header {d, dmin, scales[12]}
+    uint2 hh;      // Q6K: high bits of the lane's 32 elements
+    uint16_t sc2;  // Q6K: the lane's two group scales
+    uint16_t d;    // Q4_0 / Q8_0 / Q6K: f16 scale
+};
+
+template <int DT>
+__device__ __forceinline__ void load_unit(const cq_weight &w, int64_t row, int64_t units, int64_t u, UnitRaw<DT> &o) {
+    const int64_t g = row * units + u;
+    o.q = *(const uint4 *)(w.p0 + g * 16);
+    if (DT == CQ_DTYPE_Q4_0) o.d = ((const uint16_t *)w.p1)[g];
+    if (DT == CQ_DTYPE_Q8_0) o.d = ((const uint16_t *)w.p1)[g >> 1];
+    if (DT == CQ_DTYPE_Q4K) o.h = *(const uint4 *)(w.p1 + (g >> 3) * 16);
+    if (DT == CQ_DTYPE_Q6K) {
+        o.hh = *(const uint2 *)(w.p1 + g * 8);
+        o.sc2 = ((const uint16_t *)w.p2)[g];
+        o.d = ((const uint16_t *)w.p3)[g >> 3];
     }
 }
 
@@ -105,47 +270,36 @@ __device__ __forceinline__ int dot16(const uint32_t w[4], const int4 &a) {
     return s;
 }
 
-// The weight side of one unit, decoded once and reused for every activation row.
+// Decoded weight side of a unit, reused for every activation row.
 template <int DT> struct UnitW {
     uint32_t lo[4], hi[4];
     float dw, dmin;
-    int sc_lo, sc_hi, mn;
+    int sc_lo, sc_hi, mn_lo, mn_hi;
 };
 
-template <int DT>
-__device__ __forceinline__ void load_unit(const cq_weight &w, int64_t row, int64_t units, int64_t u, UnitW<DT> &o) {
-    const uint4 q = *(const uint4 *)(w.p0 + (row * units + u) * 16);
-    const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
-    if (DT == CQ_DTYPE_Q4_0) {
-        o.dw = cq_h2f(((const uint16_t *)w.p1)[row * units + u]);
-#pragma unroll
-        for (int i = 0; i < 4; i++) { o.lo[i] = qw[i] & 0x0F0F0F0Fu; o.hi[i] = (qw[i] >> 4) & 0x0F0F0F0Fu; }
-    } else if (DT == CQ_DTYPE_Q8_0) {
-        o.dw = cq_h2f(((const uint16_t *)w.p1)[row * (units >> 1) + (u >> 1)]);
+template <int DT> __device__ __forceinline__ void decode_unit(const UnitRaw<DT> &r, int p, UnitW<DT> &o) {
+    const uint32_t qw[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+    if (DT == CQ_DTYPE_Q8_0) {
+        o.dw = cq_h2f(r.d);
 #pragma unroll
         for (int i = 0; i < 4; i++) o.lo[i] = qw[i];
-    } else if (DT == CQ_DTYPE_Q4K) {
-        const uint4 h = *(const uint4 *)(w.p1 + (row * (units >> 3) + (u >> 3)) * 16);
-        const int p = (int)(u & 7), g = p >> 1;
-        o.dw = cq_h2f((uint16_t)(h.x & 0xffff));
-        o.dmin = cq_h2f((uint16_t)(h.x >> 16));
-        int m0, m1;
-        cq_scale_min_k4(2 * g, h.y, h.z, h.w, o.sc_lo, m0);
-        cq_scale_min_k4(2 * g + 1, h.y, h.z, h.w, o.sc_hi, m1);
-        int scp;
-        cq_scale_min_k4(p, h.y, h.z, h.w, scp, o.mn);   // lane p owns the min of sub-block p
+    } else if (DT == CQ_DTYPE_Q4_0) {
+        o.dw = cq_h2f(r.d);
 #pragma unroll
         for (int i = 0; i < 4; i++) { o.lo[i] = qw[i] & 0x0F0F0F0Fu; o.hi[i] = (qw[i] >> 4) & 0x0F0F0F0Fu; }
-    } else {  // Q6K
-        const int64_t blk = row * (units >> 3) + (u >> 3);
-        const uint2 hh = *(const uint2 *)(w.p1 + (row * units + u) * 8);
-        const int p = (int)(u & 7);
-        const int js = 8 * (p >> 2) + 2 * ((p >> 1) & 1) + (p & 1);
-        const int8_t *sc = (const int8_t *)w.p2 + blk * 16;
-        o.sc_lo = sc[js];
-        o.sc_hi = sc[js + 4];
-        o.dw = cq_h2f(((const uint16_t *)w.p3)[blk]);
-        const uint32_t hw[2] = {hh.x, hh.y};
+    } else if (DT == CQ_DTYPE_Q4K) {
+        const int g = p >> 1;
+        o.dw = cq_h2f((uint16_t)(r.h.x & 0xffff));
+        o.dmin = cq_h2f((uint16_t)(r.h.x >> 16));
+        cq_scale_min_k4(2 * g, r.h.y, r.h.z, r.h.w, o.sc_lo, o.mn_lo);
+        cq_scale_min_k4(2 * g + 1, r.h.y, r.h.z, r.h.w, o.sc_hi, o.mn_hi);
+#pragma unroll
+        for (int i = 0; i < 4; i++) { o.lo[i] = qw[i] & 0x0F0F0F0Fu; o.hi[i] = (qw[i] >> 4) & 0x0F0F0F0Fu; }
+    } else {
+        o.sc_lo = (int)(int8_t)(r.sc2 & 0xff);
+        o.sc_hi = (int)(int8_t)(r.sc2 >> 8);
+        o.dw = cq_h2f(r.d);
+        const uint32_t hw[2] = {r.hh.x, r.hh.y};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const uint32_t H = hw[i >> 1];
@@ -156,81 +310,183 @@ __device__ __forceinline__ void load_unit(const cq_weight &w, int64_t row, int64
     }
 }
 
-// Integer parts of one unit against one staged activation row.
+// Integer parts of unit u (p = u mod 8) against one activation row.
 //   Q4_0: I = sum (q-8)*a over the block.            Q8_0: I = sum q*a over half a block.
-//   Q4K : I = sc_lo*dot_lo + sc_hi*dot_hi, Mn = min_p * (bsums[2p] + bsums[2p+1]).
+//   Q4K : I = sc_lo*dot_lo + sc_hi*dot_hi over the lane's halves of sub-blocks 2g and 2g+1;
+//         Mn = min_2g * S_lo + min_2g+1 * S_hi with S = sum of the same activation quants
+//         (over the eight lanes of a block: sum_j bsums_j * min_{j/2}).
 //   Q6K : I = sc_lo*(dot_lo - 32*bsums_lo) + sc_hi*(dot_hi - 32*bsums_hi).
 template <int DT>
-__device__ __forceinline__ void unit_ints(const UnitW<DT> &w, const LdsRow &r, int64_t u, int &I, int &Mn) {
-    const int4 alo = r.lo[u];
+__device__ __forceinline__ void unit_ints(const uint8_t *smem, const UnitW<DT> &w, const LdsRow r, uint32_t u, int &I,
+                                          int &Mn) {
+    const int4 alo = lds_get<int4>(smem, r.lo + u * 16);
     Mn = 0;
     if (DT == CQ_DTYPE_Q8_0) {
         I = dot16(w.lo, alo);
         return;
     }
-    const int4 ahi = r.hi[u];
+    const int4 ahi = lds_get<int4>(smem, r.hi + u * 16);
     const int dlo = dot16(w.lo, alo), dhi = dot16(w.hi, ahi);
     if (DT == CQ_DTYPE_Q4_0) {
-        I = dlo + dhi - 8 * r.s0[u];
+        I = dlo + dhi - 8 * lds_get<int32_t>(smem, r.bs + 4 * u);
     } else if (DT == CQ_DTYPE_Q4K) {
-        I = w.sc_lo * dlo + w.sc_hi * dhi;
-        Mn = w.mn * r.s0[u];
+        I = __mul24(w.sc_lo, dlo) + __mul24(w.sc_hi, dhi);
+        // unit p = 2g + i holds elements 64g + 16i + [0,16) and 64g + 32 + 16i + [0,16):
+        // 16-element groups 4g + i (sub-block 2g) and 4g + 2 + i (sub-block 2g + 1)
+        const uint32_t p = u & 7, g = p >> 1, i = p & 1;
+        const uint32_t bs = r.bs + 32 * (u >> 3);
+        Mn = __mul24(w.mn_lo, (int)lds_get<int16_t>(smem, bs + 2 * (4 * g + i))) +
+             __mul24(w.mn_hi, (int)lds_get<int16_t>(smem, bs + 2 * (4 * g + 2 + i)));
     } else {
-        I = w.sc_lo * (dlo - 32 * r.s0[u]) + w.sc_hi * (dhi - 32 * r.s1[u]);
+        // unit p = 4h + 2t + i: low nibbles are group 8h + 2t + i, high nibbles that + 4
+        const uint32_t p = u & 7;
+        const uint32_t js = p + 4 * (p >> 2);
+        const uint32_t bs = r.bs + 32 * (u >> 3);
+        I = __mul24(w.sc_lo, dlo - 32 * (int)lds_get<int16_t>(smem, bs + 2 * js)) +
+            __mul24(w.sc_hi, dhi - 32 * (int)lds_get<int16_t>(smem, bs + 2 * (js + 4)));
     }
 }
 
 template <int DT>
-__device__ __forceinline__ float unit_value(const UnitW<DT> &w, const LdsRow &r, int64_t u) {
+__device__ __forceinline__ float unit_value(const uint8_t *smem, const UnitW<DT> &w, const LdsRow r, uint32_t u) {
     int I, Mn;
-    unit_ints<DT>(w, r, u, I, Mn);
-    const float ad = r.ad[u];
+    unit_ints<DT>(smem, w, r, u, I, Mn);
+    const float ad = lds_get<float>(smem, r.d + 4 * (DT == CQ_DTYPE_Q8_0 ? (u >> 1) : (DT == CQ_DTYPE_Q4_0 ? u : (u >> 3))));
     if (DT == CQ_DTYPE_Q4K) return ad * (w.dw * (float)I - w.dmin * (float)Mn);
     return ((float)I * w.dw) * ad;
 }
 
-// Sum over the 64 lanes of a wave, result valid in every lane.
-__device__ __forceinline__ float wave_sum(float v) {
-#define CQ_DPP_ADD(ctrl)                                                                                   \
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, true))
-    CQ_DPP_ADD(0xB1);   // quad_perm [1,0,3,2]
-    CQ_DPP_ADD(0x4E);   // quad_perm [2,3,0,1]
-    CQ_DPP_ADD(0x141);  // row_half_mirror
-    CQ_DPP_ADD(0x140);  // row_mirror
-#undef CQ_DPP_ADD
-    // every lane of a 16-lane row now holds the row's sum
-    const int iv = __builtin_bit_cast(int, v);
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 0)) +
-           __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 16)) +
-           __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 32)) +
-           __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 48));
+// --------------------------------------------------------------------- fused kernel (m = 1) ----
+// Loads of one weight row for this lane: units lane, lane + 64, ...  Lanes past the end of the row
+// re-read its last unit (same cache line as a neighbour, no extra traffic) and are masked when
+// accumulating, so the loads are unconditional and nothing waits on them early.
+template <int DT, int UPL>
+__device__ __forceinline__ void load_row(const cq_weight &w, int64_t row, uint32_t units, UnitRaw<DT> (&buf)[UPL]) {
+    const uint32_t lane = threadIdx.x & 63;
+#pragma unroll
+    for (int c = 0; c < UPL; c++) {
+        const uint32_t u = c * 64 + lane;
+        // keep u & 7 (the lane's position in its block) when clamping
+        const uint32_t uc = u < units ? u : (units - 8 + (lane & 7));
+        load_unit<DT>(w, row, units, uc, buf[c]);
+    }
 }
 
+template <int DT, int UPL>
+__device__ __forceinline__ float row_dot(const uint8_t *smem, const LdsRow r, uint32_t units,
+                                         const UnitRaw<DT> (&buf)[UPL]) {
+    const uint32_t lane = threadIdx.x & 63;
+    float acc = 0.0f;
+#pragma unroll
+    for (int c = 0; c < UPL; c++) {
+        const uint32_t u = c * 64 + lane;
+        const uint32_t uc = u < units ? u : (units - 8 + (lane & 7));
+        UnitW<DT> uw;
+        decode_unit<DT>(buf[c], lane & 7, uw);
+        const float v = unit_value<DT>(smem, uw, r, uc);
+        acc += u < units ? v : 0.0f;
+    }
+    return wave_sum(acc);
+}
+
+// Wave g of `total_waves` handles rows g, g + total_waves, ...  The launcher guarantees that every
+// wave has at least DEPTH rows, so the prologue loads are unconditional: the compiler can then
+// count outstanding loads exactly and waits for the activation chunk only (issued first; loads
+// return in order), not for the weight rows behind it.
+//   DEPTH 2 (short rows): two static register buffers, each refilled right after it is consumed.
+//   DEPTH 1 (long rows) : one buffer; a row is several KiB in flight per wave already.
+template <int DT, int UPL, int NW, int DEPTH>
+__global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float *x,
+                                                        float *__restrict__ y, int64_t total_waves,
+                                                        int64_t rows_per_wave, int64_t rows_extra) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: scalar loops and branches
+    const uint32_t units = (uint32_t)(w.k / Geo<DT>::kElems);
+    const int64_t row0 = (int64_t)blockIdx.x * NW + wave;
+    const int64_t T = total_waves;
+    // rows of this wave (>= DEPTH): n / T, plus one for the first n % T waves (both from the host)
+    const int64_t cnt = rows_per_wave + (row0 < rows_extra ? 1 : 0);
+
+    // chunks of 256 activations per wave: k/256 <= 8*UPL/NW for the 32-element unit types
+    constexpr int XCH = (((Geo<DT>::kElems == 16 ? (UPL + 1) / 2 : UPL) * 8) + NW - 1) / NW;
+    float4 fx[XCH];
+    load_x_chunks<XCH, NW>(x, w.k, wave, fx);
+    // Pin the issue order: activation loads, then weight loads, then the quantizer arithmetic.
+    // (The empty asm stops the optimizer from sinking loads past it, the scheduling barrier stops
+    // the instruction scheduler.)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    UnitRaw<DT> a[UPL], b[DEPTH == 2 ? UPL : 1];
+    load_row<DT, UPL>(w, row0, units, a);
+    if constexpr (DEPTH == 2) load_row<DT, UPL>(w, row0 + T, units, b);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    const LdsRow r = lds_row<DT>(w.k, 0);
+#ifndef CQ_EXP_SKIP_QUANT
+    quantize_row_to_lds<DT, XCH, NW>(smem, w.k, wave, r, fx);
+#endif
+    __syncthreads();
+
+    if constexpr (DEPTH == 1) {
+        for (int64_t i = 0; i < cnt; i++) {
+            const float s = row_dot<DT, UPL>(smem, r, units, a);
+            if (i + 1 < cnt) load_row<DT, UPL>(w, row0 + (i + 1) * T, units, a);
+            if (lane == 0) y[row0 + i * T] = s;
+        }
+    } else {
+        int64_t i = 0;
+        // steady state: rows i and i+1 are in a and b, rows i+2 and i+3 exist
+        for (; i + 3 < cnt; i += 2) {
+            const float s0 = row_dot<DT, UPL>(smem, r, units, a);
+            load_row<DT, UPL>(w, row0 + (i + 2) * T, units, a);
+            const float s1 = row_dot<DT, UPL>(smem, r, units, b);
+            load_row<DT, UPL>(w, row0 + (i + 3) * T, units, b);
+            if (lane == 0) { y[row0 + i * T] = s0; y[row0 + (i + 1) * T] = s1; }
+        }
+        // tail: two or three rows left (a = row i, b = row i+1, maybe row i+2 still to load)
+        const float s0 = row_dot<DT, UPL>(smem, r, units, a);
+        const bool third = i + 2 < cnt;
+        if (third) load_row<DT, UPL>(w, row0 + (i + 2) * T, units, a);
+        const float s1 = row_dot<DT, UPL>(smem, r, units, b);
+        if (lane == 0) { y[row0 + i * T] = s0; y[row0 + (i + 1) * T] = s1; }
+        if (third) {
+            const float s2 = row_dot<DT, UPL>(smem, r, units, a);
+            if (lane == 0) y[row0 + (i + 2) * T] = s2;
+        }
+    }
+}
+
+// ------------------------------------------------------------ staged kernel (m <= 4 rows) ----
+constexpr int kStagedThreads = 256;
+
 template <int DT, int MB>
-__global__ void __launch_bounds__(kThreads) matvec_kernel(cq_weight w, cq_act_view a, int64_t m0, int rows_per_wg,
-                                                          float *__restrict__ y) {
+__global__ void __launch_bounds__(kStagedThreads) staged_kernel(cq_weight w, cq_act_view a, int64_t m0,
+                                                                int rows_per_wg, float *__restrict__ y) {
     extern __shared__ __align__(16) uint8_t smem[];
     const int64_t units = w.k / Geo<DT>::kElems;
-#pragma unroll
-    for (int m = 0; m < MB; m++) stage_row<DT>(smem, units, m, a, m0 + m, w.k);
-    __syncthreads();
     LdsRow rows[MB];
 #pragma unroll
-    for (int m = 0; m < MB; m++) rows[m] = lds_row<DT>(smem, units, m);
-
+    for (int m = 0; m < MB; m++) {
+        rows[m] = lds_row<DT>(w.k, m);
+        stage_row<DT, kStagedThreads>(smem, rows[m], a, m0 + m, w.k);
+    }
+    __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t row_begin = (int64_t)blockIdx.x * rows_per_wg;
     const int64_t row_end = row_begin + rows_per_wg < w.n ? row_begin + rows_per_wg : w.n;
-    for (int64_t row = row_begin + wave; row < row_end; row += kWaves) {
+    for (int64_t row = row_begin + wave; row < row_end; row += kStagedThreads / 64) {
         float acc[MB];
 #pragma unroll
         for (int m = 0; m < MB; m++) acc[m] = 0.0f;
 #pragma unroll 2
         for (int64_t u = lane; u < units; u += 64) {
+            UnitRaw<DT> raw;
+            load_unit<DT>(w, row, units, u, raw);
             UnitW<DT> uw;
-            load_unit<DT>(w, row, units, u, uw);
+            decode_unit<DT>(raw, lane & 7, uw);
 #pragma unroll
-            for (int m = 0; m < MB; m++) acc[m] += unit_value<DT>(uw, rows[m], u);
+            for (int m = 0; m < MB; m++) acc[m] += unit_value<DT>(smem, uw, rows[m], (uint32_t)u);
         }
 #pragma unroll
         for (int m = 0; m < MB; m++) {
@@ -240,36 +496,39 @@ __global__ void __launch_bounds__(kThreads) matvec_kernel(cq_weight w, cq_act_vi
     }
 }
 
-// Per-block integer dots for verification: one wave per (activation row, weight row).
+// Per-block integer dots for verification: same unit arithmetic as the kernels above.
 template <int DT>
-__global__ void __launch_bounds__(kThreads) int_dots_kernel(cq_weight w, cq_act_view a, int64_t m0, int rows_per_wg,
-                                                            int32_t *__restrict__ out_i, int32_t *__restrict__ out_mn) {
+__global__ void __launch_bounds__(kStagedThreads) int_dots_kernel(cq_weight w, cq_act_view a, int64_t m0,
+                                                                  int rows_per_wg, int32_t *__restrict__ out_i,
+                                                                  int32_t *__restrict__ out_mn) {
     extern __shared__ __align__(16) uint8_t smem[];
     const int64_t units = w.k / Geo<DT>::kElems;
-    stage_row<DT>(smem, units, 0, a, m0, w.k);
+    const LdsRow r = lds_row<DT>(w.k, 0);
+    stage_row<DT, kStagedThreads>(smem, r, a, m0, w.k);
     __syncthreads();
-    const LdsRow r = lds_row<DT>(smem, units, 0);
-    constexpr int kUnitsPerBlock = DT == CQ_DTYPE_Q4_0 ? 1 : (DT == CQ_DTYPE_Q8_0 ? 2 : 8);
-    const int64_t kb = units / kUnitsPerBlock;
+    constexpr int kUPB = Geo<DT>::kUnitsPerBlock;
+    const int64_t kb = units / kUPB;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t row_begin = (int64_t)blockIdx.x * rows_per_wg;
     const int64_t row_end = row_begin + rows_per_wg < w.n ? row_begin + rows_per_wg : w.n;
-    for (int64_t row = row_begin + wave; row < row_end; row += kWaves) {
+    for (int64_t row = row_begin + wave; row < row_end; row += kStagedThreads / 64) {
         for (int64_t u0 = 0; u0 < units; u0 += 64) {
             const int64_t u = u0 + lane;
             int I = 0, Mn = 0;
             if (u < units) {
+                UnitRaw<DT> raw;
+                load_unit<DT>(w, row, units, u, raw);
                 UnitW<DT> uw;
-                load_unit<DT>(w, row, units, u, uw);
-                unit_ints<DT>(uw, r, u, I, Mn);
+                decode_unit<DT>(raw, lane & 7, uw);
+                unit_ints<DT>(smem, uw, r, (uint32_t)u, I, Mn);
             }
 #pragma unroll
-            for (int off = 1; off < kUnitsPerBlock; off <<= 1) {
+            for (int off = 1; off < kUPB; off <<= 1) {
                 I += __shfl_xor(I, off);
                 Mn += __shfl_xor(Mn, off);
             }
-            if (u < units && (u % kUnitsPerBlock) == 0) {
-                const int64_t o = (m0 * w.n + row) * kb + u / kUnitsPerBlock;
+            if (u < units && (u % kUPB) == 0) {
+                const int64_t o = (m0 * w.n + row) * kb + u / kUPB;
                 out_i[o] = I;
                 if (out_mn) out_mn[o] = Mn;
             }
@@ -277,30 +536,83 @@ __global__ void __launch_bounds__(kThreads) int_dots_kernel(cq_weight w, cq_act_
     }
 }
 
+// ------------------------------------------------------------------------------- launch ----
+int g_num_cus = 0;
+int num_cus() {
+    if (g_num_cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            g_num_cus = n;
+        else
+            g_num_cus = 256;
+    }
+    return g_num_cus;
+}
+
+int g_fused_wgs_per_cu = 0;  // 0 = automatic; A/B switch (CQ_MATVEC_WAVES = workgroups per CU)
+
+// Eight waves per workgroup, up to two workgroups per CU.  Whole workgroups only, and every wave
+// gets at least `depth` rows: wgs * 8 * depth <= n.
+template <int DT, int UPL>
+hipError_t launch_fused_upl(const cq_weight *w, const float *x, float *y, hipStream_t s) {
+    constexpr int NW = 8;
+    const size_t lds = lds_row_bytes<DT>(w->k);
+    const int per_cu = g_fused_wgs_per_cu > 0 ? g_fused_wgs_per_cu : 2;
+    const int64_t max_wgs = (int64_t)num_cus() * per_cu;
+    int depth = UPL <= 2 ? 2 : 1;
+    if (w->n < NW * 2) depth = 1;
+    if (w->n < NW) {  // fewer rows than one workgroup's waves: the two-launch path handles it
+        return hipErrorInvalidConfiguration;
+    }
+    int64_t wgs = w->n / (NW * depth);
+    if (wgs > max_wgs) wgs = max_wgs;
+    const int64_t tw = wgs * NW, rpw = w->n / tw, extra = w->n % tw;
+    if (depth == 2) fused_kernel<DT, UPL, NW, 2><<<(unsigned)wgs, NW * 64, lds, s>>>(*w, x, y, tw, rpw, extra);
+    else fused_kernel<DT, UPL, NW, 1><<<(unsigned)wgs, NW * 64, lds, s>>>(*w, x, y, tw, rpw, extra);
+    return hipGetLastError();
+}
+
+template <int DT>
+bool fused_ok(const cq_weight *w) {
+    // Every workgroup re-quantizes the whole activation row in its prologue; beyond 8192 elements
+    // (more than four 256-element chunks per wave) that costs more than the separate quantizer
+    // launch it saves (measured on K = 11008), so longer rows take the two-launch path.
+    return w->k <= 8192 && w->n >= 8 && lds_row_bytes<DT>(w->k) <= 64 * 1024;
+}
+
+template <int DT>
+hipError_t launch_fused(const cq_weight *w, const float *x, float *y, hipStream_t s) {
+    const int64_t units = w->k / Geo<DT>::kElems;
+    const int upl = (int)((units + 63) / 64);
+    if (upl <= 1) return launch_fused_upl<DT, 1>(w, x, y, s);
+    if (upl <= 2) return launch_fused_upl<DT, 2>(w, x, y, s);
+    if (upl <= 3) return launch_fused_upl<DT, 3>(w, x, y, s);
+    if (upl <= 4) return launch_fused_upl<DT, 4>(w, x, y, s);
+    if (upl <= 6) return launch_fused_upl<DT, 6>(w, x, y, s);
+    return launch_fused_upl<DT, 8>(w, x, y, s);
+}
+
 int pick_rows_per_wg(int64_t n) {
-    // Enough workgroups to fill 256 CUs several times over, few enough that the activation
-    // staging is amortised over several rows per wave.
     int r = 16;
     while (r > 4 && (n + r - 1) / r < 2048) r >>= 1;
     return r;
 }
 
 template <int DT>
-hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
-    const int64_t units = w->k / Geo<DT>::kElems;
+hipError_t launch_staged(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
     const int rpw = pick_rows_per_wg(w->n);
     const unsigned grid = (unsigned)((w->n + rpw - 1) / rpw);
     int64_t m0 = 0;
     while (m0 < m) {
         const int64_t left = m - m0;
-        // keep the staged rows within 64 KiB of LDS
         int mb = left >= 4 ? 4 : (left >= 2 ? 2 : 1);
-        while (mb > 1 && lds_row_bytes<DT>(units) * mb > 64 * 1024) mb >>= 1;
-        const size_t lds = lds_row_bytes<DT>(units) * mb;
-        if (lds > 150 * 1024) return hipErrorInvalidValue;
-        if (mb == 4) matvec_kernel<DT, 4><<<grid, kThreads, lds, s>>>(*w, a, m0, rpw, y);
-        else if (mb == 2) matvec_kernel<DT, 2><<<grid, kThreads, lds, s>>>(*w, a, m0, rpw, y);
-        else matvec_kernel<DT, 1><<<grid, kThreads, lds, s>>>(*w, a, m0, rpw, y);
+        while (mb > 1 && lds_row_bytes<DT>(w->k) * mb > 64 * 1024) mb >>= 1;
+        const size_t lds = lds_row_bytes<DT>(w->k) * mb;
+        if (lds > 64 * 1024) return hipErrorInvalidValue;
+        if (mb == 4) staged_kernel<DT, 4><<<grid, kStagedThreads, lds, s>>>(*w, a, m0, rpw, y);
+        else if (mb == 2) staged_kernel<DT, 2><<<grid, kStagedThreads, lds, s>>>(*w, a, m0, rpw, y);
+        else staged_kernel<DT, 1><<<grid, kStagedThreads, lds, s>>>(*w, a, m0, rpw, y);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         m0 += mb;
@@ -310,13 +622,12 @@ hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hip
 
 template <int DT>
 hipError_t launch_ints(const cq_weight *w, cq_act_view a, int64_t m, int32_t *oi, int32_t *omn, hipStream_t s) {
-    const int64_t units = w->k / Geo<DT>::kElems;
-    const size_t lds = lds_row_bytes<DT>(units);
-    if (lds > 150 * 1024) return hipErrorInvalidValue;
+    const size_t lds = lds_row_bytes<DT>(w->k);
+    if (lds > 64 * 1024) return hipErrorInvalidValue;
     const int rpw = 8;
     const unsigned grid = (unsigned)((w->n + rpw - 1) / rpw);
     for (int64_t m0 = 0; m0 < m; m0++) {
-        int_dots_kernel<DT><<<grid, kThreads, lds, s>>>(*w, a, m0, rpw, oi, omn);
+        int_dots_kernel<DT><<<grid, kStagedThreads, lds, s>>>(*w, a, m0, rpw, oi, omn);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
@@ -325,14 +636,37 @@ hipError_t launch_ints(const cq_weight *w, cq_act_view a, int64_t m, int32_t *oi
 
 }  // namespace
 
+void cq_matvec_set_waves(int nw) { g_fused_wgs_per_cu = nw; }
+
+bool cq_matvec_fused_supported(const cq_weight *w) {
+    switch (w->dtype) {
+    case CQ_DTYPE_Q4_0: return fused_ok<CQ_DTYPE_Q4_0>(w);
+    case CQ_DTYPE_Q8_0: return fused_ok<CQ_DTYPE_Q8_0>(w);
+    case CQ_DTYPE_Q4K: return fused_ok<CQ_DTYPE_Q4K>(w);
+    case CQ_DTYPE_Q6K: return fused_ok<CQ_DTYPE_Q6K>(w);
+    default: return false;
+    }
+}
+
+hipError_t cq_launch_matvec_fused(const cq_weight *w, const float *x, float *y, hipStream_t s) {
+    if (w->n == 0) return hipSuccess;
+    switch (w->dtype) {
+    case CQ_DTYPE_Q4_0: return launch_fused<CQ_DTYPE_Q4_0>(w, x, y, s);
+    case CQ_DTYPE_Q8_0: return launch_fused<CQ_DTYPE_Q8_0>(w, x, y, s);
+    case CQ_DTYPE_Q4K: return launch_fused<CQ_DTYPE_Q4K>(w, x, y, s);
+    case CQ_DTYPE_Q6K: return launch_fused<CQ_DTYPE_Q6K>(w, x, y, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+
 hipError_t cq_launch_matvec(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s) {
     (void)act_dtype;
     if (m == 0 || w->n == 0) return hipSuccess;
     switch (w->dtype) {
-    case CQ_DTYPE_Q4_0: return launch_dt<CQ_DTYPE_Q4_0>(w, a, m, y, s);
-    case CQ_DTYPE_Q8_0: return launch_dt<CQ_DTYPE_Q8_0>(w, a, m, y, s);
-    case CQ_DTYPE_Q4K: return launch_dt<CQ_DTYPE_Q4K>(w, a, m, y, s);
-    case CQ_DTYPE_Q6K: return launch_dt<CQ_DTYPE_Q6K>(w, a, m, y, s);
+    case CQ_DTYPE_Q4_0: return launch_staged<CQ_DTYPE_Q4_0>(w, a, m, y, s);
+    case CQ_DTYPE_Q8_0: return launch_staged<CQ_DTYPE_Q8_0>(w, a, m, y, s);
+    case CQ_DTYPE_Q4K: return launch_staged<CQ_DTYPE_Q4K>(w, a, m, y, s);
+    case CQ_DTYPE_Q6K: return launch_staged<CQ_DTYPE_Q6K>(w, a, m, y, s);
     default: return hipErrorInvalidValue;
     }
 }

@@ -22,7 +22,7 @@
 //          hd [n][k/256][16]      (d f16, dmin f16, scales[12]: the first 16 bytes of the GGML block)
 //   Q6K  : ql [n][k/256][128] u8  (GGML order)
 //          qh [n][k/256][64]  u8  (re-ordered, see repack.hip: 8 bytes per 16-byte ql lane)
-//          sc [n][k/256][16]  i8
+//          sc [n][k/256][16]  i8  (re-ordered: two scales per 16-byte ql lane, see repack.hip)
 //          d  [n][k/256]      f16
 // All planes live in one allocation; each plane starts 256-byte aligned and the
 // allocation carries CQ_TAIL_PAD spare bytes so that a partial tail tile can be
@@ -87,6 +87,9 @@ hipError_t cq_launch_dequantize(const cq_weight *w, float *dst32, uint16_t *dst1
 hipError_t cq_launch_matvec(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s);
 hipError_t cq_launch_int_dots(const cq_weight *w, cq_act_view a, int64_t m, int32_t *out_i, int32_t *out_mn,
                               hipStream_t s);
+bool cq_matvec_fused_supported(const cq_weight *w);   // m == 1: quantizer fused into the matvec launch
+hipError_t cq_launch_matvec_fused(const cq_weight *w, const float *x, float *y, hipStream_t s);
+void cq_matvec_set_waves(int nw);                     // A/B switch: waves per workgroup of the fused kernel
 // gemm.hip
 bool cq_gemm_supported(const cq_weight *w, int64_t m, int act_dtype);
 hipError_t cq_launch_gemm(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s);
@@ -139,13 +142,13 @@ __device__ __forceinline__ int32_t cq_clampi(int32_t v, int32_t lo, int32_t hi) 
 
 // utils.rs:49-59 on the 12 scale bytes held as three little-endian words
 __device__ __forceinline__ void cq_scale_min_k4(int j, uint32_t u0, uint32_t u1, uint32_t u2, int &sc, int &mn) {
-    const int sh = 8 * (j & 3);
-    if (j < 4) {
-        sc = (u0 >> sh) & 63;
-        mn = (u1 >> sh) & 63;
-    } else {
-        sc = ((u2 >> sh) & 0xF) | (((u0 >> (sh + 6)) & 3) << 4);
-        mn = ((u2 >> (sh + 4)) & 0xF) | (((u1 >> (sh + 6)) & 3) << 4);
-    }
+    // Branch-free (lanes of one wave differ in j): for j < 4 the value is one 6-bit field; for
+    // j >= 4 it is a 4-bit field of u2 plus the two top bits of byte j-4 of u0 / u1.
+    const bool first = j < 4;
+    const uint32_t sh = 8u * (uint32_t)(j & 3);
+    const uint32_t wlo = first ? 6u : 4u, whi = first ? 0u : 2u;   // a zero-width field reads as 0
+    sc = (int)(__builtin_amdgcn_ubfe(first ? u0 : u2, sh, wlo) | (__builtin_amdgcn_ubfe(u0, sh + 6, whi) << 4));
+    mn = (int)(__builtin_amdgcn_ubfe(first ? u1 : u2, first ? sh : sh + 4, wlo) |
+               (__builtin_amdgcn_ubfe(u1, sh + 6, whi) << 4));
 }
 #endif

@@ -61,6 +61,8 @@ __global__ void repack_q4k(const uint8_t *__restrict__ aos, uint8_t *__restrict_
 //   high nibble: element 128h + 64 + 32t + 16i + e   hi bits = qh[32h + 16i + e] >> (2t + 4)
 //   qh'[8u + 4x + c] (x < 2, c < 4) =   lo2(8x + c)       | hi2(8x + c) << 2
 //                                      | lo2(8x + 4 + c) << 4 | hi2(8x + 4 + c) << 6
+//   sc'[2u], sc'[2u + 1] = scales[js], scales[js + 4] with js = u + 4h: the scales of the lane's
+//   low-nibble and high-nibble 16-element groups, one 2-byte load per lane.
 // i.e. for the two ql words 2x and 2x+1 of the lane, (H >> {0,2,4,6}) & 0x03030303 lines the
 // two high bits up with each byte of {word 2x low, word 2x high, word 2x+1 low, word 2x+1 high}.
 __global__ void repack_q6k(const uint8_t *__restrict__ aos, uint8_t *__restrict__ ql, uint8_t *__restrict__ qh,
@@ -84,14 +86,17 @@ __global__ void repack_q6k(const uint8_t *__restrict__ aos, uint8_t *__restrict_
                                       (((s1 >> (2 * tt)) & 3) << 4) | (((s1 >> (2 * tt + 4)) & 3) << 6));
                 pqh[4 * x + c] = v;
             }
-        if (u == 0) {
-            for (int e = 0; e < 16; e++) sc[b * 16 + e] = a_sc[e];
-            d[b] = (uint16_t)(a_d[0] | (a_d[1] << 8));
-        }
+        // the lane's two 16-element scale groups (low nibbles: js, high nibbles: js + 4) side by side
+        const int js = u + 4 * h;
+        sc[b * 16 + 2 * u] = a_sc[js];
+        sc[b * 16 + 2 * u + 1] = a_sc[js + 4];
+        if (u == 0) d[b] = (uint16_t)(a_d[0] | (a_d[1] << 8));
     } else {
         for (int e = 0; e < 16; e++) a_ql[16 * u + e] = pql[e];
+        const int js = u + 4 * h;
+        a_sc[js] = sc[b * 16 + 2 * u];
+        a_sc[js + 4] = sc[b * 16 + 2 * u + 1];
         if (u == 0) {
-            for (int e = 0; e < 16; e++) a_sc[e] = sc[b * 16 + e];
             a_d[0] = (uint8_t)(d[b] & 0xff);
             a_d[1] = (uint8_t)(d[b] >> 8);
         }

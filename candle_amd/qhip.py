@@ -11,11 +11,11 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libcandle_qhip.so")
+LIB_PATH = os.environ.get("CQ_LIB_PATH", os.path.join(_HERE, "lib", "libcandle_qhip.so"))
 
 # GgmlDType ids (candle-core/src/quantized/mod.rs:173-190)
 Q4_0, Q8_0, Q8_1, Q4K, Q6K, Q8K = 2, 8, 9, 12, 14, 15
-FLAG_AUTO, FLAG_FORCE_MATVEC, FLAG_FORCE_GEMM, FLAG_ACT_Q8_1 = 0, 1, 2, 4
+FLAG_AUTO, FLAG_FORCE_MATVEC, FLAG_FORCE_GEMM, FLAG_ACT_Q8_1, FLAG_REUSE_ACT, FLAG_STAGED_ACT = 0, 1, 2, 4, 8, 16
 
 EXPORTS = [
     "cq_device_count", "cq_last_error", "cq_version", "cq_block_size", "cq_type_size", "cq_vec_dot_type",

@@ -51,8 +51,13 @@ enum {
     CQ_FLAG_AUTO = 0,
     CQ_FLAG_FORCE_MATVEC = 1, /* row-streaming kernel whatever m is (A/B runs; replaces cuda.rs:22-26 set_force_dmmv) */
     CQ_FLAG_FORCE_GEMM = 2,   /* int8-MFMA tile kernel whatever m is                                                  */
-    CQ_FLAG_ACT_Q8_1 = 4      /* K-quant weights x Q8_1 activations (the reference CUDA formulation, cuda.rs:322-326)
+    CQ_FLAG_ACT_Q8_1 = 4,     /* K-quant weights x Q8_1 activations (the reference CUDA formulation, cuda.rs:322-326)
                                  instead of the CPU formulation's Q8K; not bit-comparable with the CPU QMatMul        */
+    CQ_FLAG_REUSE_ACT = 8,    /* the workspace already holds this x, quantized by an earlier cq_qmatmul call with the
+                                 same m, k and activation format (q/k/v or gate/up share their input): skip the
+                                 quantizer launch.  No counterpart in the reference, which re-quantizes per call.     */
+    CQ_FLAG_STAGED_ACT = 16   /* m == 1 only: run the stand-alone quantizer into the workspace and the plain matvec
+                                 (two launches, as cuda.rs:249-293 does) instead of the single fused launch           */
 };
 
 typedef struct cq_weight cq_weight;

@@ -179,3 +179,35 @@ def moe_ffn(dtype13: int, dtype2: int, w1, w2, w3, hidden: int, ffn: int, xs, of
                              offsets.ctypes.data_as(i32p), row_ids.ctypes.data_as(i32p),
                              weights.ctypes.data_as(f32p), ys.ctypes.data_as(f32p)), "moe_ffn")
     return ys
+
+
+# ------------------------------------------------------------------ timed CPU baseline ----
+_BASE_PATH = os.path.join(_HERE, "libcandle_q_cpu_baseline.so")
+_base = None
+
+
+def baseline_lib():
+    """AVX2 + OpenMP restatement of the reference's CPU QMatMul (oracle/cpu_baseline.cpp)."""
+    global _base
+    if _base is None:
+        src = os.path.join(_HERE, "cpu_baseline.cpp")
+        if (not os.path.exists(_BASE_PATH)) or os.path.getmtime(_BASE_PATH) < os.path.getmtime(src):
+            subprocess.check_call(["make", "-C", _HERE, "libcandle_q_cpu_baseline.so"])
+        L = C.CDLL(_BASE_PATH)
+        L.cpub_matmul.argtypes = [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.POINTER(C.c_float), C.c_void_p,
+                                  C.POINTER(C.c_float)]
+        L.cpub_num_threads.restype = C.c_int
+        L.cpub_set_num_threads.argtypes = [C.c_int]
+        L.cpub_set_num_threads.restype = None
+        _base = L
+    return _base
+
+
+def baseline_matmul(dtype: int, lhs, rhs_blocks: np.ndarray, n: int, out=None) -> np.ndarray:
+    lhs, lp = _f32(lhs)
+    m, k = lhs.shape
+    rhs_blocks = np.ascontiguousarray(rhs_blocks, dtype=np.uint8)
+    dst = out if out is not None else np.empty((m, n), dtype=np.float32)
+    _check(baseline_lib().cpub_matmul(dtype, m, k, n, lp, rhs_blocks.ctypes.data,
+                                      dst.ctypes.data_as(C.POINTER(C.c_float))), "baseline matmul")
+    return dst

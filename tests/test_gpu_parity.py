@@ -169,6 +169,24 @@ def test_matvec_matches_oracle(qh, dt, m, k, n):
     check_f32(got, orc.matmul(dt, x, blocks, n))
 
 
+@pytest.mark.parametrize("dt", WEIGHT_DTYPES)
+@pytest.mark.parametrize("k,n", [(256, 7), (512, 300), (4096, 1000), (11008, 129), (14336, 65)])
+def test_fused_decode_equals_two_launch_path(qh, dt, k, n):
+    """m = 1 runs as one launch with the activation quantizer in the kernel prologue.  Its result
+    must equal, bit for bit, the stand-alone quantizer (checked bit-exact above) followed by the
+    plain matvec: same quantized activations, same accumulation order."""
+    w, x = make_inputs(31 * dt + k, 1, k, n, outliers=True)
+    big = np.float32(np.abs(x).max() + 1.0)          # |x| tie with opposite signs inside the first block
+    x[0, 5], x[0, 9] = big, -big
+    qw = qh.QWeight.from_ggml(dt, orc.quantize(dt, w), n, k)
+    xd = dev(x)
+    fused = qh.qmatmul(qw, xd)
+    staged = qh.qmatmul(qw, xd, qh.FLAG_STAGED_ACT)
+    assert torch.equal(fused, staged)
+    x[:] = 0.0
+    assert torch.equal(qh.qmatmul(qw, dev(x)), torch.zeros((1, n), device="cuda"))
+
+
 @pytest.mark.parametrize("dt", [orc.Q4K, orc.Q8_0])
 @pytest.mark.parametrize("m", [2, 4, 8, 16])
 @pytest.mark.parametrize("k,n", [(4096, 4096), (4096, 11008)])
