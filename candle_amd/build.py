@@ -16,11 +16,14 @@ SOURCES = ["api.hip", "repack.hip", "quantize_act.hip", "quantize_weight.hip", "
 # -packed-fp32-ops off: packed FP32 instructions are not to be generated on this hardware pool.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fno-fast-math",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function"]
+# gemm.hip: MFMA results are consumed by VALU code every block; keep the accumulators in ordinary
+# VGPRs rather than AccVGPRs, which VALU instructions cannot read.
+EXTRA_FLAGS = {"gemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 def _compile(src: str) -> str:
     obj = os.path.join(LIB_DIR, src.replace(".hip", ".o"))
-    cmd = ["hipcc", *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = ["hipcc", *FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     err = "\n".join(l for l in r.stderr.splitlines() if noise not in l)

@@ -250,7 +250,11 @@ static size_t act_ws_layout(int act_dtype, int64_t m, int64_t k, uint8_t *base, 
     if (act_dtype == CQ_DTYPE_Q8K) {
         const size_t o_d = take((size_t)(m * (k / 256)) * 4);
         const size_t o_bs = take((size_t)(m * (k / 256)) * 32);
-        if (base) { view.qs = (int8_t *)(base + o_qs); view.d = (float *)(base + o_d); view.bsums = (int16_t *)(base + o_bs); }
+        const size_t o_mp = take((size_t)(m * (k / 256)) * 32);
+        if (base) {
+            view.qs = (int8_t *)(base + o_qs); view.d = (float *)(base + o_d);
+            view.bsums = (int16_t *)(base + o_bs); view.minp = (uint16_t *)(base + o_mp);
+        }
     } else {
         const size_t o_d = take((size_t)(m * (k / 32)) * 4);
         const size_t o_s = take((size_t)(m * (k / 32)) * 4);
@@ -380,6 +384,7 @@ extern "C" int cq_qmatmul_grouped(const cq_weight *const *experts, int n_experts
         if (act == CQ_DTYPE_Q8K) {
             ve.d += r0 * (w0->k / 256);
             ve.bsums += r0 * (w0->k / 256) * 16;
+            ve.minp += r0 * (w0->k / 256) * 16;
         } else {
             ve.d += r0 * (w0->k / 32);
             ve.bsum32 += r0 * (w0->k / 32);

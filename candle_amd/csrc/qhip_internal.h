@@ -55,6 +55,7 @@ struct cq_act_view {
     int8_t *qs;
     float *d;
     int16_t *bsums;  // Q8K
+    uint16_t *minp;  // Q8K: [m][k/256][16] f16, d * sub-block sums as two f16 pieces (GEMM min term)
     int32_t *bsum32; // Q8_0 / Q8_1
     uint16_t *s16;   // Q8_1: the block's `s` field (f16 bits)
 };

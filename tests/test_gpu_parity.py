@@ -199,6 +199,49 @@ def test_small_batch_matches_oracle(qh, dt, m, k, n):
     check_f32(got, orc.matmul(dt, x, blocks, n))
 
 
+@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K])
+@pytest.mark.parametrize("m,k,n", [(9, 256, 32), (33, 512, 70), (64, 1024, 129), (130, 768, 257), (11, 512, 21)])
+def test_gemm_matches_oracle_small(qh, dt, m, k, n):
+    """The int8-MFMA tile kernel on ragged shapes (m, n not multiples of the tile; one K block)."""
+    w, x = make_inputs(3 * dt + m + k + n, m, k, n, outliers=True)
+    blocks = orc.quantize(dt, w)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    got = qh.qmatmul(qw, dev(x), qh.FLAG_FORCE_GEMM).cpu().numpy()
+    check_f32(got, orc.matmul(dt, x, blocks, n))
+
+
+@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K])
+@pytest.mark.parametrize("m,k,n", [(512, 4096, 14336), (512, 14336, 4096)])
+def test_prefill_gemm_config3(qh, dt, m, k, n):
+    """BASELINE config 3 at full size: M = 512 tokens on the Mistral FFN shapes, activations N(0,1)
+    with 1% outliers at +-8 sigma.  Weights are quantized on the device (bit-identical to the CPU
+    quantizer, checked above); the oracle evaluates a sample of 96 weight rows over all 512 tokens,
+    and the whole output is checked for batch invariance against the decode kernel on 4 rows."""
+    rng = np.random.default_rng(k + dt)
+    gen = torch.Generator(device="cuda").manual_seed(k + dt)
+    wt = torch.randn((n, k), generator=gen, device="cuda") * 0.02
+    qw = qh.QWeight.zeros(dt, n, k).quantize_(wt)
+    del wt
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    idx = rng.choice(x.size, size=x.size // 100, replace=False)
+    x.ravel()[idx] = np.where(rng.random(idx.size) < 0.5, -8.0, 8.0).astype(np.float32)
+    xd = dev(x)
+    got = qh.qmatmul(qw, xd).cpu().numpy()                      # m > 8: MFMA kernel
+    rows = np.sort(rng.choice(n, size=96, replace=False))
+    row_bytes = k // 256 * orc.TYPE_SIZE[dt]
+    blocks = qw.to_ggml().reshape(n, row_bytes)[rows].ravel()
+    want = orc.matmul(dt, x, blocks, len(rows))
+    g = got[:, rows].astype(np.float64)
+    err = np.linalg.norm(g - want) / np.linalg.norm(want)
+    assert err <= REL_L2_TOL, err
+    for r in range(0, m, 37):
+        # max-abs bar, with ||row||_2 scaled from the sampled columns to the full row
+        nrm = np.linalg.norm(want[r]) * np.sqrt(n / len(rows))
+        assert np.abs(g[r] - want[r]).max() <= MAX_ABS_FACTOR * nrm
+    mv = qh.qmatmul(qw, xd[:4].contiguous(), qh.FLAG_FORCE_MATVEC).cpu().numpy()
+    assert np.linalg.norm(got[:4] - mv) / np.linalg.norm(mv) <= 1e-5
+
+
 def test_reference_goldens_through_hip(qh, goldens, seeded_inputs):
     # quantized_tests.rs:49-64 and :109-129 (Q4_0, m=3, k=64, n=4)
     m, k, n = 3, 64, 4
