@@ -245,15 +245,20 @@ extern "C" int cq_quantize_act(int dev, int act_dtype, const float *x_dev, int64
 static size_t act_ws_layout(int act_dtype, int64_t m, int64_t k, uint8_t *base, cq_act_view *v) {
     size_t off = 0;
     auto take = [&](size_t bytes) { size_t o = off; off = cq_align_up(off + bytes, 256); return o; };
-    const size_t o_qs = take((size_t)(m * k));
+    // Q8K rows are padded (see cq_act_view::m_stride)
+    const int64_t m_pad = act_dtype == CQ_DTYPE_Q8K ? (m + 63) / 64 * 64 + 256 : m;
+    const size_t o_qs = take((size_t)(m_pad * k));
     cq_act_view view{};
+    view.m_stride = m_pad;
     if (act_dtype == CQ_DTYPE_Q8K) {
         const size_t o_d = take((size_t)(m * (k / 256)) * 4);
         const size_t o_bs = take((size_t)(m * (k / 256)) * 32);
-        const size_t o_mp = take((size_t)(m * (k / 256)) * 32);
+        const size_t o_dt = take((size_t)(m_pad * (k / 256)) * 4);
+        const size_t o_mp = take((size_t)(m_pad * (k / 256)) * 32);
         if (base) {
             view.qs = (int8_t *)(base + o_qs); view.d = (float *)(base + o_d);
-            view.bsums = (int16_t *)(base + o_bs); view.minp = (uint16_t *)(base + o_mp);
+            view.bsums = (int16_t *)(base + o_bs); view.dT = (float *)(base + o_dt);
+            view.minp = (uint16_t *)(base + o_mp);
         }
     } else {
         const size_t o_d = take((size_t)(m * (k / 32)) * 4);
@@ -384,7 +389,8 @@ extern "C" int cq_qmatmul_grouped(const cq_weight *const *experts, int n_experts
         if (act == CQ_DTYPE_Q8K) {
             ve.d += r0 * (w0->k / 256);
             ve.bsums += r0 * (w0->k / 256) * 16;
-            ve.minp += r0 * (w0->k / 256) * 16;
+            ve.dT += r0;
+            ve.minp += r0 * 16;
         } else {
             ve.d += r0 * (w0->k / 32);
             ve.bsum32 += r0 * (w0->k / 32);

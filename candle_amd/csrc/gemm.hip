@@ -17,11 +17,13 @@
 //
 // Work split: a workgroup of four waves covers BM = 32*MT activation rows x 128 weight rows; each
 // wave owns 32 weight rows (MFMA B operand: lane l holds row l%32, k = 16*(l/32)+[0,16) of a
-// 32-wide K-slice) and unpacks them from HBM straight into registers - no LDS for weights; the
-// next block's weight bytes are loaded one block ahead.  The activation tile of a block (MFMA A
-// operands, already in fragment order) goes from global memory straight into LDS with
-// global_load_lds_dwordx4, double buffered, and is shared by the four waves.  With few workgroups
-// (small n) K is split over blockIdx.z and the partial results are added atomically.
+// 32-wide K-slice) and unpacks them in registers.  Activations (shared by the four waves) and each
+// wave's packed weight bytes go from global memory straight into LDS (global_load_lds_dwordx4),
+// double buffered, one block ahead.  Every such copy instruction reads eight whole 128-byte lines
+// (8 rows x 128 B) - the texture path pays per line touched - and the 16-byte chunks of a row are
+// XOR-swizzled by the row number on the way in, so that the MFMA operand reads (lanes = rows, one
+// chunk column) spread over all LDS banks.  With few workgroups (small n) K is split over
+// blockIdx.z and the partial results are added atomically.
 #include "qhip_internal.h"
 #include <stdlib.h>
 
@@ -29,6 +31,7 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef unsigned short us2 __attribute__((ext_vector_type(2)));
@@ -39,15 +42,19 @@ typedef void __attribute__((address_space(3))) *lptr_t;
 constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * 64;
 
-// LDS image of one block's activation tile (BM = 32*MT rows):
-//   frag : [MT][8 slices][64 lanes][16 B]   A operands, lane l = row l%32, k = 32*slice + 16*(l/32) + [0,16)
+// LDS image of one pipeline stage:
+//   act  : [MT tiles][2 K-halves][4 row groups][8 rows][8 chunks of 16 B]   chunk c of row r sits at c ^ (r%8)
 //   d8   : [BM] f32
 //   minp : [BM][2 pieces][8] f16            d8 * bsum32_j split in two f16 pieces (Q4K)
-template <int MT> struct Tile {
-    static constexpr int kFrag = MT * 8 * 1024;
+//   wgt  : per wave: [4 row groups][8 rows][8 chunks] of the 128-byte qs / ql plane (same swizzle),
+//          Q6K also [2 row groups][16 rows][4 chunks] of the 64-byte qh plane (chunk c at c ^ ((r/2)%4))
+template <int DT, int MT> struct Tile {
+    static constexpr int kAct = MT * 8 * 1024;
     static constexpr int kD8 = (MT * 32 < 64 ? 64 : MT * 32) * 4;   // filled by whole-wave copies of 64 floats
-    static constexpr int kMin = MT * 32 * 32;
-    static constexpr int kBytes = kFrag + kD8 + kMin;
+    static constexpr int kMin = DT == CQ_DTYPE_Q4K ? MT * 32 * 32 : 0;
+    static constexpr int kWgtWave = DT == CQ_DTYPE_Q4K ? 4096 : 6144;
+    static constexpr int oD8 = kAct, oMin = oD8 + kD8, oWgt = oMin + kMin;
+    static constexpr int kBytes = oWgt + kWaves * kWgtWave;
 };
 
 __device__ __forceinline__ uint32_t pk_mul_u16(uint32_t a, uint32_t b) {
@@ -64,65 +71,89 @@ __device__ __forceinline__ uint32_t pk_ashr7_i16(uint32_t a) {
 }
 __device__ __forceinline__ uint32_t dup16(uint32_t v) { return (v & 0xffffu) | (v << 16); }
 
-// Asynchronous global -> LDS copies of one block's activation tile, issued by every wave for its
-// share of the 1 KiB fragments.  Lane l of a wave-wide copy lands at dst + 16*l (or 4*l), whatever
-// global address it reads from, so the fragment order is produced by the address computation
-// alone.  Rows past m read a clamped row; their outputs are never stored.
-template <int MT, bool MINS>
-__device__ __forceinline__ void stage_issue(uint8_t *buf, const cq_act_view &a, int64_t m, int64_t k, int64_t m0,
-                                            int64_t b, int wave, int lane) {
-    const int64_t kb = k >> 8;
-    const int64_t last = m - 1;
-    for (int f = wave; f < MT * 8; f += kWaves) {
-        const int mt = f >> 3, s = f & 7;
-        int64_t row = m0 + mt * 32 + (lane & 31);
-        row = row < last ? row : last;
-        const int8_t *src = a.qs + row * k + b * 256 + s * 32 + (lane >> 5) * 16;
-        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(buf + f * 1024), 16, 0, 0);
+// Asynchronous copy of 64 x 16 (or 64 x 4) bytes: lane l reads base + off and the data lands at
+// lds + 16*l (4*l).  `base` and `lds` are wave-uniform.
+__device__ __forceinline__ void dma16(const void *base, uint32_t off, uint8_t *lds) {
+    __builtin_amdgcn_global_load_lds((gptr_t)((const uint8_t *)base + off), (lptr_t)lds, 16, 0, 0);
+}
+__device__ __forceinline__ void dma4(const void *base, uint32_t off, uint8_t *lds) {
+    __builtin_amdgcn_global_load_lds((gptr_t)((const uint8_t *)base + off), (lptr_t)lds, 4, 0, 0);
+}
+
+// Per-lane constants of the copies and of the operand reads.
+struct LaneGeo {
+    uint32_t act_off;   // copy of 8 rows x 128 B of activations: (l/8)*k + ((l%8) ^ (l/8))*16
+    uint32_t wq_off;    // the same over the weights' 128-byte plane: (l/8)*kb*128 + ...
+    uint32_t wh_off;    // Q6K qh plane, 16 rows x 64 B: (l/4)*kb*64 + ((l%4) ^ ((l/8)%4))*16
+    uint32_t col[4];    // operand read: byte offset of chunk 2j+h of row l%32 inside a [4][8][8] x 16 B image
+    uint32_t qh_col[4]; // Q6K: byte offset of the 8 bytes of unit 2x+h of row l%32 inside the qh image
+};
+
+__device__ __forceinline__ LaneGeo lane_geo(int lane, int64_t k) {
+    LaneGeo g;
+    const uint32_t kb = (uint32_t)(k >> 8);
+    const uint32_t r8 = lane >> 3, c8 = lane & 7;
+    g.act_off = r8 * (uint32_t)k + ((c8 ^ r8) << 4);
+    g.wq_off = r8 * kb * 128u + ((c8 ^ r8) << 4);
+    const uint32_t r16 = lane >> 2, c4 = lane & 3;
+    g.wh_off = r16 * kb * 64u + ((c4 ^ ((r16 >> 1) & 3)) << 4);
+    const uint32_t r = lane & 31, h = lane >> 5;
+#pragma unroll
+    for (uint32_t j = 0; j < 4; j++) {
+        g.col[j] = (r >> 3) * 1024u + (r & 7) * 128u + (((2 * j + h) ^ (r & 7)) << 4);
+        g.qh_col[j] = (r >> 4) * 1024u + (r & 15) * 64u + ((j ^ ((r >> 1) & 3)) << 4) + h * 8u;
     }
-    for (int c = wave; c < (MT * 32 + 63) / 64; c += kWaves) {
-        int64_t row = m0 + c * 64 + lane;
-        row = row < last ? row : last;
-        __builtin_amdgcn_global_load_lds((gptr_t)(a.d + row * kb + b), (lptr_t)(buf + Tile<MT>::kFrag + c * 256), 4, 0, 0);
+    return g;
+}
+
+// Issues this wave's share of the copies for block b into stage `buf`.
+template <int DT, int MT>
+__device__ __forceinline__ void stage_issue(uint8_t *buf, const cq_weight &w, const cq_act_view &a, const LaneGeo &g,
+                                            int64_t m0, int64_t n_tile, bool n_ok, int64_t b, int wave, int lane) {
+    typedef Tile<DT, MT> T;
+    const int64_t k = w.k, kb = w.k >> 8;
+    // activations: MT*8 copies of 8 rows x 128 B, dealt round-robin to the waves
+#pragma unroll
+    for (int j = 0; j < MT * 8 / kWaves; j++) {
+        const int idx = wave + kWaves * j;           // = (t*2 + kh)*4 + rg
+        const int rg = idx & 3, kh = (idx >> 2) & 1, t = idx >> 3;
+        const int8_t *base = a.qs + (m0 + t * 32 + rg * 8) * k + b * 256 + kh * 128;
+        dma16(base, g.act_off, buf + idx * 1024);
     }
-    if (MINS) {
-        for (int c = wave; c < MT; c += kWaves) {
-            int64_t row = m0 + c * 32 + (lane >> 1);
-            row = row < last ? row : last;
-            const uint16_t *src = a.minp + (row * kb + b) * 16 + (lane & 1) * 8;
-            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(buf + Tile<MT>::kFrag + Tile<MT>::kD8 + c * 1024), 16,
-                                             0, 0);
+#pragma unroll
+    for (int j = 0; j < (MT * 32 + 63) / 64; j++) {
+        if ((j & 3) == wave) dma4(a.dT + b * a.m_stride + m0 + j * 64, lane * 4u, buf + T::oD8 + j * 256);
+    }
+    if (DT == CQ_DTYPE_Q4K) {
+#pragma unroll
+        for (int j = 0; j < MT; j++) {
+            if (((j + 1) & 3) == wave)
+                dma16(a.minp + (b * a.m_stride + m0 + j * 32) * 16, lane * 16u, buf + T::oMin + j * 1024);
+        }
+    }
+    // this wave's 32 weight rows
+    if (n_ok) {
+        uint8_t *wl = buf + T::oWgt + wave * T::kWgtWave;
+#pragma unroll
+        for (int rg = 0; rg < 4; rg++) dma16(w.p0 + ((n_tile + rg * 8) * kb + b) * 128, g.wq_off, wl + rg * 1024);
+        if (DT == CQ_DTYPE_Q6K) {
+#pragma unroll
+            for (int rg = 0; rg < 2; rg++)
+                dma16(w.p1 + ((n_tile + rg * 16) * kb + b) * 64, g.wh_off, wl + 4096 + rg * 1024);
         }
     }
 }
 
-// One block of one weight row as this lane needs it (row n, k-half h = lane / 32).
-template <int DT> struct WBlk;
-template <> struct WBlk<CQ_DTYPE_Q4K> {
-    uint4 q[4];   // qs bytes 32g + 16h + [0,16): low nibbles = K-slice 2g, high nibbles = slice 2g+1
-    uint4 hd;     // d, dmin, scales[12]
-};
-template <> struct WBlk<CQ_DTYPE_Q6K> {
-    uint4 q[4];   // ql lanes of the four units of this k-half: u = 4*(x/2) + 2*(x%2) + h
-    uint2 qh[4];  // their re-packed high bits
-    uint4 sc;     // re-packed scales: bytes 2u, 2u+1 = scale of the unit's low / high nibble group
-    uint32_t d;
-};
-
-__device__ __forceinline__ void load_w(const cq_weight &w, int64_t blk, int h, WBlk<CQ_DTYPE_Q4K> &r) {
+// The small per-block weight fields, loaded straight into registers one block ahead.
+template <int DT> struct WHead;
+template <> struct WHead<CQ_DTYPE_Q4K> { uint4 hd; };               // d, dmin, scales[12]
+template <> struct WHead<CQ_DTYPE_Q6K> { uint4 sc; uint32_t d; };   // re-packed scales (two per unit); d
+__device__ __forceinline__ void load_head(const cq_weight &w, int64_t blk, WHead<CQ_DTYPE_Q4K> &r) {
     r.hd = *(const uint4 *)(w.p1 + blk * 16);
-#pragma unroll
-    for (int g = 0; g < 4; g++) r.q[g] = *(const uint4 *)(w.p0 + blk * 128 + 32 * g + 16 * h);
 }
-__device__ __forceinline__ void load_w(const cq_weight &w, int64_t blk, int h, WBlk<CQ_DTYPE_Q6K> &r) {
+__device__ __forceinline__ void load_head(const cq_weight &w, int64_t blk, WHead<CQ_DTYPE_Q6K> &r) {
     r.sc = *(const uint4 *)(w.p2 + blk * 16);
     r.d = ((const uint16_t *)w.p3)[blk];
-#pragma unroll
-    for (int x = 0; x < 4; x++) {
-        const int u = 4 * (x >> 1) + 2 * (x & 1) + h;
-        r.q[x] = *(const uint4 *)(w.p0 + blk * 128 + 16 * u);
-        r.qh[x] = *(const uint2 *)(w.p1 + blk * 64 + 8 * u);
-    }
 }
 
 // One block for this wave's 32 weight rows against the MT activation tiles in `cur`, as a
@@ -131,20 +162,25 @@ __device__ __forceinline__ void load_w(const cq_weight &w, int64_t blk, int h, W
 // LDS reads run two steps ahead.  The accumulator pair alternates between two register sets.  A
 // scheduling barrier after every step keeps the compiler from hoisting all MFMAs to the front,
 // which would need MT accumulator sets at once.
-template <int MT, bool MINS, int SHIFT>
-__device__ __forceinline__ void tiles_mac(const uint8_t *cur, const v4i (&bl)[8], const v4i (&bh)[8], float dw,
-                                          v8h wmin, int lane, v16f (&out)[MT]) {
-    typedef float v4f __attribute__((ext_vector_type(4)));
+template <int DT, int MT, int SHIFT>
+__device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, const v4i (&bl)[8], const v4i (&bh)[8],
+                                          float dw, v8h wmin, int lane, v16f (&out)[MT]) {
+    typedef Tile<DT, MT> T;
+    constexpr bool MINS = DT == CQ_DTYPE_Q4K;
     const int h = lane >> 5, col = lane & 31;
-    const uint8_t *afrag = cur + lane * 16;
-    const uint8_t *d8p = cur + Tile<MT>::kFrag + h * 16;                    // rows 8j + 4h + [0,4) of a tile
-    const uint8_t *mnp = cur + Tile<MT>::kFrag + Tile<MT>::kD8 + col * 32;   // this lane's row of min pieces
+    const uint8_t *d8p = cur + T::oD8 + h * 16;        // rows 8j + 4h + [0,4) of a tile
+    const uint8_t *mnp = cur + T::oMin + col * 32;     // this lane's row of min pieces
+    // operand of tile t, K-slice s: chunk 2*(s%4) + h of K-half s/4
+    auto afrag = [&](int q) -> v4i {
+        const int t = q >> 3, s = q & 7;
+        return *(const v4i *)(cur + g.col[s & 3] + (t * 2 + (s >> 2)) * 4096);
+    };
     v16i acc_lo[2], acc_hi[2];
     v4i a[3];
     v4f dsc[2][4];
     v8h ma1, ma2;
-    a[0] = *(const v4i *)(afrag);
-    a[1] = *(const v4i *)(afrag + 1024);
+    a[0] = afrag(0);
+    a[1] = afrag(1);
     if (MINS) {
         ma1 = *(const v8h *)(mnp);
         ma2 = *(const v8h *)(mnp + 16);
@@ -152,7 +188,7 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const v4i (&bl)[8]
 #pragma unroll
     for (int q = 0; q < (MT + 1) * 8; q++) {
         const int t = q >> 3, s = q & 7;
-        if (q + 2 < MT * 8) a[(q + 2) % 3] = *(const v4i *)(afrag + (q + 2) * 1024);
+        if (q + 2 < MT * 8) a[(q + 2) % 3] = afrag(q + 2);
         if (t < MT) {
             if (s == 0) {
                 if (MINS) {
@@ -181,11 +217,7 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const v4i (&bl)[8]
         if (t > 0) {
             const int p = (t - 1) & 1;
 #pragma unroll
-#ifdef EXP_NO_EPI
-            for (int i = 2 * s; i < 2 * s + (s == 0 ? 1 : 0); i++) {
-#else
             for (int i = 2 * s; i < 2 * s + 2; i++) {
-#endif
                 const int I = (acc_hi[p][i] << SHIFT) + acc_lo[p][i];
                 float o = __builtin_fmaf((float)I * dw, dsc[p][i >> 2][i & 3], out[t - 1][i]);
                 asm volatile("" : "+v"(o));   // pins the scaling to this step (pure ops float otherwise)
@@ -197,7 +229,8 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const v4i (&bl)[8]
 }
 
 template <int MT>
-__device__ __forceinline__ void block_mac(const uint8_t *cur, const WBlk<CQ_DTYPE_Q4K> &wb, int lane, v16f (&out)[MT]) {
+__device__ __forceinline__ void block_mac(const uint8_t *cur, const uint8_t *wl, const LaneGeo &g,
+                                          const WHead<CQ_DTYPE_Q4K> &wb, int lane, v16f (&out)[MT]) {
     const int h = lane >> 5;
     const uint4 hd = wb.hd;
     const float dw = cq_h2f((uint16_t)(hd.x & 0xffff));
@@ -209,18 +242,20 @@ __device__ __forceinline__ void block_mac(const uint8_t *cur, const WBlk<CQ_DTYP
     const uint32_t mn47 = ((hd.w >> 4) & 0x0f0f0f0fu) | (((hd.z >> 6) & 0x03030303u) << 4);
     v4i bl[8], bh[8];
 #pragma unroll
-    for (int g = 0; g < 4; g++) {
-        const uint32_t scw = g < 2 ? sc03 : sc47;
-        const uint32_t s0 = (scw >> (16 * (g & 1))) & 0xff, s1 = (scw >> (16 * (g & 1) + 8)) & 0xff;
+    for (int gi = 0; gi < 4; gi++) {
+        // qs bytes 32g + 16h + [0,16): low nibbles = K-slice 2g, high nibbles = slice 2g+1
+        const uint4 q = *(const uint4 *)(wl + g.col[gi]);
+        const uint32_t scw = gi < 2 ? sc03 : sc47;
+        const uint32_t s0 = (scw >> (16 * (gi & 1))) & 0xff, s1 = (scw >> (16 * (gi & 1) + 8)) & 0xff;
         const uint32_t sl0 = dup16(s0 & 7), sh0 = dup16(s0 >> 3), sl1 = dup16(s1 & 7), sh1 = dup16(s1 >> 3);
-        const uint32_t qw[4] = {wb.q[g].x, wb.q[g].y, wb.q[g].z, wb.q[g].w};
+        const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const uint32_t lo4 = qw[i] & 0x0F0F0F0Fu, hi4 = (qw[i] >> 4) & 0x0F0F0F0Fu;
-            bl[2 * g][i] = (int)pk_mul_u16(lo4, sl0);       // sub-block 2g, low digit of the scale
-            bh[2 * g][i] = (int)pk_mul_u16(lo4, sh0);
-            bl[2 * g + 1][i] = (int)pk_mul_u16(hi4, sl1);   // sub-block 2g+1
-            bh[2 * g + 1][i] = (int)pk_mul_u16(hi4, sh1);
+            bl[2 * gi][i] = (int)pk_mul_u16(lo4, sl0);       // sub-block 2g, low digit of the scale
+            bh[2 * gi][i] = (int)pk_mul_u16(lo4, sh0);
+            bl[2 * gi + 1][i] = (int)pk_mul_u16(hi4, sl1);   // sub-block 2g+1
+            bh[2 * gi + 1][i] = (int)pk_mul_u16(hi4, sh1);
         }
     }
     v8h wmin;
@@ -231,26 +266,35 @@ __device__ __forceinline__ void block_mac(const uint8_t *cur, const WBlk<CQ_DTYP
         const _Float16 p1 = (_Float16)v;
         wmin[j] = h == 0 ? p1 : (_Float16)(v - (float)p1);
     }
-    tiles_mac<MT, true, 3>(cur, bl, bh, dw, wmin, lane, out);
+    tiles_mac<CQ_DTYPE_Q4K, MT, 3>(cur, g, bl, bh, dw, wmin, lane, out);
 }
 
 template <int MT>
-__device__ __forceinline__ void block_mac(const uint8_t *cur, const WBlk<CQ_DTYPE_Q6K> &wb, int lane, v16f (&out)[MT]) {
+__device__ __forceinline__ void block_mac(const uint8_t *cur, const uint8_t *wl, const LaneGeo &g,
+                                          const WHead<CQ_DTYPE_Q6K> &wb, int lane, v16f (&out)[MT]) {
     const int h = lane >> 5;
     const float dw = cq_h2f((uint16_t)wb.d);
     const uint32_t scw[4] = {wb.sc.x, wb.sc.y, wb.sc.z, wb.sc.w};
+    uint4 ql[4];
+    uint2 qhv[4];
+#pragma unroll
+    for (int x = 0; x < 4; x++) {
+        // ql lane of unit u = 2x + h and its re-packed high bits
+        ql[x] = *(const uint4 *)(wl + g.col[x]);
+        qhv[x] = *(const uint2 *)(wl + 4096 + g.qh_col[x]);
+    }
     v4i bl[8], bh[8];
 #pragma unroll
     for (int s = 0; s < 8; s++) {
-        // K-slice s: this lane's 16 elements are the group G = 2s + h, i.e. unit
-        // u = 4*(s/4) + 2*(s%2) + h, low nibbles when (s%4) < 2 else high nibbles
+        // K-slice s: this lane's 16 elements are the group G = 2s + h, i.e. unit u = 2x + h with
+        // x = 2*(s/4) + s%2, low nibbles when (s%4) < 2 else high nibbles
         const int x = 2 * (s >> 2) + (s & 1), nib = (s & 3) >> 1;
-        const int sb = 2 * (4 * (x >> 1) + 2 * (x & 1)) + nib;   // scale byte index for h = 0; h adds 2
-        const uint32_t sw = scw[sb >> 2];                         // bytes sb and sb + 2 are in the same word
+        const int sb = 4 * x + nib;                  // scale byte index for h = 0; h adds 2 (same word)
+        const uint32_t sw = scw[sb >> 2];
         const int sc = (int)(int8_t)((sw >> (8 * (sb & 3) + 16 * h)) & 0xff);
         const uint32_t sc16 = dup16((uint32_t)sc);
-        const uint32_t qw[4] = {wb.q[x].x, wb.q[x].y, wb.q[x].z, wb.q[x].w};
-        const uint32_t hw[2] = {wb.qh[x].x, wb.qh[x].y};
+        const uint32_t qw[4] = {ql[x].x, ql[x].y, ql[x].z, ql[x].w};
+        const uint32_t hw[2] = {qhv[x].x, qhv[x].y};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const uint32_t H = hw[i >> 1];
@@ -266,25 +310,41 @@ __device__ __forceinline__ void block_mac(const uint8_t *cur, const WBlk<CQ_DTYP
         }
     }
     v8h wmin = {};
-    tiles_mac<MT, false, 7>(cur, bl, bh, dw, wmin, lane, out);
+    tiles_mac<CQ_DTYPE_Q6K, MT, 7>(cur, g, bl, bh, dw, wmin, lane, out);
+}
+
+// Copies for block b+1 into `nxt`, then the arithmetic of block b out of `cur`.  The two stages
+// are distinct (`__restrict__`): without that knowledge the compiler makes every LDS read wait for
+// all copies in flight, which would serialise the pipeline.
+template <int DT, int MT>
+__device__ __forceinline__ void block_step(const uint8_t *__restrict__ cur, uint8_t *__restrict__ nxt,
+                                           const cq_weight &w, const cq_act_view &a, const LaneGeo &g, int64_t m0,
+                                           int64_t n_tile, bool n_ok, bool more, int64_t b, int wave, int lane,
+                                           const WHead<DT> &hcur, v16f (&out)[MT]) {
+    typedef Tile<DT, MT> T;
+    if (more) stage_issue<DT, MT>(nxt, w, a, g, m0, n_tile, n_ok, b + 1, wave, lane);
+    if (n_ok) block_mac<MT>(cur, cur + T::oWgt + wave * T::kWgtWave, g, hcur, lane, out);
 }
 
 // ------------------------------------------------------------------ kernel ----
+// Requires n % 32 == 0 and an activation workspace with padded rows (cq_act_view::m_stride).
 template <int DT, int MT>
 __global__ void __launch_bounds__(kThreads) gemm_kernel(cq_weight w, cq_act_view a, int64_t m, float *__restrict__ y,
                                                         int ksplit) {
+    typedef Tile<DT, MT> T;
     extern __shared__ __align__(16) uint8_t smem[];
-    constexpr bool MINS = DT == CQ_DTYPE_Q4K;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int h = lane >> 5, col = lane & 31;
     const int64_t kb = w.k >> 8;
     const int64_t m0 = (int64_t)blockIdx.y * (MT * 32);
     const int64_t n_tile = ((int64_t)blockIdx.x * kWaves + wave) * 32;
+    const bool n_ok = n_tile < w.n;   // wave-uniform; a wave past the last row only helps with the copies
     const int64_t n = n_tile + col;
-    const int64_t nc = n < w.n ? n : w.n - 1;   // clamped row for loads; stores are masked
+    const int64_t nc = n_ok ? n : 0;
     // this workgroup's range of K blocks
     const int64_t b0 = kb * blockIdx.z / ksplit, b1 = kb * (blockIdx.z + 1) / ksplit;
+    const LaneGeo g = lane_geo(lane, w.k);
 
     v16f out[MT];
 #pragma unroll
@@ -292,34 +352,26 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(cq_weight w, cq_act_view
 #pragma unroll
         for (int i = 0; i < 16; i++) out[t][i] = 0.0f;
 
-    WBlk<DT> wcur, wnxt;
-    stage_issue<MT, MINS>(smem, a, m, w.k, m0, b0, wave, lane);
-    load_w(w, nc * kb + b0, h, wcur);
+    WHead<DT> hcur, hnxt;
+    stage_issue<DT, MT>(smem, w, a, g, m0, n_tile, n_ok, b0, wave, lane);
+    load_head(w, nc * kb + b0, hcur);
+    hnxt = hcur;
     __builtin_amdgcn_s_waitcnt(0);   // the LDS copies above (and everything else outstanding)
     __syncthreads();
 
     for (int64_t b = b0; b < b1; b++) {
         const int par = (int)((b - b0) & 1);
-        uint8_t *cur = smem + par * Tile<MT>::kBytes;
-        uint8_t *nxt = smem + (par ^ 1) * Tile<MT>::kBytes;
+        uint8_t *cur = smem + par * T::kBytes;
+        uint8_t *nxt = smem + (par ^ 1) * T::kBytes;
         const bool more = b + 1 < b1;
-        if (more) {
-#ifndef EXP_NO_STAGE
-            stage_issue<MT, MINS>(nxt, a, m, w.k, m0, b + 1, wave, lane);
-#endif
-#ifndef EXP_NO_WLOAD
-            load_w(w, nc * kb + b + 1, h, wnxt);
-#else
-            wnxt = wcur;
-#endif
-        }
-        block_mac<MT>(cur, wcur, lane, out);
-        if (more) wcur = wnxt;
-        __builtin_amdgcn_s_waitcnt(0);   // next tile has landed in LDS
+        if (more) load_head(w, nc * kb + b + 1, hnxt);
+        block_step<DT, MT>(cur, nxt, w, a, g, m0, n_tile, n_ok, more, b, wave, lane, hcur, out);
+        hcur = hnxt;
+        __builtin_amdgcn_s_waitcnt(0);   // the next stage has landed in LDS
         __syncthreads();
     }
 
-    if (n < w.n) {
+    if (n_ok) {
 #pragma unroll
         for (int t = 0; t < MT; t++) {
 #pragma unroll
@@ -349,7 +401,7 @@ int num_cus() {
 
 template <int DT, int MT>
 hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
-    const size_t lds = 2 * Tile<MT>::kBytes;
+    const size_t lds = 2 * Tile<DT, MT>::kBytes;
     static bool attr_set = false;
     if (!attr_set && lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)gemm_kernel<DT, MT>,
@@ -375,21 +427,22 @@ template <int DT>
 hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
     if (m <= 32) return launch_mt<DT, 1>(w, a, m, y, s);
     if (m <= 64) return launch_mt<DT, 2>(w, a, m, y, s);
-    static const char *force8 = getenv("CQ_GEMM_MT8");
-    if (m <= 128 || !force8) return launch_mt<DT, 4>(w, a, m, y, s);
-    return launch_mt<DT, 8>(w, a, m, y, s);
+    return launch_mt<DT, 4>(w, a, m, y, s);
 }
 
 }  // namespace
 
 bool cq_gemm_supported(const cq_weight *w, int64_t m, int act_dtype) {
     (void)m;
-    return (w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q6K) && act_dtype == CQ_DTYPE_Q8K && w->k >= 256;
+    // the copies address rows with 32-bit offsets: 8 rows of activations, 16 rows of a weight plane
+    return (w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q6K) && act_dtype == CQ_DTYPE_Q8K && w->k >= 256 &&
+           w->k <= (1 << 24) && w->n % 32 == 0;
 }
 
 hipError_t cq_launch_gemm(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s) {
     if (!cq_gemm_supported(w, m, act_dtype)) return hipErrorNotSupported;
     if (m == 0 || w->n == 0) return hipSuccess;
+    if (a.m_stride < (m + 127) / 128 * 128) return hipErrorInvalidValue;   // rows the last tile may read
     if (w->dtype == CQ_DTYPE_Q4K) return launch_dt<CQ_DTYPE_Q4K>(w, a, m, y, s);
     return launch_dt<CQ_DTYPE_Q6K>(w, a, m, y, s);
 }

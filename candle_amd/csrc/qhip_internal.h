@@ -47,7 +47,7 @@ struct cq_weight {
 // Device activation storage used between the quantizer and the matmul kernels
 // (workspace layout).  Same numbers as the GGML activation blocks, split so
 // that int8 values are 16-byte aligned:
-//   Q8K : qs [m][k] i8 ; d [m][k/256] f32 ; bsums [m][k/256][16] i16
+//   Q8K : qs [m_stride][k] i8 ; d [m][k/256] f32 ; bsums [m][k/256][16] i16
 //   Q8_0: qs [m][k] i8 ; d [m][k/32]  f32 (the f16-rounded scale widened) ;
 //         bsum [m][k/32] i32 (sum of the 32 quants, for the Q4_0 "-8" term)
 // ---------------------------------------------------------------------------
@@ -55,7 +55,11 @@ struct cq_act_view {
     int8_t *qs;
     float *d;
     int16_t *bsums;  // Q8K
-    uint16_t *minp;  // Q8K: [m][k/256][16] f16, d * sub-block sums as two f16 pieces (GEMM min term)
+    // Q8K, for the GEMM only (block-major so that a tile of rows is contiguous per block):
+    float *dT;         // [k/256][m_stride] f32, the same values as d
+    uint16_t *minp;    // [k/256][m_stride][16] f16, d * sub-block sums as two f16 pieces p1[8] | p2[8]
+    int64_t m_stride;  // rows allocated: at least 256 more than the rows quantized, so that the GEMM
+                       // may read (and ignore) whole 128-row tiles past the last row
     int32_t *bsum32; // Q8_0 / Q8_1
     uint16_t *s16;   // Q8_1: the block's `s` field (f16 bits)
 };

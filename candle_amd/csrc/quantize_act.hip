@@ -134,14 +134,16 @@ __global__ void __launch_bounds__(256) quantize_q8k_kernel(const float *__restri
         *(uint32_t *)(out.v.qs + row * k + b_in_row * 256 + 4 * lane) = packed;
         if (lane == 0) out.v.d[blk] = d;
         if ((lane & 3) == 0) out.v.bsums[blk * 16 + (lane >> 2)] = (int16_t)sum;
-        // For the GEMM's min term: d * (sum of the 32 quants of sub-block j) as two f16 pieces
-        // p1 + p2 (22 significant bits), laid out [p1[8] | p2[8]] per block.
+        // For the GEMM (block-major copies): d again, and for the min term d * (sum of the 32
+        // quants of sub-block j) as two f16 pieces p1 + p2 (22 significant bits), [p1[8] | p2[8]].
+        const int64_t tb = b_in_row * out.v.m_stride + row;
+        if (lane == 0) out.v.dT[tb] = d;
         const int sum32 = sum + __shfl_xor(sum, 4);
         if ((lane & 7) == 0) {
             const float v = d * (float)sum32;
             const _Float16 p1 = (_Float16)v;
             const _Float16 p2 = (_Float16)(v - (float)p1);
-            _Float16 *mp = (_Float16 *)out.v.minp + blk * 16;
+            _Float16 *mp = (_Float16 *)out.v.minp + tb * 16;
             mp[lane >> 3] = p1;
             mp[8 + (lane >> 3)] = p2;
         }

@@ -200,14 +200,29 @@ def test_small_batch_matches_oracle(qh, dt, m, k, n):
 
 
 @pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K])
-@pytest.mark.parametrize("m,k,n", [(9, 256, 32), (33, 512, 70), (64, 1024, 129), (130, 768, 257), (11, 512, 21)])
+@pytest.mark.parametrize("m,k,n", [(9, 256, 32), (33, 512, 96), (64, 1024, 160), (130, 768, 288), (11, 512, 64),
+                                   (1, 256, 32), (129, 2048, 416)])
 def test_gemm_matches_oracle_small(qh, dt, m, k, n):
-    """The int8-MFMA tile kernel on ragged shapes (m, n not multiples of the tile; one K block)."""
+    """The int8-MFMA tile kernel on ragged shapes (m any, n a multiple of 32 but not of the
+    128-row workgroup tile; from one K block up)."""
     w, x = make_inputs(3 * dt + m + k + n, m, k, n, outliers=True)
     blocks = orc.quantize(dt, w)
     qw = qh.QWeight.from_ggml(dt, blocks, n, k)
     got = qh.qmatmul(qw, dev(x), qh.FLAG_FORCE_GEMM).cpu().numpy()
     check_f32(got, orc.matmul(dt, x, blocks, n))
+
+
+@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K])
+def test_gemm_needs_32_row_multiple(qh, dt):
+    """Weight row counts that are not a multiple of 32 take the dot-product kernels: forcing the
+    tile kernel is an error, the automatic choice still matches the oracle."""
+    m, k, n = 33, 512, 70
+    w, x = make_inputs(5 * dt + 1, m, k, n)
+    blocks = orc.quantize(dt, w)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    with pytest.raises(qh.QHipError):
+        qh.qmatmul(qw, dev(x), qh.FLAG_FORCE_GEMM)
+    check_f32(qh.qmatmul(qw, dev(x)).cpu().numpy(), orc.matmul(dt, x, blocks, n))
 
 
 @pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K])
