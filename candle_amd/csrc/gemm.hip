@@ -15,44 +15,46 @@
 // eight sub-blocks; it runs on the f16 MFMA with both factors split in two f16 pieces (products
 // exact to ~2^-22) and accumulates straight into the f32 result.
 //
-// Work split: a workgroup of four waves covers BM = 32*MT activation rows x 128 weight rows; each
-// wave owns 32 weight rows (MFMA B operand: lane l holds row l%32, k = 16*(l/32)+[0,16) of a
-// 32-wide K-slice) and unpacks them in registers.  Activations (shared by the four waves) and each
-// wave's packed weight bytes go from global memory straight into LDS (global_load_lds_dwordx4),
-// double buffered, one block ahead.  Every such copy instruction reads eight whole 128-byte lines
-// (8 rows x 128 B) - the texture path pays per line touched - and the 16-byte chunks of a row are
-// XOR-swizzled by the row number on the way in, so that the MFMA operand reads (lanes = rows, one
-// chunk column) spread over all LDS banks.  With few workgroups (small n) K is split over
-// blockIdx.z and the partial results are added atomically.
+// Work split: a workgroup of eight waves (two per SIMD, so that one wave's scaling arithmetic runs
+// under the other's MFMAs) covers BM = 32*MT activation rows x 128 weight rows.  Each wave owns 16
+// weight rows and works with the 16x16x64 MFMA: operand lane l holds row l%16 and the 16
+// consecutive k of quarter l/16 of a 64-wide K-slice; result lane l holds column l%16, rows
+// 4*(l/16)+[0,4).  The wave unpacks its weight operands in registers once per block and reuses
+// them for all BM rows.  Activations (shared by the waves) and each wave's packed weight bytes go
+// from global memory straight into LDS (global_load_lds_dwordx4), double buffered, one block
+// ahead.  Every such copy instruction reads eight whole 128-byte lines (8 rows x 128 B) - the
+// texture path pays per line touched - and the 16-byte chunks of a row are XOR-swizzled by the
+// row number on the way in, so that the operand reads (lanes = rows, one chunk column) spread
+// over all LDS banks.  With few workgroups (small n) K is split over blockIdx.z and the partial
+// results are added atomically.
 #include "qhip_internal.h"
-#include <stdlib.h>
 
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
-typedef float v16f __attribute__((ext_vector_type(16)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef unsigned short us2 __attribute__((ext_vector_type(2)));
 typedef short ss2 __attribute__((ext_vector_type(2)));
 typedef const void __attribute__((address_space(1))) *gptr_t;
 typedef void __attribute__((address_space(3))) *lptr_t;
 
-constexpr int kWaves = 4;
+constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
+constexpr int kRowsPerWave = 16;
+constexpr int kBN = kWaves * kRowsPerWave;
 
 // LDS image of one pipeline stage:
-//   act  : [MT tiles][2 K-halves][4 row groups][8 rows][8 chunks of 16 B]   chunk c of row r sits at c ^ (r%8)
+//   act  : [MT][2 K-halves][4 row groups][8 rows][8 chunks of 16 B]   chunk c of row r sits at c ^ (r%8)
 //   d8   : [BM] f32
 //   minp : [BM][2 pieces][8] f16            d8 * bsum32_j split in two f16 pieces (Q4K)
-//   wgt  : per wave: [4 row groups][8 rows][8 chunks] of the 128-byte qs / ql plane (same swizzle),
-//          Q6K also [2 row groups][16 rows][4 chunks] of the 64-byte qh plane (chunk c at c ^ ((r/2)%4))
+//   wgt  : per wave: [2 row groups][8 rows][8 chunks] of the 128-byte qs / ql plane (same swizzle),
+//          Q6K also [16 rows][4 chunks] of the 64-byte qh plane (chunk c at c ^ ((r/2)%4))
 template <int DT, int MT> struct Tile {
     static constexpr int kAct = MT * 8 * 1024;
     static constexpr int kD8 = (MT * 32 < 64 ? 64 : MT * 32) * 4;   // filled by whole-wave copies of 64 floats
     static constexpr int kMin = DT == CQ_DTYPE_Q4K ? MT * 32 * 32 : 0;
-    static constexpr int kWgtWave = DT == CQ_DTYPE_Q4K ? 4096 : 6144;
+    static constexpr int kWgtWave = DT == CQ_DTYPE_Q4K ? 2048 : 3072;
     static constexpr int oD8 = kAct, oMin = oD8 + kD8, oWgt = oMin + kMin;
     static constexpr int kBytes = oWgt + kWaves * kWgtWave;
 };
@@ -80,14 +82,20 @@ __device__ __forceinline__ void dma4(const void *base, uint32_t off, uint8_t *ld
     __builtin_amdgcn_global_load_lds((gptr_t)((const uint8_t *)base + off), (lptr_t)lds, 4, 0, 0);
 }
 
-// Per-lane constants of the copies and of the operand reads.
+// Per-lane constants of the copies and of the operand reads (r = l%16: row, kq = l/16: k quarter).
 struct LaneGeo {
-    uint32_t act_off;   // copy of 8 rows x 128 B of activations: (l/8)*k + ((l%8) ^ (l/8))*16
-    uint32_t wq_off;    // the same over the weights' 128-byte plane: (l/8)*kb*128 + ...
-    uint32_t wh_off;    // Q6K qh plane, 16 rows x 64 B: (l/4)*kb*64 + ((l%4) ^ ((l/8)%4))*16
-    uint32_t col[4];    // operand read: byte offset of chunk 2j+h of row l%32 inside a [4][8][8] x 16 B image
-    uint32_t qh_col[4]; // Q6K: byte offset of the 8 bytes of unit 2x+h of row l%32 inside the qh image
+    uint32_t act_off;    // copy of 8 rows x 128 B of activations: (l/8)*k + ((l%8) ^ (l/8))*16
+    uint32_t wq_off;     // the same over the weights' 128-byte plane: (l/8)*kb*128 + ...
+    uint32_t wh_off;     // Q6K qh plane, 16 rows x 64 B: (l/4)*kb*64 + ((l%4) ^ ((l/8)%4))*16
+    uint32_t a_col[2];   // activation operand of K-slice S: chunk 4*(S%2) + kq of K-half S/2, row r
+    uint32_t w_col4[4];  // Q4K weight chunk 2g + kq%2 of row r
+    uint32_t w_col6[2];  // Q6K ql chunk (unit) 4*hf + kq of row r
+    uint32_t qh_col[2];  // Q6K: the 8 bytes of high bits of unit 4*hf + kq of row r
 };
+
+__device__ __forceinline__ uint32_t swz_col(uint32_t r, uint32_t c) {
+    return (r >> 3) * 1024u + (r & 7) * 128u + ((c ^ (r & 7)) << 4);
+}
 
 __device__ __forceinline__ LaneGeo lane_geo(int lane, int64_t k) {
     LaneGeo g;
@@ -97,12 +105,15 @@ __device__ __forceinline__ LaneGeo lane_geo(int lane, int64_t k) {
     g.wq_off = r8 * kb * 128u + ((c8 ^ r8) << 4);
     const uint32_t r16 = lane >> 2, c4 = lane & 3;
     g.wh_off = r16 * kb * 64u + ((c4 ^ ((r16 >> 1) & 3)) << 4);
-    const uint32_t r = lane & 31, h = lane >> 5;
+    const uint32_t r = lane & 15, kq = lane >> 4;
 #pragma unroll
-    for (uint32_t j = 0; j < 4; j++) {
-        g.col[j] = (r >> 3) * 1024u + (r & 7) * 128u + (((2 * j + h) ^ (r & 7)) << 4);
-        g.qh_col[j] = (r >> 4) * 1024u + (r & 15) * 64u + ((j ^ ((r >> 1) & 3)) << 4) + h * 8u;
+    for (uint32_t e = 0; e < 2; e++) {
+        g.a_col[e] = swz_col(r, 4 * e + kq);
+        g.w_col6[e] = swz_col(r, 4 * e + kq);
+        g.qh_col[e] = r * 64u + (((2 * e + (kq >> 1)) ^ ((r >> 1) & 3)) << 4) + (kq & 1) * 8u;
     }
+#pragma unroll
+    for (uint32_t gi = 0; gi < 4; gi++) g.w_col4[gi] = swz_col(r, 2 * gi + (kq & 1));
     return g;
 }
 
@@ -122,25 +133,21 @@ __device__ __forceinline__ void stage_issue(uint8_t *buf, const cq_weight &w, co
     }
 #pragma unroll
     for (int j = 0; j < (MT * 32 + 63) / 64; j++) {
-        if ((j & 3) == wave) dma4(a.dT + b * a.m_stride + m0 + j * 64, lane * 4u, buf + T::oD8 + j * 256);
+        if (j == wave) dma4(a.dT + b * a.m_stride + m0 + j * 64, lane * 4u, buf + T::oD8 + j * 256);
     }
     if (DT == CQ_DTYPE_Q4K) {
 #pragma unroll
         for (int j = 0; j < MT; j++) {
-            if (((j + 1) & 3) == wave)
+            if (j + 4 == wave)
                 dma16(a.minp + (b * a.m_stride + m0 + j * 32) * 16, lane * 16u, buf + T::oMin + j * 1024);
         }
     }
-    // this wave's 32 weight rows
+    // this wave's 16 weight rows
     if (n_ok) {
         uint8_t *wl = buf + T::oWgt + wave * T::kWgtWave;
 #pragma unroll
-        for (int rg = 0; rg < 4; rg++) dma16(w.p0 + ((n_tile + rg * 8) * kb + b) * 128, g.wq_off, wl + rg * 1024);
-        if (DT == CQ_DTYPE_Q6K) {
-#pragma unroll
-            for (int rg = 0; rg < 2; rg++)
-                dma16(w.p1 + ((n_tile + rg * 16) * kb + b) * 64, g.wh_off, wl + 4096 + rg * 1024);
-        }
+        for (int rg = 0; rg < 2; rg++) dma16(w.p0 + ((n_tile + rg * 8) * kb + b) * 128, g.wq_off, wl + rg * 1024);
+        if (DT == CQ_DTYPE_Q6K) dma16(w.p1 + (n_tile * kb + b) * 64, g.wh_off, wl + 2048);
     }
 }
 
@@ -156,72 +163,57 @@ __device__ __forceinline__ void load_head(const cq_weight &w, int64_t blk, WHead
     r.d = ((const uint16_t *)w.p3)[blk];
 }
 
-// One block for this wave's 32 weight rows against the MT activation tiles in `cur`, as a
-// hand-laid software pipeline of 8*(MT+1) steps.  Step (t, s) issues the two int8 MFMAs of tile t,
-// K-slice s, and, in their shadow, the scaling of two of the sixteen integers of tile t-1 (VALU);
-// LDS reads run two steps ahead.  The accumulator pair alternates between two register sets.  A
-// scheduling barrier after every step keeps the compiler from hoisting all MFMAs to the front,
-// which would need MT accumulator sets at once.
+// One block for this wave's 16 weight rows against the 2*MT sixteen-row activation tiles in `cur`,
+// as a software pipeline: step t issues the MFMAs of tile t (four K-slices x two digits, plus the
+// min term), the scaling of the four integers of tile t-2 (VALU) and the LDS reads of tile t+1.
+// The accumulator pair rotates through three register sets.  A scheduling barrier after every
+// step keeps the compiler from hoisting all MFMAs to the front.
 template <int DT, int MT, int SHIFT>
-__device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, const v4i (&bl)[8], const v4i (&bh)[8],
-                                          float dw, v8h wmin, int lane, v16f (&out)[MT]) {
+__device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, const v4i (&bl)[4], const v4i (&bh)[4],
+                                          float dw, v8h wmin, int lane, v4f (&out)[2 * MT]) {
     typedef Tile<DT, MT> T;
     constexpr bool MINS = DT == CQ_DTYPE_Q4K;
-    const int h = lane >> 5, col = lane & 31;
-    const uint8_t *d8p = cur + T::oD8 + h * 16;        // rows 8j + 4h + [0,4) of a tile
-    const uint8_t *mnp = cur + T::oMin + col * 32;     // this lane's row of min pieces
-    // operand of tile t, K-slice s: chunk 2*(s%4) + h of K-half s/4
-    auto afrag = [&](int q) -> v4i {
-        const int t = q >> 3, s = q & 7;
-        return *(const v4i *)(cur + g.col[s & 3] + (t * 2 + (s >> 2)) * 4096);
+    constexpr int NT = 2 * MT;
+    const int r = lane & 15, kq = lane >> 4;
+    const uint8_t *d8p = cur + T::oD8 + kq * 16;                     // rows 4*kq + [0,4) of a tile
+    const uint8_t *mnp = cur + T::oMin + r * 32 + (kq >> 1) * 16;    // piece 1 for kq < 2, piece 2 above
+    v4i a[2][4];
+    v4f dsc[4];   // read one step ahead, used two steps behind
+    v8h ma[2];
+    v4i acc_lo[3], acc_hi[3];   // written in step t, read in step t+2, when the MFMAs are long done
+    auto load_tile = [&](int t) {
+        const uint8_t *base = cur + (t >> 1) * 8192 + (t & 1) * 2048;
+#pragma unroll
+        for (int s = 0; s < 4; s++) a[t & 1][s] = *(const v4i *)(base + (s >> 1) * 4096 + g.a_col[s & 1]);
+        dsc[t % 4] = *(const v4f *)(d8p + t * 64);
+        if (MINS) ma[t & 1] = *(const v8h *)(mnp + t * 512);
     };
-    v16i acc_lo[2], acc_hi[2];
-    v4i a[3];
-    v4f dsc[2][4];
-    v8h ma1, ma2;
-    a[0] = afrag(0);
-    a[1] = afrag(1);
-    if (MINS) {
-        ma1 = *(const v8h *)(mnp);
-        ma2 = *(const v8h *)(mnp + 16);
-    }
+    load_tile(0);
 #pragma unroll
-    for (int q = 0; q < (MT + 1) * 8; q++) {
-        const int t = q >> 3, s = q & 7;
-        if (q + 2 < MT * 8) a[(q + 2) % 3] = afrag(q + 2);
-        if (t < MT) {
-            if (s == 0) {
-                if (MINS) {
-                    // min term: out -= sum_j (dmin*min_j) * (d8*bsum32_j).  K-slots 0..7 carry piece 1
-                    // of the weight factor, slots 8..15 piece 2; the activation operand carries one of
-                    // its pieces in both halves.
-                    out[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma1, wmin, out[t], 0, 0, 0);
-                    out[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma2, wmin, out[t], 0, 0, 0);
-                }
-                const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                acc_lo[t & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[q % 3], bl[0], zero, 0, 0, 0);
-                acc_hi[t & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[q % 3], bh[0], zero, 0, 0, 0);
-            } else {
-                acc_lo[t & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[q % 3], bl[s], acc_lo[t & 1], 0, 0, 0);
-                acc_hi[t & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[q % 3], bh[s], acc_hi[t & 1], 0, 0, 0);
-            }
-            if (s == 4) {
+    for (int t = 0; t <= NT + 1; t++) {
+        if (t + 1 < NT) load_tile(t + 1);
+        if (t < NT) {
+            const int p = t & 1, c = t % 3;
+            // min term: out -= sum_j (dmin*min_j) * (d8*bsum32_j); the 32 K-slots are the four
+            // products of pieces: activation pieces [1,1,2,2] against weight pieces [1,2,1,2]
+            if (MINS) out[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ma[p], wmin, out[t], 0, 0, 0);
+            const v4i zero = {0, 0, 0, 0};
+            acc_lo[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[p][0], bl[0], zero, 0, 0, 0);
+            acc_hi[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[p][0], bh[0], zero, 0, 0, 0);
 #pragma unroll
-                for (int j = 0; j < 4; j++) dsc[t & 1][j] = *(const v4f *)(d8p + (t * 32 + 8 * j) * 4);
-            }
-            if (s == 6 && MINS && t + 1 < MT) {
-                ma1 = *(const v8h *)(mnp + (t + 1) * 1024);
-                ma2 = *(const v8h *)(mnp + (t + 1) * 1024 + 16);
+            for (int s = 1; s < 4; s++) {
+                acc_lo[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[p][s], bl[s], acc_lo[c], 0, 0, 0);
+                acc_hi[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[p][s], bh[s], acc_hi[c], 0, 0, 0);
             }
         }
-        if (t > 0) {
-            const int p = (t - 1) & 1;
+        if (t > 1) {
+            const int c = (t - 2) % 3;
 #pragma unroll
-            for (int i = 2 * s; i < 2 * s + 2; i++) {
-                const int I = (acc_hi[p][i] << SHIFT) + acc_lo[p][i];
-                float o = __builtin_fmaf((float)I * dw, dsc[p][i >> 2][i & 3], out[t - 1][i]);
+            for (int i = 0; i < 4; i++) {
+                const int I = (acc_hi[c][i] << SHIFT) + acc_lo[c][i];
+                float o = __builtin_fmaf((float)I * dw, dsc[(t - 2) % 4][i], out[t - 2][i]);
                 asm volatile("" : "+v"(o));   // pins the scaling to this step (pure ops float otherwise)
-                out[t - 1][i] = o;
+                out[t - 2][i] = o;
             }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -230,8 +222,8 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, 
 
 template <int MT>
 __device__ __forceinline__ void block_mac(const uint8_t *cur, const uint8_t *wl, const LaneGeo &g,
-                                          const WHead<CQ_DTYPE_Q4K> &wb, int lane, v16f (&out)[MT]) {
-    const int h = lane >> 5;
+                                          const WHead<CQ_DTYPE_Q4K> &wb, int lane, v4f (&out)[2 * MT]) {
+    const uint32_t kq = lane >> 4;
     const uint4 hd = wb.hd;
     const float dw = cq_h2f((uint16_t)(hd.x & 0xffff));
     const float dmin = cq_h2f((uint16_t)(hd.x >> 16));
@@ -240,22 +232,22 @@ __device__ __forceinline__ void block_mac(const uint8_t *cur, const uint8_t *wl,
     const uint32_t sc47 = (hd.w & 0x0f0f0f0fu) | (((hd.y >> 6) & 0x03030303u) << 4);
     const uint32_t mn03 = hd.z & 0x3f3f3f3fu;
     const uint32_t mn47 = ((hd.w >> 4) & 0x0f0f0f0fu) | (((hd.z >> 6) & 0x03030303u) << 4);
-    v4i bl[8], bh[8];
+    // K-slice g = elements 64g..64g+63 = qs bytes 32g..32g+31, low nibbles for the first 32 elements
+    // (quarters 0,1: sub-block 2g), high nibbles for the last 32 (quarters 2,3: sub-block 2g+1)
+    const uint32_t hi = kq >> 1, nsh = hi * 4;
+    v4i bl[4], bh[4];
 #pragma unroll
     for (int gi = 0; gi < 4; gi++) {
-        // qs bytes 32g + 16h + [0,16): low nibbles = K-slice 2g, high nibbles = slice 2g+1
-        const uint4 q = *(const uint4 *)(wl + g.col[gi]);
+        const uint4 q = *(const uint4 *)(wl + g.w_col4[gi]);
         const uint32_t scw = gi < 2 ? sc03 : sc47;
-        const uint32_t s0 = (scw >> (16 * (gi & 1))) & 0xff, s1 = (scw >> (16 * (gi & 1) + 8)) & 0xff;
-        const uint32_t sl0 = dup16(s0 & 7), sh0 = dup16(s0 >> 3), sl1 = dup16(s1 & 7), sh1 = dup16(s1 >> 3);
+        const uint32_t sj = (scw >> (16 * (gi & 1) + 8 * hi)) & 0xff;
+        const uint32_t sl = dup16(sj & 7), sh = dup16(sj >> 3);
         const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const uint32_t lo4 = qw[i] & 0x0F0F0F0Fu, hi4 = (qw[i] >> 4) & 0x0F0F0F0Fu;
-            bl[2 * gi][i] = (int)pk_mul_u16(lo4, sl0);       // sub-block 2g, low digit of the scale
-            bh[2 * gi][i] = (int)pk_mul_u16(lo4, sh0);
-            bl[2 * gi + 1][i] = (int)pk_mul_u16(hi4, sl1);   // sub-block 2g+1
-            bh[2 * gi + 1][i] = (int)pk_mul_u16(hi4, sh1);
+            const uint32_t v = (qw[i] >> nsh) & 0x0F0F0F0Fu;
+            bl[gi][i] = (int)pk_mul_u16(v, sl);   // low digit of the scale
+            bh[gi][i] = (int)pk_mul_u16(v, sh);
         }
     }
     v8h wmin;
@@ -264,49 +256,45 @@ __device__ __forceinline__ void block_mac(const uint8_t *cur, const uint8_t *wl,
         const uint32_t mw = j < 4 ? mn03 : mn47;
         const float v = -dmin * (float)((mw >> (8 * (j & 3))) & 0xff);
         const _Float16 p1 = (_Float16)v;
-        wmin[j] = h == 0 ? p1 : (_Float16)(v - (float)p1);
+        wmin[j] = (kq & 1) == 0 ? p1 : (_Float16)(v - (float)p1);
     }
     tiles_mac<CQ_DTYPE_Q4K, MT, 3>(cur, g, bl, bh, dw, wmin, lane, out);
 }
 
 template <int MT>
 __device__ __forceinline__ void block_mac(const uint8_t *cur, const uint8_t *wl, const LaneGeo &g,
-                                          const WHead<CQ_DTYPE_Q6K> &wb, int lane, v16f (&out)[MT]) {
-    const int h = lane >> 5;
+                                          const WHead<CQ_DTYPE_Q6K> &wb, int lane, v4f (&out)[2 * MT]) {
+    const uint32_t kq = lane >> 4;
     const float dw = cq_h2f((uint16_t)wb.d);
-    const uint32_t scw[4] = {wb.sc.x, wb.sc.y, wb.sc.z, wb.sc.w};
-    uint4 ql[4];
-    uint2 qhv[4];
+    v4i bl[4], bh[4];
 #pragma unroll
-    for (int x = 0; x < 4; x++) {
-        // ql lane of unit u = 2x + h and its re-packed high bits
-        ql[x] = *(const uint4 *)(wl + g.col[x]);
-        qhv[x] = *(const uint2 *)(wl + 4096 + g.qh_col[x]);
-    }
-    v4i bl[8], bh[8];
+    for (int hf = 0; hf < 2; hf++) {
+        // K-slices 2hf (low nibbles) and 2hf+1 (high nibbles) of unit u = 4hf + kq: 16 bytes of ql,
+        // 8 bytes of re-packed high bits, scale bytes 2u and 2u+1
+        const uint4 ql = *(const uint4 *)(wl + g.w_col6[hf]);
+        const uint2 qh = *(const uint2 *)(wl + 2048 + g.qh_col[hf]);
+        const uint32_t s_even = hf ? wb.sc.z : wb.sc.x, s_odd = hf ? wb.sc.w : wb.sc.y;
+        const uint32_t sw = s_even ^ ((s_even ^ s_odd) & (0u - (kq >> 1)));   // word 2hf + kq/2, branch-free
+        const uint32_t qw[4] = {ql.x, ql.y, ql.z, ql.w};
+        const uint32_t hw[2] = {qh.x, qh.y};
 #pragma unroll
-    for (int s = 0; s < 8; s++) {
-        // K-slice s: this lane's 16 elements are the group G = 2s + h, i.e. unit u = 2x + h with
-        // x = 2*(s/4) + s%2, low nibbles when (s%4) < 2 else high nibbles
-        const int x = 2 * (s >> 2) + (s & 1), nib = (s & 3) >> 1;
-        const int sb = 4 * x + nib;                  // scale byte index for h = 0; h adds 2 (same word)
-        const uint32_t sw = scw[sb >> 2];
-        const int sc = (int)(int8_t)((sw >> (8 * (sb & 3) + 16 * h)) & 0xff);
-        const uint32_t sc16 = dup16((uint32_t)sc);
-        const uint32_t qw[4] = {ql[x].x, ql[x].y, ql[x].z, ql[x].w};
-        const uint32_t hw[2] = {qhv[x].x, qhv[x].y};
+        for (int nib = 0; nib < 2; nib++) {
+            const int s = 2 * hf + nib;
+            const int sc = (int)(int8_t)((sw >> (16 * (kq & 1) + 8 * nib)) & 0xff);
+            const uint32_t sc16 = dup16((uint32_t)sc);
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t H = hw[i >> 1];
-            const int sh = (i & 1) * 4 + 2 * nib;
-            const uint32_t q6 = ((qw[i] >> (4 * nib)) & 0x0F0F0F0Fu) | (((H >> sh) & 0x03030303u) << 4);
-            // the four elements as 16-bit lanes, minus 32, times the group scale (low 16 bits kept)
-            const uint32_t e02 = pk_sub_u16(q6 & 0x00FF00FFu, 0x00200020u);
-            const uint32_t e13 = pk_sub_u16((q6 >> 8) & 0x00FF00FFu, 0x00200020u);
-            const uint32_t p02 = pk_mul_u16(e02, sc16), p13 = pk_mul_u16(e13, sc16);
-            // gather bytes [p02.0, p13.0, p02.2, p13.2]
-            bl[s][i] = (int)(__builtin_amdgcn_perm(p13, p02, 0x06020400u) & 0x7F7F7F7Fu);
-            bh[s][i] = (int)__builtin_amdgcn_perm(pk_ashr7_i16(p13), pk_ashr7_i16(p02), 0x06020400u);
+            for (int i = 0; i < 4; i++) {
+                const uint32_t H = hw[i >> 1];
+                const int sh = (i & 1) * 4 + 2 * nib;
+                const uint32_t q6 = ((qw[i] >> (4 * nib)) & 0x0F0F0F0Fu) | (((H >> sh) & 0x03030303u) << 4);
+                // the four elements as 16-bit lanes, minus 32, times the group scale (low 16 bits kept)
+                const uint32_t e02 = pk_sub_u16(q6 & 0x00FF00FFu, 0x00200020u);
+                const uint32_t e13 = pk_sub_u16((q6 >> 8) & 0x00FF00FFu, 0x00200020u);
+                const uint32_t p02 = pk_mul_u16(e02, sc16), p13 = pk_mul_u16(e13, sc16);
+                // gather bytes [p02.0, p13.0, p02.2, p13.2]
+                bl[s][i] = (int)(__builtin_amdgcn_perm(p13, p02, 0x06020400u) & 0x7F7F7F7Fu);
+                bh[s][i] = (int)__builtin_amdgcn_perm(pk_ashr7_i16(p13), pk_ashr7_i16(p02), 0x06020400u);
+            }
         }
     }
     v8h wmin = {};
@@ -320,14 +308,14 @@ template <int DT, int MT>
 __device__ __forceinline__ void block_step(const uint8_t *__restrict__ cur, uint8_t *__restrict__ nxt,
                                            const cq_weight &w, const cq_act_view &a, const LaneGeo &g, int64_t m0,
                                            int64_t n_tile, bool n_ok, bool more, int64_t b, int wave, int lane,
-                                           const WHead<DT> &hcur, v16f (&out)[MT]) {
+                                           const WHead<DT> &hcur, v4f (&out)[2 * MT]) {
     typedef Tile<DT, MT> T;
     if (more) stage_issue<DT, MT>(nxt, w, a, g, m0, n_tile, n_ok, b + 1, wave, lane);
     if (n_ok) block_mac<MT>(cur, cur + T::oWgt + wave * T::kWgtWave, g, hcur, lane, out);
 }
 
 // ------------------------------------------------------------------ kernel ----
-// Requires n % 32 == 0 and an activation workspace with padded rows (cq_act_view::m_stride).
+// Requires n % 16 == 0 and an activation workspace with padded rows (cq_act_view::m_stride).
 template <int DT, int MT>
 __global__ void __launch_bounds__(kThreads) gemm_kernel(cq_weight w, cq_act_view a, int64_t m, float *__restrict__ y,
                                                         int ksplit) {
@@ -335,22 +323,20 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(cq_weight w, cq_act_view
     extern __shared__ __align__(16) uint8_t smem[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int h = lane >> 5, col = lane & 31;
+    const int r = lane & 15, kq = lane >> 4;
     const int64_t kb = w.k >> 8;
     const int64_t m0 = (int64_t)blockIdx.y * (MT * 32);
-    const int64_t n_tile = ((int64_t)blockIdx.x * kWaves + wave) * 32;
+    const int64_t n_tile = ((int64_t)blockIdx.x * kWaves + wave) * kRowsPerWave;
     const bool n_ok = n_tile < w.n;   // wave-uniform; a wave past the last row only helps with the copies
-    const int64_t n = n_tile + col;
+    const int64_t n = n_tile + r;
     const int64_t nc = n_ok ? n : 0;
     // this workgroup's range of K blocks
     const int64_t b0 = kb * blockIdx.z / ksplit, b1 = kb * (blockIdx.z + 1) / ksplit;
     const LaneGeo g = lane_geo(lane, w.k);
 
-    v16f out[MT];
+    v4f out[2 * MT];
 #pragma unroll
-    for (int t = 0; t < MT; t++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) out[t][i] = 0.0f;
+    for (int t = 0; t < 2 * MT; t++) out[t] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
 
     WHead<DT> hcur, hnxt;
     stage_issue<DT, MT>(smem, w, a, g, m0, n_tile, n_ok, b0, wave, lane);
@@ -373,10 +359,10 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(cq_weight w, cq_act_view
 
     if (n_ok) {
 #pragma unroll
-        for (int t = 0; t < MT; t++) {
+        for (int t = 0; t < 2 * MT; t++) {
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int64_t row = m0 + t * 32 + (i >> 2) * 8 + h * 4 + (i & 3);
+            for (int i = 0; i < 4; i++) {
+                const int64_t row = m0 + t * 16 + kq * 4 + i;
                 if (row < m) {
                     if (ksplit == 1) y[row * w.n + n] = out[t][i];
                     else unsafeAtomicAdd(&y[row * w.n + n], out[t][i]);
@@ -409,7 +395,7 @@ hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hip
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    const int64_t gx = (w->n + kWaves * 32 - 1) / (kWaves * 32), gy = (m + MT * 32 - 1) / (MT * 32);
+    const int64_t gx = (w->n + kBN - 1) / kBN, gy = (m + MT * 32 - 1) / (MT * 32);
     // too few workgroups for the machine: split K (at least four blocks per part)
     int ksplit = 1;
     const int64_t kb = w->k >> 8;
@@ -432,11 +418,12 @@ hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hip
 
 }  // namespace
 
+
 bool cq_gemm_supported(const cq_weight *w, int64_t m, int act_dtype) {
     (void)m;
     // the copies address rows with 32-bit offsets: 8 rows of activations, 16 rows of a weight plane
     return (w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q6K) && act_dtype == CQ_DTYPE_Q8K && w->k >= 256 &&
-           w->k <= (1 << 24) && w->n % 32 == 0;
+           w->k <= (1 << 24) && w->n % kRowsPerWave == 0;
 }
 
 hipError_t cq_launch_gemm(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s) {
