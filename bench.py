@@ -9,8 +9,8 @@ streams from HBM and not from the 256 MB Infinity Cache).  Weights are random N(
 quantized on the device (bit-identical to the CPU quantizer, see tests).
 
 Prints ONE JSON line.  `value` = GGML weight bytes per step / time per step (inputs resident in
-HBM).  `roofline` covers the dominant kernel, the Q4_K matvec: algorithmic bytes per launch
-divided by its average launch duration, measured here with HIP events around single launches.
+HBM).  `roofline` covers the dominant kernel, the Q4_K decode matvec: algorithmic bytes per launch
+divided by its average launch duration, measured here with HIP events recorded around each launch.
 `cpu_baseline` times the restated candle CPU QMatMul (AVX2 + threads) on a bounded sample.
 """
 from __future__ import annotations
@@ -26,6 +26,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+# HBM bytes per Q4_K decode launch (mean over the step's 192 launches), from two rocprofv3 --pmc runs
+# of this script (FETCH_SIZE, then WRITE_SIZE), each scaled by what the counter reads for a plain
+# 256 MiB device copy (x2.000 and x1.000); see profiles/decode_stack_q4k_matvec_hbm_traffic.md.
+Q4K_DECODE_TRAFFIC_BYTES_PER_LAUNCH = 15_020_032
 
 LAYERS = 32
 HIDDEN, FFN, VOCAB = 4096, 11008, 32000
@@ -51,6 +55,9 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=LAYERS, help="(debug) fewer layers; the result is then not a bench line")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain device copy of 256 MiB three times (a kernel of known HBM traffic, to "
+                         "calibrate FETCH_SIZE / WRITE_SIZE counters in a profiler run)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (one process, one MI355X); --gpus must be 1", file=sys.stderr)
@@ -107,6 +114,14 @@ def main() -> int:
         for i in range(len(calls)):
             run_call(i, 0, s)
 
+    if args.copy_probe:
+        src = torch.full((64 * 1024 * 1024,), 1.0, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     # ---- timed region ----------------------------------------------------------------------
     side = torch.cuda.Stream()
     graph = None
@@ -136,34 +151,82 @@ def main() -> int:
         torch.cuda.synchronize()
         ms_per_step = e0.elapsed_time(e1) / args.steps
 
-        # ---- dominant kernel: Q4_K matvec, one launch at a time between two events ---------
+        # ---- dominant kernel: the Q4_K decode matvec (activation quantizer fused in) ----------
+        # Each Q4_K launch of the step is timed once per pass by a pair of HIP events that the
+        # library records around that kernel on its stream, while the whole step runs eagerly
+        # around it, so the kernel sees the same cache and clock state as in the timed region.
         q4k_calls = [i for i, c in enumerate(calls) if c[2] == "q4k"]
         durs, alg_bytes = [], []
-        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in q4k_calls]
-        for rep in range(3):
-            last_in = None
-            for (a, b), i in zip(evs, q4k_calls):
-                xin = calls[i][1]
-                if xin != last_in:  # quantize this input into the workspace outside the event pair
-                    run_call(i, 0)
-                    last_in = xin
-                a.record()
-                run_call(i, qhip.FLAG_REUSE_ACT)
-                b.record()
+        s_here = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        for rep in range(2):
+            for target in q4k_calls:
+                for i in range(len(calls)):
+                    if i == target:
+                        us = qhip.timed_kernel_us(lambda: run_call(i, 0, s_here))
+                    else:
+                        run_call(i, 0, s_here)
+                if rep == 0:
+                    continue  # first pass warms the instrumented path
+                _, _, dt, n, k = calls[target]
+                durs.append(us * 1e-6)
+                # weights + f32 activations read + f32 outputs written
+                alg_bytes.append(ggml_bytes(dt, n, k) + 4 * k + 4 * n)
             torch.cuda.synchronize()
-            if rep == 0:
-                continue  # first pass warms the instrumented path
-            for (a, b), i in zip(evs, q4k_calls):
-                _, _, dt, n, k = calls[i]
-                durs.append(a.elapsed_time(b) * 1e-3)
-                # weights + quantized activations read (Q8K: k + k/256*(4+32) bytes) + f32 outputs written
-                alg_bytes.append(ggml_bytes(dt, n, k) + k + k // 256 * 36 + 4 * n)
-    avg_dur = sum(durs) / len(durs)
+        eager_avg_dur = sum(durs) / len(durs)
+        # The same launches back to back, as in the timed region: a HIP graph of the Q4_K calls
+        # alone, replayed between two events on this stream; time / launches bounds the kernel's
+        # average duration from above (it includes the dispatch gaps between kernels).
+        avg_dur = eager_avg_dur
+        if graph is not None:
+            g4 = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g4, stream=side):
+                s_cap = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+                for i in q4k_calls:
+                    run_call(i, 0, s_cap)
+            for _ in range(3):
+                g4.replay()
+            torch.cuda.synchronize()
+            f0, f1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            f0.record()
+            for _ in range(args.steps):
+                g4.replay()
+            f1.record()
+            torch.cuda.synchronize()
+            avg_dur = f0.elapsed_time(f1) * 1e-3 / (args.steps * len(q4k_calls))
     avg_bytes = sum(alg_bytes) / len(alg_bytes)
     achieved = avg_bytes / avg_dur / 1e9
     # headline shape alone (gate/up, 11008x4096)
     big = [(d, b) for d, b in zip(durs, alg_bytes) if b > 20_000_000]
     big_gbs = (sum(b for _, b in big) / sum(d for d, _ in big) / 1e9) if big else None
+    small = [(d, b) for d, b in zip(durs, alg_bytes) if b <= 20_000_000]
+    small_gbs = (sum(b for _, b in small) / sum(d for d, _ in small) / 1e9) if small else None
+
+    # ---- the other half of the metric: Q4_K prefill GEMM, M = 512 on the Mistral FFN shape ----
+    # (BASELINE.json configs[2]; reported beside the headline, not as `value`)
+    gm, gk, gn = 512, 4096, 14336
+    gen.manual_seed(4242)
+    gw = torch.randn((gn, gk), generator=gen, device=dev, dtype=torch.float32) * 0.02
+    gq = qhip.QWeight.zeros(qhip.Q4K, gn, gk).quantize_(gw)
+    del gw
+    gx = torch.randn((gm, gk), generator=gen, device=dev, dtype=torch.float32)
+    gy = torch.empty((gm, gn), device=dev, dtype=torch.float32)
+    gws = torch.empty(gq.workspace_bytes(gm), dtype=torch.uint8, device=dev)
+
+    def gemm_call(flags):
+        qhip.check(L.cq_qmatmul(gq.handle, C.c_void_p(gx.data_ptr()), gm, C.c_void_p(gy.data_ptr()), flags,
+                                C.c_void_p(gws.data_ptr()), gws.numel(),
+                                C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+
+    gemm_us = []
+    for rep in range(12):
+        for _ in range(4):
+            gemm_call(0)
+        us = qhip.timed_kernel_us(lambda: gemm_call(0))
+        if rep >= 2:
+            gemm_us.append(us)
+    gemm_avg_us = sum(gemm_us) / len(gemm_us)
+    gemm_tops = 2.0 * gm * gk * gn / (gemm_avg_us * 1e-6) / 1e12
+    del gq, gx, gy, gws
 
     value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
     result = {
@@ -188,17 +251,29 @@ def main() -> int:
             "setup_s": round(t_setup, 1),
         },
         "roofline": {
-            "kernel": "matvec_kernel<Q4K, 1>",
+            "kernel": "fused_kernel<Q4K> (decode matvec, all Q4_K launches of the step)",
             "bound": "hbm",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": Q4K_DECODE_TRAFFIC_BYTES_PER_LAUNCH if args.layers == LAYERS else None,
             "avg_launch_us": round(avg_dur * 1e6, 3),
             "alg_bytes_per_launch": int(avg_bytes),
             "launches_timed": len(durs),
-            "gate_up_11008x4096_GBs": round(big_gbs, 1) if big_gbs else None,
+            "timing": "graph replay of the 192 Q4_K launches between two HIP events, time / launches"
+                      if graph is not None else "per-kernel HIP event pairs, eager launches",
+            "per_kernel_events_avg_launch_us": round(eager_avg_dur * 1e6, 3),
+            "per_kernel_events_gate_up_11008x4096_GBs": round(big_gbs, 1) if big_gbs else None,
+            "per_kernel_events_attn_4096x4096_GBs": round(small_gbs, 1) if small_gbs else None,
+        },
+        "prefill_gemm": {
+            "workload": "configs[2]: Q4_K [14336x4096] x Q8_K activations, M=512 (Mistral-7B FFN up/gate)",
+            "kernel": "gemm_kernel<Q4K> (int8 MFMA, quantizer launch not included)",
+            "avg_launch_us": round(gemm_avg_us, 2),
+            "tops": round(gemm_tops, 1),
+            "peak_tops": 5000.0,
+            "frac_of_int8_mfma_peak": round(gemm_tops / 5000.0, 4),
         },
     }
 
@@ -206,7 +281,7 @@ def main() -> int:
     if not args.no_cpu:
         from oracle import cpu_oracle as orc
         threads = orc.baseline_lib().cpub_num_threads()
-        sample_layers = min(2, args.layers)
+        sample_layers = min(8, args.layers)  # ~1 GB of weights: larger than the host's last-level cache
         host = []
         for i in range(sample_layers * len(LAYER_SHAPES)):
             qw, xin, dt, n, k = calls[i]

@@ -11,6 +11,24 @@
 // ------------------------------------------------------------------ errors ----
 static thread_local char g_err[512] = "";
 
+// ---- kernel timing hook ------------------------------------------------------------------------
+namespace {
+struct KernelTimer {
+    hipEvent_t start = nullptr, stop = nullptr;
+    bool armed = false, pending = false;
+};
+thread_local KernelTimer g_timer;
+}  // namespace
+
+bool cq_timing_take(hipEvent_t *start, hipEvent_t *stop) {
+    if (!g_timer.armed) return false;
+    g_timer.armed = false;
+    g_timer.pending = true;
+    *start = g_timer.start;
+    *stop = g_timer.stop;
+    return true;
+}
+
 int cq_set_error(int code, const char *fmt, ...) {
     va_list ap;
     va_start(ap, fmt);
@@ -421,5 +439,26 @@ extern "C" int cq_moe_scatter_add(int dev, const float *y, const int32_t *row_id
     if (!ys || (total_rows && (!y || !row_ids || !weights))) return cq_set_error(CQ_ERR_INVALID, "null argument");
     CQ_HIP_CHECK(hipSetDevice(dev));
     CQ_HIP_CHECK(cq_launch_scatter_add(y, row_ids, weights, total_rows, hidden, ys, tokens, (hipStream_t)stream));
+    return CQ_OK;
+}
+
+extern "C" int cq_timing_arm(void) {
+    if (!g_timer.start) {
+        CQ_HIP_CHECK(hipEventCreate(&g_timer.start));
+        CQ_HIP_CHECK(hipEventCreate(&g_timer.stop));
+    }
+    g_timer.armed = true;
+    g_timer.pending = false;
+    return CQ_OK;
+}
+
+extern "C" int cq_timing_elapsed_us(double *us) {
+    if (!us) return cq_set_error(CQ_ERR_INVALID, "us is null");
+    if (!g_timer.pending) return cq_set_error(CQ_ERR_INVALID, "no armed kernel launch to read");
+    g_timer.pending = false;
+    CQ_HIP_CHECK(hipEventSynchronize(g_timer.stop));
+    float ms = 0.0f;
+    CQ_HIP_CHECK(hipEventElapsedTime(&ms, g_timer.start, g_timer.stop));
+    *us = (double)ms * 1e3;
     return CQ_OK;
 }

@@ -405,7 +405,7 @@ hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hip
         if (e != hipSuccess) return e;
     }
     dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)ksplit);
-    gemm_kernel<DT, MT><<<grid, kThreads, lds, s>>>(*w, a, m, y, ksplit);
+    CQ_LAUNCH((gemm_kernel<DT, MT>), grid, kThreads, lds, s, *w, a, m, y, ksplit);
     return hipGetLastError();
 }
 

@@ -568,8 +568,8 @@ hipError_t launch_fused_upl(const cq_weight *w, const float *x, float *y, hipStr
     int64_t wgs = w->n / (NW * depth);
     if (wgs > max_wgs) wgs = max_wgs;
     const int64_t tw = wgs * NW, rpw = w->n / tw, extra = w->n % tw;
-    if (depth == 2) fused_kernel<DT, UPL, NW, 2><<<(unsigned)wgs, NW * 64, lds, s>>>(*w, x, y, tw, rpw, extra);
-    else fused_kernel<DT, UPL, NW, 1><<<(unsigned)wgs, NW * 64, lds, s>>>(*w, x, y, tw, rpw, extra);
+    if (depth == 2) CQ_LAUNCH((fused_kernel<DT, UPL, NW, 2>), (unsigned)wgs, NW * 64, lds, s, *w, x, y, tw, rpw, extra);
+    else CQ_LAUNCH((fused_kernel<DT, UPL, NW, 1>), (unsigned)wgs, NW * 64, lds, s, *w, x, y, tw, rpw, extra);
     return hipGetLastError();
 }
 
@@ -610,9 +610,9 @@ hipError_t launch_staged(const cq_weight *w, cq_act_view a, int64_t m, float *y,
         while (mb > 1 && lds_row_bytes<DT>(w->k) * mb > 64 * 1024) mb >>= 1;
         const size_t lds = lds_row_bytes<DT>(w->k) * mb;
         if (lds > 64 * 1024) return hipErrorInvalidValue;
-        if (mb == 4) staged_kernel<DT, 4><<<grid, kStagedThreads, lds, s>>>(*w, a, m0, rpw, y);
-        else if (mb == 2) staged_kernel<DT, 2><<<grid, kStagedThreads, lds, s>>>(*w, a, m0, rpw, y);
-        else staged_kernel<DT, 1><<<grid, kStagedThreads, lds, s>>>(*w, a, m0, rpw, y);
+        if (mb == 4) CQ_LAUNCH((staged_kernel<DT, 4>), grid, kStagedThreads, lds, s, *w, a, m0, rpw, y);
+        else if (mb == 2) CQ_LAUNCH((staged_kernel<DT, 2>), grid, kStagedThreads, lds, s, *w, a, m0, rpw, y);
+        else CQ_LAUNCH((staged_kernel<DT, 1>), grid, kStagedThreads, lds, s, *w, a, m0, rpw, y);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         m0 += mb;

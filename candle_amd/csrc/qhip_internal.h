@@ -76,6 +76,10 @@ int cq_set_error(int code, const char *fmt, ...);
                                 __FILE__, __LINE__);                                             \
     } while (0)
 
+// Kernel timing hook (api.hip): true when the calling thread armed the timer; the launch then goes
+// through CQ_LAUNCH below with the two events.  Disarms.
+bool cq_timing_take(hipEvent_t *start, hipEvent_t *stop);
+
 // ---- launchers implemented in the .hip files -------------------------------
 // repack.hip
 hipError_t cq_launch_repack(const cq_weight *w, const uint8_t *aos_dev, hipStream_t s);   // GGML AoS -> planes
@@ -104,6 +108,20 @@ hipError_t cq_launch_scatter_add(const float *y, const int32_t *row_ids, const f
                                  int64_t hidden, float *ys, int64_t tokens, hipStream_t s);
 
 hipError_t cq_launch_fill_zero(float *p, int64_t count, hipStream_t s);
+
+#if defined(__HIPCC__)
+#include <hip/hip_ext.h>
+// Kernel launch that honours the timing hook.  `kernel` in parentheses when it contains commas.
+#define CQ_LAUNCH(kernel, grid, block, lds, stream, ...)                                                  \
+    do {                                                                                                  \
+        hipEvent_t _ea, _eb;                                                                              \
+        if (cq_timing_take(&_ea, &_eb))                                                                   \
+            hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(block), (uint32_t)(lds), stream, _ea, _eb, 0,  \
+                                  __VA_ARGS__);                                                           \
+        else                                                                                              \
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), (uint32_t)(lds), stream, __VA_ARGS__);    \
+    } while (0)
+#endif
 
 // ---- small device helpers ---------------------------------------------------
 #if defined(__HIPCC__)

@@ -23,7 +23,7 @@ EXPORTS = [
     "cq_weight_dequantize_f16", "cq_weight_to_ggml", "cq_weight_size_in_bytes", "cq_weight_dtype",
     "cq_weight_device", "cq_weight_shape", "cq_weight_destroy", "cq_act_bytes", "cq_quantize_act",
     "cq_workspace_bytes", "cq_qmatmul", "cq_qmatmul_int_dots", "cq_grouped_workspace_bytes",
-    "cq_qmatmul_grouped", "cq_silu_mul", "cq_moe_scatter_add",
+    "cq_qmatmul_grouped", "cq_silu_mul", "cq_moe_scatter_add", "cq_timing_arm", "cq_timing_elapsed_us",
 ]
 
 
@@ -70,6 +70,8 @@ def load():
     L.cq_qmatmul_grouped.argtypes = [C.POINTER(vp), ci, vp, vp, C.POINTER(C.c_int32), vp, ci, vp, sz, vp]
     L.cq_silu_mul.argtypes = [ci, vp, vp, vp, i64, vp]
     L.cq_moe_scatter_add.argtypes = [ci, vp, vp, vp, i64, i64, vp, i64, vp]
+    L.cq_timing_arm.argtypes = []
+    L.cq_timing_elapsed_us.argtypes = [C.POINTER(C.c_double)]
     _lib = L
     return L
 
@@ -289,3 +291,14 @@ def moe_scatter_add(y, row_ids, weights, tokens: int):
                                     C.c_void_p(weights.data_ptr()), total, hidden, C.c_void_p(ys.data_ptr()),
                                     tokens, _stream_ptr()))
     return ys
+
+
+def timed_kernel_us(launch) -> float:
+    """Runs `launch()` (which must call cq_qmatmul once on this thread) with the library's kernel
+    timer armed and returns the duration of its matmul kernel in microseconds."""
+    L = load()
+    check(L.cq_timing_arm())
+    launch()
+    us = C.c_double()
+    check(L.cq_timing_elapsed_us(C.byref(us)))
+    return us.value

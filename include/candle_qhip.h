@@ -143,6 +143,15 @@ int cq_silu_mul(int dev, const float *a_dev, const float *b_dev, float *h_dev, i
 int cq_moe_scatter_add(int dev, const float *y_dev, const int32_t *row_ids_dev, const float *weights_dev,
                        int64_t total_rows, int64_t hidden, float *ys_dev, int64_t tokens, void *stream);
 
+/* ---- measurement aid (no counterpart in the reference) ---------------------------------------
+ * cq_timing_arm(): the next matmul kernel this host thread launches through cq_qmatmul (the
+ * matvec / GEMM kernel proper, not a separate activation-quantizer launch) is bracketed by a pair
+ * of HIP events owned by the library, recorded on the stream of that launch.
+ * cq_timing_elapsed_us(): waits for that kernel and returns its duration in microseconds;
+ * CQ_ERR_INVALID when no armed launch has happened since the last call. */
+int cq_timing_arm(void);
+int cq_timing_elapsed_us(double *us);
+
 #ifdef __cplusplus
 }
 #endif
