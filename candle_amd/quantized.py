@@ -1,0 +1,177 @@
+"""The reference's quantized-tensor surface on top of libcandle_qhip.so.
+
+Mirrors, name for name:
+  * `GgmlDType` (candle-core/src/quantized/mod.rs:133-247): ids, `block_size`, `type_size`,
+  * `QTensor` (mod.rs:35-38, 318-392): `quantize`, `dtype`, `shape`, `rank`, `dequantize`,
+    `dequantize_f16`, `storage_size_in_bytes`,
+  * `QMatMul` (mod.rs:394-462, 527-550): `from_qtensor`, `forward`,
+  * the Python binding's `QTensor.matmul_t` (candle-pyo3/src/lib.rs:1250-1255) and
+    `Tensor.quantize(str)` (lib.rs:1079-1102).
+Tensors are torch CUDA tensors (torch only owns the memory and the stream); every operation runs in
+the HIP library, and fails if that library or a GPU is missing.
+"""
+from __future__ import annotations
+
+import enum
+
+import numpy as np
+
+from . import qhip
+
+
+class GgmlDType(enum.IntEnum):
+    """GGML type ids as stored in GGUF files (mod.rs:152-171 `from_u32`, :173-190 `to_u32`).
+    Only the types this library computes with are listed."""
+    F32 = 0
+    F16 = 1
+    Q4_0 = 2
+    Q8_0 = 8
+    Q8_1 = 9
+    Q4K = 12
+    Q6K = 14
+    Q8K = 15
+
+    @classmethod
+    def from_str(cls, name: str) -> "GgmlDType":
+        """Names accepted by the reference's Python `Tensor.quantize` (lib.rs:1082-1098)."""
+        table = {"q4_0": cls.Q4_0, "q8_0": cls.Q8_0, "q8_1": cls.Q8_1, "q4k": cls.Q4K, "q6k": cls.Q6K,
+                 "q8k": cls.Q8K, "f32": cls.F32, "f16": cls.F16}
+        key = name.lower()
+        if key not in table:
+            raise ValueError(f"'{name}' is not a valid quantization type or is not supported by this build")
+        return table[key]
+
+    def block_size(self) -> int:
+        """mod.rs:234-246."""
+        if self in (GgmlDType.F32, GgmlDType.F16):
+            return 1
+        return qhip.load().cq_block_size(int(self))
+
+    def type_size(self) -> int:
+        """Bytes per block (mod.rs:212-232)."""
+        if self == GgmlDType.F32:
+            return 4
+        if self == GgmlDType.F16:
+            return 2
+        return qhip.load().cq_type_size(int(self))
+
+    def vec_dot_type(self) -> "GgmlDType":
+        """The activation type `matmul` quantizes to (`GgmlType::VecDotType`, k_quants.rs)."""
+        return GgmlDType(qhip.load().cq_vec_dot_type(int(self)))
+
+
+_WEIGHT_TYPES = (GgmlDType.Q4_0, GgmlDType.Q8_0, GgmlDType.Q4K, GgmlDType.Q6K)
+
+
+class QTensor:
+    """A quantized tensor on the device (mod.rs:318-392).  The matmul path takes rank-2 `[n, k]`
+    tensors; higher ranks are kept as their shape with the leading dims flattened into `n`."""
+
+    def __init__(self, weight: qhip.QWeight, shape):
+        self._w = weight
+        self._shape = tuple(int(s) for s in shape)
+
+    # ---- constructors ---------------------------------------------------------------------
+    @classmethod
+    def quantize(cls, src, dtype) -> "QTensor":
+        """`QTensor::quantize(src, dtype)` (mod.rs:325-343): src f32, last dim a multiple of the
+        block size.  Quantizes on the device, bit-identical to the CPU `from_float`."""
+        dtype = GgmlDType.from_str(dtype) if isinstance(dtype, str) else GgmlDType(dtype)
+        if dtype not in _WEIGHT_TYPES:
+            raise qhip.QHipError(f"quantize: unsupported dtype {dtype.name}")
+        shape = tuple(src.shape)
+        _check_shape(shape, dtype.block_size())
+        k = shape[-1]
+        n = int(np.prod(shape[:-1])) if len(shape) > 1 else 1
+        w = qhip.QWeight.zeros(int(dtype), n, k, dev=src.device.index or 0)
+        w.quantize_(src.contiguous() if not src.is_contiguous() else src)
+        return cls(w, shape)
+
+    @classmethod
+    def from_ggml(cls, dtype, blocks: np.ndarray, shape, dev: int = 0) -> "QTensor":
+        """Host GGML blocks -> device (the loader funnel `ggml_file.rs:120-135` -> `cuda.rs:591-612`)."""
+        dtype = GgmlDType(dtype)
+        shape = tuple(int(s) for s in shape)
+        _check_shape(shape, dtype.block_size())
+        k = shape[-1]
+        n = int(np.prod(shape[:-1])) if len(shape) > 1 else 1
+        return cls(qhip.QWeight.from_ggml(int(dtype), blocks, n, k, dev), shape)
+
+    # ---- getters (mod.rs:345-359; lib.rs:1214-1240) ---------------------------------------------
+    @property
+    def ggml_dtype(self) -> str:
+        return GgmlDType(self._w.dtype).name
+
+    def dtype(self) -> GgmlDType:
+        return GgmlDType(self._w.dtype)
+
+    @property
+    def shape(self):
+        return self._shape
+
+    def rank(self) -> int:
+        return len(self._shape)
+
+    def storage_size_in_bytes(self) -> int:
+        return self._w.size_in_bytes
+
+    @property
+    def weight(self) -> qhip.QWeight:
+        return self._w
+
+    # ---- operations -----------------------------------------------------------------------------
+    def dequantize(self):
+        """mod.rs:361-365."""
+        return self._w.dequantize().reshape(self._shape)
+
+    def dequantize_f16(self):
+        """mod.rs:367-382: equals `dequantize().to(f16)` bit for bit."""
+        return self._w.dequantize_f16().reshape(self._shape)
+
+    def data(self) -> np.ndarray:
+        """The GGML blocks on the host (`QTensor::data`, mod.rs:388-391).  The reference's device
+        backends bail here; this build offers the inverse re-pack instead."""
+        return self._w.to_ggml()
+
+    def matmul_t(self, lhs):
+        """`lhs @ self.T` (lib.rs:1250-1255)."""
+        return QMatMul.from_qtensor(self).forward(lhs)
+
+    def __repr__(self) -> str:
+        return f"QTensor[{self._shape}; {self.ggml_dtype.lower()}]"
+
+
+def _check_shape(shape, block_size: int):
+    """`check_shape` (mod.rs:304-316)."""
+    if len(shape) == 0:
+        raise qhip.QHipError("scalar tensor cannot be quantized")
+    if shape[-1] % block_size != 0:
+        raise qhip.QHipError(f"quantized tensor must have their last dim divisible by block size "
+                             f"{tuple(shape)} {block_size}")
+
+
+class QMatMul:
+    """`QMatMul::QTensor` arm (mod.rs:394-462): y = x . W^T with W quantized, computed by the
+    device kernels without dequantizing W."""
+
+    def __init__(self, qtensor: QTensor):
+        if qtensor.rank() != 2:
+            raise qhip.QHipError(f"QMatMul needs a rank-2 weight, got {qtensor.shape}")
+        self.qtensor = qtensor
+        self._ws = qhip.Workspace()
+
+    @classmethod
+    def from_qtensor(cls, qtensor: QTensor) -> "QMatMul":
+        return cls(qtensor)
+
+    @classmethod
+    def from_arc(cls, qtensor: QTensor) -> "QMatMul":
+        return cls(qtensor)
+
+    def forward(self, xs):
+        """mod.rs:528-550 -> `cpu_fwd` semantics (mod.rs:469-500): xs f32, contiguous, rank >= 2,
+        last dim == k; result has xs' shape with the last dim replaced by n."""
+        return qhip.qmatmul(self.qtensor.weight, xs, workspace=self._ws)
+
+    def dequantize_f16(self):
+        return self.qtensor.dequantize_f16()
