@@ -110,7 +110,7 @@ static int weight_alloc(int dev, int dt, int64_t n, int64_t k, cq_weight **out) 
     switch (dt) {
     case CQ_DTYPE_Q4_0: s0 = (size_t)nb * 16; s1 = (size_t)nb * 2; break;
     case CQ_DTYPE_Q8_0: s0 = (size_t)nb * 32; s1 = (size_t)nb * 2; break;
-    case CQ_DTYPE_Q4K: s0 = (size_t)nb * 128; s1 = (size_t)nb * 16; break;
+    case CQ_DTYPE_Q4K: s0 = (size_t)nb * 128; s1 = (size_t)nb * CQ_Q4K_HDR; break;
     case CQ_DTYPE_Q6K: s0 = (size_t)nb * 128; s1 = (size_t)nb * 64; s2 = (size_t)nb * 16; s3 = (size_t)nb * 2; break;
     }
     const size_t o1 = cq_align_up(s0 + CQ_TAIL_PAD, 256);

@@ -54,11 +54,11 @@ __global__ void dequant_q4k(const uint8_t *__restrict__ qs, const uint8_t *__res
     const int64_t b = u >> 3;
     const int p = (int)(u & 7), g = p >> 1, half = p & 1;
     const uint4 q = *(const uint4 *)(qs + u * 16);
-    const uint4 h = *(const uint4 *)(hd + b * 16);
-    const float d = cq_h2f((uint16_t)(h.x & 0xffff)), dmin = cq_h2f((uint16_t)(h.x >> 16));
-    int sc1, m1, sc2, m2;
-    cq_scale_min_k4(2 * g, h.y, h.z, h.w, sc1, m1);
-    cq_scale_min_k4(2 * g + 1, h.y, h.z, h.w, sc2, m2);
+    const uint32_t *h = (const uint32_t *)(hd + b * CQ_Q4K_HDR);
+    const uint32_t dd = h[0], rec = h[1 + g];
+    const float d = cq_h2f((uint16_t)(dd & 0xffff)), dmin = cq_h2f((uint16_t)(dd >> 16));
+    const int sc1 = (int)(rec & 0xff), sc2 = (int)((rec >> 8) & 0xff);
+    const int m1 = (int)((rec >> 16) & 0xff), m2 = (int)(rec >> 24);
     const float d1 = d * (float)sc1, mm1 = dmin * (float)m1;
     const float d2 = d * (float)sc2, mm2 = dmin * (float)m2;
     const uint32_t w[4] = {q.x, q.y, q.z, q.w};

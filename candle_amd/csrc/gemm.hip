@@ -153,10 +153,12 @@ __device__ __forceinline__ void stage_issue(uint8_t *buf, const cq_weight &w, co
 
 // The small per-block weight fields, loaded straight into registers one block ahead.
 template <int DT> struct WHead;
-template <> struct WHead<CQ_DTYPE_Q4K> { uint4 hd; };               // d, dmin, scales[12]
+template <> struct WHead<CQ_DTYPE_Q4K> { uint32_t dd; uint4 rec; };   // d | dmin << 16; records {sc, sc, mn, mn} per 32 qs bytes
 template <> struct WHead<CQ_DTYPE_Q6K> { uint4 sc; uint32_t d; };   // re-packed scales (two per unit); d
 __device__ __forceinline__ void load_head(const cq_weight &w, int64_t blk, WHead<CQ_DTYPE_Q4K> &r) {
-    r.hd = *(const uint4 *)(w.p1 + blk * 16);
+    const uint32_t *h = (const uint32_t *)(w.p1 + blk * CQ_Q4K_HDR);
+    r.dd = h[0];
+    r.rec = make_uint4(h[1], h[2], h[3], h[4]);
 }
 __device__ __forceinline__ void load_head(const cq_weight &w, int64_t blk, WHead<CQ_DTYPE_Q6K> &r) {
     r.sc = *(const uint4 *)(w.p2 + blk * 16);
@@ -224,14 +226,9 @@ template <int MT>
 __device__ __forceinline__ void block_mac(const uint8_t *cur, const uint8_t *wl, const LaneGeo &g,
                                           const WHead<CQ_DTYPE_Q4K> &wb, int lane, v4f (&out)[2 * MT]) {
     const uint32_t kq = lane >> 4;
-    const uint4 hd = wb.hd;
-    const float dw = cq_h2f((uint16_t)(hd.x & 0xffff));
-    const float dmin = cq_h2f((uint16_t)(hd.x >> 16));
-    // all eight scales and mins as bytes (k_quants.rs:1209-1219)
-    const uint32_t sc03 = hd.y & 0x3f3f3f3fu;
-    const uint32_t sc47 = (hd.w & 0x0f0f0f0fu) | (((hd.y >> 6) & 0x03030303u) << 4);
-    const uint32_t mn03 = hd.z & 0x3f3f3f3fu;
-    const uint32_t mn47 = ((hd.w >> 4) & 0x0f0f0f0fu) | (((hd.z >> 6) & 0x03030303u) << 4);
+    const float dw = cq_h2f((uint16_t)(wb.dd & 0xffff));
+    const float dmin = cq_h2f((uint16_t)(wb.dd >> 16));
+    const uint32_t rec[4] = {wb.rec.x, wb.rec.y, wb.rec.z, wb.rec.w};
     // K-slice g = elements 64g..64g+63 = qs bytes 32g..32g+31, low nibbles for the first 32 elements
     // (quarters 0,1: sub-block 2g), high nibbles for the last 32 (quarters 2,3: sub-block 2g+1)
     const uint32_t hi = kq >> 1, nsh = hi * 4;
@@ -239,8 +236,7 @@ __device__ __forceinline__ void block_mac(const uint8_t *cur, const uint8_t *wl,
 #pragma unroll
     for (int gi = 0; gi < 4; gi++) {
         const uint4 q = *(const uint4 *)(wl + g.w_col4[gi]);
-        const uint32_t scw = gi < 2 ? sc03 : sc47;
-        const uint32_t sj = (scw >> (16 * (gi & 1) + 8 * hi)) & 0xff;
+        const uint32_t sj = (rec[gi] >> (8 * hi)) & 0xff;   // scale of sub-block 2g + hi
         const uint32_t sl = dup16(sj & 7), sh = dup16(sj >> 3);
         const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
@@ -253,8 +249,7 @@ __device__ __forceinline__ void block_mac(const uint8_t *cur, const uint8_t *wl,
     v8h wmin;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
-        const uint32_t mw = j < 4 ? mn03 : mn47;
-        const float v = -dmin * (float)((mw >> (8 * (j & 3))) & 0xff);
+        const float v = -dmin * (float)((rec[j >> 1] >> (16 + 8 * (j & 1))) & 0xff);
         const _Float16 p1 = (_Float16)v;
         wmin[j] = (kq & 1) == 0 ? p1 : (_Float16)(v - (float)p1);
     }

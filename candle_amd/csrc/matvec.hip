@@ -4,8 +4,9 @@
 // (k_quants.rs:237-254, :631-649, :1171-1250, :1585-1641): integer block dots against Q8_0 / Q8K
 // activations, then f32 scales.
 //
-// Work split: a "unit" is one 16-byte lane of a row's main plane (32 elements for Q4_0, Q4K and
-// Q6K, 16 for Q8_0).  A wave walks one row 64 units (1 KiB, eight 128-byte lines) at a time;
+// Work split: a "unit" is what one lane takes of a row's main plane per step: 16 bytes (32 elements
+// for Q4_0 and Q6K, 16 for Q8_0), or 32 bytes for Q4K (64 elements = two whole sub-blocks, so the
+// lane's scale/min record is decoded once for them).  A wave walks one row 64 units at a time;
 // nibbles are split in registers and contracted with v_dot4_i32_i8; the lane sums are reduced
 // with DPP.  Quantized activations sit in LDS, permuted so that lane l of a chunk reads its
 // operands at l * 16 bytes (no bank conflicts).
@@ -22,20 +23,21 @@
 namespace {
 
 template <int DT> struct Geo;
-template <> struct Geo<CQ_DTYPE_Q4_0> { static constexpr int kElems = 32; static constexpr bool kHi = true;  static constexpr int kUnitsPerBlock = 1; static constexpr bool kActK = false; };
-template <> struct Geo<CQ_DTYPE_Q8_0> { static constexpr int kElems = 16; static constexpr bool kHi = false; static constexpr int kUnitsPerBlock = 2; static constexpr bool kActK = false; };
-template <> struct Geo<CQ_DTYPE_Q4K>  { static constexpr int kElems = 32; static constexpr bool kHi = true;  static constexpr int kUnitsPerBlock = 8; static constexpr bool kActK = true; };
-template <> struct Geo<CQ_DTYPE_Q6K>  { static constexpr int kElems = 32; static constexpr bool kHi = true;  static constexpr int kUnitsPerBlock = 8; static constexpr bool kActK = true; };
+template <> struct Geo<CQ_DTYPE_Q4_0> { static constexpr int kElems = 32;  static constexpr int kUnitsPerBlock = 1; static constexpr bool kActK = false; };
+template <> struct Geo<CQ_DTYPE_Q8_0> { static constexpr int kElems = 16;  static constexpr int kUnitsPerBlock = 2; static constexpr bool kActK = false; };
+template <> struct Geo<CQ_DTYPE_Q4K>  { static constexpr int kElems = 64;  static constexpr int kUnitsPerBlock = 4; static constexpr bool kActK = true; };
+template <> struct Geo<CQ_DTYPE_Q6K>  { static constexpr int kElems = 32;  static constexpr int kUnitsPerBlock = 8; static constexpr bool kActK = true; };
 
 // ---------------------------------------------------------------------------------------------
 // LDS image of one quantized activation row:
 //   lo [units] int4, hi [units] int4 (nibble types), d [blocks] f32,
-//   bs: Q8K activations: bsums [blocks][16] i16 ; Q8_0 activations: sum of the 32 quants [blocks] i32
+//   bs: Q6K: bsums [blocks][16] i16 ; Q8_0 activations: sum of the 32 quants [blocks] i32
+//   Q4K: four planes [units] int4 (elements 64u + 16j + [0,16) in plane j), d [blocks] f32,
+//        bs [units] {i16 sum of elements 64u..64u+31, i16 sum of elements 64u+32..64u+63}
 // ---------------------------------------------------------------------------------------------
 template <int DT> __host__ __device__ constexpr int64_t act_blocks(int64_t k) { return Geo<DT>::kActK ? k / 256 : k / 32; }
 template <int DT> __host__ __device__ constexpr size_t lds_row_bytes(int64_t k) {
-    const int64_t units = k / Geo<DT>::kElems;
-    return (size_t)units * (Geo<DT>::kHi ? 32 : 16) + (size_t)act_blocks<DT>(k) * (Geo<DT>::kActK ? 4 + 32 : 4 + 4);
+    return (size_t)k + (size_t)act_blocks<DT>(k) * (DT == CQ_DTYPE_Q4K ? 4 + 16 : (Geo<DT>::kActK ? 4 + 32 : 4 + 4));
 }
 
 // Byte offsets from the start of dynamic LDS (plain integers: every access below is then a
@@ -48,8 +50,9 @@ template <int DT> __device__ __forceinline__ LdsRow lds_row(int64_t k, int m) {
     const uint32_t units = (uint32_t)(k / Geo<DT>::kElems);
     uint32_t p = (uint32_t)m * (uint32_t)lds_row_bytes<DT>(k);
     LdsRow r;
-    r.lo = p; p += units * 16;
-    r.hi = p; if (Geo<DT>::kHi) p += units * 16;
+    r.lo = p;
+    r.hi = p + units * 16;
+    p += (uint32_t)k;
     r.d = p; p += (uint32_t)act_blocks<DT>(k) * 4;
     r.bs = p;
     return r;
@@ -58,23 +61,16 @@ template <int DT> __device__ __forceinline__ LdsRow lds_row(int64_t k, int m) {
 template <typename T> __device__ __forceinline__ T lds_get(const uint8_t *smem, uint32_t off) { return *(const T *)(smem + off); }
 template <typename T> __device__ __forceinline__ void lds_put(uint8_t *smem, uint32_t off, T v) { *(T *)(smem + off) = v; }
 
-// Where the 16 consecutive activation elements [16*piece, 16*piece+16) of a row go.
-template <int DT> __device__ __forceinline__ void piece_slot(int64_t piece, int64_t &unit, bool &hi) {
-    if (DT == CQ_DTYPE_Q8_0) { unit = piece; hi = false; return; }
-    if (DT == CQ_DTYPE_Q4_0) { unit = piece >> 1; hi = piece & 1; return; }
+// Byte offset in LDS of the 16 consecutive activation elements [16*piece, 16*piece+16) of a row.
+template <int DT> __device__ __forceinline__ uint32_t piece_off(const LdsRow r, int64_t piece, uint32_t units) {
+    if (DT == CQ_DTYPE_Q8_0) return r.lo + (uint32_t)piece * 16;
+    if (DT == CQ_DTYPE_Q4_0) return ((piece & 1) ? r.hi : r.lo) + (uint32_t)(piece >> 1) * 16;
+    if (DT == CQ_DTYPE_Q4K) return r.lo + (uint32_t)(piece & 3) * units * 16 + (uint32_t)(piece >> 2) * 16;
+    // Q6K: unit p = 4h + 2t + i covers 128h + 32t + 16i + [0,16) (low) and + 64 (high)
     const int64_t b = piece >> 4;
     const int w = (int)(piece & 15);
-    if (DT == CQ_DTYPE_Q4K) {
-        // unit p = 2g + r covers elements 64g + 16r + [0,16) (low nibbles) and + 32 (high nibbles)
-        const int g = w >> 2, r = w & 3;
-        unit = 8 * b + 2 * g + (r & 1);
-        hi = r >= 2;
-    } else {
-        // Q6K: unit p = 4h + 2t + i covers 128h + 32t + 16i + [0,16) (low) and + 64 (high)
-        const int h = w >> 3, o = w & 7;
-        unit = 8 * b + 4 * h + (o & 3);
-        hi = o >= 4;
-    }
+    const int h = w >> 3, o = w & 7;
+    return (o >= 4 ? r.hi : r.lo) + (uint32_t)(8 * b + 4 * h + (o & 3)) * 16;
 }
 
 // ------------------------------------------------------------------ wave reductions (DPP) ----
@@ -127,7 +123,7 @@ __device__ __forceinline__ uint32_t pack4(int8_t a, int8_t b, int8_t c, int8_t d
 // One 256-element chunk (chunk index c, this lane's four elements f at e0 = 256c + 4*lane).
 template <int DT>
 __device__ __forceinline__ void quantize_chunk_to_lds(uint8_t *smem, const float4 fin, int c, int e0, bool active,
-                                                      bool chunk_ok, const LdsRow r) {
+                                                      bool chunk_ok, const LdsRow r, uint32_t units) {
     const int lane = threadIdx.x & 63;
     const float4 f = active ? fin : make_float4(0.f, 0.f, 0.f, 0.f);
     {
@@ -160,7 +156,12 @@ __device__ __forceinline__ void quantize_chunk_to_lds(uint8_t *smem, const float
             sum4 += dpp_i<kQuadSwap1>(sum4);
             sum4 += dpp_i<kQuadSwap2>(sum4);  // the four lanes of a 16-element group hold its sum
             if (chunk_ok && lane == 0) lds_put<float>(smem, r.d + 4 * c, d);
-            if (chunk_ok && (lane & 3) == 0) lds_put<int16_t>(smem, r.bs + 2 * (c * 16 + (lane >> 2)), (int16_t)sum4);
+            if (DT == CQ_DTYPE_Q4K) {
+                sum4 += dpp_i<kHalfMirror>(sum4);   // eight lanes = one 32-element sub-block
+                if (chunk_ok && (lane & 7) == 0) lds_put<int16_t>(smem, r.bs + 2 * (c * 8 + (lane >> 3)), (int16_t)sum4);
+            } else if (chunk_ok && (lane & 3) == 0) {
+                lds_put<int16_t>(smem, r.bs + 2 * (c * 16 + (lane >> 2)), (int16_t)sum4);
+            }
         } else {
             float amax = fmaxf(fmaxf(fmaxf(fmaxf(0.0f, fabsf(f.x)), fabsf(f.y)), fabsf(f.z)), fabsf(f.w));
             amax = fmaxf(amax, dpp_f<kQuadSwap1>(amax));
@@ -180,11 +181,7 @@ __device__ __forceinline__ void quantize_chunk_to_lds(uint8_t *smem, const float
                 lds_put<int32_t>(smem, r.bs + 4 * (e0 >> 5), sum4);
             }
         }
-        if (active) {
-            int64_t unit; bool hi;
-            piece_slot<DT>(e0 >> 4, unit, hi);
-            lds_put<uint32_t>(smem, (hi ? r.hi : r.lo) + (uint32_t)unit * 16 + 4 * (lane & 3), packed);
-        }
+        if (active) lds_put<uint32_t>(smem, piece_off<DT>(r, e0 >> 4, units) + 4 * (lane & 3), packed);
     }
 }
 
@@ -214,7 +211,7 @@ __device__ __forceinline__ void quantize_row_to_lds(uint8_t *smem, int64_t k, in
     for (int i = 0; i < XCH; i++) {
         const int c = wave + i * NW;
         const int e0 = c * 256 + 4 * lane;
-        quantize_chunk_to_lds<DT>(smem, fx[i], c, e0, c < chunks && e0 < k, c < chunks, r);
+        quantize_chunk_to_lds<DT>(smem, fx[i], c, e0, c < chunks && e0 < k, c < chunks, r, (uint32_t)(k / Geo<DT>::kElems));
     }
 }
 
@@ -222,11 +219,9 @@ __device__ __forceinline__ void quantize_row_to_lds(uint8_t *smem, int64_t k, in
 template <int DT, int NT>
 __device__ __forceinline__ void stage_row(uint8_t *smem, const LdsRow r, const cq_act_view &a, int64_t row, int64_t k) {
     const int4 *src = (const int4 *)(a.qs + row * k);
-    for (int piece = threadIdx.x; piece < (int)(k / 16); piece += NT) {
-        int64_t unit; bool hi;
-        piece_slot<DT>(piece, unit, hi);
-        lds_put<int4>(smem, (hi ? r.hi : r.lo) + (uint32_t)unit * 16, src[piece]);
-    }
+    const uint32_t units = (uint32_t)(k / Geo<DT>::kElems);
+    for (int piece = threadIdx.x; piece < (int)(k / 16); piece += NT)
+        lds_put<int4>(smem, piece_off<DT>(r, piece, units), src[piece]);
     const int nb = (int)act_blocks<DT>(k);
     for (int b = threadIdx.x; b < nb; b += NT) {
         lds_put<float>(smem, r.d + 4 * b, a.d[row * nb + b]);
@@ -234,7 +229,11 @@ __device__ __forceinline__ void stage_row(uint8_t *smem, const LdsRow r, const c
     }
     if (Geo<DT>::kActK) {
         const int32_t *bs = (const int32_t *)(a.bsums + row * nb * 16);  // 8 words per block
-        for (int i = threadIdx.x; i < nb * 8; i += NT) lds_put<int32_t>(smem, r.bs + 4 * i, bs[i]);
+        for (int i = threadIdx.x; i < nb * 8; i += NT) {
+            const int32_t two = bs[i];   // bsums 2i and 2i+1: the two halves of 32-element sub-block i
+            if (DT == CQ_DTYPE_Q4K) lds_put<int16_t>(smem, r.bs + 2 * i, (int16_t)((int16_t)(two & 0xffff) + (int16_t)(two >> 16)));
+            else lds_put<int32_t>(smem, r.bs + 4 * i, two);
+        }
     }
 }
 
@@ -242,7 +241,8 @@ __device__ __forceinline__ void stage_row(uint8_t *smem, const LdsRow r, const c
 // Raw bytes of one unit as loaded from the planes (decoded later, so loads can run ahead).
 template <int DT> struct UnitRaw {
     uint4 q;       // main plane lane
-    uint4 h;       // Q4K: block header {d, dmin, scales[12]}
+    uint4 q2;      // Q4K: the second 16 bytes of the lane's 32
+    uint2 h;       // Q4K: {d | dmin << 16, record {sc[2g], sc[2g+1], mn[2g], mn[2g+1]}}
     uint2 hh;      // Q6K: high bits of the lane's 32 elements
     uint16_t sc2;  // Q6K: the lane's two group scales
     uint16_t d;    // Q4_0 / Q8_0 / Q6K: f16 scale
@@ -251,10 +251,17 @@ template <int DT> struct UnitRaw {
 template <int DT>
 __device__ __forceinline__ void load_unit(const cq_weight &w, int64_t row, int64_t units, int64_t u, UnitRaw<DT> &o) {
     const int64_t g = row * units + u;
+    if (DT == CQ_DTYPE_Q4K) {
+        o.q = *(const uint4 *)(w.p0 + g * 32);
+        o.q2 = *(const uint4 *)(w.p0 + g * 32 + 16);
+        const uint32_t *h = (const uint32_t *)(w.p1 + (g >> 2) * CQ_Q4K_HDR);
+        o.h.x = h[0];
+        o.h.y = h[1 + (g & 3)];   // units per row is a multiple of 4, so g & 3 == u & 3
+        return;
+    }
     o.q = *(const uint4 *)(w.p0 + g * 16);
     if (DT == CQ_DTYPE_Q4_0) o.d = ((const uint16_t *)w.p1)[g];
     if (DT == CQ_DTYPE_Q8_0) o.d = ((const uint16_t *)w.p1)[g >> 1];
-    if (DT == CQ_DTYPE_Q4K) o.h = *(const uint4 *)(w.p1 + (g >> 3) * 16);
     if (DT == CQ_DTYPE_Q6K) {
         o.hh = *(const uint2 *)(w.p1 + g * 8);
         o.sc2 = ((const uint16_t *)w.p2)[g];
@@ -272,7 +279,7 @@ __device__ __forceinline__ int dot16(const uint32_t w[4], const int4 &a) {
 
 // Decoded weight side of a unit, reused for every activation row.
 template <int DT> struct UnitW {
-    uint32_t lo[4], hi[4];
+    uint32_t lo[8], hi[8];   // Q4K uses all eight words (32 bytes of nibbles), the others four
     float dw, dmin;
     int sc_lo, sc_hi, mn_lo, mn_hi;
 };
@@ -288,13 +295,17 @@ template <int DT> __device__ __forceinline__ void decode_unit(const UnitRaw<DT> 
 #pragma unroll
         for (int i = 0; i < 4; i++) { o.lo[i] = qw[i] & 0x0F0F0F0Fu; o.hi[i] = (qw[i] >> 4) & 0x0F0F0F0Fu; }
     } else if (DT == CQ_DTYPE_Q4K) {
-        const int g = p >> 1;
+        (void)p;
         o.dw = cq_h2f((uint16_t)(r.h.x & 0xffff));
         o.dmin = cq_h2f((uint16_t)(r.h.x >> 16));
-        cq_scale_min_k4(2 * g, r.h.y, r.h.z, r.h.w, o.sc_lo, o.mn_lo);
-        cq_scale_min_k4(2 * g + 1, r.h.y, r.h.z, r.h.w, o.sc_hi, o.mn_hi);
+        o.sc_lo = (int)(r.h.y & 0xff); o.sc_hi = (int)((r.h.y >> 8) & 0xff);
+        o.mn_lo = (int)((r.h.y >> 16) & 0xff); o.mn_hi = (int)(r.h.y >> 24);
+        const uint32_t q2[4] = {r.q2.x, r.q2.y, r.q2.z, r.q2.w};
 #pragma unroll
-        for (int i = 0; i < 4; i++) { o.lo[i] = qw[i] & 0x0F0F0F0Fu; o.hi[i] = (qw[i] >> 4) & 0x0F0F0F0Fu; }
+        for (int i = 0; i < 4; i++) {
+            o.lo[i] = qw[i] & 0x0F0F0F0Fu; o.hi[i] = (qw[i] >> 4) & 0x0F0F0F0Fu;
+            o.lo[4 + i] = q2[i] & 0x0F0F0F0Fu; o.hi[4 + i] = (q2[i] >> 4) & 0x0F0F0F0Fu;
+        }
     } else {
         o.sc_lo = (int)(int8_t)(r.sc2 & 0xff);
         o.sc_hi = (int)(int8_t)(r.sc2 >> 8);
@@ -312,13 +323,26 @@ template <int DT> __device__ __forceinline__ void decode_unit(const UnitRaw<DT> 
 
 // Integer parts of unit u (p = u mod 8) against one activation row.
 //   Q4_0: I = sum (q-8)*a over the block.            Q8_0: I = sum q*a over half a block.
-//   Q4K : I = sc_lo*dot_lo + sc_hi*dot_hi over the lane's halves of sub-blocks 2g and 2g+1;
-//         Mn = min_2g * S_lo + min_2g+1 * S_hi with S = sum of the same activation quants
-//         (over the eight lanes of a block: sum_j bsums_j * min_{j/2}).
+//   Q4K : I = sc_2g*dot_lo + sc_2g+1*dot_hi over sub-blocks 2g and 2g+1;
+//         Mn = min_2g * S_lo + min_2g+1 * S_hi with S = sum of the sub-block's activation quants
+//         (over the four lanes of a block: sum_j bsums_j * min_{j/2}).
 //   Q6K : I = sc_lo*(dot_lo - 32*bsums_lo) + sc_hi*(dot_hi - 32*bsums_hi).
 template <int DT>
-__device__ __forceinline__ void unit_ints(const uint8_t *smem, const UnitW<DT> &w, const LdsRow r, uint32_t u, int &I,
-                                          int &Mn) {
+__device__ __forceinline__ void unit_ints(const uint8_t *smem, const UnitW<DT> &w, const LdsRow r, uint32_t u,
+                                          uint32_t units, int &I, int &Mn) {
+    if (DT == CQ_DTYPE_Q4K) {
+        // unit u = 32 qs bytes: low nibbles are elements 64u + [0,32) (sub-block 2g, planes 0 and 1),
+        // high nibbles elements 64u + 32 + [0,32) (sub-block 2g+1, planes 2 and 3)
+        const uint32_t plane = units * 16, at = r.lo + u * 16;
+        const int4 a0 = lds_get<int4>(smem, at), a1 = lds_get<int4>(smem, at + plane);
+        const int4 a2 = lds_get<int4>(smem, at + 2 * plane), a3 = lds_get<int4>(smem, at + 3 * plane);
+        const int dlo = dot16(w.lo, a0) + dot16(w.lo + 4, a1);
+        const int dhi = dot16(w.hi, a2) + dot16(w.hi + 4, a3);
+        I = __mul24(w.sc_lo, dlo) + __mul24(w.sc_hi, dhi);
+        const uint32_t ss = lds_get<uint32_t>(smem, r.bs + 4 * u);   // {sum of sub-block 2g, sum of 2g+1} as i16
+        Mn = __mul24(w.mn_lo, (int)(int16_t)(ss & 0xffff)) + __mul24(w.mn_hi, (int)ss >> 16);
+        return;
+    }
     const int4 alo = lds_get<int4>(smem, r.lo + u * 16);
     Mn = 0;
     if (DT == CQ_DTYPE_Q8_0) {
@@ -329,14 +353,6 @@ __device__ __forceinline__ void unit_ints(const uint8_t *smem, const UnitW<DT> &
     const int dlo = dot16(w.lo, alo), dhi = dot16(w.hi, ahi);
     if (DT == CQ_DTYPE_Q4_0) {
         I = dlo + dhi - 8 * lds_get<int32_t>(smem, r.bs + 4 * u);
-    } else if (DT == CQ_DTYPE_Q4K) {
-        I = __mul24(w.sc_lo, dlo) + __mul24(w.sc_hi, dhi);
-        // unit p = 2g + i holds elements 64g + 16i + [0,16) and 64g + 32 + 16i + [0,16):
-        // 16-element groups 4g + i (sub-block 2g) and 4g + 2 + i (sub-block 2g + 1)
-        const uint32_t p = u & 7, g = p >> 1, i = p & 1;
-        const uint32_t bs = r.bs + 32 * (u >> 3);
-        Mn = __mul24(w.mn_lo, (int)lds_get<int16_t>(smem, bs + 2 * (4 * g + i))) +
-             __mul24(w.mn_hi, (int)lds_get<int16_t>(smem, bs + 2 * (4 * g + 2 + i)));
     } else {
         // unit p = 4h + 2t + i: low nibbles are group 8h + 2t + i, high nibbles that + 4
         const uint32_t p = u & 7;
@@ -348,10 +364,11 @@ __device__ __forceinline__ void unit_ints(const uint8_t *smem, const UnitW<DT> &
 }
 
 template <int DT>
-__device__ __forceinline__ float unit_value(const uint8_t *smem, const UnitW<DT> &w, const LdsRow r, uint32_t u) {
+__device__ __forceinline__ float unit_value(const uint8_t *smem, const UnitW<DT> &w, const LdsRow r, uint32_t u,
+                                            uint32_t units) {
     int I, Mn;
-    unit_ints<DT>(smem, w, r, u, I, Mn);
-    const float ad = lds_get<float>(smem, r.d + 4 * (DT == CQ_DTYPE_Q8_0 ? (u >> 1) : (DT == CQ_DTYPE_Q4_0 ? u : (u >> 3))));
+    unit_ints<DT>(smem, w, r, u, units, I, Mn);
+    const float ad = lds_get<float>(smem, r.d + 4 * (u / Geo<DT>::kUnitsPerBlock));
     if (DT == CQ_DTYPE_Q4K) return ad * (w.dw * (float)I - w.dmin * (float)Mn);
     return ((float)I * w.dw) * ad;
 }
@@ -363,11 +380,12 @@ __device__ __forceinline__ float unit_value(const uint8_t *smem, const UnitW<DT>
 template <int DT, int UPL>
 __device__ __forceinline__ void load_row(const cq_weight &w, int64_t row, uint32_t units, UnitRaw<DT> (&buf)[UPL]) {
     const uint32_t lane = threadIdx.x & 63;
+    constexpr uint32_t kB = Geo<DT>::kUnitsPerBlock;
 #pragma unroll
     for (int c = 0; c < UPL; c++) {
         const uint32_t u = c * 64 + lane;
-        // keep u & 7 (the lane's position in its block) when clamping
-        const uint32_t uc = u < units ? u : (units - 8 + (lane & 7));
+        // keep the lane's position in its block when clamping (rows hold whole blocks)
+        const uint32_t uc = u < units ? u : (units - kB + (lane & (kB - 1)));
         load_unit<DT>(w, row, units, uc, buf[c]);
     }
 }
@@ -376,14 +394,15 @@ template <int DT, int UPL>
 __device__ __forceinline__ float row_dot(const uint8_t *smem, const LdsRow r, uint32_t units,
                                          const UnitRaw<DT> (&buf)[UPL]) {
     const uint32_t lane = threadIdx.x & 63;
+    constexpr uint32_t kB = Geo<DT>::kUnitsPerBlock;
     float acc = 0.0f;
 #pragma unroll
     for (int c = 0; c < UPL; c++) {
         const uint32_t u = c * 64 + lane;
-        const uint32_t uc = u < units ? u : (units - 8 + (lane & 7));
+        const uint32_t uc = u < units ? u : (units - kB + (lane & (kB - 1)));
         UnitW<DT> uw;
         decode_unit<DT>(buf[c], lane & 7, uw);
-        const float v = unit_value<DT>(smem, uw, r, uc);
+        const float v = unit_value<DT>(smem, uw, r, uc, units);
         acc += u < units ? v : 0.0f;
     }
     return wave_sum(acc);
@@ -409,7 +428,7 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
     const int64_t cnt = rows_per_wave + (row0 < rows_extra ? 1 : 0);
 
     // chunks of 256 activations per wave: k/256 <= 8*UPL/NW for the 32-element unit types
-    constexpr int XCH = (((Geo<DT>::kElems == 16 ? (UPL + 1) / 2 : UPL) * 8) + NW - 1) / NW;
+    constexpr int XCH = (UPL * Geo<DT>::kElems / 4 + NW - 1) / NW;   // 64 * UPL units * kElems / 256 chunks
     float4 fx[XCH];
     load_x_chunks<XCH, NW>(x, w.k, wave, fx);
     // Pin the issue order: activation loads, then weight loads, then the quantizer arithmetic.
@@ -486,7 +505,7 @@ __global__ void __launch_bounds__(kStagedThreads) staged_kernel(cq_weight w, cq_
             UnitW<DT> uw;
             decode_unit<DT>(raw, lane & 7, uw);
 #pragma unroll
-            for (int m = 0; m < MB; m++) acc[m] += unit_value<DT>(smem, uw, rows[m], (uint32_t)u);
+            for (int m = 0; m < MB; m++) acc[m] += unit_value<DT>(smem, uw, rows[m], (uint32_t)u, (uint32_t)units);
         }
 #pragma unroll
         for (int m = 0; m < MB; m++) {
@@ -520,7 +539,7 @@ __global__ void __launch_bounds__(kStagedThreads) int_dots_kernel(cq_weight w, c
                 load_unit<DT>(w, row, units, u, raw);
                 UnitW<DT> uw;
                 decode_unit<DT>(raw, lane & 7, uw);
-                unit_ints<DT>(smem, uw, r, (uint32_t)u, I, Mn);
+                unit_ints<DT>(smem, uw, r, (uint32_t)u, (uint32_t)units, I, Mn);
             }
 #pragma unroll
             for (int off = 1; off < kUPB; off <<= 1) {

@@ -19,7 +19,9 @@
 //   Q8_0 : qs [n][k/32][32]  i8
 //          d  [n][k/32]      f16
 //   Q4K  : qs [n][k/256][128] u8  (GGML order: byte 32g+l = elem 64g+l | elem 64g+32+l << 4)
-//          hd [n][k/256][16]      (d f16, dmin f16, scales[12]: the first 16 bytes of the GGML block)
+//          hd [n][k/256][20]      (d f16, dmin f16, then four records {sc[2g], sc[2g+1], mn[2g], mn[2g+1]}:
+//                                  the 6-bit scales and mins of the GGML scales[12] unpacked to bytes,
+//                                  grouped by the 32 qs bytes g they belong to)
 //   Q6K  : ql [n][k/256][128] u8  (GGML order)
 //          qh [n][k/256][64]  u8  (re-ordered, see repack.hip: 8 bytes per 16-byte ql lane)
 //          sc [n][k/256][16]  i8  (re-ordered: two scales per 16-byte ql lane, see repack.hip)
@@ -29,6 +31,7 @@
 // read with full-width loads.
 // ---------------------------------------------------------------------------
 #define CQ_TAIL_PAD 4096
+#define CQ_Q4K_HDR 20   // bytes per block in the Q4K header plane
 
 struct cq_weight {
     int dev;

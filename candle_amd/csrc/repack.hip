@@ -41,7 +41,10 @@ __global__ void repack_q8_0(const uint8_t *__restrict__ aos, uint8_t *__restrict
 }
 
 // ---- Q4K: 144-byte blocks {f16 d; f16 dmin; u8 scales[12]; u8 qs[128]} ------
-// One thread per 16-byte unit: unit 0 is the header, units 1..8 the nibbles.
+// One thread per 16-byte unit: unit 0 is the header, units 1..8 the nibbles.  The header's twelve
+// bytes of 6-bit fields (utils.rs:49-59 get_scale_min_k4) are unpacked to one byte per field and
+// grouped per 32 qs bytes: record g = {sc[2g], sc[2g+1], mn[2g], mn[2g+1]}; the inverse packs them
+// back (every one of the 96 bits is a field bit, so the round trip is exact).
 __global__ void repack_q4k(const uint8_t *__restrict__ aos, uint8_t *__restrict__ qs, uint8_t *__restrict__ hd,
                            int64_t nblocks, bool inverse) {
     int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -49,8 +52,39 @@ __global__ void repack_q4k(const uint8_t *__restrict__ aos, uint8_t *__restrict_
     int u = (int)(t - b * 9);
     if (b >= nblocks) return;
     uint4 *a = (uint4 *)(aos + b * 144) + u;      // 144 = 9 * 16, base is 256-byte aligned
-    uint4 *p = (u == 0) ? (uint4 *)(hd + b * 16) : (uint4 *)(qs + b * 128) + (u - 1);
-    if (!inverse) *p = *a; else *a = *p;
+    if (u != 0) {
+        uint4 *p = (uint4 *)(qs + b * 128) + (u - 1);
+        if (!inverse) *p = *a; else *a = *p;
+        return;
+    }
+    uint32_t *h = (uint32_t *)(hd + b * CQ_Q4K_HDR);
+    if (!inverse) {
+        const uint4 v = *a;
+        h[0] = v.x;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            int s0, m0, s1, m1;
+            cq_scale_min_k4(2 * g, v.y, v.z, v.w, s0, m0);
+            cq_scale_min_k4(2 * g + 1, v.y, v.z, v.w, s1, m1);
+            h[1 + g] = (uint32_t)s0 | ((uint32_t)s1 << 8) | ((uint32_t)m0 << 16) | ((uint32_t)m1 << 24);
+        }
+    } else {
+        uint32_t sc[8], mn[8];
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const uint32_t r = h[1 + g];
+            sc[2 * g] = r & 0xff; sc[2 * g + 1] = (r >> 8) & 0xff;
+            mn[2 * g] = (r >> 16) & 0xff; mn[2 * g + 1] = r >> 24;
+        }
+        uint32_t w[3] = {0, 0, 0};   // scales[0..3], scales[4..7], scales[8..11]
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            w[0] |= ((sc[j] & 63) | ((sc[j + 4] >> 4) << 6)) << (8 * j);
+            w[1] |= ((mn[j] & 63) | ((mn[j + 4] >> 4) << 6)) << (8 * j);
+            w[2] |= ((sc[j + 4] & 15) | ((mn[j + 4] & 15) << 4)) << (8 * j);
+        }
+        *a = make_uint4(h[0], w[0], w[1], w[2]);
+    }
 }
 
 // ---- Q6K: 210-byte blocks {u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d} -----
