@@ -215,6 +215,111 @@ __device__ __forceinline__ void quantize_row_to_lds(uint8_t *smem, int64_t k, in
     }
 }
 
+// ---- Q8K activations, two chunks per wave ------------------------------------------------------
+// Lane l takes the eight consecutive elements 8*(l%32) + [0,8) of chunk 2*pair + l/32, so a wave
+// covers two 256-element chunks and the per-chunk work (maximum search, the two divisions) is
+// paid once per eight elements instead of once per four.  Same arithmetic as above.
+struct X8 {
+    float4 a, b;
+};
+
+template <int XP, int NW>
+__device__ __forceinline__ void load_x_pairs(const float *x, int64_t k, int wave, X8 (&fx)[XP]) {
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int i = 0; i < XP; i++) {
+        const int e0 = (2 * (wave + i * NW) + (lane >> 5)) * 256 + 8 * (lane & 31);
+        const float *p = x + (e0 < k ? e0 : 0);   // k is a multiple of 256: a chunk is inside or outside as a whole
+        fx[i].a = *(const float4 *)p;
+        fx[i].b = *(const float4 *)(p + 4);
+    }
+}
+
+// Maximum / minimum over each half of the wave (lanes 0..31 and 32..63), valid in every lane.
+__device__ __forceinline__ float half_max(float v) {
+    v = fmaxf(v, dpp_f<kQuadSwap1>(v));
+    v = fmaxf(v, dpp_f<kQuadSwap2>(v));
+    v = fmaxf(v, dpp_f<kHalfMirror>(v));
+    v = fmaxf(v, dpp_f<kRowMirror>(v));
+    const float lo = fmaxf(readlane_f(v, 0), readlane_f(v, 16)), hi = fmaxf(readlane_f(v, 32), readlane_f(v, 48));
+    return (threadIdx.x & 32) ? hi : lo;
+}
+__device__ __forceinline__ int half_min_i(int v) {
+    v = min(v, dpp_i<kQuadSwap1>(v));
+    v = min(v, dpp_i<kQuadSwap2>(v));
+    v = min(v, dpp_i<kHalfMirror>(v));
+    v = min(v, dpp_i<kRowMirror>(v));
+    const int lo = min(__builtin_amdgcn_readlane(v, 0), __builtin_amdgcn_readlane(v, 16));
+    const int hi = min(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48));
+    return (threadIdx.x & 32) ? hi : lo;
+}
+
+template <int DT>
+__device__ __forceinline__ void quantize_pair_to_lds(uint8_t *smem, const X8 &fin, int c, bool chunk_ok,
+                                                     const LdsRow r, uint32_t units) {
+    const int lane = threadIdx.x & 63, hl = lane & 31;
+    float v[8] = {fin.a.x, fin.a.y, fin.a.z, fin.a.w, fin.b.x, fin.b.y, fin.b.z, fin.b.w};
+    float av[8];
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        if (!chunk_ok) v[i] = 0.0f;
+        av[i] = fabsf(v[i]);
+        amax = fmaxf(amax, av[i]);
+    }
+    amax = half_max(amax);
+    // the first element of the chunk whose |x| equals the maximum decides the sign of the scale
+    int idx = 0x7fffffff;
+    float cand = 0.0f;
+#pragma unroll
+    for (int i = 7; i >= 0; i--) {
+        if (av[i] == amax) { idx = 8 * hl + i; cand = v[i]; }
+    }
+    idx = half_min_i(idx);
+    const int src_lo = (__builtin_amdgcn_readlane(idx, 0) >> 3) & 31;
+    const int src_hi = 32 + ((__builtin_amdgcn_readlane(idx, 32) >> 3) & 31);
+    const float max_lo = readlane_f(cand, src_lo), max_hi = readlane_f(cand, src_hi);
+    const float max = (lane & 32) ? max_hi : max_lo;
+    uint32_t w0 = 0, w1 = 0;
+    int sum = 0;
+    float d = 0.0f;
+    if (amax != 0.0f) {
+        const float iscale = -128.0f / max;
+        int8_t q[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            q[i] = cq_as_i8(fminf(roundf(iscale * v[i]), 127.0f));
+            sum += (int)q[i];
+        }
+        w0 = pack4(q[0], q[1], q[2], q[3]);
+        w1 = pack4(q[4], q[5], q[6], q[7]);
+        d = 1.0f / iscale;
+    }
+    sum += dpp_i<kQuadSwap1>(sum);   // two lanes = one 16-element group
+    if (DT == CQ_DTYPE_Q4K) {
+        sum += dpp_i<kQuadSwap2>(sum);   // four lanes = one 32-element sub-block
+        if (chunk_ok && (hl & 3) == 0) lds_put<int16_t>(smem, r.bs + 2 * (c * 8 + (hl >> 2)), (int16_t)sum);
+    } else if (chunk_ok && (hl & 1) == 0) {
+        lds_put<int16_t>(smem, r.bs + 2 * (c * 16 + (hl >> 1)), (int16_t)sum);
+    }
+    if (chunk_ok) {
+        if (hl == 0) lds_put<float>(smem, r.d + 4 * c, d);
+        lds_put<uint2>(smem, piece_off<DT>(r, c * 16 + (hl >> 1), units) + 8 * (hl & 1), make_uint2(w0, w1));
+    }
+}
+
+template <int DT, int XP, int NW>
+__device__ __forceinline__ void quantize_pairs_to_lds(uint8_t *smem, int64_t k, int wave, const LdsRow r,
+                                                      const X8 (&fx)[XP]) {
+    const int lane = threadIdx.x & 63;
+    const int chunks = (int)(k / 256);
+#pragma unroll
+    for (int i = 0; i < XP; i++) {
+        const int c = 2 * (wave + i * NW) + (lane >> 5);
+        quantize_pair_to_lds<DT>(smem, fx[i], c, c < chunks, r, (uint32_t)(k / Geo<DT>::kElems));
+    }
+}
+
 // Copy an already-quantized activation row from the workspace into its LDS image.
 template <int DT, int NT>
 __device__ __forceinline__ void stage_row(uint8_t *smem, const LdsRow r, const cq_act_view &a, int64_t row, int64_t k) {
@@ -427,10 +532,14 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
     // rows of this wave (>= DEPTH): n / T, plus one for the first n % T waves (both from the host)
     const int64_t cnt = rows_per_wave + (row0 < rows_extra ? 1 : 0);
 
-    // chunks of 256 activations per wave: k/256 <= 8*UPL/NW for the 32-element unit types
-    constexpr int XCH = (UPL * Geo<DT>::kElems / 4 + NW - 1) / NW;   // 64 * UPL units * kElems / 256 chunks
-    float4 fx[XCH];
-    load_x_chunks<XCH, NW>(x, w.k, wave, fx);
+    // chunks of 256 activations: at most 64 * UPL units * kElems / 256; a wave quantizes one chunk
+    // per step for Q8_0 activations, two for Q8K
+    constexpr bool kPairs = Geo<DT>::kActK;
+    constexpr int XCH = (UPL * Geo<DT>::kElems / (kPairs ? 8 : 4) + NW - 1) / NW;
+    float4 fx[kPairs ? 1 : XCH];
+    X8 fx8[kPairs ? XCH : 1];
+    if constexpr (kPairs) load_x_pairs<XCH, NW>(x, w.k, wave, fx8);
+    else load_x_chunks<XCH, NW>(x, w.k, wave, fx);
     // Pin the issue order: activation loads, then weight loads, then the quantizer arithmetic.
     // (The empty asm stops the optimizer from sinking loads past it, the scheduling barrier stops
     // the instruction scheduler.)
@@ -442,9 +551,8 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     const LdsRow r = lds_row<DT>(w.k, 0);
-#ifndef CQ_EXP_SKIP_QUANT
-    quantize_row_to_lds<DT, XCH, NW>(smem, w.k, wave, r, fx);
-#endif
+    if constexpr (kPairs) quantize_pairs_to_lds<DT, XCH, NW>(smem, w.k, wave, r, fx8);
+    else quantize_row_to_lds<DT, XCH, NW>(smem, w.k, wave, r, fx);
     __syncthreads();
 
     if constexpr (DEPTH == 1) {
@@ -577,7 +685,8 @@ template <int DT, int UPL>
 hipError_t launch_fused_upl(const cq_weight *w, const float *x, float *y, hipStream_t s) {
     constexpr int NW = 8;
     const size_t lds = lds_row_bytes<DT>(w->k);
-    const int per_cu = g_fused_wgs_per_cu > 0 ? g_fused_wgs_per_cu : 2;
+    // every workgroup quantizes the whole activation row: one workgroup per CU for long rows
+    const int per_cu = g_fused_wgs_per_cu > 0 ? g_fused_wgs_per_cu : (w->k > 8192 ? 1 : 2);
     const int64_t max_wgs = (int64_t)num_cus() * per_cu;
     int depth = UPL <= 2 ? 2 : 1;
     if (w->n < NW * 2) depth = 1;
@@ -594,10 +703,10 @@ hipError_t launch_fused_upl(const cq_weight *w, const float *x, float *y, hipStr
 
 template <int DT>
 bool fused_ok(const cq_weight *w) {
-    // Every workgroup re-quantizes the whole activation row in its prologue; beyond 8192 elements
-    // (more than four 256-element chunks per wave) that costs more than the separate quantizer
-    // launch it saves (measured on K = 11008), so longer rows take the two-launch path.
-    return w->k <= 8192 && w->n >= 8 && lds_row_bytes<DT>(w->k) <= 64 * 1024;
+    // Every workgroup re-quantizes the whole activation row in its prologue, which pays off against a
+    // separate quantizer launch up to the row lengths measured (K = 11008: 12.0 us against 11.6 + 3.1 us).
+    // The launcher instantiates up to eight units per lane (512 units per row).
+    return w->k <= 16384 && w->k / Geo<DT>::kElems <= 512 && w->n >= 8 && lds_row_bytes<DT>(w->k) <= 64 * 1024;
 }
 
 template <int DT>
