@@ -143,24 +143,22 @@ __device__ __forceinline__ uint16_t cq_f2h(float f) {  // round-to-nearest-even
     __builtin_memcpy(&h, &v, 2);
     return h;
 }
-// Rust `as i8` / `as u8` / `as i32` on f32: truncate toward zero, saturate, NaN -> 0.
+// Rust `as i8` / `as u8` / `as i32` on f32: truncate toward zero, saturate, NaN -> 0.  That is
+// what the hardware conversions do for the 32-bit range (v_cvt_i32_f32 / v_cvt_u32_f32 round toward
+// zero, clamp, and turn NaN into 0), so the narrow types only add an integer clamp; no branches.
+__device__ __forceinline__ int32_t cq_as_i32(float v) {
+    int32_t r;
+    asm("v_cvt_i32_f32_e32 %0, %1" : "=v"(r) : "v"(v));
+    return r;
+}
 __device__ __forceinline__ int8_t cq_as_i8(float v) {
-    if (!(v == v)) return 0;
-    if (v <= -128.0f) return -128;
-    if (v >= 127.0f) return 127;
-    return (int8_t)(int)v;
+    const int32_t r = cq_as_i32(v);
+    return (int8_t)(r < -128 ? -128 : (r > 127 ? 127 : r));
 }
 __device__ __forceinline__ uint8_t cq_as_u8(float v) {
-    if (!(v == v)) return 0;
-    if (v <= 0.0f) return 0;
-    if (v >= 255.0f) return 255;
-    return (uint8_t)(int)v;
-}
-__device__ __forceinline__ int32_t cq_as_i32(float v) {
-    if (!(v == v)) return 0;
-    if (v >= 2147483648.0f) return 2147483647;
-    if (v <= -2147483648.0f) return (-2147483647 - 1);
-    return (int32_t)v;
+    uint32_t r;
+    asm("v_cvt_u32_f32_e32 %0, %1" : "=v"(r) : "v"(v));
+    return (uint8_t)(r > 255u ? 255u : r);
 }
 // utils.rs:3-5 nearest_int = v.round() as i32 (round half away from zero)
 __device__ __forceinline__ int32_t cq_nearest_int(float v) { return cq_as_i32(roundf(v)); }
