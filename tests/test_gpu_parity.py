@@ -213,8 +213,8 @@ def test_gemm_matches_oracle_small(qh, dt, m, k, n):
 
 
 @pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K])
-def test_gemm_needs_16_row_multiple(qh, dt):
-    """Weight row counts that are not a multiple of 16 take the dot-product kernels: forcing the
+def test_gemm_needs_32_row_multiple(qh, dt):
+    """Weight row counts that are not a multiple of 32 take the dot-product kernels: forcing the
     tile kernel is an error, the automatic choice still matches the oracle."""
     m, k, n = 33, 512, 70
     w, x = make_inputs(5 * dt + 1, m, k, n)
