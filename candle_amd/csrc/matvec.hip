@@ -584,6 +584,74 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
     }
 }
 
+// ------------------------------------------------------ batched kernel (2 <= m <= 8 rows) ----
+// The same persistent structure as fused_kernel for a few activation rows: one workgroup per CU
+// copies the MB quantized rows from the workspace into LDS once, then every wave streams its weight
+// rows (next row's loads in flight) and contracts each decoded unit against all MB rows, so the
+// weights are read and unpacked once.  Rows m0 + MB and beyond of the call are masked (their LDS
+// image is a copy of the last valid row).
+template <int DT, int UPL, int MB>
+__device__ __forceinline__ void row_dot_mb(const uint8_t *smem, const LdsRow (&rows)[MB], uint32_t units,
+                                           const UnitRaw<DT> (&buf)[UPL], float (&out)[MB]) {
+    const uint32_t lane = threadIdx.x & 63;
+    constexpr uint32_t kB = Geo<DT>::kUnitsPerBlock;
+    float acc[MB];
+#pragma unroll
+    for (int m = 0; m < MB; m++) acc[m] = 0.0f;
+#pragma unroll
+    for (int c = 0; c < UPL; c++) {
+        const uint32_t u = c * 64 + lane;
+        const uint32_t uc = u < units ? u : (units - kB + (lane & (kB - 1)));
+        UnitW<DT> uw;
+        decode_unit<DT>(buf[c], lane & 7, uw);
+#pragma unroll
+        for (int m = 0; m < MB; m++) {
+            const float v = unit_value<DT>(smem, uw, rows[m], uc, units);
+            acc[m] += u < units ? v : 0.0f;
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MB; m++) out[m] = wave_sum(acc[m]);
+}
+
+template <int DT, int UPL, int NW, int MB>
+__global__ void __launch_bounds__(NW * 64) batched_kernel(cq_weight w, cq_act_view a, int64_t m0, int64_t m,
+                                                          float *__restrict__ y, int64_t total_waves,
+                                                          int64_t rows_per_wave, int64_t rows_extra) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t units = (uint32_t)(w.k / Geo<DT>::kElems);
+    const int64_t row0 = (int64_t)blockIdx.x * NW + wave;
+    const int64_t T = total_waves;
+    const int64_t cnt = rows_per_wave + (row0 < rows_extra ? 1 : 0);   // >= 1
+
+    UnitRaw<DT> cur[UPL], nxt[UPL];
+    load_row<DT, UPL>(w, row0, units, cur);
+    LdsRow rows[MB];
+#pragma unroll
+    for (int i = 0; i < MB; i++) {
+        rows[i] = lds_row<DT>(w.k, i);
+        const int64_t src = m0 + i < m ? m0 + i : m - 1;
+        stage_row<DT, NW * 64>(smem, rows[i], a, src, w.k);
+    }
+    __syncthreads();
+    for (int64_t i = 0; i < cnt; i++) {
+        const int64_t row = row0 + i * T;
+        const bool more = i + 1 < cnt;
+        load_row<DT, UPL>(w, more ? row + T : row, units, nxt);   // unconditional: the last one re-reads its own row
+        float out[MB];
+        row_dot_mb<DT, UPL, MB>(smem, rows, units, cur, out);
+        if (lane == 0) {
+#pragma unroll
+            for (int j = 0; j < MB; j++)
+                if (m0 + j < m) y[(m0 + j) * w.n + row] = out[j];
+        }
+#pragma unroll
+        for (int c = 0; c < UPL; c++) cur[c] = nxt[c];
+    }
+}
+
 // ------------------------------------------------------------ staged kernel (m <= 4 rows) ----
 constexpr int kStagedThreads = 256;
 
@@ -677,6 +745,7 @@ int num_cus() {
     return g_num_cus;
 }
 
+bool g_no_batched = false;   // A/B switch: rows of up to four on the simple kernel only
 int g_fused_wgs_per_cu = 0;  // 0 = automatic; A/B switch (CQ_MATVEC_WAVES = workgroups per CU)
 
 // Eight waves per workgroup, one workgroup per CU.  Whole workgroups only, and every wave
@@ -728,8 +797,59 @@ int pick_rows_per_wg(int64_t n) {
     return r;
 }
 
+template <int DT, int UPL, int MB>
+hipError_t launch_batched_upl(const cq_weight *w, cq_act_view a, int64_t m0, int64_t m, float *y, hipStream_t s) {
+    constexpr int NW = 8;
+    const size_t lds = lds_row_bytes<DT>(w->k) * MB;
+    static bool attr_set = false;
+    if (!attr_set && lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void *)batched_kernel<DT, UPL, NW, MB>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    int64_t wgs = w->n / NW;
+    if (wgs > num_cus()) wgs = num_cus();
+    const int64_t tw = wgs * NW, rpw = w->n / tw, extra = w->n % tw;
+    CQ_LAUNCH((batched_kernel<DT, UPL, NW, MB>), (unsigned)wgs, NW * 64, lds, s, *w, a, m0, m, y, tw, rpw, extra);
+    return hipGetLastError();
+}
+
+template <int DT, int MB>
+hipError_t launch_batched(const cq_weight *w, cq_act_view a, int64_t m0, int64_t m, float *y, hipStream_t s) {
+    const int64_t units = w->k / Geo<DT>::kElems;
+    const int upl = (int)((units + 63) / 64);
+    if (upl <= 1) return launch_batched_upl<DT, 1, MB>(w, a, m0, m, y, s);
+    if (upl <= 2) return launch_batched_upl<DT, 2, MB>(w, a, m0, m, y, s);
+    if (upl <= 3) return launch_batched_upl<DT, 3, MB>(w, a, m0, m, y, s);
+    if (upl <= 4) return launch_batched_upl<DT, 4, MB>(w, a, m0, m, y, s);
+    if (upl <= 6) return launch_batched_upl<DT, 6, MB>(w, a, m0, m, y, s);
+    return launch_batched_upl<DT, 8, MB>(w, a, m0, m, y, s);
+}
+
+// Rows of eight (or four) per launch on the persistent kernel when the row fits its unit and LDS
+// budget, else the simple kernel below.
+template <int DT>
+bool batched_ok(const cq_weight *w, int mb) {
+    return w->k / Geo<DT>::kElems <= 512 && w->n >= 8 && lds_row_bytes<DT>(w->k) * mb <= 128 * 1024;
+}
+
 template <int DT>
 hipError_t launch_staged(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
+    if (m >= 2 && !g_no_batched) {
+        int64_t m0 = 0;
+        bool done = true;
+        while (m0 < m) {
+            const int64_t left = m - m0;
+            hipError_t e;
+            if (left > 4 && batched_ok<DT>(w, 8)) e = launch_batched<DT, 8>(w, a, m0, m, y, s), m0 += 8;
+            else if (batched_ok<DT>(w, 4)) e = launch_batched<DT, 4>(w, a, m0, m, y, s), m0 += 4;
+            else { done = false; break; }
+            if (e != hipSuccess) return e;
+        }
+        if (done) return hipSuccess;
+        if (m0 != 0) return hipErrorInvalidValue;   // unreachable: the checks above do not depend on m0
+    }
     const int rpw = pick_rows_per_wg(w->n);
     const unsigned grid = (unsigned)((w->n + rpw - 1) / rpw);
     int64_t m0 = 0;
@@ -765,7 +885,7 @@ hipError_t launch_ints(const cq_weight *w, cq_act_view a, int64_t m, int32_t *oi
 
 }  // namespace
 
-void cq_matvec_set_waves(int nw) { g_fused_wgs_per_cu = nw; }
+void cq_matvec_set_waves(int nw) { g_no_batched = nw >= 100; g_fused_wgs_per_cu = nw % 100; }
 
 bool cq_matvec_fused_supported(const cq_weight *w) {
     switch (w->dtype) {
