@@ -199,6 +199,39 @@ def test_small_batch_matches_oracle(qh, dt, m, k, n):
     check_f32(got, orc.matmul(dt, x, blocks, n))
 
 
+@pytest.mark.parametrize("dt", WEIGHT_DTYPES)
+@pytest.mark.parametrize("m,k,n", [(3, 512, 37), (5, 1024, 64), (7, 2048, 9), (9, 256, 130), (12, 11008, 24),
+                                   (2, 256, 8), (8, 14336, 16)])
+def test_ragged_batches_match_oracle(qh, dt, m, k, n):
+    """Row counts that do not fill the 4- and 8-row batches of the dot-product kernels, weight row
+    counts that are not a multiple of the waves per workgroup, the shortest rows (one K block) and
+    rows longer than the single-launch decode path takes."""
+    w, x = make_inputs(11 * dt + m + k + n, m, k, n, outliers=True)
+    blocks = orc.quantize(dt, w)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    got = qh.qmatmul(qw, dev(x), qh.FLAG_FORCE_MATVEC).cpu().numpy()
+    check_f32(got, orc.matmul(dt, x, blocks, n))
+    # the same rows one at a time (decode kernel) give the same values: batch invariance
+    one = np.concatenate([qh.qmatmul(qw, dev(x[r:r + 1])).cpu().numpy() for r in range(m)])
+    check_f32(got, one)
+
+
+@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K])
+def test_gemm_ragged_rows_large(qh, dt):
+    """M = 300 (not a multiple of the 128-row workgroup tile) on a K-split shape: every output row
+    of the tile kernel equals the dot-product kernels' result for that row within tolerance."""
+    m, k, n = 300, 4096, 512
+    w, x = make_inputs(13 * dt + 2, m, k, n, outliers=True)
+    blocks = orc.quantize(dt, w)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    got = qh.qmatmul(qw, dev(x)).cpu().numpy()
+    rows = [0, 1, 127, 128, 255, 256, 298, 299]
+    want = orc.matmul(dt, x[rows], blocks, n)
+    check_f32(got[rows], want)
+    ref = qh.qmatmul(qw, dev(x), qh.FLAG_FORCE_MATVEC).cpu().numpy()
+    check_f32(got, ref)
+
+
 @pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K])
 @pytest.mark.parametrize("m,k,n", [(9, 256, 32), (33, 512, 96), (64, 1024, 160), (130, 768, 288), (11, 512, 64),
                                    (1, 256, 32), (129, 2048, 416)])
@@ -310,14 +343,21 @@ def test_forward_shape_and_errors(qh):
 
 
 # ------------------------------------------------------------------------- MoE ----
-def test_moe_ffn_matches_oracle(qh):
+@pytest.mark.parametrize("tokens,starve", [(24, False), (64, True)])
+def test_moe_ffn_matches_oracle(qh, tokens, starve):
     """Mixtral-shaped expert FFN at reduced width: routed top-2, per-expert gathered QMatMul,
-    silu(w1 x) * w3 x, w2, scaled scatter-add (quantized_llama.rs:75-143)."""
-    rng = np.random.default_rng(23)
-    tokens, hidden, ffn, n_e, top_k = 24, 512, 1024, 8, 2
+    silu(w1 x) * w3 x, w2, scaled scatter-add (quantized_llama.rs:75-143).  24 tokens keep every
+    expert on the dot-product kernels (at most 8 rows each); 64 tokens (BASELINE config 4's count)
+    with one expert that no token picks give experts on the tile kernel and an empty slice."""
+    rng = np.random.default_rng(23 + tokens)
+    hidden, ffn, n_e, top_k = 512, 1024, 8, 2
     xs = rng.standard_normal((tokens, hidden)).astype(np.float32)
     logits = rng.standard_normal((tokens, n_e)).astype(np.float32)
+    if starve:
+        logits[:, 5] = -30.0
     offsets, row_ids, weights = orc.moe_route(orc.softmax_last_dim(logits), top_k)
+    if starve:
+        assert offsets[6] == offsets[5] and max(np.diff(offsets)) > 8
     w1 = [orc.quantize(orc.Q4K, (rng.standard_normal((ffn, hidden)) * 0.05).astype(np.float32)) for _ in range(n_e)]
     w3 = [orc.quantize(orc.Q4K, (rng.standard_normal((ffn, hidden)) * 0.05).astype(np.float32)) for _ in range(n_e)]
     w2 = [orc.quantize(orc.Q6K, (rng.standard_normal((hidden, ffn)) * 0.05).astype(np.float32)) for _ in range(n_e)]
