@@ -399,6 +399,14 @@ extern "C" int cq_qmatmul_grouped(const cq_weight *const *experts, int n_experts
     act_ws_layout(act, total, w0->k, (uint8_t *)ws, &v);
     // gather + quantize every routed row once, then one matmul per non-empty expert over its slice
     CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, row_ids_dev, total, w0->k, v, s));
+    // experts with more than eight rows among them: one tile-kernel launch for all experts
+    int64_t most = 0;
+    for (int e = 0; e < n_experts; e++) most = offsets[e + 1] - offsets[e] > most ? offsets[e + 1] - offsets[e] : most;
+    const bool want_gemm = (flags & CQ_FLAG_FORCE_GEMM) ? true : (flags & CQ_FLAG_FORCE_MATVEC) ? false : most > 8;
+    if (want_gemm && cq_gemm_grouped_supported(experts, n_experts, offsets, act)) {
+        CQ_HIP_CHECK(cq_launch_gemm_grouped(experts, n_experts, offsets, v, y_dev, s));
+        return CQ_OK;
+    }
     for (int e = 0; e < n_experts; e++) {
         const int64_t r0 = offsets[e], te = offsets[e + 1] - offsets[e];
         if (te == 0) continue;

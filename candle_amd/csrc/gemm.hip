@@ -331,16 +331,17 @@ __device__ __forceinline__ void block_step(const uint8_t *__restrict__ cur, uint
 
 // ------------------------------------------------------------------ kernel ----
 // Requires n % 32 == 0 and an activation workspace with padded rows (cq_act_view::m_stride).
+// One workgroup: activation rows [m0, m0 + 32*MT) (stored up to row m - 1) x the 256 weight rows of
+// blockIdx.x, K blocks of part blockIdx.z.
 template <int DT, int MT>
-__global__ void __launch_bounds__(kThreads) gemm_kernel(cq_weight w, cq_act_view a, int64_t m, float *__restrict__ y,
-                                                        int ksplit) {
+__device__ __forceinline__ void gemm_body(const cq_weight &w, const cq_act_view &a, int64_t m0, int64_t m,
+                                          float *__restrict__ y, int ksplit) {
     typedef Tile<DT, MT> T;
     extern __shared__ __align__(16) uint8_t smem[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int h = lane >> 5, col = lane & 31;
     const int64_t kb = w.k >> 8;
-    const int64_t m0 = (int64_t)blockIdx.y * (MT * 32);
     const int64_t n_tile = ((int64_t)blockIdx.x * kWaves + wave) * 32;
     const bool n_ok = n_tile < w.n;   // wave-uniform; a wave past the last row only helps with the copies
     const int64_t n = n_tile + col;
@@ -391,6 +392,30 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(cq_weight w, cq_act_view
     }
 }
 
+template <int DT, int MT>
+__global__ void __launch_bounds__(kThreads) gemm_kernel(cq_weight w, cq_act_view a, int64_t m, float *__restrict__ y,
+                                                        int ksplit) {
+    gemm_body<DT, MT>(w, a, (int64_t)blockIdx.y * (MT * 32), m, y, ksplit);
+}
+
+// Grouped (mixture-of-experts) variant: one launch for every expert.  blockIdx.y walks a table of
+// 32-row tiles of the expert-sorted activation rows; each tile names its expert's weights.
+constexpr int kMaxGroupExperts = 16, kMaxGroupTiles = 96;
+struct GroupArgs {
+    cq_weight w[kMaxGroupExperts];
+    int32_t row0[kMaxGroupTiles];      // first activation row of the tile
+    int32_t row_end[kMaxGroupTiles];   // end of its expert's rows
+    int8_t expert[kMaxGroupTiles];
+};
+
+template <int DT>
+__global__ void __launch_bounds__(kThreads) gemm_grouped_kernel(GroupArgs ga, cq_act_view a, float *__restrict__ y,
+                                                                int ksplit) {
+    const int tile = blockIdx.y;
+    const cq_weight w = ga.w[ga.expert[tile]];
+    gemm_body<DT, 1>(w, a, ga.row0[tile], ga.row_end[tile], y, ksplit);
+}
+
 int g_cus = 0;
 int num_cus() {
     if (g_cus == 0) {
@@ -435,7 +460,59 @@ hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hip
     return launch_mt<DT, 4>(w, a, m, y, s);
 }
 
+template <int DT>
+hipError_t launch_grouped(const cq_weight *const *experts, int n_experts, const int32_t *offsets, cq_act_view a,
+                          float *y, hipStream_t s) {
+    GroupArgs ga;
+    int ntiles = 0;
+    for (int e = 0; e < n_experts; e++) {
+        ga.w[e] = *experts[e];
+        for (int32_t r = offsets[e]; r < offsets[e + 1]; r += 32) {
+            if (ntiles == kMaxGroupTiles) return hipErrorInvalidConfiguration;
+            ga.row0[ntiles] = r;
+            ga.row_end[ntiles] = offsets[e + 1];
+            ga.expert[ntiles] = (int8_t)e;
+            ntiles++;
+        }
+    }
+    if (ntiles == 0) return hipSuccess;
+    const cq_weight *w = experts[0];
+    const size_t lds = Tile<DT, 1>::kTotal;
+    static bool attr_set = false;
+    if (!attr_set && lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void *)gemm_grouped_kernel<DT>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int64_t gx = (w->n + kWaves * 32 - 1) / (kWaves * 32);
+    int ksplit = 1;
+    const int64_t kb = w->k >> 8;
+    while (gx * ntiles * ksplit * 2 <= 2 * num_cus() && kb / (ksplit * 2) >= 4 && ksplit < 16) ksplit *= 2;
+    if (ksplit > 1) {
+        hipError_t e = cq_launch_fill_zero(y, (int64_t)offsets[n_experts] * w->n, s);
+        if (e != hipSuccess) return e;
+    }
+    dim3 grid((unsigned)gx, (unsigned)ntiles, (unsigned)ksplit);
+    CQ_LAUNCH((gemm_grouped_kernel<DT>), grid, kThreads, lds, s, ga, a, y, ksplit);
+    return hipGetLastError();
+}
+
 }  // namespace
+
+bool cq_gemm_grouped_supported(const cq_weight *const *experts, int n_experts, const int32_t *offsets, int act_dtype) {
+    if (n_experts > kMaxGroupExperts || !cq_gemm_supported(experts[0], 0, act_dtype)) return false;
+    int64_t tiles = 0;
+    for (int e = 0; e < n_experts; e++) tiles += (offsets[e + 1] - offsets[e] + 31) / 32;
+    return tiles <= kMaxGroupTiles;
+}
+
+hipError_t cq_launch_gemm_grouped(const cq_weight *const *experts, int n_experts, const int32_t *offsets, cq_act_view a,
+                                  float *y, hipStream_t s) {
+    if (a.m_stride < ((int64_t)offsets[n_experts] + 31) / 32 * 32) return hipErrorInvalidValue;
+    if (experts[0]->dtype == CQ_DTYPE_Q4K) return launch_grouped<CQ_DTYPE_Q4K>(experts, n_experts, offsets, a, y, s);
+    return launch_grouped<CQ_DTYPE_Q6K>(experts, n_experts, offsets, a, y, s);
+}
 
 bool cq_gemm_supported(const cq_weight *w, int64_t m, int act_dtype) {
     (void)m;
