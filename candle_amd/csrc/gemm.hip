@@ -432,13 +432,7 @@ int num_cus() {
 template <int DT, int MT>
 hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
     const size_t lds = Tile<DT, MT>::kTotal;
-    static bool attr_set = false;
-    if (!attr_set && lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void *)gemm_kernel<DT, MT>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    if (hipError_t e = cq_ensure_lds<gemm_kernel<DT, MT>>(w->dev, lds); e != hipSuccess) return e;
     const int64_t gx = (w->n + kWaves * 32 - 1) / (kWaves * 32), gy = (m + MT * 32 - 1) / (MT * 32);
     // too few workgroups for the machine: split K (at least four blocks per part)
     int ksplit = 1;
@@ -478,13 +472,7 @@ hipError_t launch_grouped(const cq_weight *const *experts, int n_experts, const 
     if (ntiles == 0) return hipSuccess;
     const cq_weight *w = experts[0];
     const size_t lds = Tile<DT, 1>::kTotal;
-    static bool attr_set = false;
-    if (!attr_set && lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void *)gemm_grouped_kernel<DT>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    if (hipError_t e = cq_ensure_lds<gemm_grouped_kernel<DT>>(w->dev, lds); e != hipSuccess) return e;
     const int64_t gx = (w->n + kWaves * 32 - 1) / (kWaves * 32);
     int ksplit = 1;
     const int64_t kb = w->k >> 8;

@@ -801,13 +801,7 @@ template <int DT, int UPL, int MB>
 hipError_t launch_batched_upl(const cq_weight *w, cq_act_view a, int64_t m0, int64_t m, float *y, hipStream_t s) {
     constexpr int NW = 8;
     const size_t lds = lds_row_bytes<DT>(w->k) * MB;
-    static bool attr_set = false;
-    if (!attr_set && lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void *)batched_kernel<DT, UPL, NW, MB>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    if (hipError_t e = cq_ensure_lds<batched_kernel<DT, UPL, NW, MB>>(w->dev, lds); e != hipSuccess) return e;
     int64_t wgs = w->n / NW;
     if (wgs > num_cus()) wgs = num_cus();
     const int64_t tw = wgs * NW, rpw = w->n / tw, extra = w->n % tw;

@@ -118,6 +118,7 @@ hipError_t cq_launch_fill_zero(float *p, int64_t count, hipStream_t s);
 
 #if defined(__HIPCC__)
 #include <hip/hip_ext.h>
+#include <atomic>
 // Kernel launch that honours the timing hook.  `kernel` in parentheses when it contains commas.
 #define CQ_LAUNCH(kernel, grid, block, lds, stream, ...)                                                  \
     do {                                                                                                  \
@@ -128,6 +129,19 @@ hipError_t cq_launch_fill_zero(float *p, int64_t count, hipStream_t s);
         else                                                                                              \
             hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), (uint32_t)(lds), stream, __VA_ARGS__);    \
     } while (0)
+
+// Raises the dynamic-LDS limit of `Kernel` on device `dev` when a launch needs more than the
+// default 48 KiB; remembers, per kernel and device, the largest size already granted.
+template <auto Kernel> hipError_t cq_ensure_lds(int dev, size_t lds) {
+    constexpr int kMaxDev = 32;
+    static std::atomic<size_t> granted[kMaxDev];
+    if (lds <= 48 * 1024) return hipSuccess;
+    const int slot = dev >= 0 && dev < kMaxDev ? dev : -1;
+    if (slot >= 0 && granted[slot].load(std::memory_order_relaxed) >= lds) return hipSuccess;
+    hipError_t e = hipFuncSetAttribute((const void *)Kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e == hipSuccess && slot >= 0) granted[slot].store(lds, std::memory_order_relaxed);
+    return e;
+}
 #endif
 
 // ---- small device helpers ---------------------------------------------------
