@@ -337,6 +337,21 @@ extern "C" int cq_qmatmul(const cq_weight *w, const float *x_dev, int64_t m, flo
     cq_act_view v;
     act_ws_layout(act, m, w->k, (uint8_t *)ws, &v);
     if (!(flags & CQ_FLAG_REUSE_ACT)) CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, nullptr, m, w->k, v, s));
+    if (flags & CQ_FLAG_FORCE_SKINNY) {
+        if (!cq_skinny_supported(w, act))
+            return cq_set_error(CQ_ERR_UNSUPPORTED, "no split-K MFMA kernel for dtype %d with activation dtype %d and n = %lld",
+                                w->dtype, act, (long long)w->n);
+        CQ_HIP_CHECK(cq_launch_skinny(w, v, act, m, y_dev, s));
+        return CQ_OK;
+    }
+    // Few rows: split K over the waves instead of tiling rows.  Measured faster than the dot-product
+    // kernels from 2 rows on and than the tile kernel up to 32 rows (up to 128 rows when n is small
+    // and the tile kernel cannot fill the machine).
+    if (!(flags & (CQ_FLAG_FORCE_GEMM | CQ_FLAG_FORCE_MATVEC)) && m >= 2 && cq_skinny_supported(w, act) &&
+        (m <= 32 || (m <= 128 && w->n < 8192))) {
+        CQ_HIP_CHECK(cq_launch_skinny(w, v, act, m, y_dev, s));
+        return CQ_OK;
+    }
     bool use_gemm = false;
     if (flags & CQ_FLAG_FORCE_GEMM) {
         if (!cq_gemm_supported(w, m, act))

@@ -1,0 +1,292 @@
+// Skinny matmul on int8 MFMA for 2..32 activation rows: y[m, n] = x[m, k] . W[n, k]^T with K-quant
+// weights and Q8K activations (k_quants.rs:1842-1883 with vec_dot :1171-1250 for Q4K, :1585-1641
+// for Q6K) - the small-batch decode and the per-expert shapes of a mixture-of-experts layer, where
+// the weights are still read once and the job stays bound by HBM.  The arithmetic is that of the
+// prefill GEMM (gemm.hip): sub-block scales folded into the int8 weight operands as two digits,
+// exact block integers I = 8*hi + lo (Q4K) / 128*hi + lo (Q6K), the Q4K min term on the f16 MFMA.
+//
+// Work split: with so few activation rows there is no tile to reuse weights over, so the K
+// dimension is split instead.  A workgroup owns 16 weight rows (one 16x16x64 MFMA operand); its
+// eight waves take the 256-element K blocks round-robin (wave w: blocks w, w+8, ...).  Per block a
+// wave copies its 16 x 144 (210) weight bytes and the block's activation slice from global memory
+// straight into its own LDS buffer (global_load_lds, whole 128-byte lines, XOR-swizzled as in
+// gemm.hip), unpacks, and issues eight MFMAs per 16 activation rows.  The waves' partial 16 x 16
+// results are summed through LDS in wave order (deterministic; no atomics).  Many small workgroups
+// (n / 16) and one block in flight per wave keep enough bytes outstanding per CU.
+#include "qhip_internal.h"
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+typedef short ss2 __attribute__((ext_vector_type(2)));
+typedef const void __attribute__((address_space(1))) *gptr_t;
+typedef void __attribute__((address_space(3))) *lptr_t;
+
+constexpr int kWaves = 8;
+constexpr int kThreads = kWaves * 64;
+
+__device__ __forceinline__ uint32_t pk_mul_u16(uint32_t a, uint32_t b) {
+    const us2 r = __builtin_bit_cast(us2, a) * __builtin_bit_cast(us2, b);
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ uint32_t pk_sub_u16(uint32_t a, uint32_t b) {
+    const us2 r = __builtin_bit_cast(us2, a) - __builtin_bit_cast(us2, b);
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ uint32_t pk_ashr7_i16(uint32_t a) {
+    const ss2 r = __builtin_bit_cast(ss2, a) >> (ss2){7, 7};
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ uint32_t dup16(uint32_t v) { return (v & 0xffffu) | (v << 16); }
+
+__device__ __forceinline__ void dma16(const void *base, uint32_t off, uint8_t *lds) {
+    __builtin_amdgcn_global_load_lds((gptr_t)((const uint8_t *)base + off), (lptr_t)lds, 16, 0, 0);
+}
+__device__ __forceinline__ void dma4(const void *base, uint32_t off, uint8_t *lds) {
+    __builtin_amdgcn_global_load_lds((gptr_t)((const uint8_t *)base + off), (lptr_t)lds, 4, 0, 0);
+}
+
+// Per-wave LDS buffer for RT groups of eight activation rows:
+//   wgt : [2 row groups][8 rows][8 chunks of 16 B] of the 128-byte qs / ql plane, chunk c of row r at c ^ (r%8);
+//         Q6K also [16 rows][4 chunks] of the 64-byte qh plane (chunk c at c ^ ((r/2)%4))
+//   act : [RT row groups][2 K-halves][8 rows][8 chunks], same swizzle
+//   d8  : [8*RT] f32         minp : [8*RT][2 pieces][8] f16 (Q4K)
+template <int DT, int RT> struct Buf {
+    static constexpr int kWgt = DT == CQ_DTYPE_Q4K ? 2048 : 3072;
+    static constexpr int oAct = kWgt, kAct = RT * 2048;
+    static constexpr int oD8 = oAct + kAct, kD8 = RT * 32;
+    static constexpr int oMin = oD8 + kD8, kMin = DT == CQ_DTYPE_Q4K ? RT * 256 : 0;
+    static constexpr int kRaw = oMin + kMin;
+    // the buffer also carries the wave's partial results at the end: 1 KiB per 16 activation rows
+    static constexpr int kBytes = kRaw < 2048 ? 2048 : kRaw;
+};
+
+__device__ __forceinline__ uint32_t swz_col(uint32_t r, uint32_t c) {
+    return (r >> 3) * 1024u + (r & 7) * 128u + ((c ^ (r & 7)) << 4);
+}
+
+template <int DT> struct WHead;
+template <> struct WHead<CQ_DTYPE_Q4K> { uint32_t dd; uint4 rec; };   // d | dmin << 16; records {sc, sc, mn, mn} per 32 qs bytes
+template <> struct WHead<CQ_DTYPE_Q6K> { uint4 sc; uint32_t d; };     // re-packed scales (two per unit); d
+__device__ __forceinline__ void load_head(const cq_weight &w, int64_t blk, WHead<CQ_DTYPE_Q4K> &r) {
+    const uint32_t *h = (const uint32_t *)(w.p1 + blk * CQ_Q4K_HDR);
+    r.dd = h[0];
+    r.rec = make_uint4(h[1], h[2], h[3], h[4]);
+}
+__device__ __forceinline__ void load_head(const cq_weight &w, int64_t blk, WHead<CQ_DTYPE_Q6K> &r) {
+    r.sc = *(const uint4 *)(w.p2 + blk * 16);
+    r.d = ((const uint16_t *)w.p3)[blk];
+}
+
+// Weight operands of one block for lane (row r = l%16, k quarter kq = l/16): the two digit operands
+// of the four 64-wide K-slices, the block scale and the Q4K min-term operand.
+__device__ __forceinline__ void block_unpack(const uint8_t *wl, int lane, const WHead<CQ_DTYPE_Q4K> &wb, v4i (&bl)[4],
+                                             v4i (&bh)[4], float &dw, v8h &wmin) {
+    const uint32_t r = lane & 15, kq = lane >> 4;
+    dw = cq_h2f((uint16_t)(wb.dd & 0xffff));
+    const float dmin = cq_h2f((uint16_t)(wb.dd >> 16));
+    const uint32_t rec[4] = {wb.rec.x, wb.rec.y, wb.rec.z, wb.rec.w};
+    // K-slice g = elements 64g..64g+63 = qs bytes 32g..32g+31, low nibbles for the first 32 elements
+    // (quarters 0,1: sub-block 2g), high nibbles for the last 32 (quarters 2,3: sub-block 2g+1)
+    const uint32_t hi = kq >> 1, nsh = hi * 4;
+#pragma unroll
+    for (int gi = 0; gi < 4; gi++) {
+        const uint4 q = *(const uint4 *)(wl + swz_col(r, 2 * gi + (kq & 1)));
+        const uint32_t sj = (rec[gi] >> (8 * hi)) & 0xff;   // scale of sub-block 2g + hi
+        const uint32_t sl = dup16(sj & 7), sh = dup16(sj >> 3);
+        const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t v = (qw[i] >> nsh) & 0x0F0F0F0Fu;
+            bl[gi][i] = (int)pk_mul_u16(v, sl);   // low digit of the scale
+            bh[gi][i] = (int)pk_mul_u16(v, sh);
+        }
+    }
+    // min term operand: 32 K-slots = activation pieces [1,1,2,2] x weight pieces [1,2,1,2] of the
+    // eight sub-block values -dmin*min_j
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const float v = -dmin * (float)((rec[j >> 1] >> (16 + 8 * (j & 1))) & 0xff);
+        const _Float16 p1 = (_Float16)v;
+        wmin[j] = (kq & 1) == 0 ? p1 : (_Float16)(v - (float)p1);
+    }
+}
+
+__device__ __forceinline__ void block_unpack(const uint8_t *wl, int lane, const WHead<CQ_DTYPE_Q6K> &wb, v4i (&bl)[4],
+                                             v4i (&bh)[4], float &dw, v8h &wmin) {
+    const uint32_t r = lane & 15, kq = lane >> 4;
+    dw = cq_h2f((uint16_t)wb.d);
+#pragma unroll
+    for (int hf = 0; hf < 2; hf++) {
+        // K-slices 2hf (low nibbles) and 2hf+1 (high nibbles) of unit u = 4hf + kq: 16 bytes of ql,
+        // 8 bytes of re-packed high bits, scale bytes 2u and 2u+1
+        const uint4 ql = *(const uint4 *)(wl + swz_col(r, 4 * hf + kq));
+        const uint2 qh = *(const uint2 *)(wl + 2048 + r * 64u + (((2 * hf + (kq >> 1)) ^ ((r >> 1) & 3)) << 4) + (kq & 1) * 8u);
+        const uint32_t s_even = hf ? wb.sc.z : wb.sc.x, s_odd = hf ? wb.sc.w : wb.sc.y;
+        const uint32_t sw = s_even ^ ((s_even ^ s_odd) & (0u - (kq >> 1)));   // word 2hf + kq/2, branch-free
+        const uint32_t qw[4] = {ql.x, ql.y, ql.z, ql.w};
+        const uint32_t hw[2] = {qh.x, qh.y};
+#pragma unroll
+        for (int nib = 0; nib < 2; nib++) {
+            const int s = 2 * hf + nib;
+            const int sc = (int)(int8_t)((sw >> (16 * (kq & 1) + 8 * nib)) & 0xff);
+            const uint32_t sc16 = dup16((uint32_t)sc);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t H = hw[i >> 1];
+                const int sh = (i & 1) * 4 + 2 * nib;
+                const uint32_t q6 = ((qw[i] >> (4 * nib)) & 0x0F0F0F0Fu) | (((H >> sh) & 0x03030303u) << 4);
+                // the four elements as 16-bit lanes, minus 32, times the group scale (low 16 bits kept)
+                const uint32_t e02 = pk_sub_u16(q6 & 0x00FF00FFu, 0x00200020u);
+                const uint32_t e13 = pk_sub_u16((q6 >> 8) & 0x00FF00FFu, 0x00200020u);
+                const uint32_t p02 = pk_mul_u16(e02, sc16), p13 = pk_mul_u16(e13, sc16);
+                // gather bytes [p02.0, p13.0, p02.2, p13.2]
+                bl[s][i] = (int)(__builtin_amdgcn_perm(p13, p02, 0x06020400u) & 0x7F7F7F7Fu);
+                bh[s][i] = (int)__builtin_amdgcn_perm(pk_ashr7_i16(p13), pk_ashr7_i16(p02), 0x06020400u);
+            }
+        }
+    }
+    wmin = v8h{};
+}
+
+// RT = groups of eight activation rows held (rows m0 .. m0 + 8*RT - 1; the workspace pads rows, so
+// whole groups can be copied); results are stored for rows < m.  Requires n % 16 == 0.
+template <int DT, int RT>
+__global__ void __launch_bounds__(kThreads) skinny_kernel(cq_weight w, cq_act_view a, int64_t m0, int64_t m,
+                                                          float *__restrict__ y) {
+    typedef Buf<DT, RT> B;
+    constexpr bool MINS = DT == CQ_DTYPE_Q4K;
+    constexpr int NT = (RT + 1) / 2;   // 16-row tiles
+    constexpr int SHIFT = DT == CQ_DTYPE_Q4K ? 3 : 7;
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t r = lane & 15, kq = lane >> 4;
+    const int64_t k = w.k, kb = w.k >> 8;
+    const int64_t n_tile = (int64_t)blockIdx.x * 16;
+    uint8_t *buf = smem + wave * B::kBytes;
+
+    // copy offsets: 8 rows x 128 B per instruction, chunks swizzled by the row
+    const uint32_t r8 = lane >> 3, c8 = lane & 7;
+    const uint32_t act_off = r8 * (uint32_t)k + ((c8 ^ r8) << 4);
+    const uint32_t wq_off = r8 * (uint32_t)kb * 128u + ((c8 ^ r8) << 4);
+    const uint32_t r16 = lane >> 2, c4 = lane & 3;
+    const uint32_t wh_off = r16 * (uint32_t)kb * 64u + ((c4 ^ ((r16 >> 1) & 3)) << 4);
+    // activation operand reads: row of tile t clamped to the rows held
+    uint32_t a_col[NT][2];
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const uint32_t row = t * 16 + r < 8u * RT ? t * 16 + r : 8u * RT - 1;
+#pragma unroll
+        for (uint32_t e = 0; e < 2; e++)
+            a_col[t][e] = B::oAct + (row >> 3) * 2048u + (row & 7) * 128u + (((4 * e + kq) ^ (row & 7)) << 4);
+    }
+
+    v4f out[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) out[t] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+
+    for (int64_t b = wave; b < kb; b += kWaves) {
+        // ---- copies of block b: weights of the 16 rows, activation rows, their scales
+#pragma unroll
+        for (int rg = 0; rg < 2; rg++) dma16(w.p0 + ((n_tile + rg * 8) * kb + b) * 128, wq_off, buf + rg * 1024);
+        if (DT == CQ_DTYPE_Q6K) dma16(w.p1 + (n_tile * kb + b) * 64, wh_off, buf + 2048);
+#pragma unroll
+        for (int i = 0; i < 2 * RT; i++) {
+            const int rg = i >> 1, kh = i & 1;
+            dma16(a.qs + (m0 + rg * 8) * k + b * 256 + kh * 128, act_off, buf + B::oAct + i * 1024);
+        }
+        if (lane < 8 * RT) dma4(a.dT + b * a.m_stride + m0, lane * 4u, buf + B::oD8);
+        if (MINS && lane < 16 * RT) dma16(a.minp + (b * a.m_stride + m0) * 16, lane * 16u, buf + B::oMin);
+        WHead<DT> head;
+        load_head(w, (n_tile + r) * kb + b, head);
+        __builtin_amdgcn_s_waitcnt(0);   // everything above has landed
+
+        // ---- arithmetic of block b
+        v4i bl[4], bh[4];
+        float dw;
+        v8h wmin;
+        block_unpack(buf, lane, head, bl, bh, dw, wmin);
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const v4f d8 = *(const v4f *)(buf + B::oD8 + (t * 16 + 4 * kq < 8u * RT ? t * 16 + 4 * kq : 0) * 4);
+            if (MINS) {
+                const uint32_t row = t * 16 + r < 8u * RT ? t * 16 + r : 8u * RT - 1;
+                const v8h ma = *(const v8h *)(buf + B::oMin + row * 32 + (kq >> 1) * 16);
+                out[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ma, wmin, out[t], 0, 0, 0);
+            }
+            v4i acc_lo = {0, 0, 0, 0}, acc_hi = {0, 0, 0, 0};
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                const v4i av = *(const v4i *)(buf + a_col[t][s & 1] + (s >> 1) * 1024);
+                acc_lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bl[s], acc_lo, 0, 0, 0);
+                acc_hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bh[s], acc_hi, 0, 0, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int I = (acc_hi[i] << SHIFT) + acc_lo[i];
+                out[t][i] = __builtin_fmaf((float)I * dw, d8[i], out[t][i]);
+            }
+        }
+    }
+
+    // ---- sum the eight waves' partial tiles in wave order
+#pragma unroll
+    for (int t = 0; t < NT; t++) *(v4f *)(buf + t * 1024 + lane * 16) = out[t];
+    __syncthreads();
+    if (wave < NT) {
+        v4f s = *(const v4f *)(smem + wave * 1024 + lane * 16);
+#pragma unroll
+        for (int o = 1; o < kWaves; o++) {
+            const v4f p = *(const v4f *)(smem + o * B::kBytes + wave * 1024 + lane * 16);
+            s += p;
+        }
+        const int64_t col = n_tile + r;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int64_t row = m0 + wave * 16 + kq * 4 + i;
+            if (row < m) y[row * w.n + col] = s[i];
+        }
+    }
+}
+
+template <int DT, int RT>
+hipError_t launch_rt(const cq_weight *w, cq_act_view a, int64_t m0, int64_t m, float *y, hipStream_t s) {
+    const size_t lds = (size_t)Buf<DT, RT>::kBytes * kWaves;
+    if (hipError_t e = cq_ensure_lds<skinny_kernel<DT, RT>>(w->dev, lds); e != hipSuccess) return e;
+    CQ_LAUNCH((skinny_kernel<DT, RT>), (unsigned)(w->n / 16), kThreads, lds, s, *w, a, m0, m, y);
+    return hipGetLastError();
+}
+
+template <int DT>
+hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
+    for (int64_t m0 = 0; m0 < m; m0 += 32) {
+        const int64_t left = m - m0;
+        hipError_t e;
+        if (left <= 8) e = launch_rt<DT, 1>(w, a, m0, m, y, s);
+        else if (left <= 16) e = launch_rt<DT, 2>(w, a, m0, m, y, s);
+        else if (left <= 24) e = launch_rt<DT, 3>(w, a, m0, m, y, s);
+        else e = launch_rt<DT, 4>(w, a, m0, m, y, s);
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+}  // namespace
+
+bool cq_skinny_supported(const cq_weight *w, int act_dtype) {
+    // the copies address 8 rows of activations and 16 rows of a weight plane with 32-bit offsets
+    return (w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q6K) && act_dtype == CQ_DTYPE_Q8K && w->k >= 256 &&
+           w->k <= (1 << 24) && w->n % 16 == 0 && w->n > 0;
+}
+
+hipError_t cq_launch_skinny(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s) {
+    if (!cq_skinny_supported(w, act_dtype)) return hipErrorNotSupported;
+    if (m == 0) return hipSuccess;
+    if (a.m_stride < (m + 31) / 32 * 32) return hipErrorInvalidValue;   // whole 8-row groups are copied
+    if (w->dtype == CQ_DTYPE_Q4K) return launch_dt<CQ_DTYPE_Q4K>(w, a, m, y, s);
+    return launch_dt<CQ_DTYPE_Q6K>(w, a, m, y, s);
+}

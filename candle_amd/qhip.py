@@ -16,6 +16,7 @@ LIB_PATH = os.environ.get("CQ_LIB_PATH", os.path.join(_HERE, "lib", "libcandle_q
 # GgmlDType ids (candle-core/src/quantized/mod.rs:173-190)
 Q4_0, Q8_0, Q8_1, Q4K, Q6K, Q8K = 2, 8, 9, 12, 14, 15
 FLAG_AUTO, FLAG_FORCE_MATVEC, FLAG_FORCE_GEMM, FLAG_ACT_Q8_1, FLAG_REUSE_ACT, FLAG_STAGED_ACT = 0, 1, 2, 4, 8, 16
+FLAG_FORCE_SKINNY = 32
 
 EXPORTS = [
     "cq_device_count", "cq_last_error", "cq_version", "cq_block_size", "cq_type_size", "cq_vec_dot_type",

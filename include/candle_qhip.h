@@ -56,6 +56,7 @@ enum {
     CQ_FLAG_REUSE_ACT = 8,    /* the workspace already holds this x, quantized by an earlier cq_qmatmul call with the
                                  same m, k and activation format (q/k/v or gate/up share their input): skip the
                                  quantizer launch.  No counterpart in the reference, which re-quantizes per call.     */
+    CQ_FLAG_FORCE_SKINNY = 32, /* the split-K MFMA kernel for few rows whatever m is (A/B runs)                                */
     CQ_FLAG_STAGED_ACT = 16   /* m == 1 only: run the stand-alone quantizer into the workspace and the plain matvec
                                  (two launches, as cuda.rs:249-293 does) instead of the single fused launch           */
 };

@@ -217,6 +217,20 @@ def test_ragged_batches_match_oracle(qh, dt, m, k, n):
 
 
 @pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K])
+@pytest.mark.parametrize("m,k,n", [(2, 256, 16), (3, 512, 48), (8, 4096, 64), (9, 1024, 32), (16, 2048, 80),
+                                   (17, 768, 16), (24, 11008, 32), (32, 4096, 16), (33, 2304, 48), (5, 14336, 16)])
+def test_skinny_matches_oracle(qh, dt, m, k, n):
+    """The split-K MFMA kernel for few rows: every row-group count (1-4 groups of eight rows), more
+    than 32 rows (two launches), fewer K blocks than waves, K blocks not a multiple of the waves."""
+    w, x = make_inputs(17 * dt + m + k + n, m, k, n, outliers=True)
+    blocks = orc.quantize(dt, w)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    got = qh.qmatmul(qw, dev(x), qh.FLAG_FORCE_SKINNY)
+    check_f32(got.cpu().numpy(), orc.matmul(dt, x, blocks, n))
+    assert torch.equal(got, qh.qmatmul(qw, dev(x), qh.FLAG_FORCE_SKINNY))   # deterministic: no atomics
+
+
+@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K])
 def test_gemm_ragged_rows_large(qh, dt):
     """M = 300 (not a multiple of the 128-row workgroup tile) on a K-split shape: every output row
     of the tile kernel equals the dot-product kernels' result for that row within tolerance."""
