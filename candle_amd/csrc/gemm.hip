@@ -20,7 +20,7 @@
 // owns 32 weight rows (32x32x32 MFMA, B operand: lane l holds row l%32, k = 16*(l/32)+[0,16) of a
 // 32-wide K-slice), unpacks them in registers once per block and reuses them for all BM rows.
 // Activations (shared by the waves) and each wave's packed weight bytes go from global memory
-// straight into LDS (global_load_lds_dwordx4), double buffered, one block ahead.  Every such copy
+// straight into LDS (buffer_load_dwordx4 ... lds), double buffered, one block ahead.  Every such copy
 // instruction reads eight whole 128-byte lines (8 rows x 128 B) - the texture path pays per line
 // touched - and the 16-byte chunks of a row are XOR-swizzled by the row number on the way in, so
 // that the MFMA operand reads (lanes = rows, one chunk column) spread over all LDS banks.  With few
@@ -54,8 +54,8 @@ template <int DT, int MT> struct Tile {
     static constexpr int kMin = DT == CQ_DTYPE_Q4K ? MT * 32 * 32 : 0;
     static constexpr int kWgtWave = DT == CQ_DTYPE_Q4K ? 4096 : 6144;
     static constexpr int oD8 = kAct, oMin = oD8 + kD8;
-    static constexpr int kBytes = oMin + kMin;                                  // one activation stage (two of them)
-    static constexpr int oWgt = 2 * kBytes;                                     // weights: one buffer per wave
+    static constexpr int kBytes = oMin + kMin;                                  // one activation stage (three of them)
+    static constexpr int oWgt = 3 * kBytes;                                     // weights: one buffer per wave
     static constexpr int kTotal = oWgt + kWaves * kWgtWave;
 };
 
@@ -73,13 +73,22 @@ __device__ __forceinline__ uint32_t pk_ashr7_i16(uint32_t a) {
 }
 __device__ __forceinline__ uint32_t dup16(uint32_t v) { return (v & 0xffffu) | (v << 16); }
 
+// Buffer descriptor over `base` (wave-uniform): raw bytes, no stride, no bounds.  The copies below
+// are buffer loads rather than global loads on purpose: with a global (FLAT-encoded) LDS copy in
+// flight the compiler treats the LDS counter as out of order and turns every wait on an operand
+// read into a wait for all of them, which serialises the software-pipelined LDS reads; a buffer
+// load leaves the LDS counter alone and takes its per-lane offset without 64-bit vector adds.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t wave_rsrc(const void *base) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, -1, 0x00020000);
+}
+
 // Asynchronous copy of 64 x 16 (or 64 x 4) bytes: lane l reads base + off and the data lands at
 // lds + 16*l (4*l).  `base` and `lds` are wave-uniform.
 __device__ __forceinline__ void dma16(const void *base, uint32_t off, uint8_t *lds) {
-    __builtin_amdgcn_global_load_lds((gptr_t)((const uint8_t *)base + off), (lptr_t)lds, 16, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(wave_rsrc(base), (lptr_t)lds, 16, (int)off, 0, 0, 0);
 }
 __device__ __forceinline__ void dma4(const void *base, uint32_t off, uint8_t *lds) {
-    __builtin_amdgcn_global_load_lds((gptr_t)((const uint8_t *)base + off), (lptr_t)lds, 4, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(wave_rsrc(base), (lptr_t)lds, 4, (int)off, 0, 0, 0);
 }
 
 // Per-lane constants of the copies and of the operand reads.
@@ -171,10 +180,11 @@ __device__ __forceinline__ void load_head(const cq_weight &w, int64_t blk, WHead
 // LDS reads run two steps ahead.  The accumulator pair alternates between two register sets.  A
 // scheduling barrier after every step keeps the compiler from hoisting all MFMAs to the front,
 // which would need MT accumulator sets at once.
-template <int DT, int MT, int SHIFT>
+template <int DT, int MT, int T0, int T1, int SHIFT>
 __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, const v4i (&bl)[8], const v4i (&bh)[8],
                                           float dw, v8h wmin, int lane, v16f (&out)[MT]) {
     typedef Tile<DT, MT> T;
+    if constexpr (T0 >= T1) return;
     constexpr bool MINS = DT == CQ_DTYPE_Q4K;
     const int h = lane >> 5, col = lane & 31;
     const uint8_t *d8p = cur + T::oD8 + h * 16;        // rows 8j + 4h + [0,4) of a tile
@@ -188,17 +198,17 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, 
     v4i a[3];
     v4f dreg[2];   // d8 of four rows each, read two steps before the scaling that needs them
     v8h ma1, ma2;
-    a[0] = afrag(0);
-    a[1] = afrag(1);
+    a[(T0 * 8) % 3] = afrag(T0 * 8);
+    a[(T0 * 8 + 1) % 3] = afrag(T0 * 8 + 1);
     if (MINS) {
-        ma1 = *(const v8h *)(mnp);
-        ma2 = *(const v8h *)(mnp + 16);
+        ma1 = *(const v8h *)(mnp + T0 * 1024);
+        ma2 = *(const v8h *)(mnp + T0 * 1024 + 16);
     }
 #pragma unroll
-    for (int q = 0; q < (MT + 1) * 8; q++) {
+    for (int q = T0 * 8; q < (T1 + 1) * 8; q++) {
         const int t = q >> 3, s = q & 7;
-        if (q + 2 < MT * 8) a[(q + 2) % 3] = afrag(q + 2);
-        if (t < MT) {
+        if (q + 2 < T1 * 8) a[(q + 2) % 3] = afrag(q + 2);
+        if (t < T1) {
             if (s == 0) {
                 if (MINS) {
                     // min term: out -= sum_j (dmin*min_j) * (d8*bsum32_j).  K-slots 0..7 carry piece 1
@@ -215,12 +225,12 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, 
                 acc_hi[t & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[q % 3], bh[s], acc_hi[t & 1], 0, 0, 0);
             }
             if (s == 6) dreg[0] = *(const v4f *)(d8p + (t * 32) * 4);
-            if (s == 6 && MINS && t + 1 < MT) {
+            if (s == 6 && MINS && t + 1 < T1) {
                 ma1 = *(const v8h *)(mnp + (t + 1) * 1024);
                 ma2 = *(const v8h *)(mnp + (t + 1) * 1024 + 16);
             }
         }
-        if (t > 0) {
+        if (t > T0) {
             const int p = (t - 1) & 1;
             if ((s & 1) == 0 && s < 6) dreg[((s >> 1) + 1) & 1] = *(const v4f *)(d8p + ((t - 1) * 32 + 8 * ((s >> 1) + 1)) * 4);
 #pragma unroll
@@ -308,25 +318,36 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g
     wmin = v8h{};
 }
 
-// Activation copies for block b+1 into `nxt`, weight operands of block b out of `wl`, the copies of
-// the wave's weights for block b+1 into `wl` again (its bytes are in registers by then), then the
-// arithmetic of block b out of `cur`.  The three LDS regions are distinct (`__restrict__`): without
-// that knowledge the compiler makes every LDS read wait for all copies in flight, which would
-// serialise the pipeline.
-template <int DT, int MT>
+// One K block of one wave.  The two waves of a SIMD (waves w and w + 4 of the workgroup) run half a
+// block apart: a leading wave unpacks block b, contracts all of its tiles and meets the others at
+// the block barrier; a trailing wave goes through the barrier after the lower half of the tiles and
+// contracts the upper half behind it, while the leading waves already unpack block b+1.  The
+// unpacking is pure VALU work and the contraction mostly MFMA, so one wave's unpacking runs under
+// the other's MFMAs instead of both alternating between the two in lockstep.  Activations
+// therefore live in three stages: block b+1 lands in `nxt` while block b is read from `cur` and the
+// trailing waves may still read block b-1.  The wave's weight bytes of block b come out of `wl`,
+// which is refilled for block b+1 as soon as they are in registers.  The LDS regions are distinct
+// (`__restrict__`): without that knowledge the compiler makes every LDS read wait for all copies in
+// flight, which would serialise the pipeline.
+template <int DT, int MT, bool TRAIL>
 __device__ __forceinline__ void block_step(const uint8_t *__restrict__ cur, uint8_t *__restrict__ nxt,
                                            uint8_t *__restrict__ wl, const cq_weight &w, const cq_act_view &a,
                                            const LaneGeo &g, int64_t m0, int64_t n_tile, bool n_ok, bool more, int64_t b,
                                            int wave, int lane, const WHead<DT> &hcur, v16f (&out)[MT]) {
+    constexpr int SHIFT = DT == CQ_DTYPE_Q4K ? 3 : 7;
+    constexpr int SPLIT = TRAIL ? MT / 2 : MT;   // tiles [SPLIT, MT) follow the barrier
+    v4i bl[8], bh[8];
+    float dw = 0.0f;
+    v8h wmin = {};
     if (more) stage_issue<DT, MT>(nxt, w, a, g, m0, b + 1, wave, lane);
     if (n_ok) {
-        v4i bl[8], bh[8];
-        float dw;
-        v8h wmin;
         block_unpack(wl, g, hcur, lane, bl, bh, dw, wmin);
         if (more) stage_weights<DT>(wl, w, g, n_tile, b + 1);
-        tiles_mac<DT, MT, (DT == CQ_DTYPE_Q4K ? 3 : 7)>(cur, g, bl, bh, dw, wmin, lane, out);
+        tiles_mac<DT, MT, 0, SPLIT, SHIFT>(cur, g, bl, bh, dw, wmin, lane, out);
     }
+    __builtin_amdgcn_s_waitcnt(0);   // the next stage and the wave's next weights have landed in LDS
+    __syncthreads();
+    if (TRAIL && n_ok) tiles_mac<DT, MT, SPLIT, MT, SHIFT>(cur, g, bl, bh, dw, wmin, lane, out);
 }
 
 // ------------------------------------------------------------------ kernel ----
@@ -365,16 +386,32 @@ __device__ __forceinline__ void gemm_body(const cq_weight &w, const cq_act_view 
     __builtin_amdgcn_s_waitcnt(0);   // the LDS copies above (and everything else outstanding)
     __syncthreads();
 
-    for (int64_t b = b0; b < b1; b++) {
-        const int par = (int)((b - b0) & 1);
-        uint8_t *cur = smem + par * T::kBytes;
-        uint8_t *nxt = smem + (par ^ 1) * T::kBytes;
-        const bool more = b + 1 < b1;
-        if (more) load_head(w, nc * kb + b + 1, hnxt);
-        block_step<DT, MT>(cur, nxt, wl, w, a, g, m0, n_tile, n_ok, more, b, wave, lane, hcur, out);
-        hcur = hnxt;
-        __builtin_amdgcn_s_waitcnt(0);   // the next stage has landed in LDS
-        __syncthreads();
+    // Stage of block b: (b - b0) % 3.  Both loops pass the same number of barriers.
+    int ic = 0, in = 1, ifree = 2;
+    auto rotate = [&]() {
+        const int t = ic;
+        ic = in;
+        in = ifree;
+        ifree = t;
+    };
+    if (wave < kWaves / 2) {
+        for (int64_t b = b0; b < b1; b++) {
+            const bool more = b + 1 < b1;
+            if (more) load_head(w, nc * kb + b + 1, hnxt);
+            block_step<DT, MT, false>(smem + ic * T::kBytes, smem + in * T::kBytes, wl, w, a, g, m0, n_tile, n_ok, more, b,
+                                      wave, lane, hcur, out);
+            hcur = hnxt;
+            rotate();
+        }
+    } else {
+        for (int64_t b = b0; b < b1; b++) {
+            const bool more = b + 1 < b1;
+            if (more) load_head(w, nc * kb + b + 1, hnxt);
+            block_step<DT, MT, true>(smem + ic * T::kBytes, smem + in * T::kBytes, wl, w, a, g, m0, n_tile, n_ok, more, b,
+                                     wave, lane, hcur, out);
+            hcur = hnxt;
+            rotate();
+        }
     }
 
     if (n_ok) {

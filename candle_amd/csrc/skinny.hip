@@ -9,7 +9,7 @@
 // dimension is split instead.  A workgroup owns 16 weight rows (one 16x16x64 MFMA operand); its
 // eight waves take the 256-element K blocks round-robin (wave w: blocks w, w+8, ...).  Per block a
 // wave copies its 16 x 144 (210) weight bytes and the block's activation slice from global memory
-// straight into its own LDS buffer (global_load_lds, whole 128-byte lines, XOR-swizzled as in
+// straight into its own LDS buffer (buffer_load ... lds, whole 128-byte lines, XOR-swizzled as in
 // gemm.hip), unpacks, and issues eight MFMAs per 16 activation rows.  The waves' partial 16 x 16
 // results are summed through LDS in wave order (deterministic; no atomics).  Many small workgroups
 // (n / 16) and one block in flight per wave keep enough bytes outstanding per CU.
@@ -42,11 +42,20 @@ __device__ __forceinline__ uint32_t pk_ashr7_i16(uint32_t a) {
 }
 __device__ __forceinline__ uint32_t dup16(uint32_t v) { return (v & 0xffffu) | (v << 16); }
 
+// Buffer descriptor over `base` (wave-uniform): raw bytes, no stride, no bounds.  The copies below
+// are buffer loads rather than global loads on purpose: with a global (FLAT-encoded) LDS copy in
+// flight the compiler treats the LDS counter as out of order and turns every wait on an operand
+// read into a wait for all of them, which serialises the software-pipelined LDS reads; a buffer
+// load leaves the LDS counter alone and takes its per-lane offset without 64-bit vector adds.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t wave_rsrc(const void *base) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, -1, 0x00020000);
+}
+
 __device__ __forceinline__ void dma16(const void *base, uint32_t off, uint8_t *lds) {
-    __builtin_amdgcn_global_load_lds((gptr_t)((const uint8_t *)base + off), (lptr_t)lds, 16, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(wave_rsrc(base), (lptr_t)lds, 16, (int)off, 0, 0, 0);
 }
 __device__ __forceinline__ void dma4(const void *base, uint32_t off, uint8_t *lds) {
-    __builtin_amdgcn_global_load_lds((gptr_t)((const uint8_t *)base + off), (lptr_t)lds, 4, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(wave_rsrc(base), (lptr_t)lds, 4, (int)off, 0, 0, 0);
 }
 
 // Per-wave LDS buffer for RT groups of eight activation rows:
