@@ -263,8 +263,9 @@ extern "C" int cq_quantize_act(int dev, int act_dtype, const float *x_dev, int64
 static size_t act_ws_layout(int act_dtype, int64_t m, int64_t k, uint8_t *base, cq_act_view *v) {
     size_t off = 0;
     auto take = [&](size_t bytes) { size_t o = off; off = cq_align_up(off + bytes, 256); return o; };
-    // Q8K rows are padded (see cq_act_view::m_stride)
-    const int64_t m_pad = act_dtype == CQ_DTYPE_Q8K ? (m + 63) / 64 * 64 + 256 : m;
+    // Q8K rows are padded (see cq_act_view::m_stride); the others to whole 32-row groups, which the
+    // split-K MFMA kernel copies without looking at the row count
+    const int64_t m_pad = act_dtype == CQ_DTYPE_Q8K ? (m + 63) / 64 * 64 + 256 : (m + 31) / 32 * 32;
     const size_t o_qs = take((size_t)(m_pad * k));
     cq_act_view view{};
     view.m_stride = m_pad;

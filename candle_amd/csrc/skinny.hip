@@ -1,5 +1,5 @@
 // Skinny matmul on int8 MFMA for 2..32 activation rows: y[m, n] = x[m, k] . W[n, k]^T with K-quant
-// weights and Q8K activations (k_quants.rs:1842-1883 with vec_dot :1171-1250 for Q4K, :1585-1641
+// weights and Q8K activations (Q8_0 weights with Q8_0 activations: second kernel below) (k_quants.rs:1842-1883 with vec_dot :1171-1250 for Q4K, :1585-1641
 // for Q6K) - the small-batch decode and the per-expert shapes of a mixture-of-experts layer, where
 // the weights are still read once and the job stays bound by HBM.  The arithmetic is that of the
 // prefill GEMM (gemm.hip): sub-block scales folded into the int8 weight operands as two digits,
@@ -262,6 +262,136 @@ __global__ void __launch_bounds__(kThreads) skinny_kernel(cq_weight w, cq_act_vi
     }
 }
 
+// ------------------------------------------------------------ Q8_0 weights x Q8_0 activations ----
+// The same work split for 32-element blocks (k_quants.rs:618-649: sumf += sumi * d_w * d_x per
+// block).  The weights are int8 already, so the operands go from LDS straight into the 16x16x32
+// MFMA, one per block, and each block's 16 x 16 integers are scaled by the two block scales on the
+// way into the f32 result.  A wave takes 256 elements (eight blocks) per step.
+//   wgt : [2 row groups][2 K-halves][8 rows][8 chunks of 16 B], chunk c of row r at c ^ (r%8)
+//   act : [RT row groups][2 K-halves][8 rows][8 chunks], same swizzle
+template <int RT> struct BufQ8 {
+    static constexpr int oAct = 4096, kRaw = oAct + RT * 2048;
+    static constexpr int kBytes = kRaw;   // >= 2 KiB of partial results
+};
+
+template <int RT>
+__global__ void __launch_bounds__(kThreads) skinny_q8_0_kernel(cq_weight w, cq_act_view a, int64_t m0, int64_t m,
+                                                               float *__restrict__ y) {
+    typedef BufQ8<RT> B;
+    constexpr int NT = (RT + 1) / 2;   // 16-row tiles
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t r = lane & 15, kq = lane >> 4;
+    const int64_t k = w.k, kg = w.k >> 8, kb = w.k >> 5;
+    const int64_t n_tile = (int64_t)blockIdx.x * 16;
+    uint8_t *buf = smem + wave * B::kBytes;
+
+    // copy offsets: 8 rows x 128 B per instruction, chunks swizzled by the row
+    const uint32_t r8 = lane >> 3, c8 = lane & 7;
+    const uint32_t row_off = r8 * (uint32_t)k + ((c8 ^ r8) << 4);
+    // operand reads: 8 bytes [32b + 8kq, +8) of a row = half b/4, chunk 2(b%4) + kq/2, byte 8(kq%2)
+    uint32_t w_col[4], a_col[NT][4];
+    int64_t a_row[NT][4];   // rows whose scales this lane applies (results rows 4kq + i of tile t)
+#pragma unroll
+    for (uint32_t c = 0; c < 4; c++) w_col[c] = (r >> 3) * 2048u + (r & 7) * 128u + (((2 * c + (kq >> 1)) ^ (r & 7)) << 4) + (kq & 1) * 8u;
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const uint32_t row = t * 16 + r < 8u * RT ? t * 16 + r : 8u * RT - 1;
+#pragma unroll
+        for (uint32_t c = 0; c < 4; c++)
+            a_col[t][c] = B::oAct + (row >> 3) * 2048u + (row & 7) * 128u + (((2 * c + (kq >> 1)) ^ (row & 7)) << 4) + (kq & 1) * 8u;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int64_t row_i = m0 + t * 16 + 4 * kq + i;
+            a_row[t][i] = row_i < m ? row_i : m - 1;
+        }
+    }
+
+    v4f out[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) out[t] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+
+    for (int64_t g = wave; g < kg; g += kWaves) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int rg = i >> 1, kh = i & 1;
+            dma16(w.p0 + (n_tile + rg * 8) * k + g * 256 + kh * 128, row_off, buf + i * 1024);
+        }
+#pragma unroll
+        for (int i = 0; i < 2 * RT; i++) {
+            const int rg = i >> 1, kh = i & 1;
+            dma16(a.qs + (m0 + rg * 8) * k + g * 256 + kh * 128, row_off, buf + B::oAct + i * 1024);
+        }
+        // the eight block scales of this lane's weight row, and of the activation rows it scales
+        const uint4 dwv = *(const uint4 *)(w.p1 + ((n_tile + r) * kb + g * 8) * 2);
+        v4f da[NT][4][2];
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const v4f *p = (const v4f *)(a.d + a_row[t][i] * kb + g * 8);
+                da[t][i][0] = p[0];
+                da[t][i][1] = p[1];
+            }
+        __builtin_amdgcn_s_waitcnt(0);   // everything above has landed
+
+        const uint32_t dww[4] = {dwv.x, dwv.y, dwv.z, dwv.w};
+#pragma unroll
+        for (int b = 0; b < 8; b++) {
+            const float dw = cq_h2f((uint16_t)(dww[b >> 1] >> (16 * (b & 1))));
+            const long wv = *(const long *)(buf + w_col[b & 3] + (b >> 2) * 1024);
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const long av = *(const long *)(buf + a_col[t][b & 3] + (b >> 2) * 1024);
+                const v4i acc = __builtin_amdgcn_mfma_i32_16x16x32_i8(av, wv, (v4i){0, 0, 0, 0}, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 4; i++) out[t][i] = __builtin_fmaf((float)acc[i] * dw, da[t][i][b >> 2][b & 3], out[t][i]);
+            }
+        }
+    }
+
+    // ---- sum the eight waves' partial tiles in wave order
+#pragma unroll
+    for (int t = 0; t < NT; t++) *(v4f *)(buf + t * 1024 + lane * 16) = out[t];
+    __syncthreads();
+    if (wave < NT) {
+        v4f s = *(const v4f *)(smem + wave * 1024 + lane * 16);
+#pragma unroll
+        for (int o = 1; o < kWaves; o++) {
+            const v4f p = *(const v4f *)(smem + o * B::kBytes + wave * 1024 + lane * 16);
+            s += p;
+        }
+        const int64_t col = n_tile + r;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int64_t row = m0 + wave * 16 + kq * 4 + i;
+            if (row < m) y[row * w.n + col] = s[i];
+        }
+    }
+}
+
+template <int RT>
+hipError_t launch_q8_rt(const cq_weight *w, cq_act_view a, int64_t m0, int64_t m, float *y, hipStream_t s) {
+    const size_t lds = (size_t)BufQ8<RT>::kBytes * kWaves;
+    if (hipError_t e = cq_ensure_lds<skinny_q8_0_kernel<RT>>(w->dev, lds); e != hipSuccess) return e;
+    CQ_LAUNCH((skinny_q8_0_kernel<RT>), (unsigned)(w->n / 16), kThreads, lds, s, *w, a, m0, m, y);
+    return hipGetLastError();
+}
+
+hipError_t launch_q8(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
+    for (int64_t m0 = 0; m0 < m; m0 += 32) {
+        const int64_t left = m - m0;
+        hipError_t e;
+        if (left <= 8) e = launch_q8_rt<1>(w, a, m0, m, y, s);
+        else if (left <= 16) e = launch_q8_rt<2>(w, a, m0, m, y, s);
+        else if (left <= 24) e = launch_q8_rt<3>(w, a, m0, m, y, s);
+        else e = launch_q8_rt<4>(w, a, m0, m, y, s);
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
 template <int DT, int RT>
 hipError_t launch_rt(const cq_weight *w, cq_act_view a, int64_t m0, int64_t m, float *y, hipStream_t s) {
     const size_t lds = (size_t)Buf<DT, RT>::kBytes * kWaves;
@@ -288,14 +418,16 @@ hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hip
 
 bool cq_skinny_supported(const cq_weight *w, int act_dtype) {
     // the copies address 8 rows of activations and 16 rows of a weight plane with 32-bit offsets
-    return (w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q6K) && act_dtype == CQ_DTYPE_Q8K && w->k >= 256 &&
-           w->k <= (1 << 24) && w->n % 16 == 0 && w->n > 0;
+    const bool kquant = (w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q6K) && act_dtype == CQ_DTYPE_Q8K;
+    const bool q8 = w->dtype == CQ_DTYPE_Q8_0 && act_dtype == CQ_DTYPE_Q8_0 && w->k % 256 == 0;
+    return (kquant || q8) && w->k >= 256 && w->k <= (1 << 24) && w->n % 16 == 0 && w->n > 0;
 }
 
 hipError_t cq_launch_skinny(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s) {
     if (!cq_skinny_supported(w, act_dtype)) return hipErrorNotSupported;
     if (m == 0) return hipSuccess;
     if (a.m_stride < (m + 31) / 32 * 32) return hipErrorInvalidValue;   // whole 8-row groups are copied
+    if (w->dtype == CQ_DTYPE_Q8_0) return launch_q8(w, a, m, y, s);
     if (w->dtype == CQ_DTYPE_Q4K) return launch_dt<CQ_DTYPE_Q4K>(w, a, m, y, s);
     return launch_dt<CQ_DTYPE_Q6K>(w, a, m, y, s);
 }
