@@ -486,3 +486,37 @@ extern "C" int cq_timing_elapsed_us(double *us) {
     *us = (double)ms * 1e3;
     return CQ_OK;
 }
+
+// ---- hardware self-check of the quantizers' rounding instruction -------------------------------
+namespace {
+__global__ void selfcheck_round_kernel(uint32_t last_bits, unsigned long long *bad) {
+    const unsigned long long stride = (unsigned long long)gridDim.x * blockDim.x;
+    unsigned long long mine = 0;
+    for (unsigned long long b = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x; b <= last_bits; b += stride) {
+        const float t = __builtin_bit_cast(float, (uint32_t)b);
+        // exact: t has 24 significant bits, so t + 0.5 is exact in double
+        const int want = (int)floor((double)t + 0.5);
+        if (cq_round_away_i32(t) != want) mine++;
+        if (cq_round_away_i32(-t) != -want) mine++;
+    }
+    if (mine) atomicAdd(bad, mine);
+}
+}  // namespace
+
+extern "C" int cq_selfcheck_round(int dev, uint64_t *mismatches) {
+    if (!mismatches) return cq_set_error(CQ_ERR_INVALID, "mismatches is null");
+    CQ_HIP_CHECK(hipSetDevice(dev));
+    unsigned long long *bad = nullptr;
+    CQ_HIP_CHECK(hipMalloc((void **)&bad, sizeof(*bad)));
+    hipError_t e = hipMemset(bad, 0, sizeof(*bad));
+    if (e == hipSuccess) {
+        hipLaunchKernelGGL(selfcheck_round_kernel, dim3(4096), dim3(256), 0, 0, 0x43020000u /* 130.0f */, bad);
+        e = hipGetLastError();
+    }
+    unsigned long long host = 0;
+    if (e == hipSuccess) e = hipMemcpy(&host, bad, sizeof(host), hipMemcpyDeviceToHost);
+    (void)hipFree(bad);
+    CQ_HIP_CHECK(e);
+    *mismatches = host;
+    return CQ_OK;
+}

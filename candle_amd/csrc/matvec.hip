@@ -235,14 +235,27 @@ __device__ __forceinline__ void load_x_pairs(const float *x, int64_t k, int wave
     }
 }
 
-// Maximum / minimum over each half of the wave (lanes 0..31 and 32..63), valid in every lane.
-__device__ __forceinline__ float half_max(float v) {
-    v = fmaxf(v, dpp_f<kQuadSwap1>(v));
-    v = fmaxf(v, dpp_f<kQuadSwap2>(v));
-    v = fmaxf(v, dpp_f<kHalfMirror>(v));
-    v = fmaxf(v, dpp_f<kRowMirror>(v));
-    const float lo = fmaxf(readlane_f(v, 0), readlane_f(v, 16)), hi = fmaxf(readlane_f(v, 32), readlane_f(v, 48));
-    return (threadIdx.x & 32) ? hi : lo;
+// Maxima over the two halves of the wave (lanes 0..31 and 32..63) of non-negative floats, as two
+// wave-uniform values.  Non-negative floats order like their bit patterns, so the steps are single
+// integer max instructions with a DPP operand.
+__device__ __forceinline__ void half_max_bits(uint32_t v, uint32_t &lo, uint32_t &hi) {
+    v = max(v, (uint32_t)dpp_i<kQuadSwap1>((int)v));
+    v = max(v, (uint32_t)dpp_i<kQuadSwap2>((int)v));
+    v = max(v, (uint32_t)dpp_i<kHalfMirror>((int)v));
+    v = max(v, (uint32_t)dpp_i<kRowMirror>((int)v));
+    lo = max((uint32_t)__builtin_amdgcn_readlane((int)v, 0), (uint32_t)__builtin_amdgcn_readlane((int)v, 16));
+    hi = max((uint32_t)__builtin_amdgcn_readlane((int)v, 32), (uint32_t)__builtin_amdgcn_readlane((int)v, 48));
+}
+// max / min of three floats in one instruction (NaN operands lose against numbers)
+__device__ __forceinline__ float max3f(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+__device__ __forceinline__ float min3f(float a, float b, float c) {
+    float r;
+    asm("v_min3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
 }
 __device__ __forceinline__ int half_min_i(int v) {
     v = min(v, dpp_i<kQuadSwap1>(v));
@@ -254,45 +267,66 @@ __device__ __forceinline__ int half_min_i(int v) {
     return (threadIdx.x & 32) ? hi : lo;
 }
 
+// Low bytes of four integers as one word.
+__device__ __forceinline__ uint32_t pack4i(int a, int b, int c, int d) {
+    const uint32_t lo = __builtin_amdgcn_perm((uint32_t)b, (uint32_t)a, 0x0c0c0400u);
+    const uint32_t hi = __builtin_amdgcn_perm((uint32_t)d, (uint32_t)c, 0x0c0c0400u);
+    return __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+}
+
 template <int DT>
 __device__ __forceinline__ void quantize_pair_to_lds(uint8_t *smem, const X8 &fin, int c, bool chunk_ok,
                                                      const LdsRow r, uint32_t units) {
     const int lane = threadIdx.x & 63, hl = lane & 31;
-    float v[8] = {fin.a.x, fin.a.y, fin.a.z, fin.a.w, fin.b.x, fin.b.y, fin.b.z, fin.b.w};
-    float av[8];
-    float amax = 0.0f;
+    const float v[8] = {fin.a.x, fin.a.y, fin.a.z, fin.a.w, fin.b.x, fin.b.y, fin.b.z, fin.b.w};
+    // magnitude of the lane's largest positive and largest negative value (zero if it has none), then
+    // of the chunk (an out-of-range chunk goes through the arithmetic on the bytes of chunk 0; nothing
+    // of it is stored)
+    const float vmax = max3f(max3f(v[0], v[1], v[2]), max3f(v[3], v[4], v[5]), max3f(v[6], v[7], v[7]));
+    const float vmin = min3f(min3f(v[0], v[1], v[2]), min3f(v[3], v[4], v[5]), min3f(v[6], v[7], v[7]));
+    const uint32_t pbits = (uint32_t)max(__builtin_bit_cast(int, vmax), 0);
+    const uint32_t nbits = (uint32_t)max(__builtin_bit_cast(int, vmin) ^ (int)0x80000000, 0);
+    uint32_t a_lo, a_hi;
+    half_max_bits(max(pbits, nbits), a_lo, a_hi);
+    const bool upper = (lane & 32) != 0;
+    const uint32_t abits = upper ? a_hi : a_lo;
+    // The first element of the chunk whose |x| equals the maximum decides the sign of the scale.
+    // Unless the maximum occurs with both signs that is simply the sign it occurs with; all of this
+    // is wave-uniform (scalar) work on the two lane masks.
+    const uint64_t pos_hit = __builtin_amdgcn_ballot_w64(pbits == abits);
+    const uint64_t neg_hit = __builtin_amdgcn_ballot_w64(nbits == abits);
+    const bool pos_lo = (uint32_t)pos_hit != 0, pos_hi = (uint32_t)(pos_hit >> 32) != 0;
+    const bool neg_lo = (uint32_t)neg_hit != 0, neg_hi = (uint32_t)(neg_hit >> 32) != 0;
+    const uint32_t m_lo = a_lo | (neg_lo ? 0x80000000u : 0u), m_hi = a_hi | (neg_hi ? 0x80000000u : 0u);
+    uint32_t mbits = upper ? m_hi : m_lo;
+    if ((pos_lo && neg_lo && a_lo != 0) || (pos_hi && neg_hi && a_hi != 0)) {
+        // both signs in one of the chunks: search the first index the long way
+        int idx = 0x7fffffff;
+        float cand = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        if (!chunk_ok) v[i] = 0.0f;
-        av[i] = fabsf(v[i]);
-        amax = fmaxf(amax, av[i]);
+        for (int i = 7; i >= 0; i--) {
+            if ((__builtin_bit_cast(uint32_t, v[i]) & 0x7fffffffu) == abits) { idx = 8 * hl + i; cand = v[i]; }
+        }
+        idx = half_min_i(idx);
+        const int src_lo = (__builtin_amdgcn_readlane(idx, 0) >> 3) & 31;
+        const int src_hi = 32 + ((__builtin_amdgcn_readlane(idx, 32) >> 3) & 31);
+        const float max_lo = readlane_f(cand, src_lo), max_hi = readlane_f(cand, src_hi);
+        mbits = __builtin_bit_cast(uint32_t, upper ? max_hi : max_lo);
     }
-    amax = half_max(amax);
-    // the first element of the chunk whose |x| equals the maximum decides the sign of the scale
-    int idx = 0x7fffffff;
-    float cand = 0.0f;
-#pragma unroll
-    for (int i = 7; i >= 0; i--) {
-        if (av[i] == amax) { idx = 8 * hl + i; cand = v[i]; }
-    }
-    idx = half_min_i(idx);
-    const int src_lo = (__builtin_amdgcn_readlane(idx, 0) >> 3) & 31;
-    const int src_hi = 32 + ((__builtin_amdgcn_readlane(idx, 32) >> 3) & 31);
-    const float max_lo = readlane_f(cand, src_lo), max_hi = readlane_f(cand, src_hi);
-    const float max = (lane & 32) ? max_hi : max_lo;
+    const float max = __builtin_bit_cast(float, mbits);
     uint32_t w0 = 0, w1 = 0;
     int sum = 0;
     float d = 0.0f;
-    if (amax != 0.0f) {
+    if (abits != 0) {
         const float iscale = -128.0f / max;
-        int8_t q[8];
+        int q[8];
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            q[i] = cq_as_i8(fminf(roundf(iscale * v[i]), 127.0f));
-            sum += (int)q[i];
+            q[i] = min(cq_round_away_i32(iscale * v[i]), 127);
+            sum += q[i];
         }
-        w0 = pack4(q[0], q[1], q[2], q[3]);
-        w1 = pack4(q[4], q[5], q[6], q[7]);
+        w0 = pack4i(q[0], q[1], q[2], q[3]);
+        w1 = pack4i(q[4], q[5], q[6], q[7]);
         d = 1.0f / iscale;
     }
     sum += dpp_i<kQuadSwap1>(sum);   // two lanes = one 16-element group
@@ -353,25 +387,44 @@ template <int DT> struct UnitRaw {
     uint16_t d;    // Q4_0 / Q8_0 / Q6K: f16 scale
 };
 
-template <int DT>
-__device__ __forceinline__ void load_unit(const cq_weight &w, int64_t row, int64_t units, int64_t u, UnitRaw<DT> &o) {
-    const int64_t g = row * units + u;
+// Plane pointers of one weight row (wave-uniform: they stay in scalar registers and the loads take
+// them as scalar base plus a 32-bit lane offset, without 64-bit vector address arithmetic).
+struct RowPtr {
+    const uint8_t *p0, *p1, *p2, *p3;
+};
+template <int DT> __device__ __forceinline__ RowPtr row_ptr(const cq_weight &w, int64_t row, uint32_t units) {
+    constexpr int kB = Geo<DT>::kUnitsPerBlock;
+    const int64_t g0 = row * units;   // units per row is a multiple of the units per block
+    RowPtr rp;
+    rp.p0 = w.p0 + g0 * (DT == CQ_DTYPE_Q4K ? 32 : 16);
+    rp.p1 = w.p1 + (DT == CQ_DTYPE_Q4K ? (g0 / kB) * CQ_Q4K_HDR : DT == CQ_DTYPE_Q6K ? g0 * 8 : DT == CQ_DTYPE_Q4_0 ? g0 * 2 : g0);
+    rp.p2 = DT == CQ_DTYPE_Q6K ? w.p2 + g0 * 2 : nullptr;
+    rp.p3 = DT == CQ_DTYPE_Q6K ? w.p3 + (g0 / kB) * 2 : nullptr;
+    return rp;
+}
+
+template <int DT> __device__ __forceinline__ void load_unit(const RowPtr &rp, uint32_t u, UnitRaw<DT> &o) {
     if (DT == CQ_DTYPE_Q4K) {
-        o.q = *(const uint4 *)(w.p0 + g * 32);
-        o.q2 = *(const uint4 *)(w.p0 + g * 32 + 16);
-        const uint32_t *h = (const uint32_t *)(w.p1 + (g >> 2) * CQ_Q4K_HDR);
-        o.h.x = h[0];
-        o.h.y = h[1 + (g & 3)];   // units per row is a multiple of 4, so g & 3 == u & 3
+        o.q = *(const uint4 *)(rp.p0 + u * 32u);
+        o.q2 = *(const uint4 *)(rp.p0 + u * 32u + 16u);
+        const uint8_t *h = rp.p1 + (u >> 2) * (uint32_t)CQ_Q4K_HDR;
+        o.h.x = *(const uint32_t *)h;
+        o.h.y = *(const uint32_t *)(h + 4u + (u & 3u) * 4u);
         return;
     }
-    o.q = *(const uint4 *)(w.p0 + g * 16);
-    if (DT == CQ_DTYPE_Q4_0) o.d = ((const uint16_t *)w.p1)[g];
-    if (DT == CQ_DTYPE_Q8_0) o.d = ((const uint16_t *)w.p1)[g >> 1];
+    o.q = *(const uint4 *)(rp.p0 + u * 16u);
+    if (DT == CQ_DTYPE_Q4_0) o.d = *(const uint16_t *)(rp.p1 + u * 2u);
+    if (DT == CQ_DTYPE_Q8_0) o.d = *(const uint16_t *)(rp.p1 + (u >> 1) * 2u);
     if (DT == CQ_DTYPE_Q6K) {
-        o.hh = *(const uint2 *)(w.p1 + g * 8);
-        o.sc2 = ((const uint16_t *)w.p2)[g];
-        o.d = ((const uint16_t *)w.p3)[g >> 3];
+        o.hh = *(const uint2 *)(rp.p1 + u * 8u);
+        o.sc2 = *(const uint16_t *)(rp.p2 + u * 2u);
+        o.d = *(const uint16_t *)(rp.p3 + (u >> 3) * 2u);
     }
+}
+
+template <int DT>
+__device__ __forceinline__ void load_unit(const cq_weight &w, int64_t row, int64_t units, int64_t u, UnitRaw<DT> &o) {
+    load_unit<DT>(row_ptr<DT>(w, row, (uint32_t)units), (uint32_t)u, o);
 }
 
 __device__ __forceinline__ int dot16(const uint32_t w[4], const int4 &a) {
@@ -486,12 +539,13 @@ template <int DT, int UPL>
 __device__ __forceinline__ void load_row(const cq_weight &w, int64_t row, uint32_t units, UnitRaw<DT> (&buf)[UPL]) {
     const uint32_t lane = threadIdx.x & 63;
     constexpr uint32_t kB = Geo<DT>::kUnitsPerBlock;
+    const RowPtr rp = row_ptr<DT>(w, row, units);
 #pragma unroll
     for (int c = 0; c < UPL; c++) {
         const uint32_t u = c * 64 + lane;
         // keep the lane's position in its block when clamping (rows hold whole blocks)
         const uint32_t uc = u < units ? u : (units - kB + (lane & (kB - 1)));
-        load_unit<DT>(w, row, units, uc, buf[c]);
+        load_unit<DT>(rp, uc, buf[c]);
     }
 }
 
@@ -565,10 +619,19 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
         int64_t i = 0;
         // steady state: rows i and i+1 are in a and b, rows i+2 and i+3 exist
         for (; i + 3 < cnt; i += 2) {
-            const float s0 = row_dot<DT, UPL>(smem, r, units, a);
+            // the refill of a buffer is issued before the arithmetic on its old contents (which move
+            // to other registers), so a wave keeps up to three rows in flight
+            UnitRaw<DT> ta[UPL], tb[UPL];
+#pragma unroll
+            for (int c = 0; c < UPL; c++) ta[c] = a[c];
             load_row<DT, UPL>(w, row0 + (i + 2) * T, units, a);
-            const float s1 = row_dot<DT, UPL>(smem, r, units, b);
+            __builtin_amdgcn_sched_barrier(0);
+            const float s0 = row_dot<DT, UPL>(smem, r, units, ta);
+#pragma unroll
+            for (int c = 0; c < UPL; c++) tb[c] = b[c];
             load_row<DT, UPL>(w, row0 + (i + 3) * T, units, b);
+            __builtin_amdgcn_sched_barrier(0);
+            const float s1 = row_dot<DT, UPL>(smem, r, units, tb);
             if (lane == 0) { y[row0 + i * T] = s0; y[row0 + (i + 1) * T] = s1; }
         }
         // tail: two or three rows left (a = row i, b = row i+1, maybe row i+2 still to load)

@@ -176,6 +176,16 @@ __device__ __forceinline__ int8_t cq_as_i8(float v) {
     const int32_t r = cq_as_i32(v);
     return (int8_t)(r < -128 ? -128 : (r > 127 ? 127 : r));
 }
+// round(t) (half away from zero) as an integer, for |t| <= 130: v_cvt_rpi_i32_f32 is floor(|t| + 0.5)
+// computed exactly (no rounded intermediate sum; checked against the exact value for every float
+// in [0, 130] by cq_selfcheck_round), the sign goes back on in integers.
+__device__ __forceinline__ int cq_round_away_i32(float t) {
+    int m;
+    asm("v_cvt_rpi_i32_f32_e64 %0, |%1|" : "=v"(m) : "v"(t));
+    const int sgn = __builtin_bit_cast(int, t) >> 31;
+    return (m ^ sgn) - sgn;
+}
+
 __device__ __forceinline__ uint8_t cq_as_u8(float v) {
     uint32_t r;
     asm("v_cvt_u32_f32_e32 %0, %1" : "=v"(r) : "v"(v));

@@ -25,6 +25,7 @@ EXPORTS = [
     "cq_weight_device", "cq_weight_shape", "cq_weight_destroy", "cq_act_bytes", "cq_quantize_act",
     "cq_workspace_bytes", "cq_qmatmul", "cq_qmatmul_int_dots", "cq_grouped_workspace_bytes",
     "cq_qmatmul_grouped", "cq_silu_mul", "cq_moe_scatter_add", "cq_timing_arm", "cq_timing_elapsed_us",
+    "cq_selfcheck_round",
 ]
 
 
@@ -73,6 +74,7 @@ def load():
     L.cq_moe_scatter_add.argtypes = [ci, vp, vp, vp, i64, i64, vp, i64, vp]
     L.cq_timing_arm.argtypes = []
     L.cq_timing_elapsed_us.argtypes = [C.POINTER(C.c_double)]
+    L.cq_selfcheck_round.argtypes = [ci, C.POINTER(C.c_uint64)]
     _lib = L
     return L
 

@@ -153,6 +153,14 @@ int cq_moe_scatter_add(int dev, const float *y_dev, const int32_t *row_ids_dev, 
 int cq_timing_arm(void);
 int cq_timing_elapsed_us(double *us);
 
+/* ---- hardware self-check (no counterpart in the reference) -------------------------------------
+ * The activation quantizers round with `f32::round` (half away from zero; k_quants.rs:605, :1812).
+ * On the device that is one conversion instruction (floor(|t| + 0.5) without an intermediate
+ * rounding) plus the sign.  This call compares it with round-half-away computed the long way for
+ * every f32 t with |t| <= 130 (both signs, denormals included) and stores the number of
+ * mismatches, which must be zero on any device the library is used on. */
+int cq_selfcheck_round(int dev, uint64_t *mismatches);
+
 #ifdef __cplusplus
 }
 #endif

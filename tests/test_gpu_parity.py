@@ -187,6 +187,42 @@ def test_fused_decode_equals_two_launch_path(qh, dt, k, n):
     assert torch.equal(qh.qmatmul(qw, dev(x)), torch.zeros((1, n), device="cuda"))
 
 
+@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K])
+def test_fused_decode_sign_of_scale_cases(qh, dt):
+    """The Q8K scale takes the sign of the FIRST element with the largest magnitude.  Blocks where
+    that magnitude occurs with both signs (negative first, positive first, in the same eight
+    elements, in either half of a wave's pair of blocks), with one sign only, all-zero blocks beside
+    non-zero ones, and values that round at a tie: the one-launch decode path must still equal the
+    stand-alone quantizer plus matvec bit for bit, and that quantizer the oracle."""
+    k, n = 2048, 64
+    w, x = make_inputs(77 + dt, 1, k, n)
+    x[0] = np.round(x[0] * 8) / 8                       # many products land on exact .5 ties
+    big = np.float32(9.5)
+    x[0, 0 * 256 + 200], x[0, 0 * 256 + 17] = big, -big          # block 0: negative first
+    x[0, 1 * 256 + 3], x[0, 1 * 256 + 250] = big, -big           # block 1 (upper half-wave): positive first
+    x[0, 2 * 256 + 8], x[0, 2 * 256 + 9] = -big, big             # block 2: both inside one lane's eight
+    x[0, 3 * 256 + 100] = -big                                   # block 3: negative only
+    x[0, 4 * 256:5 * 256] = 0.0                                  # block 4: all zero, block 5 not
+    x[0, 6 * 256:7 * 256] = -0.0                                 # block 6: all minus zero
+    x[0, 7 * 256 + 255] = big                                    # block 7: positive only, last element
+    xd = dev(x)
+    got = qh.quantize_act(orc.Q8K, xd).cpu().numpy()
+    want = orc.quantize(orc.Q8K, x[0])
+    assert got.size == want.size and np.array_equal(got, want)
+    qw = qh.QWeight.from_ggml(dt, orc.quantize(dt, w), n, k)
+    fused = qh.qmatmul(qw, xd)
+    assert torch.equal(fused, qh.qmatmul(qw, xd, qh.FLAG_STAGED_ACT))
+    check_f32(fused.cpu().numpy(), orc.matmul(dt, x, orc.quantize(dt, w), n))
+
+
+def test_rounding_instruction_selfcheck(qh):
+    """Every f32 in [-130, 130]: the device's one-instruction rounding equals round-half-away."""
+    import ctypes as C
+    bad = C.c_uint64(123)
+    qh.check(qh.load().cq_selfcheck_round(0, C.byref(bad)))
+    assert bad.value == 0
+
+
 @pytest.mark.parametrize("dt", [orc.Q4K, orc.Q8_0])
 @pytest.mark.parametrize("m", [2, 4, 8, 16])
 @pytest.mark.parametrize("k,n", [(4096, 4096), (4096, 11008)])
