@@ -621,17 +621,25 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
         for (; i + 3 < cnt; i += 2) {
             // the refill of a buffer is issued before the arithmetic on its old contents (which move
             // to other registers), so a wave keeps up to three rows in flight
-            UnitRaw<DT> ta[UPL], tb[UPL];
+            float s0, s1;
+            if constexpr (UPL <= 2) {
+                UnitRaw<DT> ta[UPL], tb[UPL];
 #pragma unroll
-            for (int c = 0; c < UPL; c++) ta[c] = a[c];
-            load_row<DT, UPL>(w, row0 + (i + 2) * T, units, a);
-            __builtin_amdgcn_sched_barrier(0);
-            const float s0 = row_dot<DT, UPL>(smem, r, units, ta);
+                for (int c = 0; c < UPL; c++) ta[c] = a[c];
+                load_row<DT, UPL>(w, row0 + (i + 2) * T, units, a);
+                __builtin_amdgcn_sched_barrier(0);
+                s0 = row_dot<DT, UPL>(smem, r, units, ta);
 #pragma unroll
-            for (int c = 0; c < UPL; c++) tb[c] = b[c];
-            load_row<DT, UPL>(w, row0 + (i + 3) * T, units, b);
-            __builtin_amdgcn_sched_barrier(0);
-            const float s1 = row_dot<DT, UPL>(smem, r, units, tb);
+                for (int c = 0; c < UPL; c++) tb[c] = b[c];
+                load_row<DT, UPL>(w, row0 + (i + 3) * T, units, b);
+                __builtin_amdgcn_sched_barrier(0);
+                s1 = row_dot<DT, UPL>(smem, r, units, tb);
+            } else {
+                s0 = row_dot<DT, UPL>(smem, r, units, a);
+                load_row<DT, UPL>(w, row0 + (i + 2) * T, units, a);
+                s1 = row_dot<DT, UPL>(smem, r, units, b);
+                load_row<DT, UPL>(w, row0 + (i + 3) * T, units, b);
+            }
             if (lane == 0) { y[row0 + i * T] = s0; y[row0 + (i + 1) * T] = s1; }
         }
         // tail: two or three rows left (a = row i, b = row i+1, maybe row i+2 still to load)
