@@ -41,12 +41,6 @@ extern "C" const char *cq_last_error(void) { return g_err; }
 extern "C" const char *cq_version(void) { return "candle_qhip 0.1 (gfx950)"; }
 
 extern "C" int cq_device_count(void) {
-    static bool env_read = false;
-    if (!env_read) {  // A/B switch for tuning runs: waves per workgroup of the fused decode kernel
-        env_read = true;
-        const char *e = getenv("CQ_MATVEC_WAVES");
-        if (e && *e) cq_matvec_set_waves(atoi(e));
-    }
     int n = 0;
     if (hipGetDeviceCount(&n) != hipSuccess) {
         (void)hipGetLastError();

@@ -11,13 +11,17 @@
 // with DPP.  Quantized activations sit in LDS, permuted so that lane l of a chunk reads its
 // operands at l * 16 bytes (no bank conflicts).
 //
-// Two kernels:
-//   fused_kernel  (m == 1): one launch per QMatMul call.  Each wave first issues the loads of its
-//       first weight row, then the workgroup quantizes the f32 activation row into LDS
+// Kernels:
+//   fused_kernel   (m == 1): one launch per QMatMul call.  Each wave first issues the loads of its
+//       first weight rows, then the workgroup quantizes the f32 activation row into LDS
 //       (BlockQ8K / BlockQ8_0::from_float, bit-identical to quantize_act.hip), then rows are
 //       processed with the next row's loads in flight (register double buffering).
-//   staged_kernel (m <= 4 rows per launch): activations come from the workspace written by the
-//       stand-alone quantizer.
+//   batched_kernel (2..8 rows per pass): the same persistent structure with the quantized rows
+//       copied from the workspace of the stand-alone quantizer; a weight unit is unpacked once for
+//       all rows.
+//   staged_kernel  (up to 4 rows per launch): the simple fallback for rows too long for the LDS
+//       budget of the above.
+//   int_dots_kernel: the per-block integers of the dot products, for the bit-exactness test.
 #include "qhip_internal.h"
 
 namespace {
@@ -816,9 +820,6 @@ int num_cus() {
     return g_num_cus;
 }
 
-bool g_no_batched = false;   // A/B switch: rows of up to four on the simple kernel only
-int g_fused_wgs_per_cu = 0;  // 0 = automatic; A/B switch (CQ_MATVEC_WAVES = workgroups per CU)
-
 // Eight waves per workgroup, one workgroup per CU.  Whole workgroups only, and every wave
 // gets at least `depth` rows: wgs * 8 * depth <= n.
 template <int DT, int UPL>
@@ -827,8 +828,7 @@ hipError_t launch_fused_upl(const cq_weight *w, const float *x, float *y, hipStr
     const size_t lds = lds_row_bytes<DT>(w->k);
     // every workgroup quantizes the whole activation row, so fewer, longer-lived workgroups win: one
     // per CU measured faster than two on every decode shape (11008 x 4096 Q4K: 7.0 us against 7.6 us)
-    const int per_cu = g_fused_wgs_per_cu > 0 ? g_fused_wgs_per_cu : 1;
-    const int64_t max_wgs = (int64_t)num_cus() * per_cu;
+    const int64_t max_wgs = num_cus();
     int depth = UPL <= 2 ? 2 : 1;
     if (w->n < NW * 2) depth = 1;
     if (w->n < NW) {  // fewer rows than one workgroup's waves: the two-launch path handles it
@@ -901,7 +901,7 @@ bool batched_ok(const cq_weight *w, int mb) {
 
 template <int DT>
 hipError_t launch_staged(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
-    if (m >= 2 && !g_no_batched) {
+    if (m >= 2) {
         int64_t m0 = 0;
         bool done = true;
         while (m0 < m) {
@@ -949,8 +949,6 @@ hipError_t launch_ints(const cq_weight *w, cq_act_view a, int64_t m, int32_t *oi
 }
 
 }  // namespace
-
-void cq_matvec_set_waves(int nw) { g_no_batched = nw >= 100; g_fused_wgs_per_cu = nw % 100; }
 
 bool cq_matvec_fused_supported(const cq_weight *w) {
     switch (w->dtype) {

@@ -101,7 +101,6 @@ hipError_t cq_launch_int_dots(const cq_weight *w, cq_act_view a, int64_t m, int3
                               hipStream_t s);
 bool cq_matvec_fused_supported(const cq_weight *w);   // m == 1: quantizer fused into the matvec launch
 hipError_t cq_launch_matvec_fused(const cq_weight *w, const float *x, float *y, hipStream_t s);
-void cq_matvec_set_waves(int nw);                     // A/B switch: waves per workgroup of the fused kernel
 // gemm.hip
 bool cq_gemm_supported(const cq_weight *w, int64_t m, int act_dtype);
 hipError_t cq_launch_gemm(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s);
