@@ -169,6 +169,29 @@ def test_matvec_matches_oracle(qh, dt, m, k, n):
     check_f32(got, orc.matmul(dt, x, blocks, n))
 
 
+@pytest.mark.parametrize("dt,k,n", [(orc.Q6K, 4096, 32000), (orc.Q6K, 11008, 4096), (orc.Q4K, 4096, 11008),
+                                     (orc.Q4K, 14336, 4096)])
+def test_decode_full_size_row_samples(qh, dt, k, n):
+    """The largest decode shapes of the configurations at their full size (lm_head, down and gate/up
+    projections, an expert's w2-shaped tensor).  Weights are quantized on the device (bit-exact with
+    the oracle's quantizer, checked above); the oracle then recomputes blocks of rows taken from the
+    start, the middle and the end of the result out of the very same GGML bytes, and every row of the
+    one-launch path must equal the two-launch path bit for bit."""
+    rng = np.random.default_rng(dt * 7 + k)
+    w = torch.randn((n, k), device="cuda", generator=torch.Generator(device="cuda").manual_seed(dt + n)) * 0.02
+    qw = qh.QWeight.zeros(dt, n, k).quantize_(w)
+    del w
+    x = rng.standard_normal((1, k)).astype(np.float32)
+    xd = dev(x)
+    y = qh.qmatmul(qw, xd)
+    assert torch.equal(y, qh.qmatmul(qw, xd, qh.FLAG_STAGED_ACT))
+    got = y.cpu().numpy()
+    blocks = qw.to_ggml().reshape(n, -1)
+    for r0 in (0, n // 2 - 32, n - 64):
+        rows = blocks[r0:r0 + 64].reshape(-1)
+        check_f32(got[:, r0:r0 + 64], orc.matmul(dt, x, rows, 64))
+
+
 @pytest.mark.parametrize("dt", WEIGHT_DTYPES)
 @pytest.mark.parametrize("k,n", [(256, 7), (512, 300), (4096, 1000), (11008, 129), (14336, 65)])
 def test_fused_decode_equals_two_launch_path(qh, dt, k, n):
