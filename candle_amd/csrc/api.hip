@@ -182,6 +182,7 @@ extern "C" int cq_weight_quantize(cq_weight *w, const float *src_dev, void *stre
 
 extern "C" int cq_weight_dequantize(const cq_weight *w, float *dst_dev, void *stream) {
     if (!w || !dst_dev) return cq_set_error(CQ_ERR_INVALID, "null argument");
+    if ((uintptr_t)dst_dev & 15) return cq_set_error(CQ_ERR_INVALID, "dst must be 16-byte aligned");
     CQ_HIP_CHECK(hipSetDevice(w->dev));
     CQ_HIP_CHECK(cq_launch_dequantize(w, dst_dev, nullptr, (hipStream_t)stream));
     return CQ_OK;
@@ -189,6 +190,7 @@ extern "C" int cq_weight_dequantize(const cq_weight *w, float *dst_dev, void *st
 
 extern "C" int cq_weight_dequantize_f16(const cq_weight *w, uint16_t *dst_dev, void *stream) {
     if (!w || !dst_dev) return cq_set_error(CQ_ERR_INVALID, "null argument");
+    if ((uintptr_t)dst_dev & 15) return cq_set_error(CQ_ERR_INVALID, "dst must be 16-byte aligned");
     CQ_HIP_CHECK(hipSetDevice(w->dev));
     CQ_HIP_CHECK(cq_launch_dequantize(w, nullptr, dst_dev, (hipStream_t)stream));
     return CQ_OK;

@@ -9,9 +9,22 @@
 
 namespace {
 
+// Sixteen consecutive results starting at element i (a multiple of 16): 64 or 32 bytes in
+// 16-byte stores.
 template <bool F16>
-__device__ __forceinline__ void put(float *d32, uint16_t *d16, int64_t i, float v) {
-    if (F16) d16[i] = cq_f2h(v); else d32[i] = v;
+__device__ __forceinline__ void put16(float *d32, uint16_t *d16, int64_t i, const float (&v)[16]) {
+    if (F16) {
+        uint32_t w[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) w[j] = (uint32_t)cq_f2h(v[2 * j]) | ((uint32_t)cq_f2h(v[2 * j + 1]) << 16);
+        uint4 *dst = (uint4 *)(d16 + i);
+        dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
+        dst[1] = make_uint4(w[4], w[5], w[6], w[7]);
+    } else {
+        float4 *dst = (float4 *)(d32 + i);
+#pragma unroll
+        for (int j = 0; j < 4; j++) dst[j] = make_float4(v[4 * j], v[4 * j + 1], v[4 * j + 2], v[4 * j + 3]);
+    }
 }
 
 template <bool F16>
@@ -22,13 +35,16 @@ __global__ void dequant_q4_0(const uint8_t *__restrict__ qs, const uint16_t *__r
     const uint4 q = *(const uint4 *)(qs + b * 16);
     const float d = cq_h2f(dpl[b]);
     const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+    float lo[16], hi[16];
 #pragma unroll
     for (int j = 0; j < 16; j++) {
         const uint32_t byte = (w[j >> 2] >> (8 * (j & 3))) & 0xff;
         const int x0 = (int)(byte & 0xF) - 8, x1 = (int)(byte >> 4) - 8;
-        put<F16>(d32, d16, b * 32 + j, (float)x0 * d);
-        put<F16>(d32, d16, b * 32 + j + 16, (float)x1 * d);
+        lo[j] = (float)x0 * d;
+        hi[j] = (float)x1 * d;
     }
+    put16<F16>(d32, d16, b * 32, lo);
+    put16<F16>(d32, d16, b * 32 + 16, hi);
 }
 
 template <bool F16>
@@ -39,11 +55,13 @@ __global__ void dequant_q8_0(const uint8_t *__restrict__ qs, const uint16_t *__r
     const uint4 q = *(const uint4 *)(qs + u * 16);
     const float d = cq_h2f(dpl[u >> 1]);
     const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+    float out[16];
 #pragma unroll
     for (int j = 0; j < 16; j++) {
         const int8_t v = (int8_t)((w[j >> 2] >> (8 * (j & 3))) & 0xff);
-        put<F16>(d32, d16, u * 16 + j, (float)v * d);
+        out[j] = (float)v * d;
     }
+    put16<F16>(d32, d16, u * 16, out);
 }
 
 template <bool F16>
@@ -63,12 +81,15 @@ __global__ void dequant_q4k(const uint8_t *__restrict__ qs, const uint8_t *__res
     const float d2 = d * (float)sc2, mm2 = dmin * (float)m2;
     const uint32_t w[4] = {q.x, q.y, q.z, q.w};
     const int64_t base = b * 256 + 64 * g + 16 * half;
+    float lo[16], hi[16];
 #pragma unroll
     for (int j = 0; j < 16; j++) {
         const uint32_t byte = (w[j >> 2] >> (8 * (j & 3))) & 0xff;
-        put<F16>(d32, d16, base + j, d1 * (float)(byte & 0xF) - mm1);
-        put<F16>(d32, d16, base + 32 + j, d2 * (float)(byte >> 4) - mm2);
+        lo[j] = d1 * (float)(byte & 0xF) - mm1;
+        hi[j] = d2 * (float)(byte >> 4) - mm2;
     }
+    put16<F16>(d32, d16, base, lo);
+    put16<F16>(d32, d16, base + 32, hi);
 }
 
 template <bool F16>
@@ -87,6 +108,7 @@ __global__ void dequant_q6k(const uint8_t *__restrict__ ql, const uint8_t *__res
     const uint32_t w[4] = {q.x, q.y, q.z, q.w};
     const uint32_t hw[2] = {hh.x, hh.y};
     const int64_t base = b * 256 + 128 * h + 32 * t + i0;
+    float lo[16], hi[16];
 #pragma unroll
     for (int e = 0; e < 16; e++) {
         const int wi = e >> 2, c = e & 3;
@@ -95,9 +117,11 @@ __global__ void dequant_q6k(const uint8_t *__restrict__ ql, const uint8_t *__res
         const int sh = (wi & 1) * 4;
         const int q_lo = (int)((byte & 0xF) | (((hb >> sh) & 3) << 4)) - 32;
         const int q_hi = (int)((byte >> 4) | (((hb >> (sh + 2)) & 3) << 4)) - 32;
-        put<F16>(d32, d16, base + e, d * s_lo * (float)q_lo);
-        put<F16>(d32, d16, base + 64 + e, d * s_hi * (float)q_hi);
+        lo[e] = d * s_lo * (float)q_lo;
+        hi[e] = d * s_hi * (float)q_hi;
     }
+    put16<F16>(d32, d16, base, lo);
+    put16<F16>(d32, d16, base + 64, hi);
 }
 
 template <bool F16>

@@ -88,7 +88,8 @@ int cq_weight_zeros(int dev, int ggml_dtype, int64_t n, int64_t k, cq_weight **o
  * reference copies to the host and runs T::from_float there; here the same arithmetic runs in
  * a HIP kernel and yields the same bytes. */
 int cq_weight_quantize(cq_weight *w, const float *src_dev, void *stream);
-/* QCudaStorage::dequantize / dequantize_f16 (cuda.rs:391-446): dst has n*k elements. */
+/* QCudaStorage::dequantize / dequantize_f16 (cuda.rs:391-446): dst has n*k elements and is
+ * 16-byte aligned (the kernels store whole 16-byte groups). */
 int cq_weight_dequantize(const cq_weight *w, float *dst_dev, void *stream);
 int cq_weight_dequantize_f16(const cq_weight *w, uint16_t *dst_dev, void *stream);
 /* Inverse re-pack: the exact GGML bytes back on the host (QStorage::data, mod.rs:118-130; what
