@@ -491,3 +491,22 @@ def test_moe_ffn_matches_oracle(qh, tokens, starve):
     assert np.array_equal(ys, acc)
     # end to end: only as loose as the re-quantization effect described above
     assert np.linalg.norm(ys - want) / np.linalg.norm(want) < 5e-3
+
+
+@pytest.mark.parametrize("tokens,total,hidden", [(5, 9, 6), (7, 200, 8), (64, 128, 4096), (3, 70, 1028), (4, 0, 16)])
+def test_moe_scatter_add_order_and_shapes(qh, tokens, total, hidden):
+    """ys[row_ids[p]] += weights[p] * y[p] for p in increasing order (cpu_backend/mod.rs:619-653): both
+    kernels (hidden a multiple of 4 or not), more rows than one 64-row search step, tokens that
+    receive nothing, no rows at all.  Sums are compared bit for bit with the same sequential loop."""
+    rng = np.random.default_rng(tokens * 1000 + total)
+    y = rng.standard_normal((total, hidden)).astype(np.float32)
+    rid = rng.integers(0, max(tokens - 1, 1), size=total).astype(np.int32)     # the last token gets no row
+    wt = rng.random(total).astype(np.float32)
+    want = np.zeros((tokens, hidden), np.float32)
+    for p in range(total):
+        want[rid[p]] = want[rid[p]] + y[p] * wt[p]
+    y_d = dev(y) if total else torch.zeros((0, hidden), device="cuda")
+    rid_d = dev(rid) if total else torch.zeros((0,), dtype=torch.int32, device="cuda")
+    wt_d = dev(wt) if total else torch.zeros((0,), device="cuda")
+    got = qh.moe_scatter_add(y_d, rid_d, wt_d, tokens).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
