@@ -25,6 +25,8 @@
 // touched - and the 16-byte chunks of a row are XOR-swizzled by the row number on the way in, so
 // that the MFMA operand reads (lanes = rows, one chunk column) spread over all LDS banks.  With few
 // workgroups (small n) K is split over blockIdx.z and the partial results are added atomically.
+#include <type_traits>
+
 #include "qhip_internal.h"
 
 namespace {
@@ -180,7 +182,7 @@ __device__ __forceinline__ void load_head(const cq_weight &w, int64_t blk, WHead
 // LDS reads run two steps ahead.  The accumulator pair alternates between two register sets.  A
 // scheduling barrier after every step keeps the compiler from hoisting all MFMAs to the front,
 // which would need MT accumulator sets at once.
-template <int DT, int MT, int T0, int T1, int SHIFT>
+template <int DT, int MT, int T0, int T1, int SHIFT, bool HALF>
 __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, const v4i (&bl)[8], const v4i (&bh)[8],
                                           float dw, v8h wmin, int lane, v16f (&out)[MT]) {
     typedef Tile<DT, MT> T;
@@ -235,6 +237,7 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, 
             if ((s & 1) == 0 && s < 6) dreg[((s >> 1) + 1) & 1] = *(const v4f *)(d8p + ((t - 1) * 32 + 8 * ((s >> 1) + 1)) * 4);
 #pragma unroll
             for (int i = 2 * s; i < 2 * s + 2; i++) {
+                if (HALF && i >= 8) continue;   // rows 16..31 of the tile are not wanted
                 const int I = (acc_hi[p][i] << SHIFT) + acc_lo[p][i];
                 float o = __builtin_fmaf((float)I * dw, dreg[(i >> 2) & 1][i & 3], out[t - 1][i]);
                 asm volatile("" : "+v"(o));   // pins the scaling to this step (pure ops float otherwise)
@@ -329,7 +332,7 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g
 // which is refilled for block b+1 as soon as they are in registers.  The LDS regions are distinct
 // (`__restrict__`): without that knowledge the compiler makes every LDS read wait for all copies in
 // flight, which would serialise the pipeline.
-template <int DT, int MT, bool TRAIL>
+template <int DT, int MT, bool TRAIL, bool HALF>
 __device__ __forceinline__ void block_step(const uint8_t *__restrict__ cur, uint8_t *__restrict__ nxt,
                                            uint8_t *__restrict__ wl, const cq_weight &w, const cq_act_view &a,
                                            const LaneGeo &g, int64_t m0, int64_t n_tile, bool n_ok, bool more, int64_t b,
@@ -343,11 +346,11 @@ __device__ __forceinline__ void block_step(const uint8_t *__restrict__ cur, uint
     if (n_ok) {
         block_unpack(wl, g, hcur, lane, bl, bh, dw, wmin);
         if (more) stage_weights<DT>(wl, w, g, n_tile, b + 1);
-        tiles_mac<DT, MT, 0, SPLIT, SHIFT>(cur, g, bl, bh, dw, wmin, lane, out);
+        tiles_mac<DT, MT, 0, SPLIT, SHIFT, HALF>(cur, g, bl, bh, dw, wmin, lane, out);
     }
     __builtin_amdgcn_s_waitcnt(0);   // the next stage and the wave's next weights have landed in LDS
     __syncthreads();
-    if (TRAIL && n_ok) tiles_mac<DT, MT, SPLIT, MT, SHIFT>(cur, g, bl, bh, dw, wmin, lane, out);
+    if (TRAIL && n_ok) tiles_mac<DT, MT, SPLIT, MT, SHIFT, HALF>(cur, g, bl, bh, dw, wmin, lane, out);
 }
 
 // ------------------------------------------------------------------ kernel ----
@@ -394,24 +397,28 @@ __device__ __forceinline__ void gemm_body(const cq_weight &w, const cq_act_view 
         in = ifree;
         ifree = t;
     };
+    auto run = [&](auto trail, auto half) {
+        for (int64_t b = b0; b < b1; b++) {
+            const bool more = b + 1 < b1;
+            if (more) load_head(w, nc * kb + b + 1, hnxt);
+            block_step<DT, MT, decltype(trail)::value, decltype(half)::value>(smem + ic * T::kBytes, smem + in * T::kBytes, wl, w,
+                                                                              a, g, m0, n_tile, n_ok, more, b, wave, lane,
+                                                                              hcur, out);
+            hcur = hnxt;
+            rotate();
+        }
+    };
+    // a single 32-row tile of which at most 16 rows exist (an expert with few tokens): the scaling of
+    // the other half of the accumulators is skipped
+    const bool half = MT == 1 && m - m0 <= 16;
+    using T_ = std::true_type;
+    using F_ = std::false_type;
     if (wave < kWaves / 2) {
-        for (int64_t b = b0; b < b1; b++) {
-            const bool more = b + 1 < b1;
-            if (more) load_head(w, nc * kb + b + 1, hnxt);
-            block_step<DT, MT, false>(smem + ic * T::kBytes, smem + in * T::kBytes, wl, w, a, g, m0, n_tile, n_ok, more, b,
-                                      wave, lane, hcur, out);
-            hcur = hnxt;
-            rotate();
-        }
+        if (MT == 1 && half) run(F_{}, std::integral_constant<bool, MT == 1>{});
+        else run(F_{}, F_{});
     } else {
-        for (int64_t b = b0; b < b1; b++) {
-            const bool more = b + 1 < b1;
-            if (more) load_head(w, nc * kb + b + 1, hnxt);
-            block_step<DT, MT, true>(smem + ic * T::kBytes, smem + in * T::kBytes, wl, w, a, g, m0, n_tile, n_ok, more, b,
-                                     wave, lane, hcur, out);
-            hcur = hnxt;
-            rotate();
-        }
+        if (MT == 1 && half) run(T_{}, std::integral_constant<bool, MT == 1>{});
+        else run(T_{}, F_{});
     }
 
     if (n_ok) {
