@@ -647,12 +647,18 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
             if (lane == 0) { y[row0 + i * T] = s0; y[row0 + (i + 1) * T] = s1; }
         }
         // tail: two or three rows left (a = row i, b = row i+1, maybe row i+2 still to load)
-        const float s0 = row_dot<DT, UPL>(smem, r, units, a);
         const bool third = i + 2 < cnt;
-        if (third) load_row<DT, UPL>(w, row0 + (i + 2) * T, units, a);
-        const float s1 = row_dot<DT, UPL>(smem, r, units, b);
-        if (lane == 0) { y[row0 + i * T] = s0; y[row0 + (i + 1) * T] = s1; }
-        if (third) {
+        if (!third) {
+            // two rows in one stretch of straight-line code: their dependent chains (dot products,
+            // wave reductions) interleave
+            const float s0 = row_dot<DT, UPL>(smem, r, units, a);
+            const float s1 = row_dot<DT, UPL>(smem, r, units, b);
+            if (lane == 0) { y[row0 + i * T] = s0; y[row0 + (i + 1) * T] = s1; }
+        } else {
+            const float s0 = row_dot<DT, UPL>(smem, r, units, a);
+            load_row<DT, UPL>(w, row0 + (i + 2) * T, units, a);
+            const float s1 = row_dot<DT, UPL>(smem, r, units, b);
+            if (lane == 0) { y[row0 + i * T] = s0; y[row0 + (i + 1) * T] = s1; }
             const float s2 = row_dot<DT, UPL>(smem, r, units, a);
             if (lane == 0) y[row0 + (i + 2) * T] = s2;
         }
