@@ -344,7 +344,10 @@ extern "C" int cq_qmatmul(const cq_weight *w, const float *x_dev, int64_t m, flo
     // Few rows: split K over the waves instead of tiling rows.  Measured faster than the dot-product
     // kernels from 2 rows on and than the tile kernel up to 32 rows (up to 128 rows when n is small
     // and the tile kernel cannot fill the machine).
-    if (!(flags & (CQ_FLAG_FORCE_GEMM | CQ_FLAG_FORCE_MATVEC)) && m >= 2 && cq_skinny_supported(w, act) &&
+    // (the 32-element-block types from 4 rows (Q8_0) or 5 rows (Q4_0) on: below that the batched
+    // dot-product kernel is as fast or faster, it has no per-block scaling of MFMA results to do)
+    const int64_t skinny_from = w->dtype == CQ_DTYPE_Q8_0 ? 4 : w->dtype == CQ_DTYPE_Q4_0 ? 5 : 2;
+    if (!(flags & (CQ_FLAG_FORCE_GEMM | CQ_FLAG_FORCE_MATVEC)) && m >= skinny_from && cq_skinny_supported(w, act) &&
         (m <= 32 || (m <= 128 && w->n < 8192))) {
         CQ_HIP_CHECK(cq_launch_skinny(w, v, act, m, y_dev, s));
         return CQ_OK;

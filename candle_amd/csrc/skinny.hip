@@ -262,22 +262,26 @@ __global__ void __launch_bounds__(kThreads) skinny_kernel(cq_weight w, cq_act_vi
     }
 }
 
-// ------------------------------------------------------------ Q8_0 weights x Q8_0 activations ----
-// The same work split for 32-element blocks (k_quants.rs:618-649: sumf += sumi * d_w * d_x per
-// block).  The weights are int8 already, so the operands go from LDS straight into the 16x16x32
-// MFMA, one per block, and each block's 16 x 16 integers are scaled by the two block scales on the
-// way into the f32 result.  A wave takes 256 elements (eight blocks) per step.
-//   wgt : [2 row groups][2 K-halves][8 rows][8 chunks of 16 B], chunk c of row r at c ^ (r%8)
+// ---------------------------------------------------- Q8_0 / Q4_0 weights x Q8_0 activations ----
+// The same work split for 32-element blocks (k_quants.rs:618-649, :224-254: sumf += sumi * d_w *
+// d_x per block).  Q8_0 weights are int8 already and Q4_0 weights are one mask away from it, so the
+// operands go from LDS (almost) straight into the 16x16x32 MFMA, one per block, and each block's
+// 16 x 16 integers are scaled by the two block scales on the way into the f32 result.  Q4_0 holds
+// q - 8; the MFMA contracts q and 8 * (sum of the block's activations) comes off afterwards.  A wave
+// takes 256 elements (eight blocks) per step.
+//   wgt : Q8_0 [2 row groups][2 K-halves][8 rows][8 chunks of 16 B], Q4_0 [2 row groups][8 rows][8 chunks
+//         = blocks]; chunk c of row r at c ^ (r%8)
 //   act : [RT row groups][2 K-halves][8 rows][8 chunks], same swizzle
 template <int RT> struct BufQ8 {
     static constexpr int oAct = 4096, kRaw = oAct + RT * 2048;
     static constexpr int kBytes = kRaw;   // >= 2 KiB of partial results
 };
 
-template <int RT>
-__global__ void __launch_bounds__(kThreads) skinny_q8_0_kernel(cq_weight w, cq_act_view a, int64_t m0, int64_t m,
-                                                               float *__restrict__ y) {
+template <int DT, int RT>
+__global__ void __launch_bounds__(kThreads) skinny_blk32_kernel(cq_weight w, cq_act_view a, int64_t m0, int64_t m,
+                                                                float *__restrict__ y) {
     typedef BufQ8<RT> B;
+    constexpr bool Q4 = DT == CQ_DTYPE_Q4_0;
     constexpr int NT = (RT + 1) / 2;   // 16-row tiles
     extern __shared__ __align__(16) uint8_t smem[];
     const int lane = threadIdx.x & 63;
@@ -290,7 +294,10 @@ __global__ void __launch_bounds__(kThreads) skinny_q8_0_kernel(cq_weight w, cq_a
     // copy offsets: 8 rows x 128 B per instruction, chunks swizzled by the row
     const uint32_t r8 = lane >> 3, c8 = lane & 7;
     const uint32_t row_off = r8 * (uint32_t)k + ((c8 ^ r8) << 4);
-    // operand reads: 8 bytes [32b + 8kq, +8) of a row = half b/4, chunk 2(b%4) + kq/2, byte 8(kq%2)
+    const uint32_t q4_off = r8 * (uint32_t)(k >> 1) + ((c8 ^ r8) << 4);   // Q4_0: 128 bytes per row and step
+    // operand reads: 8 bytes [32b + 8kq, +8) of a row = half b/4, chunk 2(b%4) + kq/2, byte 8(kq%2);
+    // Q4_0 weights: chunk b, bytes 8(kq%2) .. +8, low nibbles for kq < 2, high nibbles above
+    const uint32_t w4_col = (r >> 3) * 1024u + (r & 7) * 128u + (kq & 1) * 8u, w4_shift = 4 * (kq >> 1);
     uint32_t w_col[4], a_col[NT][4];
     int64_t a_row[NT][4];   // rows whose scales this lane applies (results rows 4kq + i of tile t)
 #pragma unroll
@@ -313,10 +320,15 @@ __global__ void __launch_bounds__(kThreads) skinny_q8_0_kernel(cq_weight w, cq_a
     for (int t = 0; t < NT; t++) out[t] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
 
     for (int64_t g = wave; g < kg; g += kWaves) {
+        if (Q4) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int rg = i >> 1, kh = i & 1;
-            dma16(w.p0 + (n_tile + rg * 8) * k + g * 256 + kh * 128, row_off, buf + i * 1024);
+            for (int rg = 0; rg < 2; rg++) dma16(w.p0 + (n_tile + rg * 8) * (k >> 1) + g * 128, q4_off, buf + rg * 1024);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int rg = i >> 1, kh = i & 1;
+                dma16(w.p0 + (n_tile + rg * 8) * k + g * 256 + kh * 128, row_off, buf + i * 1024);
+            }
         }
 #pragma unroll
         for (int i = 0; i < 2 * RT; i++) {
@@ -326,6 +338,7 @@ __global__ void __launch_bounds__(kThreads) skinny_q8_0_kernel(cq_weight w, cq_a
         // the eight block scales of this lane's weight row, and of the activation rows it scales
         const uint4 dwv = *(const uint4 *)(w.p1 + ((n_tile + r) * kb + g * 8) * 2);
         v4f da[NT][4][2];
+        v4i bs[Q4 ? NT : 1][4][2];   // Q4_0: the sums of the activation blocks
 #pragma unroll
         for (int t = 0; t < NT; t++)
 #pragma unroll
@@ -333,6 +346,11 @@ __global__ void __launch_bounds__(kThreads) skinny_q8_0_kernel(cq_weight w, cq_a
                 const v4f *p = (const v4f *)(a.d + a_row[t][i] * kb + g * 8);
                 da[t][i][0] = p[0];
                 da[t][i][1] = p[1];
+                if (Q4) {
+                    const v4i *q = (const v4i *)(a.bsum32 + a_row[t][i] * kb + g * 8);
+                    bs[t][i][0] = q[0];
+                    bs[t][i][1] = q[1];
+                }
             }
         __builtin_amdgcn_s_waitcnt(0);   // everything above has landed
 
@@ -340,13 +358,23 @@ __global__ void __launch_bounds__(kThreads) skinny_q8_0_kernel(cq_weight w, cq_a
 #pragma unroll
         for (int b = 0; b < 8; b++) {
             const float dw = cq_h2f((uint16_t)(dww[b >> 1] >> (16 * (b & 1))));
-            const long wv = *(const long *)(buf + w_col[b & 3] + (b >> 2) * 1024);
+            long wv;
+            if (Q4) {
+                const uint2 raw = *(const uint2 *)(buf + w4_col + (((uint32_t)b ^ (r & 7)) << 4));
+                const uint32_t lo = (raw.x >> w4_shift) & 0x0F0F0F0Fu, hi = (raw.y >> w4_shift) & 0x0F0F0F0Fu;
+                wv = (long)(((uint64_t)hi << 32) | lo);
+            } else {
+                wv = *(const long *)(buf + w_col[b & 3] + (b >> 2) * 1024);
+            }
 #pragma unroll
             for (int t = 0; t < NT; t++) {
                 const long av = *(const long *)(buf + a_col[t][b & 3] + (b >> 2) * 1024);
                 const v4i acc = __builtin_amdgcn_mfma_i32_16x16x32_i8(av, wv, (v4i){0, 0, 0, 0}, 0, 0, 0);
 #pragma unroll
-                for (int i = 0; i < 4; i++) out[t][i] = __builtin_fmaf((float)acc[i] * dw, da[t][i][b >> 2][b & 3], out[t][i]);
+                for (int i = 0; i < 4; i++) {
+                    const int I = Q4 ? acc[i] - 8 * bs[Q4 ? t : 0][i][b >> 2][b & 3] : acc[i];
+                    out[t][i] = __builtin_fmaf((float)I * dw, da[t][i][b >> 2][b & 3], out[t][i]);
+                }
             }
         }
     }
@@ -371,22 +399,22 @@ __global__ void __launch_bounds__(kThreads) skinny_q8_0_kernel(cq_weight w, cq_a
     }
 }
 
-template <int RT>
-hipError_t launch_q8_rt(const cq_weight *w, cq_act_view a, int64_t m0, int64_t m, float *y, hipStream_t s) {
+template <int DT, int RT>
+hipError_t launch_blk32_rt(const cq_weight *w, cq_act_view a, int64_t m0, int64_t m, float *y, hipStream_t s) {
     const size_t lds = (size_t)BufQ8<RT>::kBytes * kWaves;
-    if (hipError_t e = cq_ensure_lds<skinny_q8_0_kernel<RT>>(w->dev, lds); e != hipSuccess) return e;
-    CQ_LAUNCH((skinny_q8_0_kernel<RT>), (unsigned)(w->n / 16), kThreads, lds, s, *w, a, m0, m, y);
+    if (hipError_t e = cq_ensure_lds<skinny_blk32_kernel<DT, RT>>(w->dev, lds); e != hipSuccess) return e;
+    CQ_LAUNCH((skinny_blk32_kernel<DT, RT>), (unsigned)(w->n / 16), kThreads, lds, s, *w, a, m0, m, y);
     return hipGetLastError();
 }
 
-hipError_t launch_q8(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
+template <int DT> hipError_t launch_blk32(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
     for (int64_t m0 = 0; m0 < m; m0 += 32) {
         const int64_t left = m - m0;
         hipError_t e;
-        if (left <= 8) e = launch_q8_rt<1>(w, a, m0, m, y, s);
-        else if (left <= 16) e = launch_q8_rt<2>(w, a, m0, m, y, s);
-        else if (left <= 24) e = launch_q8_rt<3>(w, a, m0, m, y, s);
-        else e = launch_q8_rt<4>(w, a, m0, m, y, s);
+        if (left <= 8) e = launch_blk32_rt<DT, 1>(w, a, m0, m, y, s);
+        else if (left <= 16) e = launch_blk32_rt<DT, 2>(w, a, m0, m, y, s);
+        else if (left <= 24) e = launch_blk32_rt<DT, 3>(w, a, m0, m, y, s);
+        else e = launch_blk32_rt<DT, 4>(w, a, m0, m, y, s);
         if (e != hipSuccess) return e;
     }
     return hipSuccess;
@@ -419,7 +447,7 @@ hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hip
 bool cq_skinny_supported(const cq_weight *w, int act_dtype) {
     // the copies address 8 rows of activations and 16 rows of a weight plane with 32-bit offsets
     const bool kquant = (w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q6K) && act_dtype == CQ_DTYPE_Q8K;
-    const bool q8 = w->dtype == CQ_DTYPE_Q8_0 && act_dtype == CQ_DTYPE_Q8_0 && w->k % 256 == 0;
+    const bool q8 = (w->dtype == CQ_DTYPE_Q8_0 || w->dtype == CQ_DTYPE_Q4_0) && act_dtype == CQ_DTYPE_Q8_0 && w->k % 256 == 0;
     return (kquant || q8) && w->k >= 256 && w->k <= (1 << 24) && w->n % 16 == 0 && w->n > 0;
 }
 
@@ -427,7 +455,8 @@ hipError_t cq_launch_skinny(const cq_weight *w, cq_act_view a, int act_dtype, in
     if (!cq_skinny_supported(w, act_dtype)) return hipErrorNotSupported;
     if (m == 0) return hipSuccess;
     if (a.m_stride < (m + 31) / 32 * 32) return hipErrorInvalidValue;   // whole 8-row groups are copied
-    if (w->dtype == CQ_DTYPE_Q8_0) return launch_q8(w, a, m, y, s);
+    if (w->dtype == CQ_DTYPE_Q8_0) return launch_blk32<CQ_DTYPE_Q8_0>(w, a, m, y, s);
+    if (w->dtype == CQ_DTYPE_Q4_0) return launch_blk32<CQ_DTYPE_Q4_0>(w, a, m, y, s);
     if (w->dtype == CQ_DTYPE_Q4K) return launch_dt<CQ_DTYPE_Q4K>(w, a, m, y, s);
     return launch_dt<CQ_DTYPE_Q6K>(w, a, m, y, s);
 }
