@@ -228,6 +228,82 @@ def main() -> int:
     gemm_tops = 2.0 * gm * gk * gn / (gemm_avg_us * 1e-6) / 1e12
     del gq, gx, gy, gws
 
+    # ---- the same step with the model's neighbours of each matmul (reported beside the headline) ----
+    # Per layer rms_norm -> q, k, v; o; rms_norm -> gate, up; silu(gate) * up -> down; final rms_norm
+    # -> lm_head (quantized_llama.rs:453-511 without attention and residuals).  "separate": one more
+    # launch per rms_norm (torch's kernel) and per silu * mul (cq_silu_mul); "fused": those steps inside
+    # the matmul launches (cq_qmatmul_fused).  Same weights as the headline step, HIP graph replay.
+    neighbours = None
+    try:
+        alpha = torch.ones(HIDDEN, device=dev, dtype=torch.float32)
+        h_buf = torch.empty((1, FFN), device=dev, dtype=torch.float32)
+        eps = 1e-5
+
+        def fused_call(i, pre, x, aux, s):
+            qhip.check(L.cq_qmatmul_fused(calls[i][0].handle, pre, C.c_void_p(x.data_ptr()), C.c_void_p(aux.data_ptr()),
+                                          eps, 1, C.c_void_p(outputs[i].data_ptr()), 0, C.c_void_p(ws.data_ptr()),
+                                          ws.numel(), s))
+
+        def plain_call(i, x, s):
+            qhip.check(L.cq_qmatmul(calls[i][0].handle, C.c_void_p(x.data_ptr()), 1, C.c_void_p(outputs[i].data_ptr()),
+                                    0, C.c_void_p(ws.data_ptr()), ws.numel(), s))
+
+        def chain(fused):
+            s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+            norm = lambda x: torch.nn.functional.rms_norm(x, (HIDDEN,), alpha, eps)
+            for layer in range(args.layers):
+                b = layer * len(LAYER_SHAPES)
+                if fused:
+                    for j in range(3):
+                        fused_call(b + j, qhip.PRE_RMS_NORM, inputs["x_attn"], alpha, s)
+                    plain_call(b + 3, inputs["x_o"], s)
+                    for j in (4, 5):
+                        fused_call(b + j, qhip.PRE_RMS_NORM, outputs[b + 3], alpha, s)
+                    fused_call(b + 6, qhip.PRE_SILU_MUL, outputs[b + 4], outputs[b + 5], s)
+                else:
+                    xn = norm(inputs["x_attn"])
+                    for j in range(3):
+                        plain_call(b + j, xn, s)
+                    plain_call(b + 3, inputs["x_o"], s)
+                    xn = norm(outputs[b + 3])
+                    for j in (4, 5):
+                        plain_call(b + j, xn, s)
+                    qhip.check(L.cq_silu_mul(0, C.c_void_p(outputs[b + 4].data_ptr()), C.c_void_p(outputs[b + 5].data_ptr()),
+                                             C.c_void_p(h_buf.data_ptr()), FFN, s))
+                    plain_call(b + 6, h_buf, s)
+            last = len(calls) - 1
+            if fused:
+                fused_call(last, qhip.PRE_RMS_NORM, inputs["x_head"], alpha, s)
+            else:
+                plain_call(last, norm(inputs["x_head"]), s)
+
+        times = {}
+        with torch.cuda.stream(side):
+            for name, fused in (("separate", False), ("fused", True)):
+                chain(fused)
+                torch.cuda.synchronize()
+                gn_ = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gn_, stream=side):
+                    chain(fused)
+                for _ in range(3):
+                    gn_.replay()
+                torch.cuda.synchronize()
+                n0, n1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                n0.record()
+                for _ in range(args.steps):
+                    gn_.replay()
+                n1.record()
+                torch.cuda.synchronize()
+                times[name] = n0.elapsed_time(n1) / args.steps
+        neighbours = {
+            "workload": "the headline step plus per layer 2 x rms_norm and silu * mul, and the final rms_norm",
+            "matmuls_only_ms": round(ms_per_step, 4),
+            "separate_launches_ms": round(times["separate"], 4),
+            "fused_ms": round(times["fused"], 4),
+        }
+    except Exception as e:  # reported beside the headline only: never fails the bench line
+        print(f"bench.py: neighbour chain not measured ({e})", file=sys.stderr)
+
     value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
     result = {
         "metric": "Q4_K matvec HBM GB/s (% of peak); Q4_K M=512 GEMM TOPS (% int8 MFMA peak)",
@@ -276,6 +352,9 @@ def main() -> int:
             "frac_of_int8_mfma_peak": round(gemm_tops / 5000.0, 4),
         },
     }
+
+    if neighbours is not None:
+        result["fused_neighbours"] = neighbours
 
     # ---- CPU baseline: restated candle CPU QMatMul (AVX2 + threads) on a bounded sample ----
     if not args.no_cpu:

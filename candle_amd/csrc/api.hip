@@ -239,8 +239,18 @@ extern "C" size_t cq_act_bytes(int act_dtype, int64_t m, int64_t k) {
     return (size_t)(m * (k / cq_block_size(act_dtype))) * (size_t)cq_type_size(act_dtype);
 }
 
-extern "C" int cq_quantize_act(int dev, int act_dtype, const float *x_dev, int64_t m, int64_t k, void *dst,
-                               void *stream) {
+// Checks the description of a fused step; a null aux or an unknown kind is the caller's error.
+static int check_pre(const cq_pre &pre) {
+    if (pre.kind == CQ_PRE_NONE) return CQ_OK;
+    if (pre.kind != CQ_PRE_RMS_NORM && pre.kind != CQ_PRE_SILU_MUL)
+        return cq_set_error(CQ_ERR_INVALID, "unknown fused step %d", pre.kind);
+    if (!pre.aux) return cq_set_error(CQ_ERR_INVALID, "null argument");
+    if ((uintptr_t)pre.aux & 15) return cq_set_error(CQ_ERR_INVALID, "aux must be 16-byte aligned");
+    return CQ_OK;
+}
+
+static int quantize_act_impl(int dev, int act_dtype, const float *x_dev, int64_t m, int64_t k, cq_pre pre, void *dst,
+                             void *stream) {
     if (!is_act_dtype(act_dtype)) return cq_set_error(CQ_ERR_UNSUPPORTED, "unsupported activation dtype %d", act_dtype);
     if (m < 0 || k < 0) return cq_set_error(CQ_ERR_INVALID, "negative shape");
     if (k % cq_block_size(act_dtype) != 0)
@@ -250,9 +260,20 @@ extern "C" int cq_quantize_act(int dev, int act_dtype, const float *x_dev, int64
     if (!x_dev || !dst) return cq_set_error(CQ_ERR_INVALID, "null argument");
     if (((uintptr_t)x_dev & 15) || ((uintptr_t)dst & 3))
         return cq_set_error(CQ_ERR_INVALID, "x must be 16-byte aligned and dst 4-byte aligned");
+    if (int rc = check_pre(pre)) return rc;
     CQ_HIP_CHECK(hipSetDevice(dev));
-    CQ_HIP_CHECK(cq_launch_quantize_act_aos(act_dtype, x_dev, m, k, dst, (hipStream_t)stream));
+    CQ_HIP_CHECK(cq_launch_quantize_act_aos(act_dtype, x_dev, m, k, pre, dst, (hipStream_t)stream));
     return CQ_OK;
+}
+
+extern "C" int cq_quantize_act(int dev, int act_dtype, const float *x_dev, int64_t m, int64_t k, void *dst,
+                               void *stream) {
+    return quantize_act_impl(dev, act_dtype, x_dev, m, k, cq_no_pre(), dst, stream);
+}
+
+extern "C" int cq_quantize_act_fused(int dev, int act_dtype, int pre, const float *x_dev, const float *aux_dev,
+                                     float eps, int64_t m, int64_t k, void *dst, void *stream) {
+    return quantize_act_impl(dev, act_dtype, x_dev, m, k, cq_pre{pre, aux_dev, eps}, dst, stream);
 }
 
 // Workspace layout for m rows of K elements (see cq_act_view).
@@ -312,11 +333,14 @@ static int check_matmul_args(const cq_weight *w, const float *x, int64_t m, cons
     return CQ_OK;
 }
 
-extern "C" int cq_qmatmul(const cq_weight *w, const float *x_dev, int64_t m, float *y_dev, int flags, void *ws,
-                          size_t ws_bytes, void *stream) {
+static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int64_t m, float *y_dev, int flags,
+                        void *ws, size_t ws_bytes, void *stream) {
     const size_t need = cq_workspace_bytes(w, m, flags);
     int rc = check_matmul_args(w, x_dev, m, y_dev, ws, ws_bytes, need);
     if (rc || m == 0 || w->n == 0) return rc;
+    if ((rc = check_pre(pre))) return rc;
+    if (pre.kind != CQ_PRE_NONE && (flags & CQ_FLAG_REUSE_ACT))
+        return cq_set_error(CQ_ERR_INVALID, "a fused step and a reused workspace exclude each other");
     if (w->k == 0) {
         CQ_HIP_CHECK(hipSetDevice(w->dev));
         CQ_HIP_CHECK(cq_launch_fill_zero(y_dev, m * w->n, (hipStream_t)stream));
@@ -328,12 +352,12 @@ extern "C" int cq_qmatmul(const cq_weight *w, const float *x_dev, int64_t m, flo
     // decode (one activation row): a single launch that quantizes x in its prologue
     if (m == 1 && !(flags & (CQ_FLAG_REUSE_ACT | CQ_FLAG_FORCE_GEMM | CQ_FLAG_STAGED_ACT | CQ_FLAG_ACT_Q8_1)) &&
         cq_matvec_fused_supported(w)) {
-        CQ_HIP_CHECK(cq_launch_matvec_fused(w, x_dev, y_dev, s));
+        CQ_HIP_CHECK(cq_launch_matvec_fused(w, x_dev, pre, y_dev, s));
         return CQ_OK;
     }
     cq_act_view v;
     act_ws_layout(act, m, w->k, (uint8_t *)ws, &v);
-    if (!(flags & CQ_FLAG_REUSE_ACT)) CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, nullptr, m, w->k, v, s));
+    if (!(flags & CQ_FLAG_REUSE_ACT)) CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, nullptr, m, w->k, pre, v, s));
     if (flags & CQ_FLAG_FORCE_SKINNY) {
         if (!cq_skinny_supported(w, act))
             return cq_set_error(CQ_ERR_UNSUPPORTED, "no split-K MFMA kernel for dtype %d with activation dtype %d and n = %lld",
@@ -367,6 +391,16 @@ extern "C" int cq_qmatmul(const cq_weight *w, const float *x_dev, int64_t m, flo
     return CQ_OK;
 }
 
+extern "C" int cq_qmatmul(const cq_weight *w, const float *x_dev, int64_t m, float *y_dev, int flags, void *ws,
+                          size_t ws_bytes, void *stream) {
+    return qmatmul_impl(w, x_dev, cq_no_pre(), m, y_dev, flags, ws, ws_bytes, stream);
+}
+
+extern "C" int cq_qmatmul_fused(const cq_weight *w, int pre, const float *x_dev, const float *aux_dev, float eps,
+                                int64_t m, float *y_dev, int flags, void *ws, size_t ws_bytes, void *stream) {
+    return qmatmul_impl(w, x_dev, cq_pre{pre, aux_dev, eps}, m, y_dev, flags, ws, ws_bytes, stream);
+}
+
 extern "C" int cq_qmatmul_int_dots(const cq_weight *w, const float *x_dev, int64_t m, int32_t *out_i, int32_t *out_mn,
                                    void *ws, size_t ws_bytes, void *stream) {
     const size_t need = cq_workspace_bytes(w, m, 0);
@@ -377,7 +411,7 @@ extern "C" int cq_qmatmul_int_dots(const cq_weight *w, const float *x_dev, int64
     hipStream_t s = (hipStream_t)stream;
     cq_act_view v;
     act_ws_layout(act, m, w->k, (uint8_t *)ws, &v);
-    CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, nullptr, m, w->k, v, s));
+    CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, nullptr, m, w->k, cq_no_pre(), v, s));
     CQ_HIP_CHECK(cq_launch_int_dots(w, v, m, out_i, w->dtype == CQ_DTYPE_Q4K ? out_mn : nullptr, s));
     return CQ_OK;
 }
@@ -389,9 +423,9 @@ extern "C" size_t cq_grouped_workspace_bytes(const cq_weight *const *experts, in
     return act_ws_layout(act_dtype_for(experts[0], flags), total_rows, experts[0]->k, nullptr, nullptr);
 }
 
-extern "C" int cq_qmatmul_grouped(const cq_weight *const *experts, int n_experts, const float *x_dev,
-                                  const int32_t *row_ids_dev, const int32_t *offsets, float *y_dev, int flags,
-                                  void *ws, size_t ws_bytes, void *stream) {
+static int grouped_impl(const cq_weight *const *experts, int n_experts, const float *x_dev, cq_pre pre,
+                        const int32_t *row_ids_dev, const int32_t *offsets, float *y_dev, int flags, void *ws,
+                        size_t ws_bytes, void *stream) {
     if (!experts || n_experts <= 0 || !offsets) return cq_set_error(CQ_ERR_INVALID, "null argument");
     const cq_weight *w0 = experts[0];
     if (!w0) return cq_set_error(CQ_ERR_INVALID, "null expert");
@@ -408,12 +442,13 @@ extern "C" int cq_qmatmul_grouped(const cq_weight *const *experts, int n_experts
     if (rc || total == 0 || w0->n == 0 || w0->k == 0) return rc;
     const int act = act_dtype_for(w0, flags);
     if (act == CQ_DTYPE_Q8_1) return cq_set_error(CQ_ERR_UNSUPPORTED, "grouped matmul takes the CPU formulation only");
+    if ((rc = check_pre(pre))) return rc;
     CQ_HIP_CHECK(hipSetDevice(w0->dev));
     hipStream_t s = (hipStream_t)stream;
     cq_act_view v;
     act_ws_layout(act, total, w0->k, (uint8_t *)ws, &v);
     // gather + quantize every routed row once, then one matmul per non-empty expert over its slice
-    CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, row_ids_dev, total, w0->k, v, s));
+    CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, row_ids_dev, total, w0->k, pre, v, s));
     // experts with more than eight rows among them: one tile-kernel launch for all experts
     int64_t most = 0;
     for (int e = 0; e < n_experts; e++) most = offsets[e + 1] - offsets[e] > most ? offsets[e + 1] - offsets[e] : most;
@@ -444,6 +479,20 @@ extern "C" int cq_qmatmul_grouped(const cq_weight *const *experts, int n_experts
         else CQ_HIP_CHECK(cq_launch_matvec(experts[e], ve, act, te, ye, s));
     }
     return CQ_OK;
+}
+
+extern "C" int cq_qmatmul_grouped(const cq_weight *const *experts, int n_experts, const float *x_dev,
+                                  const int32_t *row_ids_dev, const int32_t *offsets, float *y_dev, int flags,
+                                  void *ws, size_t ws_bytes, void *stream) {
+    return grouped_impl(experts, n_experts, x_dev, cq_no_pre(), row_ids_dev, offsets, y_dev, flags, ws, ws_bytes, stream);
+}
+
+extern "C" int cq_qmatmul_grouped_fused(const cq_weight *const *experts, int n_experts, int pre, const float *x_dev,
+                                        const float *aux_dev, float eps, const int32_t *row_ids_dev,
+                                        const int32_t *offsets, float *y_dev, int flags, void *ws, size_t ws_bytes,
+                                        void *stream) {
+    return grouped_impl(experts, n_experts, x_dev, cq_pre{pre, aux_dev, eps}, row_ids_dev, offsets, y_dev, flags, ws,
+                        ws_bytes, stream);
 }
 
 extern "C" int cq_silu_mul(int dev, const float *a, const float *b, float *h, int64_t count, void *stream) {

@@ -219,6 +219,30 @@ __device__ __forceinline__ void quantize_row_to_lds(uint8_t *smem, int64_t k, in
     }
 }
 
+// ---- model steps in front of the quantizer (cq_pre) --------------------------------------------
+// silu(v) = v / (1 + exp(-v)) (candle-core/src/op.rs:607-609), every operation single and in the
+// reference's order; rms_norm as the reference's device kernel writes it, scale * x * alpha
+// (candle-kernels/src/reduce.cu:161-172), with scale = 1 / sqrt(mean + eps) from two correctly
+// rounded operations (the CPU code divides each element by sqrt(mean + eps) instead,
+// candle-nn/src/ops.rs:491-494: a difference of a unit in the last place of some elements).
+__device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v)); }
+__device__ __forceinline__ float4 silu_mul4(float4 f, float4 a) {
+    return make_float4(silu_f(f.x) * a.x, silu_f(f.y) * a.y, silu_f(f.z) * a.z, silu_f(f.w) * a.w);
+}
+__device__ __forceinline__ float4 rms_scale4(float4 f, float scale, float4 a) {
+    return make_float4(scale * f.x * a.x, scale * f.y * a.y, scale * f.z * a.z, scale * f.w * a.w);
+}
+__device__ __forceinline__ float4 mul4(float4 f, float4 a) { return make_float4(f.x * a.x, f.y * a.y, f.z * a.z, f.w * a.w); }
+__device__ __forceinline__ float sum_sq4(float4 f) {
+    float t = f.x * f.x;
+    t += f.y * f.y;
+    t += f.z * f.z;
+    t += f.w * f.w;
+    return t;
+}
+// LDS offset of the per-chunk sums of squares: behind the activation image
+template <int DT> __host__ __device__ constexpr size_t fused_red_offset(int64_t k) { return (lds_row_bytes<DT>(k) + 15) / 16 * 16; }
+
 // ---- Q8K activations, two chunks per wave ------------------------------------------------------
 // Lane l takes the eight consecutive elements 8*(l%32) + [0,8) of chunk 2*pair + l/32, so a wave
 // covers two 256-element chunks and the per-chunk work (maximum search, the two divisions) is
@@ -577,8 +601,12 @@ __device__ __forceinline__ float row_dot(const uint8_t *smem, const LdsRow r, ui
 // return in order), not for the weight rows behind it.
 //   DEPTH 2 (short rows): two static register buffers, each refilled right after it is consumed.
 //   DEPTH 1 (long rows) : one buffer; a row is several KiB in flight per wave already.
-template <int DT, int UPL, int NW, int DEPTH>
-__global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float *x,
+//
+// PRE: the model step computed on the loaded activations before they are quantized (cq_pre):
+// silu(x) * x2 elementwise, or rms_norm, for which the waves first add up the squares of their
+// chunks and exchange the chunk sums through LDS, at the price of one more workgroup barrier.
+template <int DT, int UPL, int NW, int DEPTH, int PRE>
+__global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float *x, cq_pre pre,
                                                         float *__restrict__ y, int64_t total_waves,
                                                         int64_t rows_per_wave, int64_t rows_extra) {
     extern __shared__ __align__(16) uint8_t smem[];
@@ -598,6 +626,12 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
     X8 fx8[kPairs ? XCH : 1];
     if constexpr (kPairs) load_x_pairs<XCH, NW>(x, w.k, wave, fx8);
     else load_x_chunks<XCH, NW>(x, w.k, wave, fx);
+    float4 gx[(PRE != CQ_PRE_NONE && !kPairs) ? XCH : 1];   // the second operand, at the same elements
+    X8 gx8[(PRE != CQ_PRE_NONE && kPairs) ? XCH : 1];
+    if constexpr (PRE != CQ_PRE_NONE) {
+        if constexpr (kPairs) load_x_pairs<XCH, NW>(pre.aux, w.k, wave, gx8);
+        else load_x_chunks<XCH, NW>(pre.aux, w.k, wave, gx);
+    }
     // Pin the issue order: activation loads, then weight loads, then the quantizer arithmetic.
     // (The empty asm stops the optimizer from sinking loads past it, the scheduling barrier stops
     // the instruction scheduler.)
@@ -609,15 +643,84 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     const LdsRow r = lds_row<DT>(w.k, 0);
+    if constexpr (PRE == CQ_PRE_SILU_MUL) {
+#pragma unroll
+        for (int i = 0; i < XCH; i++) {
+            if constexpr (kPairs) { fx8[i].a = silu_mul4(fx8[i].a, gx8[i].a); fx8[i].b = silu_mul4(fx8[i].b, gx8[i].b); }
+            else fx[i] = silu_mul4(fx[i], gx[i]);
+        }
+    }
+    // rms_norm.  Sum of squares in the order every rms_norm kernel of this library uses, so that a
+    // row gives the same bits whatever the batch: groups of 8 consecutive elements (two sequential
+    // sums of 4, added), a binary tree over the 32 groups of a 256-element chunk (group j with
+    // j^1, then ^2, ^4, ^8, ^16), then the chunks one after the other.
+    // Q8K activations: quantizing scale * z gives the quants of z and the block scales of z times
+    // `scale` (up to rounding), so the waves quantize z = x * alpha at once, leave their chunk sums
+    // in LDS for after the barrier that follows anyway, and multiply the row results by `scale`.
+    // Q8_0 activations round their block scale to f16, which does not commute with the scaling:
+    // there the elements are scaled before they are quantized, behind a barrier of its own.
+    constexpr bool kRms = PRE == CQ_PRE_RMS_NORM;
+    constexpr int kSlots = (kPairs ? 2 : 1) * XCH * NW;   // chunk slots of the workgroup (a multiple of 8)
+    const uint32_t red = (uint32_t)fused_red_offset<DT>(w.k);
+    auto row_scale = [&]() {
+        // all slots are read at once and added in order; the zeros behind the last chunk change nothing
+        float4 ps[kSlots / 4];
+#pragma unroll
+        for (int c = 0; c < kSlots / 4; c++) ps[c] = lds_get<float4>(smem, red + 16 * c);
+        float sum2 = ps[0].x;
+        sum2 += ps[0].y; sum2 += ps[0].z; sum2 += ps[0].w;
+#pragma unroll
+        for (int c = 1; c < kSlots / 4; c++) { sum2 += ps[c].x; sum2 += ps[c].y; sum2 += ps[c].z; sum2 += ps[c].w; }
+        return 1.0f / sqrtf(sum2 / (float)w.k + pre.eps);
+    };
+    if constexpr (kRms) {
+        const int chunks = (int)((w.k + 255) / 256);
+#pragma unroll
+        for (int i = 0; i < XCH; i++) {
+            if constexpr (kPairs) {
+                float t = sum_sq4(fx8[i].a) + sum_sq4(fx8[i].b);   // lane = group; 32 lanes = chunk
+                t += dpp_f<kQuadSwap1>(t);
+                t += dpp_f<kQuadSwap2>(t);
+                t += dpp_f<kHalfMirror>(t);
+                t += dpp_f<kRowMirror>(t);
+                const float p_lo = readlane_f(t, 0) + readlane_f(t, 16), p_hi = readlane_f(t, 32) + readlane_f(t, 48);
+                const int c = 2 * (wave + i * NW) + lane;   // every slot below kSlots is written: zero past the row
+                if (lane < 2) lds_put<float>(smem, red + 4 * c, c < chunks ? (lane ? p_hi : p_lo) : 0.0f);
+                fx8[i].a = mul4(fx8[i].a, gx8[i].a);
+                fx8[i].b = mul4(fx8[i].b, gx8[i].b);
+            } else {
+                const int c = wave + i * NW;
+                float t = c * 256 + 4 * lane < w.k ? sum_sq4(fx[i]) : 0.0f;   // two lanes = group
+                t += dpp_f<kQuadSwap1>(t);
+                t += dpp_f<kQuadSwap2>(t);
+                t += dpp_f<kHalfMirror>(t);
+                t += dpp_f<kRowMirror>(t);
+                const float p = (readlane_f(t, 0) + readlane_f(t, 16)) + (readlane_f(t, 32) + readlane_f(t, 48));
+                if (lane == 0) lds_put<float>(smem, red + 4 * c, c < chunks ? p : 0.0f);
+            }
+        }
+        if constexpr (!kPairs) {
+            __syncthreads();
+            const float scale = row_scale();
+#pragma unroll
+            for (int i = 0; i < XCH; i++) fx[i] = rms_scale4(fx[i], scale, gx[i]);
+        }
+    }
     if constexpr (kPairs) quantize_pairs_to_lds<DT, XCH, NW>(smem, w.k, wave, r, fx8);
     else quantize_row_to_lds<DT, XCH, NW>(smem, w.k, wave, r, fx);
     __syncthreads();
+    float yscale = 1.0f;
+    if constexpr (kRms && kPairs) yscale = row_scale();
+    auto put = [&](int64_t row, float v) {
+        if constexpr (kRms && kPairs) v *= yscale;
+        if (lane == 0) y[row] = v;
+    };
 
     if constexpr (DEPTH == 1) {
         for (int64_t i = 0; i < cnt; i++) {
             const float s = row_dot<DT, UPL>(smem, r, units, a);
             if (i + 1 < cnt) load_row<DT, UPL>(w, row0 + (i + 1) * T, units, a);
-            if (lane == 0) y[row0 + i * T] = s;
+            put(row0 + i * T, s);
         }
     } else {
         int64_t i = 0;
@@ -644,7 +747,8 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
                 s1 = row_dot<DT, UPL>(smem, r, units, b);
                 load_row<DT, UPL>(w, row0 + (i + 3) * T, units, b);
             }
-            if (lane == 0) { y[row0 + i * T] = s0; y[row0 + (i + 1) * T] = s1; }
+            put(row0 + i * T, s0);
+            put(row0 + (i + 1) * T, s1);
         }
         // tail: two or three rows left (a = row i, b = row i+1, maybe row i+2 still to load)
         const bool third = i + 2 < cnt;
@@ -653,14 +757,16 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
             // wave reductions) interleave
             const float s0 = row_dot<DT, UPL>(smem, r, units, a);
             const float s1 = row_dot<DT, UPL>(smem, r, units, b);
-            if (lane == 0) { y[row0 + i * T] = s0; y[row0 + (i + 1) * T] = s1; }
+            put(row0 + i * T, s0);
+            put(row0 + (i + 1) * T, s1);
         } else {
             const float s0 = row_dot<DT, UPL>(smem, r, units, a);
             load_row<DT, UPL>(w, row0 + (i + 2) * T, units, a);
             const float s1 = row_dot<DT, UPL>(smem, r, units, b);
-            if (lane == 0) { y[row0 + i * T] = s0; y[row0 + (i + 1) * T] = s1; }
+            put(row0 + i * T, s0);
+            put(row0 + (i + 1) * T, s1);
             const float s2 = row_dot<DT, UPL>(smem, r, units, a);
-            if (lane == 0) y[row0 + (i + 2) * T] = s2;
+            put(row0 + (i + 2) * T, s2);
         }
     }
 }
@@ -828,10 +934,12 @@ int num_cus() {
 
 // Eight waves per workgroup, one workgroup per CU.  Whole workgroups only, and every wave
 // gets at least `depth` rows: wgs * 8 * depth <= n.
-template <int DT, int UPL>
-hipError_t launch_fused_upl(const cq_weight *w, const float *x, float *y, hipStream_t s) {
+template <int DT, int UPL, int PRE>
+hipError_t launch_fused_upl(const cq_weight *w, const float *x, cq_pre pre, float *y, hipStream_t s) {
     constexpr int NW = 8;
-    const size_t lds = lds_row_bytes<DT>(w->k);
+    constexpr int kXch = (UPL * Geo<DT>::kElems / (Geo<DT>::kActK ? 8 : 4) + NW - 1) / NW;   // as in the kernel
+    const size_t lds = PRE == CQ_PRE_RMS_NORM ? fused_red_offset<DT>(w->k) + 4 * (size_t)((Geo<DT>::kActK ? 2 : 1) * kXch * NW)
+                                              : lds_row_bytes<DT>(w->k);
     // every workgroup quantizes the whole activation row, so fewer, longer-lived workgroups win: one
     // per CU measured faster than two on every decode shape (11008 x 4096 Q4K: 7.0 us against 7.6 us)
     const int64_t max_wgs = num_cus();
@@ -843,8 +951,8 @@ hipError_t launch_fused_upl(const cq_weight *w, const float *x, float *y, hipStr
     int64_t wgs = w->n / (NW * depth);
     if (wgs > max_wgs) wgs = max_wgs;
     const int64_t tw = wgs * NW, rpw = w->n / tw, extra = w->n % tw;
-    if (depth == 2) CQ_LAUNCH((fused_kernel<DT, UPL, NW, 2>), (unsigned)wgs, NW * 64, lds, s, *w, x, y, tw, rpw, extra);
-    else CQ_LAUNCH((fused_kernel<DT, UPL, NW, 1>), (unsigned)wgs, NW * 64, lds, s, *w, x, y, tw, rpw, extra);
+    if (depth == 2) CQ_LAUNCH((fused_kernel<DT, UPL, NW, 2, PRE>), (unsigned)wgs, NW * 64, lds, s, *w, x, pre, y, tw, rpw, extra);
+    else CQ_LAUNCH((fused_kernel<DT, UPL, NW, 1, PRE>), (unsigned)wgs, NW * 64, lds, s, *w, x, pre, y, tw, rpw, extra);
     return hipGetLastError();
 }
 
@@ -853,19 +961,29 @@ bool fused_ok(const cq_weight *w) {
     // Every workgroup re-quantizes the whole activation row in its prologue, which pays off against a
     // separate quantizer launch up to the row lengths measured (K = 11008: 12.0 us against 11.6 + 3.1 us).
     // The launcher instantiates up to eight units per lane (512 units per row).
-    return w->k <= 16384 && w->k / Geo<DT>::kElems <= 512 && w->n >= 8 && lds_row_bytes<DT>(w->k) <= 64 * 1024;
+    return w->k <= 16384 && w->k / Geo<DT>::kElems <= 512 && w->n >= 8 && lds_row_bytes<DT>(w->k) <= 64 * 1024 - 1024;
+}
+
+template <int DT, int PRE>
+hipError_t launch_fused_pre(const cq_weight *w, const float *x, cq_pre pre, float *y, hipStream_t s) {
+    const int64_t units = w->k / Geo<DT>::kElems;
+    const int upl = (int)((units + 63) / 64);
+    if (upl <= 1) return launch_fused_upl<DT, 1, PRE>(w, x, pre, y, s);
+    if (upl <= 2) return launch_fused_upl<DT, 2, PRE>(w, x, pre, y, s);
+    if (upl <= 3) return launch_fused_upl<DT, 3, PRE>(w, x, pre, y, s);
+    if (upl <= 4) return launch_fused_upl<DT, 4, PRE>(w, x, pre, y, s);
+    if (upl <= 6) return launch_fused_upl<DT, 6, PRE>(w, x, pre, y, s);
+    return launch_fused_upl<DT, 8, PRE>(w, x, pre, y, s);
 }
 
 template <int DT>
-hipError_t launch_fused(const cq_weight *w, const float *x, float *y, hipStream_t s) {
-    const int64_t units = w->k / Geo<DT>::kElems;
-    const int upl = (int)((units + 63) / 64);
-    if (upl <= 1) return launch_fused_upl<DT, 1>(w, x, y, s);
-    if (upl <= 2) return launch_fused_upl<DT, 2>(w, x, y, s);
-    if (upl <= 3) return launch_fused_upl<DT, 3>(w, x, y, s);
-    if (upl <= 4) return launch_fused_upl<DT, 4>(w, x, y, s);
-    if (upl <= 6) return launch_fused_upl<DT, 6>(w, x, y, s);
-    return launch_fused_upl<DT, 8>(w, x, y, s);
+hipError_t launch_fused(const cq_weight *w, const float *x, cq_pre pre, float *y, hipStream_t s) {
+    switch (pre.kind) {
+    case CQ_PRE_NONE: return launch_fused_pre<DT, CQ_PRE_NONE>(w, x, pre, y, s);
+    case CQ_PRE_RMS_NORM: return launch_fused_pre<DT, CQ_PRE_RMS_NORM>(w, x, pre, y, s);
+    case CQ_PRE_SILU_MUL: return launch_fused_pre<DT, CQ_PRE_SILU_MUL>(w, x, pre, y, s);
+    default: return hipErrorInvalidValue;
+    }
 }
 
 int pick_rows_per_wg(int64_t n) {
@@ -966,13 +1084,13 @@ bool cq_matvec_fused_supported(const cq_weight *w) {
     }
 }
 
-hipError_t cq_launch_matvec_fused(const cq_weight *w, const float *x, float *y, hipStream_t s) {
+hipError_t cq_launch_matvec_fused(const cq_weight *w, const float *x, cq_pre pre, float *y, hipStream_t s) {
     if (w->n == 0) return hipSuccess;
     switch (w->dtype) {
-    case CQ_DTYPE_Q4_0: return launch_fused<CQ_DTYPE_Q4_0>(w, x, y, s);
-    case CQ_DTYPE_Q8_0: return launch_fused<CQ_DTYPE_Q8_0>(w, x, y, s);
-    case CQ_DTYPE_Q4K: return launch_fused<CQ_DTYPE_Q4K>(w, x, y, s);
-    case CQ_DTYPE_Q6K: return launch_fused<CQ_DTYPE_Q6K>(w, x, y, s);
+    case CQ_DTYPE_Q4_0: return launch_fused<CQ_DTYPE_Q4_0>(w, x, pre, y, s);
+    case CQ_DTYPE_Q8_0: return launch_fused<CQ_DTYPE_Q8_0>(w, x, pre, y, s);
+    case CQ_DTYPE_Q4K: return launch_fused<CQ_DTYPE_Q4K>(w, x, pre, y, s);
+    case CQ_DTYPE_Q6K: return launch_fused<CQ_DTYPE_Q6K>(w, x, pre, y, s);
     default: return hipErrorInvalidValue;
     }
 }

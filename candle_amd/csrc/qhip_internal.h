@@ -87,10 +87,20 @@ bool cq_timing_take(hipEvent_t *start, hipEvent_t *stop);
 // repack.hip
 hipError_t cq_launch_repack(const cq_weight *w, const uint8_t *aos_dev, hipStream_t s);   // GGML AoS -> planes
 hipError_t cq_launch_unpack(const cq_weight *w, uint8_t *aos_dev, hipStream_t s);         // planes -> GGML AoS
+// A step of the caller's model computed on the way into the activation quantizer (CQ_PRE_*):
+// rms_norm: x / sqrt(mean(x^2) + eps) * aux[k]; silu_mul: silu(x) * aux[m][k] (aux indexed like x).
+struct cq_pre {
+    int kind;
+    const float *aux;
+    float eps;
+};
+static inline cq_pre cq_no_pre() { return cq_pre{CQ_PRE_NONE, nullptr, 0.0f}; }
+
 // quantize_act.hip
-hipError_t cq_launch_quantize_act_aos(int act_dtype, const float *x, int64_t m, int64_t k, void *dst, hipStream_t s);
+hipError_t cq_launch_quantize_act_aos(int act_dtype, const float *x, int64_t m, int64_t k, cq_pre pre, void *dst,
+                                      hipStream_t s);
 hipError_t cq_launch_quantize_act_ws(int act_dtype, const float *x, const int32_t *row_ids, int64_t m, int64_t k,
-                                     cq_act_view v, hipStream_t s);
+                                     cq_pre pre, cq_act_view v, hipStream_t s);
 // quantize_weight.hip
 hipError_t cq_launch_quantize_weight(int dtype, const float *src, int64_t nblocks, uint8_t *aos_dev, hipStream_t s);
 // dequantize.hip
@@ -100,7 +110,7 @@ hipError_t cq_launch_matvec(const cq_weight *w, cq_act_view a, int act_dtype, in
 hipError_t cq_launch_int_dots(const cq_weight *w, cq_act_view a, int64_t m, int32_t *out_i, int32_t *out_mn,
                               hipStream_t s);
 bool cq_matvec_fused_supported(const cq_weight *w);   // m == 1: quantizer fused into the matvec launch
-hipError_t cq_launch_matvec_fused(const cq_weight *w, const float *x, float *y, hipStream_t s);
+hipError_t cq_launch_matvec_fused(const cq_weight *w, const float *x, cq_pre pre, float *y, hipStream_t s);
 // gemm.hip
 bool cq_gemm_supported(const cq_weight *w, int64_t m, int act_dtype);
 hipError_t cq_launch_gemm(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s);

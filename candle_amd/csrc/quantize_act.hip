@@ -8,9 +8,23 @@
 // 4l..4l+3 (one float4 load, a whole 1 KiB line per wave).  Reductions are wave shuffles.
 // Every f32 operation is a single IEEE operation in the reference's order (this file is
 // compiled with -ffp-contract=off; `/` is correctly rounded).
+//
+// A step of the caller's model can run in front of the quantizer (cq_pre): silu(x) * x2 between the
+// feed-forward projections (candle-transformers/src/models/quantized_llama.rs:56-63, silu as in
+// candle-core/src/op.rs:607-609) is elementwise and goes into the kernels above; rms_norm
+// (candle-nn/src/ops.rs:482-495: x / sqrt(mean(x^2) + eps) * alpha) needs the whole row first and
+// has a kernel of its own with one workgroup per row.
 #include "qhip_internal.h"
 
 namespace {
+
+__device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v)); }
+__device__ __forceinline__ float4 silu_mul4(float4 f, float4 a) {
+    return make_float4(silu_f(f.x) * a.x, silu_f(f.y) * a.y, silu_f(f.z) * a.z, silu_f(f.w) * a.w);
+}
+__device__ __forceinline__ float4 rms_scale4(float4 f, float scale, float4 a) {
+    return make_float4(scale * f.x * a.x, scale * f.y * a.y, scale * f.z * a.z, scale * f.w * a.w);
+}
 
 struct Sink {
     // GGML struct layout (AOS) or the workspace layout (qhip_internal.h)
@@ -20,22 +34,10 @@ struct Sink {
 
 __device__ __forceinline__ int8_t round_to_i8(float v) { return cq_as_i8(roundf(v)); }
 
-// Q8_0 / Q8_1: eight 32-element blocks per wave, 8 lanes per block.
+// Q8_0 / Q8_1: eight 32-element blocks per wave, 8 lanes per block.  `f` = the lane's four values
+// at element e0 of `row` (zeros in a lane past the end of the row); called by all 64 lanes.
 template <bool AOS, bool Q8_1>
-__global__ void __launch_bounds__(256) quantize_q8_0_kernel(const float *__restrict__ x,
-                                                            const int32_t *__restrict__ row_ids, int64_t m,
-                                                            int64_t k, Sink out) {
-    const int lane = threadIdx.x & 63;
-    const int64_t chunks_per_row = (k + 255) / 256;
-    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    if (wave >= m * chunks_per_row) return;
-    const int64_t row = wave / chunks_per_row;
-    const int64_t e0 = (wave - row * chunks_per_row) * 256 + 4 * lane;
-    const bool active = e0 < k;  // k % 32 == 0, so a lane is either fully inside or fully outside
-    const int64_t src_row = row_ids ? (int64_t)row_ids[row] : row;
-    float4 f = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (active) f = *(const float4 *)(x + src_row * k + e0);
-
+__device__ __forceinline__ void q8_0_chunk(const float4 f, bool active, int64_t row, int64_t e0, int64_t k, const Sink &out) {
     float amax = fmaxf(fmaxf(fmaxf(fmaxf(0.0f, fabsf(f.x)), fabsf(f.y)), fabsf(f.z)), fabsf(f.w));
     amax = fmaxf(amax, __shfl_xor(amax, 1));
     amax = fmaxf(amax, __shfl_xor(amax, 2));
@@ -77,19 +79,34 @@ __global__ void __launch_bounds__(256) quantize_q8_0_kernel(const float *__restr
     }
 }
 
-// Q8K: one 256-element block per wave.
-template <bool AOS>
-__global__ void __launch_bounds__(256) quantize_q8k_kernel(const float *__restrict__ x,
-                                                           const int32_t *__restrict__ row_ids, int64_t m, int64_t k,
-                                                           Sink out) {
+template <bool AOS, bool Q8_1, bool SILU>
+__global__ void __launch_bounds__(256) quantize_q8_0_kernel(const float *__restrict__ x,
+                                                            const int32_t *__restrict__ row_ids, int64_t m,
+                                                            int64_t k, const float *__restrict__ x2, Sink out) {
     const int lane = threadIdx.x & 63;
-    const int64_t kb = k / 256;
-    const int64_t blk = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    if (blk >= m * kb) return;
-    const int64_t row = blk / kb;
-    const int64_t b_in_row = blk - row * kb;
+    const int64_t chunks_per_row = (k + 255) / 256;
+    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (wave >= m * chunks_per_row) return;
+    const int64_t row = wave / chunks_per_row;
+    const int64_t e0 = (wave - row * chunks_per_row) * 256 + 4 * lane;
+    const bool active = e0 < k;  // k % 32 == 0, so a lane is either fully inside or fully outside
     const int64_t src_row = row_ids ? (int64_t)row_ids[row] : row;
-    const float4 f = *(const float4 *)(x + src_row * k + b_in_row * 256 + 4 * lane);
+    float4 f = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (active) {
+        f = *(const float4 *)(x + src_row * k + e0);
+        if (SILU) f = silu_mul4(f, *(const float4 *)(x2 + src_row * k + e0));
+    }
+    q8_0_chunk<AOS, Q8_1>(f, active, row, e0, k, out);
+}
+
+// Q8K: one 256-element block per wave.
+// `f` = the lane's four values of block b_in_row of `row`; called by all 64 lanes.  SCALED: the
+// block's scale is multiplied by `dscale` on the way out (the block then stands for dscale * f).
+template <bool AOS, bool SCALED = false>
+__device__ __forceinline__ void q8k_chunk(const float4 f, int64_t row, int64_t b_in_row, int64_t k, const Sink &out,
+                                          float dscale = 1.0f) {
+    const int lane = threadIdx.x & 63;
+    const int64_t blk = row * (k / 256) + b_in_row;
 
     // first index with the largest |x| (strict `<` in the reference keeps the earliest)
     float amax = 0.0f, max = 0.0f;
@@ -122,6 +139,7 @@ __global__ void __launch_bounds__(256) quantize_q8k_kernel(const float *__restri
                  ((uint32_t)(uint8_t)q3 << 24);
         sum = (int)q0 + (int)q1 + (int)q2 + (int)q3;
         d = 1.0f / iscale;
+        if (SCALED) d *= dscale;
     }
     sum += __shfl_xor(sum, 1);
     sum += __shfl_xor(sum, 2);  // lanes 4j..4j+3 now hold bsums[j]
@@ -150,37 +168,116 @@ __global__ void __launch_bounds__(256) quantize_q8k_kernel(const float *__restri
     }
 }
 
+template <bool AOS, bool SILU>
+__global__ void __launch_bounds__(256) quantize_q8k_kernel(const float *__restrict__ x,
+                                                           const int32_t *__restrict__ row_ids, int64_t m, int64_t k,
+                                                           const float *__restrict__ x2, Sink out) {
+    const int lane = threadIdx.x & 63;
+    const int64_t kb = k / 256;
+    const int64_t blk = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (blk >= m * kb) return;
+    const int64_t row = blk / kb;
+    const int64_t b_in_row = blk - row * kb;
+    const int64_t src_row = row_ids ? (int64_t)row_ids[row] : row;
+    float4 f = *(const float4 *)(x + src_row * k + b_in_row * 256 + 4 * lane);
+    if (SILU) f = silu_mul4(f, *(const float4 *)(x2 + src_row * k + b_in_row * 256 + 4 * lane));
+    q8k_chunk<AOS>(f, row, b_in_row, k, out);
+}
+
+// rms_norm in front of the quantizer: one workgroup of four waves per row.  The squares are added
+// in a fixed order that does not depend on the kernel (the decode matvec's prologue follows it
+// too, so a row gives the same bits whatever the batch): groups of 8 consecutive elements as two
+// sequential sums of 4, added; a binary tree over the 32 groups of a 256-element chunk (group j
+// with j^1, then ^2, ^4, ^8, ^16); then the chunks one after the other.  The reference's CPU code
+// adds all squares one after the other: the two sums agree to rounding, not to the bit.
+// scale = 1 / sqrt(mean + eps) multiplies the elements as in the reference's device kernel
+// (candle-kernels/src/reduce.cu:161-172; its CPU code divides every element by the root).  The
+// second pass reads the row again (from L2):
+//   Q8_0 / Q8_1: quantizes scale * x * alpha chunk by chunk;
+//   Q8K: quantizes z = x * alpha and multiplies the block scales by `scale`: the quants of
+//        scale * z are those of z, and the decode matvec uses the same form.
+// ACT: 0 = Q8K, 1 = Q8_0, 2 = Q8_1.  Dynamic LDS: one float per chunk.
+template <bool AOS, int ACT>
+__global__ void __launch_bounds__(256) quantize_rms_rows_kernel(const float *__restrict__ x,
+                                                                const int32_t *__restrict__ row_ids, int64_t k,
+                                                                const float *__restrict__ alpha, float eps, Sink out) {
+    extern __shared__ float chunk_sums[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t row = blockIdx.x;
+    const int64_t src_row = row_ids ? (int64_t)row_ids[row] : row;
+    const float *xr = x + src_row * k;
+    const int64_t chunks = (k + 255) / 256;
+    for (int64_t c = wave; c < chunks; c += 4) {
+        const int64_t e0 = c * 256 + 4 * lane;
+        float t = 0.0f;
+        if (e0 < k) {
+            const float4 f = *(const float4 *)(xr + e0);
+            t = f.x * f.x;
+            t += f.y * f.y;
+            t += f.z * f.z;
+            t += f.w * f.w;
+        }
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) t += __shfl_xor(t, off);
+        if (lane == 0) chunk_sums[c] = t;
+    }
+    __syncthreads();
+    float sum2 = chunk_sums[0];
+    for (int64_t c = 1; c < chunks; c++) sum2 += chunk_sums[c];
+    const float scale = 1.0f / sqrtf(sum2 / (float)k + eps);
+    for (int64_t c = wave; c < chunks; c += 4) {
+        const int64_t e0 = c * 256 + 4 * lane;
+        const bool active = e0 < k;
+        float4 f = make_float4(0.f, 0.f, 0.f, 0.f), a = f;
+        if (active) { f = *(const float4 *)(xr + e0); a = *(const float4 *)(alpha + e0); }
+        if (ACT == 0) q8k_chunk<AOS, true>(make_float4(f.x * a.x, f.y * a.y, f.z * a.z, f.w * a.w), row, c, k, out, scale);
+        else q8_0_chunk<AOS, ACT == 2>(rms_scale4(f, scale, a), active, row, e0, k, out);
+    }
+}
+
 template <bool AOS>
-hipError_t launch(int act_dtype, const float *x, const int32_t *row_ids, int64_t m, int64_t k, Sink out,
+hipError_t launch(int act_dtype, const float *x, const int32_t *row_ids, int64_t m, int64_t k, cq_pre pre, Sink out,
                   hipStream_t s) {
     if (m == 0 || k == 0) return hipSuccess;
+    if (act_dtype != CQ_DTYPE_Q8K && act_dtype != CQ_DTYPE_Q8_0 && act_dtype != CQ_DTYPE_Q8_1) return hipErrorInvalidValue;
     const int threads = 256, waves = threads / 64;
+    if (pre.kind == CQ_PRE_RMS_NORM) {
+        const unsigned grid = (unsigned)m;
+        const size_t lds = (size_t)((k + 255) / 256) * 4;
+        if (lds > 48 * 1024) return hipErrorInvalidValue;   // rows of more than 3 million elements
+        if (act_dtype == CQ_DTYPE_Q8K) quantize_rms_rows_kernel<AOS, 0><<<grid, threads, lds, s>>>(x, row_ids, k, pre.aux, pre.eps, out);
+        else if (act_dtype == CQ_DTYPE_Q8_0) quantize_rms_rows_kernel<AOS, 1><<<grid, threads, lds, s>>>(x, row_ids, k, pre.aux, pre.eps, out);
+        else quantize_rms_rows_kernel<AOS, 2><<<grid, threads, lds, s>>>(x, row_ids, k, pre.aux, pre.eps, out);
+        return hipGetLastError();
+    }
+    const bool silu = pre.kind == CQ_PRE_SILU_MUL;
+    const int64_t nw = act_dtype == CQ_DTYPE_Q8K ? m * (k / 256) : m * ((k + 255) / 256);
+    const unsigned grid = (unsigned)((nw + waves - 1) / waves);
     if (act_dtype == CQ_DTYPE_Q8K) {
-        const int64_t nw = m * (k / 256);
-        quantize_q8k_kernel<AOS><<<(unsigned)((nw + waves - 1) / waves), threads, 0, s>>>(x, row_ids, m, k, out);
+        if (silu) quantize_q8k_kernel<AOS, true><<<grid, threads, 0, s>>>(x, row_ids, m, k, pre.aux, out);
+        else quantize_q8k_kernel<AOS, false><<<grid, threads, 0, s>>>(x, row_ids, m, k, nullptr, out);
     } else if (act_dtype == CQ_DTYPE_Q8_0) {
-        const int64_t nw = m * ((k + 255) / 256);
-        quantize_q8_0_kernel<AOS, false><<<(unsigned)((nw + waves - 1) / waves), threads, 0, s>>>(x, row_ids, m, k, out);
-    } else if (act_dtype == CQ_DTYPE_Q8_1) {
-        const int64_t nw = m * ((k + 255) / 256);
-        quantize_q8_0_kernel<AOS, true><<<(unsigned)((nw + waves - 1) / waves), threads, 0, s>>>(x, row_ids, m, k, out);
+        if (silu) quantize_q8_0_kernel<AOS, false, true><<<grid, threads, 0, s>>>(x, row_ids, m, k, pre.aux, out);
+        else quantize_q8_0_kernel<AOS, false, false><<<grid, threads, 0, s>>>(x, row_ids, m, k, nullptr, out);
     } else {
-        return hipErrorInvalidValue;
+        if (silu) quantize_q8_0_kernel<AOS, true, true><<<grid, threads, 0, s>>>(x, row_ids, m, k, pre.aux, out);
+        else quantize_q8_0_kernel<AOS, true, false><<<grid, threads, 0, s>>>(x, row_ids, m, k, nullptr, out);
     }
     return hipGetLastError();
 }
 
 }  // namespace
 
-hipError_t cq_launch_quantize_act_aos(int act_dtype, const float *x, int64_t m, int64_t k, void *dst, hipStream_t s) {
+hipError_t cq_launch_quantize_act_aos(int act_dtype, const float *x, int64_t m, int64_t k, cq_pre pre, void *dst,
+                                      hipStream_t s) {
     Sink out{};
     out.aos = (uint8_t *)dst;
-    return launch<true>(act_dtype, x, nullptr, m, k, out, s);
+    return launch<true>(act_dtype, x, nullptr, m, k, pre, out, s);
 }
 
 hipError_t cq_launch_quantize_act_ws(int act_dtype, const float *x, const int32_t *row_ids, int64_t m, int64_t k,
-                                     cq_act_view v, hipStream_t s) {
+                                     cq_pre pre, cq_act_view v, hipStream_t s) {
     Sink out{};
     out.v = v;
-    return launch<false>(act_dtype, x, row_ids, m, k, out, s);
+    return launch<false>(act_dtype, x, row_ids, m, k, pre, out, s);
 }

@@ -17,6 +17,7 @@ LIB_PATH = os.environ.get("CQ_LIB_PATH", os.path.join(_HERE, "lib", "libcandle_q
 Q4_0, Q8_0, Q8_1, Q4K, Q6K, Q8K = 2, 8, 9, 12, 14, 15
 FLAG_AUTO, FLAG_FORCE_MATVEC, FLAG_FORCE_GEMM, FLAG_ACT_Q8_1, FLAG_REUSE_ACT, FLAG_STAGED_ACT = 0, 1, 2, 4, 8, 16
 FLAG_FORCE_SKINNY = 32
+PRE_NONE, PRE_RMS_NORM, PRE_SILU_MUL = 0, 1, 2
 
 EXPORTS = [
     "cq_device_count", "cq_last_error", "cq_version", "cq_block_size", "cq_type_size", "cq_vec_dot_type",
@@ -25,7 +26,7 @@ EXPORTS = [
     "cq_weight_device", "cq_weight_shape", "cq_weight_destroy", "cq_act_bytes", "cq_quantize_act",
     "cq_workspace_bytes", "cq_qmatmul", "cq_qmatmul_int_dots", "cq_grouped_workspace_bytes",
     "cq_qmatmul_grouped", "cq_silu_mul", "cq_moe_scatter_add", "cq_timing_arm", "cq_timing_elapsed_us",
-    "cq_selfcheck_round",
+    "cq_selfcheck_round", "cq_quantize_act_fused", "cq_qmatmul_fused", "cq_qmatmul_grouped_fused",
 ]
 
 
@@ -75,6 +76,10 @@ def load():
     L.cq_timing_arm.argtypes = []
     L.cq_timing_elapsed_us.argtypes = [C.POINTER(C.c_double)]
     L.cq_selfcheck_round.argtypes = [ci, C.POINTER(C.c_uint64)]
+    L.cq_quantize_act_fused.argtypes = [ci, ci, ci, vp, vp, C.c_float, i64, i64, vp, vp]
+    L.cq_qmatmul_fused.argtypes = [vp, ci, vp, vp, C.c_float, i64, vp, ci, vp, sz, vp]
+    L.cq_qmatmul_grouped_fused.argtypes = [C.POINTER(vp), ci, ci, vp, vp, C.c_float, vp, C.POINTER(C.c_int32), vp, ci,
+                                           vp, sz, vp]
     _lib = L
     return L
 
@@ -205,27 +210,53 @@ class QWeight:
         return load().cq_workspace_bytes(self._h, m, flags)
 
 
-def quantize_act(act_dtype: int, x):
-    """T::VecDotType::from_float over the rows of x [m, k]: returns a uint8 device tensor holding
-    the GGML blocks."""
+def _check_pre(pre: int, x, aux):
+    """Shape rules of the fused steps: alpha [k] for rms_norm, a second operand shaped like x for
+    silu * mul (rms_norm's own check: candle-nn/src/ops.rs:641-650)."""
+    if pre == PRE_NONE:
+        return
+    _require_f32_cuda(aux, "aux")
+    if pre == PRE_RMS_NORM:
+        if aux.dim() != 1 or aux.shape[0] != x.shape[-1]:
+            raise QHipError(f"shape mismatch in rms-norm {tuple(x.shape)} {tuple(aux.shape)}")
+    elif pre == PRE_SILU_MUL:
+        if tuple(aux.shape) != tuple(x.shape):
+            raise QHipError(f"shape mismatch in silu-mul {tuple(x.shape)} {tuple(aux.shape)}")
+    else:
+        raise QHipError(f"unknown fused step {pre}")
+
+
+def quantize_act(act_dtype: int, x, pre: int = PRE_NONE, aux=None, eps: float = 0.0):
+    """T::VecDotType::from_float over the rows of x [m, k] (after the fused step `pre`, if any):
+    returns a uint8 device tensor holding the GGML blocks."""
     torch = _torch()
     L = load()
     _require_f32_cuda(x)
+    _check_pre(pre, x, aux)
     m, k = x.shape
     nbytes = L.cq_act_bytes(act_dtype, m, k)
     if nbytes == 0 and m * k != 0:
         raise QHipError(f"{k} is not divisible by the block size of dtype {act_dtype}")
     out = torch.zeros(max(nbytes, 4), dtype=torch.uint8, device=x.device)
-    check(L.cq_quantize_act(x.device.index or 0, act_dtype, C.c_void_p(x.data_ptr()), m, k,
-                            C.c_void_p(out.data_ptr()), _stream_ptr()))
+    if pre == PRE_NONE:
+        check(L.cq_quantize_act(x.device.index or 0, act_dtype, C.c_void_p(x.data_ptr()), m, k,
+                                C.c_void_p(out.data_ptr()), _stream_ptr()))
+    else:
+        check(L.cq_quantize_act_fused(x.device.index or 0, act_dtype, pre, C.c_void_p(x.data_ptr()),
+                                      C.c_void_p(aux.data_ptr()), eps, m, k, C.c_void_p(out.data_ptr()),
+                                      _stream_ptr()))
     return out[:nbytes]
 
 
-def qmatmul(w: QWeight, x, flags: int = 0, out=None, workspace: Workspace | None = None):
-    """QMatMul::forward for a quantized weight: x [..., k] f32 contiguous -> [..., n]."""
+def qmatmul(w: QWeight, x, flags: int = 0, out=None, workspace: Workspace | None = None, pre: int = PRE_NONE,
+            aux=None, eps: float = 0.0):
+    """QMatMul::forward for a quantized weight: x [..., k] f32 contiguous -> [..., n].  With `pre`
+    the model step in front of the matmul (rms_norm with alpha = aux, or silu(x) * aux) is computed
+    inside the same launches."""
     torch = _torch()
     L = load()
     _require_f32_cuda(x)
+    _check_pre(pre, x, aux)
     n, k = w.shape
     if x.dim() < 2:
         raise QHipError(f"input tensor has only one dimension {tuple(x.shape)}")   # mod.rs:480-482
@@ -237,8 +268,13 @@ def qmatmul(w: QWeight, x, flags: int = 0, out=None, workspace: Workspace | None
         out = torch.empty(out_shape, dtype=torch.float32, device=x.device)
     need = L.cq_workspace_bytes(w.handle, m, flags)
     ws = (workspace or _default_ws).get(need, x.device)
-    check(L.cq_qmatmul(w.handle, C.c_void_p(x.data_ptr()), m, C.c_void_p(out.data_ptr()), flags,
-                       C.c_void_p(ws.data_ptr()), ws.numel(), _stream_ptr()))
+    if pre == PRE_NONE:
+        check(L.cq_qmatmul(w.handle, C.c_void_p(x.data_ptr()), m, C.c_void_p(out.data_ptr()), flags,
+                           C.c_void_p(ws.data_ptr()), ws.numel(), _stream_ptr()))
+    else:
+        check(L.cq_qmatmul_fused(w.handle, pre, C.c_void_p(x.data_ptr()), C.c_void_p(aux.data_ptr()), eps, m,
+                                 C.c_void_p(out.data_ptr()), flags, C.c_void_p(ws.data_ptr()), ws.numel(),
+                                 _stream_ptr()))
     return out
 
 
@@ -259,11 +295,14 @@ def qmatmul_int_dots(w: QWeight, x):
     return oi, om
 
 
-def qmatmul_grouped(experts, x, row_ids, offsets, flags: int = 0, workspace: Workspace | None = None):
-    """y[p] = x[row_ids[p]] . W_e^T for p in [offsets[e], offsets[e+1]); offsets is a host int32 array."""
+def qmatmul_grouped(experts, x, row_ids, offsets, flags: int = 0, workspace: Workspace | None = None,
+                    pre: int = PRE_NONE, aux=None, eps: float = 0.0):
+    """y[p] = x[row_ids[p]] . W_e^T for p in [offsets[e], offsets[e+1]); offsets is a host int32 array.
+    With `pre`, the gathered rows go through that step first (aux rows gathered like x rows)."""
     torch = _torch()
     L = load()
     _require_f32_cuda(x)
+    _check_pre(pre, x, aux)
     n, k = experts[0].shape
     offsets = np.ascontiguousarray(offsets, dtype=np.int32)
     total = int(offsets[-1])
@@ -272,9 +311,15 @@ def qmatmul_grouped(experts, x, row_ids, offsets, flags: int = 0, workspace: Wor
     need = L.cq_grouped_workspace_bytes(arr, len(experts), total, flags)
     ws = (workspace or _default_ws).get(need, x.device)
     rid = C.c_void_p(row_ids.data_ptr()) if row_ids is not None else None
-    check(L.cq_qmatmul_grouped(arr, len(experts), C.c_void_p(x.data_ptr()), rid,
-                               offsets.ctypes.data_as(C.POINTER(C.c_int32)), C.c_void_p(y.data_ptr()), flags,
-                               C.c_void_p(ws.data_ptr()), ws.numel(), _stream_ptr()))
+    if pre == PRE_NONE:
+        check(L.cq_qmatmul_grouped(arr, len(experts), C.c_void_p(x.data_ptr()), rid,
+                                   offsets.ctypes.data_as(C.POINTER(C.c_int32)), C.c_void_p(y.data_ptr()), flags,
+                                   C.c_void_p(ws.data_ptr()), ws.numel(), _stream_ptr()))
+    else:
+        check(L.cq_qmatmul_grouped_fused(arr, len(experts), pre, C.c_void_p(x.data_ptr()), C.c_void_p(aux.data_ptr()),
+                                         eps, rid, offsets.ctypes.data_as(C.POINTER(C.c_int32)),
+                                         C.c_void_p(y.data_ptr()), flags, C.c_void_p(ws.data_ptr()), ws.numel(),
+                                         _stream_ptr()))
     return y
 
 

@@ -173,5 +173,16 @@ class QMatMul:
         last dim == k; result has xs' shape with the last dim replaced by n."""
         return qhip.qmatmul(self.qtensor.weight, xs, workspace=self._ws)
 
+    def forward_rms_norm(self, xs, alpha, eps: float):
+        """`self.forward(rms_norm(xs, alpha, eps))` (RmsNorm::forward, candle-transformers/src/
+        quantized_nn.rs:121-125, in front of a projection as in quantized_llama.rs:453-466) without
+        the normalised tensor going to memory."""
+        return qhip.qmatmul(self.qtensor.weight, xs, workspace=self._ws, pre=qhip.PRE_RMS_NORM, aux=alpha, eps=eps)
+
+    def forward_silu_mul(self, gate, up):
+        """`self.forward(silu(gate) * up)`: the feed-forward's w2 applied to silu(w1 x) * (w3 x)
+        (Mlp::forward, quantized_llama.rs:56-63)."""
+        return qhip.qmatmul(self.qtensor.weight, gate, workspace=self._ws, pre=qhip.PRE_SILU_MUL, aux=up)
+
     def dequantize_f16(self):
         return self.qtensor.dequantize_f16()

@@ -61,6 +61,13 @@ enum {
                                  (two launches, as cuda.rs:249-293 does) instead of the single fused launch           */
 };
 
+/* the model step a fused call computes on the way into the activation quantizer */
+enum {
+    CQ_PRE_NONE = 0,
+    CQ_PRE_RMS_NORM = 1, /* x / sqrt(mean(x^2) + eps) * alpha[k]   (candle-nn/src/ops.rs:482-495)                  */
+    CQ_PRE_SILU_MUL = 2  /* silu(x) * x2, x2 shaped like x         (quantized_llama.rs:56-63, candle-core op.rs:607-609) */
+};
+
 typedef struct cq_weight cq_weight;
 
 /* ---- library / device ---------------------------------------------------- */
@@ -144,6 +151,31 @@ int cq_silu_mul(int dev, const float *a_dev, const float *b_dev, float *h_dev, i
  * increasing p, which is increasing expert index, like the reference's sequential loop. */
 int cq_moe_scatter_add(int dev, const float *y_dev, const int32_t *row_ids_dev, const float *weights_dev,
                        int64_t total_rows, int64_t hidden, float *ys_dev, int64_t tokens, void *stream);
+
+/* ---- the matmul with the preceding model step fused in --------------------------------------
+ * What the quantized models run directly in front of a QMatMul, computed on the way into the
+ * activation quantizer so that the intermediate tensor never goes to memory:
+ *   CQ_PRE_RMS_NORM: RmsNorm::forward (candle-transformers/src/quantized_nn.rs:121-125 ->
+ *     candle_nn::ops::rms_norm, candle-nn/src/ops.rs:482-495) in front of the attention and
+ *     feed-forward projections (quantized_llama.rs:453-466): aux = alpha[k], eps as given.
+ *   CQ_PRE_SILU_MUL: silu(w1 x) * (w3 x) in front of w2 (Mlp::forward, quantized_llama.rs:56-63;
+ *     the expert loop :124-131): x = w1's output, aux = w3's output, both [m, k]; eps unused.
+ * Equivalent to the unfused sequence up to rounding: rms_norm is computed as the reference's device
+ * kernel does, (1 / sqrt(mean + eps)) * x * alpha (candle-kernels/src/reduce.cu:161-172), with the
+ * squares added pairwise in an order that does not depend on m; the CPU code adds them one by one
+ * and divides.  silu * mul is the reference's sequence of operations (the exp is the device's).
+ * aux is 16-byte aligned like x.  For one row this is still one launch.
+ * cq_quantize_act_fused is the quantizer half on its own, for byte comparison with the CPU path. */
+int cq_quantize_act_fused(int dev, int act_dtype, int pre, const float *x_dev, const float *aux_dev, float eps,
+                          int64_t m, int64_t k, void *dst_blocks_dev, void *stream);
+int cq_qmatmul_fused(const cq_weight *w, int pre, const float *x_dev, const float *aux_dev, float eps, int64_t m,
+                     float *y_dev, int flags, void *workspace_dev, size_t workspace_bytes, void *stream);
+/* cq_qmatmul_grouped with the same step applied to the gathered rows (row p reads x and aux at
+ * row_ids[p], or p when row_ids is NULL). */
+int cq_qmatmul_grouped_fused(const cq_weight *const *experts, int n_experts, int pre, const float *x_dev,
+                             const float *aux_dev, float eps, const int32_t *row_ids_dev,
+                             const int32_t *offsets_host, float *y_dev, int flags, void *workspace_dev,
+                             size_t workspace_bytes, void *stream);
 
 /* ---- measurement aid (no counterpart in the reference) ---------------------------------------
  * cq_timing_arm(): the next matmul kernel this host thread launches through cq_qmatmul (the

@@ -20,6 +20,11 @@
  *                                               : :647-651, :640, :666, :1122, :786-861
  *   f16 conversion                              : exhaustive comparison with numpy.float16
  *   softmax / silu / top-k MoE combine          : brute-force dense-masked MoE on tiny sizes
+ *   rms_norm (candle-nn/src/ops.rs:482-495)     : reference golden candle-nn/tests/ops.rs:55-66
+ *        (4 decimals) and the closed form x / sqrt(mean(x^2) + eps) * alpha in float64
+ *   silu_mul (op.rs:607-609, quantized_llama.rs:60-62) : closed form in float64 (no reference
+ *        golden prints silu of known inputs on this path; PARITY UNPINNED beyond that: the last
+ *        bits depend on the platform's expf)
  *   q8_1 quantize (k_quants.rs:665-691)         : PARITY UNPINNED by any reference
  *        golden (no reference test inspects its output); checked only against
  *        the closed form "q8_0 plus s = f16(f16(sum q) * d)".
@@ -1022,4 +1027,26 @@ int orc_moe_ffn(int n_experts, int dtype13, int dtype2, const void *const *w1, c
         if (rc) return rc;
     }
     return 0;
+}
+
+/* candle-nn/src/ops.rs:482-495 (RmsNorm::cpu_fwd, f32): per row of `dim` elements the squares are
+ * added one by one in f32, m = sqrt(sum / dim + eps), then dst = src / m * alpha. */
+void orc_rms_norm(const float *x, const float *alpha, float eps, int64_t rows, int64_t dim, float *out) {
+    for (int64_t r = 0; r < rows; r++) {
+        const float *src = x + r * dim;
+        float *dst = out + r * dim;
+        float sum2 = 0.0f;
+        for (int64_t i = 0; i < dim; i++) sum2 += src[i] * src[i];
+        float m = sqrtf(sum2 / (float)dim + eps);
+        for (int64_t i = 0; i < dim; i++) dst[i] = src[i] / m * alpha[i];
+    }
+}
+
+/* quantized_llama.rs:60-62: silu(w1) * w3 with silu(v) = v / (1 + exp(-v)) (op.rs:607-609). */
+void orc_silu_mul(const float *a, const float *b, int64_t count, float *out) {
+    for (int64_t i = 0; i < count; i++) {
+        float v = a[i];
+        float s = v / (1.0f + expf(-v));
+        out[i] = s * b[i];
+    }
 }

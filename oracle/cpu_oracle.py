@@ -57,6 +57,10 @@ def lib():
         L.orc_moe_route.argtypes = [f32p, i64, C.c_int, C.c_int, i32p, i32p, f32p]
         L.orc_moe_ffn.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(vp), C.POINTER(vp), C.POINTER(vp),
                                   i64, i64, f32p, i64, i32p, i32p, f32p, f32p]
+        L.orc_rms_norm.argtypes = [f32p, f32p, C.c_float, i64, i64, f32p]
+        L.orc_rms_norm.restype = None
+        L.orc_silu_mul.argtypes = [f32p, f32p, i64, f32p]
+        L.orc_silu_mul.restype = None
         _lib = L
     return _lib
 
@@ -147,6 +151,26 @@ def softmax_last_dim(x) -> np.ndarray:
     x, xp = _f32(x)
     out = np.empty_like(x)
     lib().orc_softmax_last_dim(xp, out.ctypes.data_as(C.POINTER(C.c_float)), x.size // x.shape[-1], x.shape[-1])
+    return out
+
+
+def rms_norm(x, alpha, eps: float) -> np.ndarray:
+    """candle_nn::ops::rms_norm on f32 (candle-nn/src/ops.rs:482-495) over the last dimension."""
+    x, xp = _f32(x)
+    alpha, ap = _f32(alpha)
+    assert alpha.ndim == 1 and alpha.shape[0] == x.shape[-1]
+    out = np.empty_like(x)
+    lib().orc_rms_norm(xp, ap, eps, x.size // x.shape[-1], x.shape[-1], out.ctypes.data_as(C.POINTER(C.c_float)))
+    return out
+
+
+def silu_mul(a, b) -> np.ndarray:
+    """silu(a) * b as in Mlp::forward (quantized_llama.rs:60-62, op.rs:607-609)."""
+    a, ap = _f32(a)
+    b, bp = _f32(b)
+    assert a.shape == b.shape
+    out = np.empty_like(a)
+    lib().orc_silu_mul(ap, bp, a.size, out.ctypes.data_as(C.POINTER(C.c_float)))
     return out
 
 

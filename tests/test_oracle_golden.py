@@ -379,3 +379,31 @@ def test_moe_route_and_ffn_match_dense_masked():
             mask[row_ids[p]] = weights[p]
         dense += out.astype(np.float64) * mask[:, None]
     assert np.linalg.norm(ys - dense) / np.linalg.norm(dense) < 1e-5
+
+
+# ------------------------------------------- neighbours of the matmul: rms_norm, silu * mul ----
+def test_rms_norm_golden_and_closed_form(goldens):
+    g = goldens["rms_norm_2x2x3"]
+    x = np.array(g["x"], dtype=np.float32)
+    got = orc.rms_norm(x, np.array(g["alpha"], dtype=np.float32), g["eps"])
+    assert np.round(got.astype(np.float64), 4).tolist() == g["rounded4"]
+    # closed form in float64 on a long row; a dropped eps, a missing division by the row length or
+    # alpha applied before the division by m would all show
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((3, 4096)) * 3).astype(np.float32)
+    alpha = (1 + 0.1 * rng.standard_normal(4096)).astype(np.float32)
+    want = x.astype(np.float64) / np.sqrt((x.astype(np.float64) ** 2).mean(-1, keepdims=True) + 0.5) * alpha
+    got = orc.rms_norm(x, alpha, 0.5)
+    assert np.abs(got - want).max() <= 2e-6 * np.abs(want).max()
+    assert np.abs(orc.rms_norm(x, alpha, 1e-5) - want).max() > 1e-3   # eps matters at this size
+
+
+def test_silu_mul_closed_form():
+    rng = np.random.default_rng(6)
+    a = np.concatenate([rng.standard_normal(4000) * 4, [0.0, -0.0, 30.0, -30.0, 88.0, -88.0, -104.0]]).astype(np.float32)
+    b = rng.standard_normal(a.size).astype(np.float32)
+    got = orc.silu_mul(a, b)
+    a64 = a.astype(np.float64)
+    want = a64 / (1 + np.exp(-a64)) * b
+    assert np.abs(got - want).max() <= 1e-6 * np.abs(want).max()
+    assert got[4000] == 0.0 and abs(got[4002] - 30.0 * b[4002]) < 1e-5 and abs(got[4006]) < 1e-30
