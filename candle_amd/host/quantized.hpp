@@ -154,19 +154,31 @@ class QHipStorage {
     }
     // cuda.rs:478-499 `fwd(self_shape, storage, layout)`: x contiguous f32, rank 2 or 3 (any rank >= 2
     // here, as on the CPU), last dim == k; the result owns a fresh allocation.
-    Tensor fwd(const Shape &self_shape, const Tensor &x, hipStream_t stream = nullptr) const {
+    // `pre` != CQ_PRE_NONE: the model step in front of the projection computed inside the same
+    // launches: rms_norm with alpha = *aux (candle-nn/src/ops.rs:641-652), or silu(x) * *aux
+    // (quantized_llama.rs:60-62).
+    Tensor fwd(const Shape &self_shape, const Tensor &x, hipStream_t stream = nullptr, int pre = CQ_PRE_NONE,
+               const Tensor *aux = nullptr, float eps = 0.0f) const {
         if (self_shape.size() != 2) throw Error("QHipStorage::fwd: weight must be rank 2, got " + to_string(self_shape));
         const int64_t n = self_shape[0], k = self_shape[1];
         if (x.rank() < 2) throw Error("input tensor has only one dimension " + to_string(x.shape));       // mod.rs:480-482
         if (x.shape.back() != k)
             throw Error("input tensor " + to_string(x.shape) + " incompatible with " + to_string(self_shape));  // mod.rs:485-487
+        if (pre == CQ_PRE_RMS_NORM && (!aux || aux->shape != Shape{k}))
+            throw Error("shape mismatch in rms-norm " + to_string(x.shape) + " " + (aux ? to_string(aux->shape) : "none"));  // ops.rs:644-650
+        if (pre == CQ_PRE_SILU_MUL && (!aux || aux->shape != x.shape))
+            throw Error("shape mismatch in silu-mul " + to_string(x.shape) + " " + (aux ? to_string(aux->shape) : "none"));
         const int64_t m = k ? elem_count(x.shape) / k : 0;
         Shape out_shape = x.shape;
         out_shape.back() = n;
         Tensor y{out_shape, DeviceBuffer<float>((size_t)(m * n))};
         const size_t ws_bytes = cq_workspace_bytes(w_, m, CQ_FLAG_AUTO);
         DeviceBuffer<uint8_t> ws(ws_bytes);   // per call, like the reference's quantized-activation buffer (cuda.rs:249-252)
-        check(cq_qmatmul(w_, x.data.get(), m, y.data.get(), CQ_FLAG_AUTO, ws.get(), ws_bytes, stream), "QHipStorage::fwd");
+        if (pre == CQ_PRE_NONE)
+            check(cq_qmatmul(w_, x.data.get(), m, y.data.get(), CQ_FLAG_AUTO, ws.get(), ws_bytes, stream), "QHipStorage::fwd");
+        else
+            check(cq_qmatmul_fused(w_, pre, x.data.get(), aux->data.get(), eps, m, y.data.get(), CQ_FLAG_AUTO, ws.get(),
+                                   ws_bytes, stream), "QHipStorage::fwd");
         // the workspace is freed when this returns; hipFree waits for the device, as dropping a
         // CudaSlice synchronises with its stream
         return y;
@@ -222,6 +234,15 @@ class QMatMul {
     // y = xs . W^T; xs [.., k] -> [.., n]
     Tensor forward(const Tensor &xs, hipStream_t stream = nullptr) const {
         return qtensor_->storage().fwd(qtensor_->shape(), xs, stream);
+    }
+    // forward(rms_norm(xs, alpha, eps)): RmsNorm::forward (candle-transformers/src/quantized_nn.rs:121-125)
+    // in front of a projection (quantized_llama.rs:453-466), without the normalised tensor in memory
+    Tensor forward_rms_norm(const Tensor &xs, const Tensor &alpha, float eps, hipStream_t stream = nullptr) const {
+        return qtensor_->storage().fwd(qtensor_->shape(), xs, stream, CQ_PRE_RMS_NORM, &alpha, eps);
+    }
+    // forward(silu(gate) * up): the feed-forward's w2 (Mlp::forward, quantized_llama.rs:56-63)
+    Tensor forward_silu_mul(const Tensor &gate, const Tensor &up, hipStream_t stream = nullptr) const {
+        return qtensor_->storage().fwd(qtensor_->shape(), gate, stream, CQ_PRE_SILU_MUL, &up);
     }
     const QTensor &qtensor() const { return *qtensor_; }
 

@@ -86,6 +86,39 @@ static void roundtrip() {
     EXPECT(worst < 0.017f, "Q4K round-trip max error %f", worst);
 }
 
+static void fused_neighbours() {
+    // forward_rms_norm / forward_silu_mul against forward() on inputs prepared on the host
+    const int m = 3, k = 512, n = 16;
+    std::vector<float> w((size_t)(n * k)), x((size_t)(m * k)), u((size_t)(m * k)), alpha((size_t)k);
+    for (int i = 0; i < n * k; i++) w[(size_t)i] = 0.02f * std::sin(0.37f * (float)i);
+    for (int i = 0; i < m * k; i++) { x[(size_t)i] = 2.0f * std::cos(0.11f * (float)i); u[(size_t)i] = std::sin(0.05f * (float)i); }
+    for (int i = 0; i < k; i++) alpha[(size_t)i] = 1.0f + 0.1f * std::sin((float)i);
+    QMatMul mm = QMatMul::from_qtensor(QTensor::quantize(Tensor::from_host(w, {n, k}), GgmlDType::Q4K));
+    const float eps = 1e-5f;
+    std::vector<float> xn(x.size()), su(x.size());
+    for (int r = 0; r < m; r++) {
+        float sum2 = 0.f;
+        for (int i = 0; i < k; i++) sum2 += x[(size_t)(r * k + i)] * x[(size_t)(r * k + i)];
+        const float root = std::sqrt(sum2 / (float)k + eps);
+        for (int i = 0; i < k; i++) xn[(size_t)(r * k + i)] = x[(size_t)(r * k + i)] / root * alpha[(size_t)i];
+    }
+    for (size_t i = 0; i < x.size(); i++) su[i] = x[i] / (1.0f + std::exp(-x[i])) * u[i];
+    auto close = [&](const std::vector<float> &a, const std::vector<float> &b, const char *what) {
+        double num = 0, den = 0;
+        for (size_t i = 0; i < a.size(); i++) { num += ((double)a[i] - b[i]) * ((double)a[i] - b[i]); den += (double)b[i] * b[i]; }
+        EXPECT(a.size() == b.size() && std::sqrt(num) <= 1e-4 * std::sqrt(den), "%s: relative L2 %g", what, std::sqrt(num / den));
+    };
+    Tensor xt = Tensor::from_host(x, {m, k}), ut = Tensor::from_host(u, {m, k}), at = Tensor::from_host(alpha, {k});
+    close(mm.forward_rms_norm(xt, at, eps).to_host(), mm.forward(Tensor::from_host(xn, {m, k})).to_host(), "forward_rms_norm");
+    close(mm.forward_silu_mul(xt, ut).to_host(), mm.forward(Tensor::from_host(su, {m, k})).to_host(), "forward_silu_mul");
+    Tensor one = Tensor::from_host(std::vector<float>(x.begin(), x.begin() + k), {1, k});
+    Tensor one_n = Tensor::from_host(std::vector<float>(xn.begin(), xn.begin() + k), {1, k});
+    close(mm.forward_rms_norm(one, at, eps).to_host(), mm.forward(one_n).to_host(), "forward_rms_norm, one row");
+    Tensor short_alpha = Tensor::from_host(std::vector<float>((size_t)(k - 1), 1.f), {k - 1});
+    EXPECT(throws([&] { mm.forward_rms_norm(xt, short_alpha, eps); }), "alpha of the wrong length must be an error");
+    EXPECT(throws([&] { mm.forward_silu_mul(xt, one); }), "operands of different shapes must be an error");
+}
+
 int main(int argc, char **argv) {
     const bool host = argc > 1 && std::strcmp(argv[1], "--host-only") == 0;
     try {
@@ -100,6 +133,7 @@ int main(int argc, char **argv) {
             q4_0_matmul("quantized_matmul", 0.f, 0.f, g1);
             q4_0_matmul("quantized_matmul_neg", 3 * 64 / 2.0f, 64 * 4 / 3.0f, g2);
             roundtrip();
+            fused_neighbours();
         }
     } catch (const std::exception &e) {
         std::printf("FAIL: exception: %s\n", e.what());
