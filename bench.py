@@ -304,6 +304,57 @@ def main() -> int:
     except Exception as e:  # reported beside the headline only: never fails the bench line
         print(f"bench.py: neighbour chain not measured ({e})", file=sys.stderr)
 
+    # ---- the same bytes in fewer, larger calls (reported beside the headline) -----------------------
+    # A model that keeps q|k|v and gate|up as one quantized tensor each (rows of GGML blocks simply
+    # concatenated: [12288 x 4096] and [22016 x 4096]) issues 129 QMatMul calls per step instead of 225
+    # over the same number of weight bytes.  Fresh random weights of those shapes, same kernels.
+    merged = None
+    try:
+        m_calls = []
+        for layer in range(args.layers):
+            for idx, (dt, n, k, xin) in enumerate((("q4k", 3 * HIDDEN, HIDDEN, "x_attn"), ("q4k", HIDDEN, HIDDEN, "x_o"),
+                                                   ("q4k", 2 * FFN, HIDDEN, "x_ffn"), ("q6k", HIDDEN, FFN, "x_down"))):
+                gen.manual_seed(500_000 + 10 * layer + idx)
+                w = torch.randn((n, k), generator=gen, device=dev, dtype=torch.float32) * 0.02
+                m_calls.append((qhip.QWeight.zeros(DT[dt], n, k).quantize_(w), xin, dt, n, k))
+                del w
+        m_calls.append(calls[-1])
+        m_out = [torch.empty((1, n), device=dev, dtype=torch.float32) for (_, _, _, n, _) in m_calls]
+        m_bytes = sum(ggml_bytes(dt, n, k) for (_, _, dt, n, k) in m_calls)
+
+        def m_step():
+            s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+            for (qw, xin, _, _, _), out in zip(m_calls, m_out):
+                qhip.check(L.cq_qmatmul(qw.handle, C.c_void_p(inputs[xin].data_ptr()), 1, C.c_void_p(out.data_ptr()), 0,
+                                        C.c_void_p(ws.data_ptr()), ws.numel(), s))
+
+        with torch.cuda.stream(side):
+            m_step()
+            torch.cuda.synchronize()
+            gm_ = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gm_, stream=side):
+                m_step()
+            for _ in range(3):
+                gm_.replay()
+            torch.cuda.synchronize()
+            m0, m1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            m0.record()
+            for _ in range(args.steps):
+                gm_.replay()
+            m1.record()
+            torch.cuda.synchronize()
+            m_ms = m0.elapsed_time(m1) / args.steps
+        merged = {
+            "workload": "q|k|v and gate|up stored as one tensor each: %d calls per step" % len(m_calls),
+            "weight_bytes_per_step": m_bytes,
+            "ms_per_step": round(m_ms, 4),
+            "GBs": round(m_bytes / (m_ms * 1e-3) / 1e9, 1),
+            "frac_of_hbm_peak": round(m_bytes / (m_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        }
+        del m_calls, m_out, gm_
+    except Exception as e:  # reported beside the headline only: never fails the bench line
+        print(f"bench.py: merged-projection step not measured ({e})", file=sys.stderr)
+
     value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
     result = {
         "metric": "Q4_K matvec HBM GB/s (% of peak); Q4_K M=512 GEMM TOPS (% int8 MFMA peak)",
@@ -355,6 +406,8 @@ def main() -> int:
 
     if neighbours is not None:
         result["fused_neighbours"] = neighbours
+    if merged is not None:
+        result["merged_projections"] = merged
 
     # ---- CPU baseline: restated candle CPU QMatMul (AVX2 + threads) on a bounded sample ----
     if not args.no_cpu:
