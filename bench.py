@@ -55,6 +55,9 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=LAYERS, help="(debug) fewer layers; the result is then not a bench line")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the figures reported beside the headline (fused neighbours, merged projections), "
+                         "so that a profiler run sees the headline kernels only")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain device copy of 256 MiB three times (a kernel of known HBM traffic, to "
                          "calibrate FETCH_SIZE / WRITE_SIZE counters in a profiler run)")
@@ -235,6 +238,8 @@ def main() -> int:
     # the matmul launches (cq_qmatmul_fused).  Same weights as the headline step, HIP graph replay.
     neighbours = None
     try:
+        if args.no_extras or args.no_graph:   # both extras are graph replays
+            raise RuntimeError("skipped by --no-extras / --no-graph")
         alpha = torch.ones(HIDDEN, device=dev, dtype=torch.float32)
         h_buf = torch.empty((1, FFN), device=dev, dtype=torch.float32)
         eps = 1e-5
@@ -302,7 +307,8 @@ def main() -> int:
             "fused_ms": round(times["fused"], 4),
         }
     except Exception as e:  # reported beside the headline only: never fails the bench line
-        print(f"bench.py: neighbour chain not measured ({e})", file=sys.stderr)
+        if not (args.no_extras or args.no_graph):
+            print(f"bench.py: neighbour chain not measured ({e})", file=sys.stderr)
 
     # ---- the same bytes in fewer, larger calls (reported beside the headline) -----------------------
     # A model that keeps q|k|v and gate|up as one quantized tensor each (rows of GGML blocks simply
@@ -310,6 +316,8 @@ def main() -> int:
     # over the same number of weight bytes.  Fresh random weights of those shapes, same kernels.
     merged = None
     try:
+        if args.no_extras or args.no_graph:   # both extras are graph replays
+            raise RuntimeError("skipped by --no-extras / --no-graph")
         m_calls = []
         for layer in range(args.layers):
             for idx, (dt, n, k, xin) in enumerate((("q4k", 3 * HIDDEN, HIDDEN, "x_attn"), ("q4k", HIDDEN, HIDDEN, "x_o"),
@@ -353,7 +361,8 @@ def main() -> int:
         }
         del m_calls, m_out, gm_
     except Exception as e:  # reported beside the headline only: never fails the bench line
-        print(f"bench.py: merged-projection step not measured ({e})", file=sys.stderr)
+        if not (args.no_extras or args.no_graph):
+            print(f"bench.py: merged-projection step not measured ({e})", file=sys.stderr)
 
     value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
     result = {
