@@ -16,6 +16,8 @@
  *   q8k quantize, q8k x q8k dot                 : :694-698, :1147
  *   q4k quantize (make_qkx1_quants, packing), dequant, q4k x q8k dot
  *                                               : :553-557, :546, :572, :1069, :786-861
+ *   q5k quantize (make_qkx1_quants with 31 levels), dequant, q5k x q8k dot
+ *                                               : :578-625 (spot values, < 0.009, < 2.5), :792, :1077-1098
  *   q6k quantize (make_qx_quants), dequant, q6k x q8k dot
  *                                               : :647-651, :640, :666, :1122, :786-861
  *   f16 conversion                              : exhaustive comparison with numpy.float16
@@ -60,7 +62,9 @@ typedef struct { float d; int8_t qs[QK_K]; int16_t bsums[QK_K / 16]; } block_q8k
 _Static_assert(sizeof(block_q4_0) == 18, "q4_0");
 _Static_assert(sizeof(block_q8_0) == 34, "q8_0");
 _Static_assert(sizeof(block_q8_1) == 36, "q8_1");
+typedef struct { uint16_t d; uint16_t dmin; uint8_t scales[K_SCALE_SIZE]; uint8_t qh[QK_K / 8]; uint8_t qs[QK_K / 2]; } block_q5k; /* 176, k_quants.rs:119-127 */
 _Static_assert(sizeof(block_q4k) == 144, "q4k");
+_Static_assert(sizeof(block_q5k) == 176, "q5k");
 _Static_assert(sizeof(block_q6k) == 210, "q6k");
 _Static_assert(sizeof(block_q8k) == 292, "q8k");
 
@@ -502,6 +506,142 @@ static float vec_dot_q4k_q8k(int64_t n, const block_q4k *xs, const block_q8k *ys
     return sumf + t;
 }
 
+/* ---------------------------------------------------------------- Q5K ---- */
+/* k_quants.rs:1450-1525 */
+int orc_quantize_q5k(const float *xs, void *out, int64_t k) {
+    if (k % QK_K != 0) return -1;
+    block_q5k *ys = (block_q5k *)out;
+    for (int64_t ib = 0; ib < k / QK_K; ib++) {
+        const float *x = xs + ib * QK_K;
+        block_q5k *block = &ys[ib];
+        memset(block->scales, 0, K_SCALE_SIZE); /* blocks come from zeros() in the reference */
+        float mins[8], scales[8];
+        for (int j = 0; j < 8; j++) make_qkx1_quants(31, 5, x + 32 * j, 32, &scales[j], &mins[j]);
+        float max_scale = 0.0f, max_min = 0.0f;
+        for (int j = 0; j < 8; j++) max_scale = fmaxf(scales[j], max_scale);
+        for (int j = 0; j < 8; j++) max_min = fmaxf(mins[j], max_min);
+        float inv_scale = max_scale > 0.0f ? 63.0f / max_scale : 0.0f;
+        float inv_min = max_min > 0.0f ? 63.0f / max_min : 0.0f;
+        for (int j = 0; j < 8; j++) {
+            int32_t lsi = nearest_int(inv_scale * scales[j]); if (lsi > 63) lsi = 63;
+            int32_t lmi = nearest_int(inv_min * mins[j]); if (lmi > 63) lmi = 63;
+            uint8_t ls = (uint8_t)lsi, lm = (uint8_t)lmi;
+            if (j < 4) {
+                block->scales[j] = ls;
+                block->scales[j + 4] = lm;
+            } else {
+                block->scales[j + 4] = (uint8_t)((ls & 0xF) | ((lm & 0xF) << 4));
+                block->scales[j - 4] |= (uint8_t)((ls >> 4) << 6);
+                block->scales[j] |= (uint8_t)((lm >> 4) << 6);
+            }
+        }
+        block->d = orc_f32_to_f16(max_scale / 63.0f);
+        block->dmin = orc_f32_to_f16(max_min / 63.0f);
+        uint8_t l[QK_K];
+        memset(l, 0, sizeof(l));
+        for (int j = 0; j < 8; j++) {
+            uint8_t sc, m;
+            get_scale_min_k4(j, block->scales, &sc, &m);
+            float d = orc_f16_to_f32(block->d) * (float)sc;
+            if (d != 0.0f) {
+                float dm = orc_f16_to_f32(block->dmin) * (float)m;
+                for (int ii = 0; ii < 32; ii++) {
+                    int32_t lv = nearest_int((x[32 * j + ii] + dm) / d);
+                    l[32 * j + ii] = (uint8_t)clampi(lv, 0, 31);
+                }
+            }
+        }
+        memset(block->qh, 0, sizeof(block->qh));
+        uint8_t m1 = 1, m2 = 2;
+        for (int n = 0; n < QK_K; n += 64) {
+            int offset = (n / 64) * 32;
+            for (int j = 0; j < 32; j++) {
+                uint8_t l1 = l[n + j], l2 = l[n + j + 32];
+                if (l1 > 15) { l1 -= 16; block->qh[j] |= m1; }
+                if (l2 > 15) { l2 -= 16; block->qh[j] |= m2; }
+                block->qs[offset + j] = (uint8_t)(l1 | (l2 << 4));
+            }
+            m1 <<= 2;
+            m2 <<= 2;
+        }
+    }
+    return 0;
+}
+
+/* k_quants.rs:1527-1564 */
+int orc_dequantize_q5k(const void *in, float *ys, int64_t k) {
+    if (k % QK_K != 0) return -1;
+    const block_q5k *xs = (const block_q5k *)in;
+    for (int64_t ib = 0; ib < k / QK_K; ib++) {
+        const block_q5k *b = &xs[ib];
+        float d = orc_f16_to_f32(b->d), min = orc_f16_to_f32(b->dmin);
+        float *y = ys + ib * QK_K;
+        int is = 0, yi = 0;
+        uint8_t u1 = 1, u2 = 2;
+        for (int j = 0; j < QK_K; j += 64) {
+            const uint8_t *ql = b->qs + j / 2;
+            uint8_t sc, m;
+            get_scale_min_k4(is, b->scales, &sc, &m);
+            float d1 = d * (float)sc, m1 = min * (float)m;
+            get_scale_min_k4(is + 1, b->scales, &sc, &m);
+            float d2 = d * (float)sc, m2 = min * (float)m;
+            for (int l = 0; l < 32; l++) y[yi++] = d1 * (float)((ql[l] & 0xF) + ((b->qh[l] & u1) ? 16 : 0)) - m1;
+            for (int l = 0; l < 32; l++) y[yi++] = d2 * (float)((ql[l] >> 4) + ((b->qh[l] & u2) ? 16 : 0)) - m2;
+            is += 2;
+            u1 <<= 2;
+            u2 <<= 2;
+        }
+    }
+    return 0;
+}
+
+/* Per-block integer parts of Q5K x Q8K (k_quants.rs:1380-1438), as for Q4K with the fifth bit of
+ * each quant taken from qh: bit 2g of qh[l] for element 64g + l, bit 2g+1 for element 64g + 32 + l. */
+static inline void ints_q5k_q8k(const block_q5k *x, const block_q8k *y, int32_t aux32[8], int32_t *sumi) {
+    int8_t aux8[QK_K];
+    uint8_t m = 1;
+    for (int g = 0; g < 4; g++) {
+        for (int l = 0; l < 32; l++) aux8[64 * g + l] = (int8_t)((x->qs[32 * g + l] & 0xF) + ((x->qh[l] & m) ? 16 : 0));
+        m <<= 1;
+        for (int l = 0; l < 32; l++) aux8[64 * g + 32 + l] = (int8_t)((x->qs[32 * g + l] >> 4) + ((x->qh[l] & m) ? 16 : 0));
+        m <<= 1;
+    }
+    uint8_t scales[8], mins[8];
+    for (int j = 0; j < 8; j++) get_scale_min_k4(j, x->scales, &scales[j], &mins[j]);
+    int32_t s = 0;
+    for (int j = 0; j < 16; j++) s += (int32_t)y->bsums[j] * (int32_t)mins[j / 2];
+    *sumi = s;
+    for (int l = 0; l < 8; l++) aux32[l] = 0;
+    const int8_t *a = aux8, *q8 = y->qs;
+    for (int j = 0; j < 8; j++) {
+        int32_t scale = scales[j];
+        for (int r = 0; r < 4; r++) {
+            for (int l = 0; l < 8; l++) {
+                int16_t p = (int16_t)((int16_t)q8[l] * (int16_t)a[l]);
+                aux32[l] += scale * (int32_t)p;
+            }
+            q8 += 8; a += 8;
+        }
+    }
+}
+
+/* k_quants.rs:1361-1447 (vec_dot_unopt) */
+static float vec_dot_q5k_q8k(int64_t n, const block_q5k *xs, const block_q8k *ys) {
+    float sums[8] = {0};
+    float sumf = 0.0f;
+    for (int64_t i = 0; i < n / QK_K; i++) {
+        int32_t aux32[8], sumi;
+        ints_q5k_q8k(&xs[i], &ys[i], aux32, &sumi);
+        float d = orc_f16_to_f32(xs[i].d) * ys[i].d;
+        for (int l = 0; l < 8; l++) sums[l] += d * (float)aux32[l];
+        float dmin = orc_f16_to_f32(xs[i].dmin) * ys[i].d;
+        sumf -= dmin * (float)sumi;
+    }
+    float t = 0.0f;
+    for (int l = 0; l < 8; l++) t += sums[l];
+    return sumf + t;
+}
+
 /* ---------------------------------------------------------------- Q6K ---- */
 /* utils.rs:61-198 */
 static float make_qx_quants(int n, int32_t nmax, const float *x, int8_t *ls, int rmse_type) {
@@ -740,14 +880,14 @@ static inline int32_t int_q6k_q8k(const block_q6k *x, const block_q8k *y) {
 int64_t orc_block_size(int dtype) {
     switch (dtype) {
     case ORC_Q4_0: case ORC_Q8_0: case ORC_Q8_1: return 32;
-    case ORC_Q4K: case ORC_Q6K: case ORC_Q8K: return QK_K;
+    case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return QK_K;
     default: return 0;
     }
 }
 int64_t orc_type_size(int dtype) {
     switch (dtype) {
     case ORC_Q4_0: return 18; case ORC_Q8_0: return 34; case ORC_Q8_1: return 36;
-    case ORC_Q4K: return 144; case ORC_Q6K: return 210; case ORC_Q8K: return 292;
+    case ORC_Q4K: return 144; case ORC_Q5K: return 176; case ORC_Q6K: return 210; case ORC_Q8K: return 292;
     default: return 0;
     }
 }
@@ -756,7 +896,7 @@ int64_t orc_type_size(int dtype) {
 int orc_vec_dot_type(int dtype) {
     switch (dtype) {
     case ORC_Q4_0: case ORC_Q8_0: return ORC_Q8_0;
-    case ORC_Q4K: case ORC_Q6K: case ORC_Q8K: return ORC_Q8K;
+    case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return ORC_Q8K;
     default: return -1;
     }
 }
@@ -767,6 +907,7 @@ int orc_quantize(int dtype, const float *xs, void *out, int64_t k) {
     case ORC_Q8_0: return orc_quantize_q8_0(xs, out, k);
     case ORC_Q8_1: return orc_quantize_q8_1(xs, out, k);
     case ORC_Q4K: return orc_quantize_q4k(xs, out, k);
+    case ORC_Q5K: return orc_quantize_q5k(xs, out, k);
     case ORC_Q6K: return orc_quantize_q6k(xs, out, k);
     case ORC_Q8K: memset(out, 0, (size_t)(k / QK_K) * 292); return orc_quantize_q8k(xs, out, k);
     default: return -2;
@@ -778,6 +919,7 @@ int orc_dequantize(int dtype, const void *in, float *ys, int64_t k) {
     case ORC_Q4_0: return orc_dequantize_q4_0(in, ys, k);
     case ORC_Q8_0: return orc_dequantize_q8_0(in, ys, k);
     case ORC_Q4K: return orc_dequantize_q4k(in, ys, k);
+    case ORC_Q5K: return orc_dequantize_q5k(in, ys, k);
     case ORC_Q6K: return orc_dequantize_q6k(in, ys, k);
     case ORC_Q8K: return orc_dequantize_q8k(in, ys, k);
     default: return -2;
@@ -792,6 +934,7 @@ int orc_vec_dot(int dtype, int64_t n, const void *xs, const void *ys, float *out
     case ORC_Q4_0: *out = vec_dot_q4_0_q8_0(n, xs, ys); return 0;
     case ORC_Q8_0: *out = vec_dot_q8_0_q8_0(n, xs, ys); return 0;
     case ORC_Q4K: *out = vec_dot_q4k_q8k(n, xs, ys); return 0;
+    case ORC_Q5K: *out = vec_dot_q5k_q8k(n, xs, ys); return 0;
     case ORC_Q6K: *out = vec_dot_q6k_q8k(n, xs, ys); return 0;
     case ORC_Q8K: *out = vec_dot_q8k_q8k(n, xs, ys); return 0;
     default: return -2;
@@ -855,6 +998,14 @@ int orc_block_int_dots(int dtype, int64_t m, int64_t k, int64_t n, const void *a
                 case ORC_Q4K: {
                     int32_t aux32[8], sumi, t = 0;
                     ints_q4k_q8k((const block_q4k *)w + b, (const block_q8k *)a + b, aux32, &sumi);
+                    for (int l = 0; l < 8; l++) t += aux32[l];
+                    out_i[o] = t;
+                    if (out_mn) out_mn[o] = sumi;
+                    break;
+                }
+                case ORC_Q5K: {
+                    int32_t aux32[8], sumi, t = 0;
+                    ints_q5k_q8k((const block_q5k *)w + b, (const block_q8k *)a + b, aux32, &sumi);
                     for (int l = 0; l < 8; l++) t += aux32[l];
                     out_i[o] = t;
                     if (out_mn) out_mn[o] = sumi;

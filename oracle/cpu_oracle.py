@@ -17,11 +17,11 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libcandle_q_oracle.so")
 
 # GgmlDType ids (candle-core/src/quantized/mod.rs:173-190)
-Q4_0, Q8_0, Q8_1, Q4K, Q6K, Q8K = 2, 8, 9, 12, 14, 15
-BLOCK_SIZE = {Q4_0: 32, Q8_0: 32, Q8_1: 32, Q4K: 256, Q6K: 256, Q8K: 256}
-TYPE_SIZE = {Q4_0: 18, Q8_0: 34, Q8_1: 36, Q4K: 144, Q6K: 210, Q8K: 292}
-VEC_DOT_TYPE = {Q4_0: Q8_0, Q8_0: Q8_0, Q4K: Q8K, Q6K: Q8K, Q8K: Q8K}
-NAMES = {Q4_0: "q4_0", Q8_0: "q8_0", Q8_1: "q8_1", Q4K: "q4k", Q6K: "q6k", Q8K: "q8k"}
+Q4_0, Q8_0, Q8_1, Q4K, Q5K, Q6K, Q8K = 2, 8, 9, 12, 13, 14, 15
+BLOCK_SIZE = {Q4_0: 32, Q8_0: 32, Q8_1: 32, Q4K: 256, Q5K: 256, Q6K: 256, Q8K: 256}
+TYPE_SIZE = {Q4_0: 18, Q8_0: 34, Q8_1: 36, Q4K: 144, Q5K: 176, Q6K: 210, Q8K: 292}
+VEC_DOT_TYPE = {Q4_0: Q8_0, Q8_0: Q8_0, Q4K: Q8K, Q5K: Q8K, Q6K: Q8K, Q8K: Q8K}
+NAMES = {Q4_0: "q4_0", Q8_0: "q8_0", Q8_1: "q8_1", Q4K: "q4k", Q5K: "q5k", Q6K: "q6k", Q8K: "q8k"}
 
 
 def build(force: bool = False) -> str:
@@ -139,7 +139,7 @@ def block_int_dots(dtype: int, act_blocks: np.ndarray, m: int, rhs_blocks: np.nd
     act_blocks = np.ascontiguousarray(act_blocks, dtype=np.uint8)
     rhs_blocks = np.ascontiguousarray(rhs_blocks, dtype=np.uint8)
     oi = np.zeros((m, n, kb), dtype=np.int32)
-    om = np.zeros((m, n, kb), dtype=np.int32) if dtype == Q4K else None
+    om = np.zeros((m, n, kb), dtype=np.int32) if dtype in (Q4K, Q5K) else None
     i32p = C.POINTER(C.c_int32)
     _check(lib().orc_block_int_dots(dtype, m, k, n, act_blocks.ctypes.data, rhs_blocks.ctypes.data,
                                     oi.ctypes.data_as(i32p),

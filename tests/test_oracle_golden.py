@@ -6,7 +6,7 @@ import pytest
 
 from oracle import cpu_oracle as orc
 
-DT = {"q4_0": orc.Q4_0, "q8_0": orc.Q8_0, "q4k": orc.Q4K, "q6k": orc.Q6K, "q8k": orc.Q8K}
+DT = {"q4_0": orc.Q4_0, "q8_0": orc.Q8_0, "q4k": orc.Q4K, "q5k": orc.Q5K, "q6k": orc.Q6K, "q8k": orc.Q8K}
 
 
 # ---------------------------------------------------------------- f16 ----
@@ -77,7 +77,7 @@ def _test_vector2(bound, size=1024):
     return (v - np.float32(size) / np.float32(2.0)) * np.float32(bound) / (np.float32(size) / np.float32(2.0))
 
 
-@pytest.mark.parametrize("name", ["q4k", "q6k", "q8k"])
+@pytest.mark.parametrize("name", ["q4k", "q5k", "q6k", "q8k"])
 def test_kquant_roundtrip_golden(goldens, name):
     g = goldens["kquant_roundtrip_test_vector2"]
     idx = g["indices"]
@@ -100,7 +100,7 @@ def _ggml_like(offset):
     return (np.float32(0.1) + np.float32(2.0) * np.cos(i + np.float32(offset), dtype=np.float32)).astype(np.float32)
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q4k", "q6k", "q8k", "q8_0"])
+@pytest.mark.parametrize("name", ["q4_0", "q4k", "q5k", "q6k", "q8k", "q8_0"])
 def test_quantization_total_error(goldens, name):
     src = _ggml_like(0.0)
     dst = orc.dequantize(DT[name], orc.quantize(DT[name], src))
@@ -109,7 +109,7 @@ def test_quantization_total_error(goldens, name):
 
 
 # ------------------------------------------------- G6: dot product error ----
-@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4k", "q6k", "q8k"])
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4k", "q5k", "q6k", "q8k"])
 def test_dot_product_error(goldens, name):
     g = goldens["dot_product_error"]
     ramp = (np.arange(4096, dtype=np.float32) / np.float32(4096))
@@ -125,7 +125,7 @@ def test_dot_product_error(goldens, name):
 
 
 # ------------------------------------- G7: seeded full path m=11,k=512,n=21 ----
-@pytest.mark.parametrize("name", ["q4k", "q6k", "q8k"])
+@pytest.mark.parametrize("name", ["q4k", "q5k", "q6k", "q8k"])
 def test_seeded_matmul_golden(goldens, seeded_inputs, name):
     g = goldens["seeded_matmul_m11_k512_n21"]
     lhs, rhs = seeded_inputs
@@ -137,7 +137,7 @@ def test_seeded_matmul_golden(goldens, seeded_inputs, name):
 
 
 # ------------------------------------------------ G8: batch invariance ----
-@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4k", "q6k"])
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4k", "q5k", "q6k"])
 def test_batch_invariance(seeded_inputs, name):
     lhs, rhs = seeded_inputs
     lhs, rhs = lhs[:2, :256], rhs[:6, :256]
@@ -150,7 +150,7 @@ def test_batch_invariance(seeded_inputs, name):
 
 
 # --------------------------------------------- G9: generic matmul error ----
-@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4k", "q6k"])
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4k", "q5k", "q6k"])
 def test_generic_matmul_error(goldens, name):
     m, n, k = goldens["generic_matmul_error"]["mnk"]
     lhs = (np.arange(m * k, dtype=np.float32) / np.float32(m * k)).reshape(m, k)
@@ -179,6 +179,17 @@ def _unpack_q4k(blocks):
     qs = b[:, 16:].astype(np.int32).reshape(-1, 4, 32)
     q = np.stack([qs & 0xF, qs >> 4], axis=2).reshape(-1, 8, 32)  # [block, sub-block, 32]
     return d, dmin, sc, mn, q
+
+
+def _unpack_q5k(blocks):
+    """Q5K blocks (k_quants.rs:119-127: d, dmin, scales[12], qh[32], qs[128]) unpacked with numpy;
+    sub-block j takes bit j of qh[l] as the fifth bit of its element l."""
+    b = blocks.reshape(-1, 176)
+    as_q4k = np.concatenate([b[:, :16], b[:, 48:]], axis=1)     # same header, scales and nibbles as Q4K
+    d, dmin, sc, mn, q = _unpack_q4k(as_q4k)
+    qh = b[:, 16:48].astype(np.int32)                            # [block, 32]
+    hi = np.stack([(qh >> j) & 1 for j in range(8)], axis=1)     # [block, sub-block, 32]
+    return d, dmin, sc, mn, q + 16 * hi
 
 
 def _unpack_q6k(blocks):
@@ -259,7 +270,7 @@ def test_q8_1_is_q8_0_plus_s():
     assert np.array_equal(s.view(np.uint16), want.view(np.uint16))
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4k", "q6k", "q8k"])
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4k", "q5k", "q6k", "q8k"])
 def test_int_dots_and_matmul_bruteforce(name):
     """Integer block dots recomputed by int64 numpy from independently unpacked blocks,
     and the f32 result against a float64 evaluation of the same formula."""
@@ -272,11 +283,11 @@ def test_int_dots_and_matmul_bruteforce(name):
     a = np.concatenate([orc.quantize(orc.VEC_DOT_TYPE[dt], lhs[r]) for r in range(m)])
     oi, om = orc.block_int_dots(dt, a, m, w, n, k)
     out = orc.matmul(dt, lhs, w, n)
-    if name in ("q4k", "q6k", "q8k"):
+    if name in ("q4k", "q5k", "q6k", "q8k"):
         d8, q8, bs = _unpack_q8k(a)
         d8, q8, bs = d8.reshape(m, -1), q8.reshape(m, -1, 256), bs.reshape(m, -1, 16)
-        if name == "q4k":
-            d, dmin, sc, mn, q = _unpack_q4k(w)
+        if name in ("q4k", "q5k"):
+            d, dmin, sc, mn, q = _unpack_q4k(w) if name == "q4k" else _unpack_q5k(w)
             kb = k // 256
             d, dmin = d.reshape(n, kb), dmin.reshape(n, kb)
             sc, mn, q = sc.reshape(n, kb, 8), mn.reshape(n, kb, 8), q.reshape(n, kb, 8, 32)
