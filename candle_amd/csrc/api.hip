@@ -53,7 +53,7 @@ extern "C" int cq_device_count(void) {
 extern "C" int64_t cq_block_size(int dt) {
     switch (dt) {
     case CQ_DTYPE_Q4_0: case CQ_DTYPE_Q8_0: case CQ_DTYPE_Q8_1: return 32;
-    case CQ_DTYPE_Q4K: case CQ_DTYPE_Q6K: case CQ_DTYPE_Q8K: return 256;
+    case CQ_DTYPE_Q4K: case CQ_DTYPE_Q5K: case CQ_DTYPE_Q6K: case CQ_DTYPE_Q8K: return 256;
     default: return 0;
     }
 }
@@ -63,6 +63,7 @@ extern "C" int64_t cq_type_size(int dt) {
     case CQ_DTYPE_Q8_0: return 34;
     case CQ_DTYPE_Q8_1: return 36;
     case CQ_DTYPE_Q4K: return 144;
+    case CQ_DTYPE_Q5K: return 176;
     case CQ_DTYPE_Q6K: return 210;
     case CQ_DTYPE_Q8K: return 292;
     default: return 0;
@@ -71,13 +72,13 @@ extern "C" int64_t cq_type_size(int dt) {
 extern "C" int cq_vec_dot_type(int dt) {
     switch (dt) {
     case CQ_DTYPE_Q4_0: case CQ_DTYPE_Q8_0: return CQ_DTYPE_Q8_0;
-    case CQ_DTYPE_Q4K: case CQ_DTYPE_Q6K: return CQ_DTYPE_Q8K;
+    case CQ_DTYPE_Q4K: case CQ_DTYPE_Q5K: case CQ_DTYPE_Q6K: return CQ_DTYPE_Q8K;
     default: return -1;
     }
 }
 
 static bool is_weight_dtype(int dt) {
-    return dt == CQ_DTYPE_Q4_0 || dt == CQ_DTYPE_Q8_0 || dt == CQ_DTYPE_Q4K || dt == CQ_DTYPE_Q6K;
+    return dt == CQ_DTYPE_Q4_0 || dt == CQ_DTYPE_Q8_0 || dt == CQ_DTYPE_Q4K || dt == CQ_DTYPE_Q5K || dt == CQ_DTYPE_Q6K;
 }
 
 // --------------------------------------------------------------- weights ----
@@ -105,6 +106,7 @@ static int weight_alloc(int dev, int dt, int64_t n, int64_t k, cq_weight **out) 
     case CQ_DTYPE_Q4_0: s0 = (size_t)nb * 16; s1 = (size_t)nb * 2; break;
     case CQ_DTYPE_Q8_0: s0 = (size_t)nb * 32; s1 = (size_t)nb * 2; break;
     case CQ_DTYPE_Q4K: s0 = (size_t)nb * 128; s1 = (size_t)nb * CQ_Q4K_HDR; break;
+    case CQ_DTYPE_Q5K: s0 = (size_t)nb * 128; s1 = (size_t)nb * CQ_Q4K_HDR; s2 = (size_t)nb * 32; break;
     case CQ_DTYPE_Q6K: s0 = (size_t)nb * 128; s1 = (size_t)nb * 64; s2 = (size_t)nb * 16; s3 = (size_t)nb * 2; break;
     }
     const size_t o1 = cq_align_up(s0 + CQ_TAIL_PAD, 256);
@@ -412,7 +414,7 @@ extern "C" int cq_qmatmul_int_dots(const cq_weight *w, const float *x_dev, int64
     cq_act_view v;
     act_ws_layout(act, m, w->k, (uint8_t *)ws, &v);
     CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, nullptr, m, w->k, cq_no_pre(), v, s));
-    CQ_HIP_CHECK(cq_launch_int_dots(w, v, m, out_i, w->dtype == CQ_DTYPE_Q4K ? out_mn : nullptr, s));
+    CQ_HIP_CHECK(cq_launch_int_dots(w, v, m, out_i, (w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q5K) ? out_mn : nullptr, s));
     return CQ_OK;
 }
 

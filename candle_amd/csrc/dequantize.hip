@@ -1,6 +1,6 @@
 // Device planes -> f32 / f16 (QTensor::dequantize, dequantize_f16;
 // candle-core/src/quantized/mod.rs:361-382, CUDA precedent cuda.rs:69-181).
-// The f32 values are those of T::to_float (k_quants.rs:163-183, :568-584, :1313-1341,
+// The f32 values are those of T::to_float (k_quants.rs:163-183, :568-584, :1313-1341, :1527-1564,
 // :1716-1746): same products in the same order, no contraction.  The f16 output is the
 // f32 output rounded to nearest-even, as the reference's tests require
 // (candle-core/tests/quantized_tests.rs:229-234).
@@ -64,9 +64,11 @@ __global__ void dequant_q8_0(const uint8_t *__restrict__ qs, const uint16_t *__r
     put16<F16>(d32, d16, u * 16, out);
 }
 
-template <bool F16>
-__global__ void dequant_q4k(const uint8_t *__restrict__ qs, const uint8_t *__restrict__ hd, int64_t nunits,
-                            float *d32, uint16_t *d16) {
+// Q5 (Q5K, to_float k_quants.rs:1527-1564): the fifth bits come from the re-ordered qh plane, words
+// {L, H} per 32 qs bytes, bit 8c + i for byte c of qs word i.
+template <bool F16, bool Q5>
+__global__ void dequant_q4k(const uint8_t *__restrict__ qs, const uint8_t *__restrict__ hd,
+                            const uint8_t *__restrict__ qh, int64_t nunits, float *d32, uint16_t *d16) {
     const int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // 16 bytes of qs = 32 elements
     if (u >= nunits) return;
     const int64_t b = u >> 3;
@@ -81,12 +83,15 @@ __global__ void dequant_q4k(const uint8_t *__restrict__ qs, const uint8_t *__res
     const float d2 = d * (float)sc2, mm2 = dmin * (float)m2;
     const uint32_t w[4] = {q.x, q.y, q.z, q.w};
     const int64_t base = b * 256 + 64 * g + 16 * half;
+    uint2 fifth = make_uint2(0u, 0u);
+    if (Q5) fifth = *(const uint2 *)(qh + (b * 4 + g) * 8);
     float lo[16], hi[16];
 #pragma unroll
     for (int j = 0; j < 16; j++) {
         const uint32_t byte = (w[j >> 2] >> (8 * (j & 3))) & 0xff;
-        lo[j] = d1 * (float)(byte & 0xF) - mm1;
-        hi[j] = d2 * (float)(byte >> 4) - mm2;
+        const int bit = 8 * (j & 3) + 4 * half + (j >> 2);
+        lo[j] = d1 * (float)((byte & 0xF) + (((fifth.x >> bit) & 1u) << 4)) - mm1;
+        hi[j] = d2 * (float)((byte >> 4) + (((fifth.y >> bit) & 1u) << 4)) - mm2;
     }
     put16<F16>(d32, d16, base, lo);
     put16<F16>(d32, d16, base + 32, hi);
@@ -138,7 +143,10 @@ hipError_t launch(const cq_weight *w, float *d32, uint16_t *d16, hipStream_t s) 
         dequant_q8_0<F16><<<grid(total / 16), threads, 0, s>>>(w->p0, (const uint16_t *)w->p1, total / 16, d32, d16);
         break;
     case CQ_DTYPE_Q4K:
-        dequant_q4k<F16><<<grid(total / 32), threads, 0, s>>>(w->p0, w->p1, total / 32, d32, d16);
+        dequant_q4k<F16, false><<<grid(total / 32), threads, 0, s>>>(w->p0, w->p1, nullptr, total / 32, d32, d16);
+        break;
+    case CQ_DTYPE_Q5K:
+        dequant_q4k<F16, true><<<grid(total / 32), threads, 0, s>>>(w->p0, w->p1, w->p2, total / 32, d32, d16);
         break;
     case CQ_DTYPE_Q6K:
         dequant_q6k<F16><<<grid(total / 32), threads, 0, s>>>(w->p0, w->p1, (const int8_t *)w->p2,

@@ -30,7 +30,12 @@ template <int DT> struct Geo;
 template <> struct Geo<CQ_DTYPE_Q4_0> { static constexpr int kElems = 32;  static constexpr int kUnitsPerBlock = 1; static constexpr bool kActK = false; };
 template <> struct Geo<CQ_DTYPE_Q8_0> { static constexpr int kElems = 16;  static constexpr int kUnitsPerBlock = 2; static constexpr bool kActK = false; };
 template <> struct Geo<CQ_DTYPE_Q4K>  { static constexpr int kElems = 64;  static constexpr int kUnitsPerBlock = 4; static constexpr bool kActK = true; };
+template <> struct Geo<CQ_DTYPE_Q5K>  { static constexpr int kElems = 64;  static constexpr int kUnitsPerBlock = 4; static constexpr bool kActK = true; };
 template <> struct Geo<CQ_DTYPE_Q6K>  { static constexpr int kElems = 32;  static constexpr int kUnitsPerBlock = 8; static constexpr bool kActK = true; };
+
+// Q5K is Q4K with a fifth bit per quant from a plane of its own: same units, same LDS image, same
+// scale / min records.
+constexpr bool is_k4(int dt) { return dt == CQ_DTYPE_Q4K || dt == CQ_DTYPE_Q5K; }
 
 // ---------------------------------------------------------------------------------------------
 // LDS image of one quantized activation row:
@@ -41,7 +46,7 @@ template <> struct Geo<CQ_DTYPE_Q6K>  { static constexpr int kElems = 32;  stati
 // ---------------------------------------------------------------------------------------------
 template <int DT> __host__ __device__ constexpr int64_t act_blocks(int64_t k) { return Geo<DT>::kActK ? k / 256 : k / 32; }
 template <int DT> __host__ __device__ constexpr size_t lds_row_bytes(int64_t k) {
-    return (size_t)k + (size_t)act_blocks<DT>(k) * (DT == CQ_DTYPE_Q4K ? 4 + 16 : (Geo<DT>::kActK ? 4 + 32 : 4 + 4));
+    return (size_t)k + (size_t)act_blocks<DT>(k) * (is_k4(DT) ? 4 + 16 : (Geo<DT>::kActK ? 4 + 32 : 4 + 4));
 }
 
 // Byte offsets from the start of dynamic LDS (plain integers: every access below is then a
@@ -69,7 +74,7 @@ template <typename T> __device__ __forceinline__ void lds_put(uint8_t *smem, uin
 template <int DT> __device__ __forceinline__ uint32_t piece_off(const LdsRow r, int64_t piece, uint32_t units) {
     if (DT == CQ_DTYPE_Q8_0) return r.lo + (uint32_t)piece * 16;
     if (DT == CQ_DTYPE_Q4_0) return ((piece & 1) ? r.hi : r.lo) + (uint32_t)(piece >> 1) * 16;
-    if (DT == CQ_DTYPE_Q4K) return r.lo + (uint32_t)(piece & 3) * units * 16 + (uint32_t)(piece >> 2) * 16;
+    if (is_k4(DT)) return r.lo + (uint32_t)(piece & 3) * units * 16 + (uint32_t)(piece >> 2) * 16;
     // Q6K: unit p = 4h + 2t + i covers 128h + 32t + 16i + [0,16) (low) and + 64 (high)
     const int64_t b = piece >> 4;
     const int w = (int)(piece & 15);
@@ -160,7 +165,7 @@ __device__ __forceinline__ void quantize_chunk_to_lds(uint8_t *smem, const float
             sum4 += dpp_i<kQuadSwap1>(sum4);
             sum4 += dpp_i<kQuadSwap2>(sum4);  // the four lanes of a 16-element group hold its sum
             if (chunk_ok && lane == 0) lds_put<float>(smem, r.d + 4 * c, d);
-            if (DT == CQ_DTYPE_Q4K) {
+            if (is_k4(DT)) {
                 sum4 += dpp_i<kHalfMirror>(sum4);   // eight lanes = one 32-element sub-block
                 if (chunk_ok && (lane & 7) == 0) lds_put<int16_t>(smem, r.bs + 2 * (c * 8 + (lane >> 3)), (int16_t)sum4);
             } else if (chunk_ok && (lane & 3) == 0) {
@@ -358,7 +363,7 @@ __device__ __forceinline__ void quantize_pair_to_lds(uint8_t *smem, const X8 &fi
         d = 1.0f / iscale;
     }
     sum += dpp_i<kQuadSwap1>(sum);   // two lanes = one 16-element group
-    if (DT == CQ_DTYPE_Q4K) {
+    if (is_k4(DT)) {
         sum += dpp_i<kQuadSwap2>(sum);   // four lanes = one 32-element sub-block
         if (chunk_ok && (hl & 3) == 0) lds_put<int16_t>(smem, r.bs + 2 * (c * 8 + (hl >> 2)), (int16_t)sum);
     } else if (chunk_ok && (hl & 1) == 0) {
@@ -398,7 +403,7 @@ __device__ __forceinline__ void stage_row(uint8_t *smem, const LdsRow r, const c
         const int32_t *bs = (const int32_t *)(a.bsums + row * nb * 16);  // 8 words per block
         for (int i = threadIdx.x; i < nb * 8; i += NT) {
             const int32_t two = bs[i];   // bsums 2i and 2i+1: the two halves of 32-element sub-block i
-            if (DT == CQ_DTYPE_Q4K) lds_put<int16_t>(smem, r.bs + 2 * i, (int16_t)((int16_t)(two & 0xffff) + (int16_t)(two >> 16)));
+            if (is_k4(DT)) lds_put<int16_t>(smem, r.bs + 2 * i, (int16_t)((int16_t)(two & 0xffff) + (int16_t)(two >> 16)));
             else lds_put<int32_t>(smem, r.bs + 4 * i, two);
         }
     }
@@ -410,7 +415,7 @@ template <int DT> struct UnitRaw {
     uint4 q;       // main plane lane
     uint4 q2;      // Q4K: the second 16 bytes of the lane's 32
     uint2 h;       // Q4K: {d | dmin << 16, record {sc[2g], sc[2g+1], mn[2g], mn[2g+1]}}
-    uint2 hh;      // Q6K: high bits of the lane's 32 elements
+    uint2 hh;      // Q6K: high bits of the lane's 32 elements; Q5K: fifth bits {L, H} of the lane's 64
     uint16_t sc2;  // Q6K: the lane's two group scales
     uint16_t d;    // Q4_0 / Q8_0 / Q6K: f16 scale
 };
@@ -424,20 +429,21 @@ template <int DT> __device__ __forceinline__ RowPtr row_ptr(const cq_weight &w, 
     constexpr int kB = Geo<DT>::kUnitsPerBlock;
     const int64_t g0 = row * units;   // units per row is a multiple of the units per block
     RowPtr rp;
-    rp.p0 = w.p0 + g0 * (DT == CQ_DTYPE_Q4K ? 32 : 16);
-    rp.p1 = w.p1 + (DT == CQ_DTYPE_Q4K ? (g0 / kB) * CQ_Q4K_HDR : DT == CQ_DTYPE_Q6K ? g0 * 8 : DT == CQ_DTYPE_Q4_0 ? g0 * 2 : g0);
-    rp.p2 = DT == CQ_DTYPE_Q6K ? w.p2 + g0 * 2 : nullptr;
+    rp.p0 = w.p0 + g0 * (is_k4(DT) ? 32 : 16);
+    rp.p1 = w.p1 + (is_k4(DT) ? (g0 / kB) * CQ_Q4K_HDR : DT == CQ_DTYPE_Q6K ? g0 * 8 : DT == CQ_DTYPE_Q4_0 ? g0 * 2 : g0);
+    rp.p2 = DT == CQ_DTYPE_Q6K ? w.p2 + g0 * 2 : DT == CQ_DTYPE_Q5K ? w.p2 + g0 * 8 : nullptr;
     rp.p3 = DT == CQ_DTYPE_Q6K ? w.p3 + (g0 / kB) * 2 : nullptr;
     return rp;
 }
 
 template <int DT> __device__ __forceinline__ void load_unit(const RowPtr &rp, uint32_t u, UnitRaw<DT> &o) {
-    if (DT == CQ_DTYPE_Q4K) {
+    if (is_k4(DT)) {
         o.q = *(const uint4 *)(rp.p0 + u * 32u);
         o.q2 = *(const uint4 *)(rp.p0 + u * 32u + 16u);
         const uint8_t *h = rp.p1 + (u >> 2) * (uint32_t)CQ_Q4K_HDR;
         o.h.x = *(const uint32_t *)h;
         o.h.y = *(const uint32_t *)(h + 4u + (u & 3u) * 4u);
+        if (DT == CQ_DTYPE_Q5K) o.hh = *(const uint2 *)(rp.p2 + u * 8u);
         return;
     }
     o.q = *(const uint4 *)(rp.p0 + u * 16u);
@@ -480,7 +486,7 @@ template <int DT> __device__ __forceinline__ void decode_unit(const UnitRaw<DT> 
         o.dw = cq_h2f(r.d);
 #pragma unroll
         for (int i = 0; i < 4; i++) { o.lo[i] = qw[i] & 0x0F0F0F0Fu; o.hi[i] = (qw[i] >> 4) & 0x0F0F0F0Fu; }
-    } else if (DT == CQ_DTYPE_Q4K) {
+    } else if (is_k4(DT)) {
         (void)p;
         o.dw = cq_h2f((uint16_t)(r.h.x & 0xffff));
         o.dmin = cq_h2f((uint16_t)(r.h.x >> 16));
@@ -491,6 +497,14 @@ template <int DT> __device__ __forceinline__ void decode_unit(const UnitRaw<DT> 
         for (int i = 0; i < 4; i++) {
             o.lo[i] = qw[i] & 0x0F0F0F0Fu; o.hi[i] = (qw[i] >> 4) & 0x0F0F0F0Fu;
             o.lo[4 + i] = q2[i] & 0x0F0F0F0Fu; o.hi[4 + i] = (q2[i] >> 4) & 0x0F0F0F0Fu;
+        }
+        if (DT == CQ_DTYPE_Q5K) {
+            // bit 8c + i of L (H) is the fifth bit of the low (high) nibble in byte c of qs word i
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                o.lo[i] |= ((r.hh.x >> i) & 0x01010101u) << 4;
+                o.hi[i] |= ((r.hh.y >> i) & 0x01010101u) << 4;
+            }
         }
     } else {
         o.sc_lo = (int)(int8_t)(r.sc2 & 0xff);
@@ -516,7 +530,7 @@ template <int DT> __device__ __forceinline__ void decode_unit(const UnitRaw<DT> 
 template <int DT>
 __device__ __forceinline__ void unit_ints(const uint8_t *smem, const UnitW<DT> &w, const LdsRow r, uint32_t u,
                                           uint32_t units, int &I, int &Mn) {
-    if (DT == CQ_DTYPE_Q4K) {
+    if (is_k4(DT)) {
         // unit u = 32 qs bytes: low nibbles are elements 64u + [0,32) (sub-block 2g, planes 0 and 1),
         // high nibbles elements 64u + 32 + [0,32) (sub-block 2g+1, planes 2 and 3)
         const uint32_t plane = units * 16, at = r.lo + u * 16;
@@ -555,7 +569,7 @@ __device__ __forceinline__ float unit_value(const uint8_t *smem, const UnitW<DT>
     int I, Mn;
     unit_ints<DT>(smem, w, r, u, units, I, Mn);
     const float ad = lds_get<float>(smem, r.d + 4 * (u / Geo<DT>::kUnitsPerBlock));
-    if (DT == CQ_DTYPE_Q4K) return ad * (w.dw * (float)I - w.dmin * (float)Mn);
+    if (is_k4(DT)) return ad * (w.dw * (float)I - w.dmin * (float)Mn);
     return ((float)I * w.dw) * ad;
 }
 
@@ -1079,6 +1093,7 @@ bool cq_matvec_fused_supported(const cq_weight *w) {
     case CQ_DTYPE_Q4_0: return fused_ok<CQ_DTYPE_Q4_0>(w);
     case CQ_DTYPE_Q8_0: return fused_ok<CQ_DTYPE_Q8_0>(w);
     case CQ_DTYPE_Q4K: return fused_ok<CQ_DTYPE_Q4K>(w);
+    case CQ_DTYPE_Q5K: return fused_ok<CQ_DTYPE_Q5K>(w);
     case CQ_DTYPE_Q6K: return fused_ok<CQ_DTYPE_Q6K>(w);
     default: return false;
     }
@@ -1090,6 +1105,7 @@ hipError_t cq_launch_matvec_fused(const cq_weight *w, const float *x, cq_pre pre
     case CQ_DTYPE_Q4_0: return launch_fused<CQ_DTYPE_Q4_0>(w, x, pre, y, s);
     case CQ_DTYPE_Q8_0: return launch_fused<CQ_DTYPE_Q8_0>(w, x, pre, y, s);
     case CQ_DTYPE_Q4K: return launch_fused<CQ_DTYPE_Q4K>(w, x, pre, y, s);
+    case CQ_DTYPE_Q5K: return launch_fused<CQ_DTYPE_Q5K>(w, x, pre, y, s);
     case CQ_DTYPE_Q6K: return launch_fused<CQ_DTYPE_Q6K>(w, x, pre, y, s);
     default: return hipErrorInvalidValue;
     }
@@ -1102,6 +1118,7 @@ hipError_t cq_launch_matvec(const cq_weight *w, cq_act_view a, int act_dtype, in
     case CQ_DTYPE_Q4_0: return launch_staged<CQ_DTYPE_Q4_0>(w, a, m, y, s);
     case CQ_DTYPE_Q8_0: return launch_staged<CQ_DTYPE_Q8_0>(w, a, m, y, s);
     case CQ_DTYPE_Q4K: return launch_staged<CQ_DTYPE_Q4K>(w, a, m, y, s);
+    case CQ_DTYPE_Q5K: return launch_staged<CQ_DTYPE_Q5K>(w, a, m, y, s);
     case CQ_DTYPE_Q6K: return launch_staged<CQ_DTYPE_Q6K>(w, a, m, y, s);
     default: return hipErrorInvalidValue;
     }
@@ -1114,6 +1131,7 @@ hipError_t cq_launch_int_dots(const cq_weight *w, cq_act_view a, int64_t m, int3
     case CQ_DTYPE_Q4_0: return launch_ints<CQ_DTYPE_Q4_0>(w, a, m, out_i, out_mn, s);
     case CQ_DTYPE_Q8_0: return launch_ints<CQ_DTYPE_Q8_0>(w, a, m, out_i, out_mn, s);
     case CQ_DTYPE_Q4K: return launch_ints<CQ_DTYPE_Q4K>(w, a, m, out_i, out_mn, s);
+    case CQ_DTYPE_Q5K: return launch_ints<CQ_DTYPE_Q5K>(w, a, m, out_i, out_mn, s);
     case CQ_DTYPE_Q6K: return launch_ints<CQ_DTYPE_Q6K>(w, a, m, out_i, out_mn, s);
     default: return hipErrorInvalidValue;
     }

@@ -22,6 +22,10 @@
 //          hd [n][k/256][20]      (d f16, dmin f16, then four records {sc[2g], sc[2g+1], mn[2g], mn[2g+1]}:
 //                                  the 6-bit scales and mins of the GGML scales[12] unpacked to bytes,
 //                                  grouped by the 32 qs bytes g they belong to)
+//   Q5K  : qs and hd as Q4K (the low four bits of every quant)
+//          qh [n][k/256][32]  u8  (re-ordered, see repack.hip: per 32 qs bytes g two words {L, H} with the
+//                                  fifth bits of their low-nibble and high-nibble elements, bit 8c+i of a
+//                                  word belonging to byte c of qs word i)
 //   Q6K  : ql [n][k/256][128] u8  (GGML order)
 //          qh [n][k/256][64]  u8  (re-ordered, see repack.hip: 8 bytes per 16-byte ql lane)
 //          sc [n][k/256][16]  i8  (re-ordered: two scales per 16-byte ql lane, see repack.hip)
@@ -42,7 +46,7 @@ struct cq_weight {
     size_t alloc_bytes;
     uint8_t *p0;         // qs / ql
     uint8_t *p1;         // d (Q4_0,Q8_0) / hd (Q4K) / qh (Q6K)
-    uint8_t *p2;         // sc (Q6K)
+    uint8_t *p2;         // sc (Q6K) / qh (Q5K)
     uint8_t *p3;         // d  (Q6K)
 };
 

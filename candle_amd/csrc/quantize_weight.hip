@@ -5,6 +5,7 @@
 // the host and quantizes there (cuda.rs:448-472); the bytes produced here are the same.
 //   Q4_0 k_quants.rs:185-220      Q8_0 :586-615
 //   Q4K  :1252-1311 + utils.rs:201-258 (make_qkx1_quants) + :49-59 (get_scale_min_k4)
+//   Q5K  :1450-1525, the same with 32 levels
 //   Q6K  :1643-1713 + utils.rs:61-198  (make_qx_quants, n=16, nmax=32, rmse_type=1)
 #include "qhip_internal.h"
 
@@ -50,8 +51,8 @@ __global__ void quantize_q8_0(const float *__restrict__ src, int64_t nblocks, ui
 }
 
 // utils.rs:201-258
-__device__ void make_qkx1_quants(const float *x, float &out_scale, float &out_min) {
-    const int n = 32, nmax = 15, ntry = 5;
+__device__ void make_qkx1_quants(const float *x, int nmax, float &out_scale, float &out_min) {
+    const int n = 32, ntry = 5;
     uint8_t l[32];
     for (int i = 0; i < n; i++) l[i] = 0;
     float min = x[0], max = x[0];
@@ -85,13 +86,19 @@ __device__ void make_qkx1_quants(const float *x, float &out_scale, float &out_mi
     out_min = -min;
 }
 
+// LEVELS = 16: Q4K (144-byte blocks).  LEVELS = 32: Q5K (k_quants.rs:1450-1525), the same scale search
+// with 31 as the top level, the quants' fifth bits in qh[32] between the scales and the nibbles.
+template <int LEVELS>
 __global__ void quantize_q4k(const float *__restrict__ src, int64_t nblocks, uint8_t *__restrict__ out) {
     const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (b >= nblocks) return;
     const float *x = src + b * QK_K;
-    uint8_t *y = out + b * 144;
+    constexpr int kQs = LEVELS == 16 ? 16 : 48;   // offset of the nibbles in the block
+    uint8_t *y = out + b * (LEVELS == 16 ? 144 : 176);
+    uint8_t qh[32];
+    for (int l = 0; l < 32; l++) qh[l] = 0;
     float mins[8], scales[8];
-    for (int j = 0; j < 8; j++) make_qkx1_quants(x + 32 * j, scales[j], mins[j]);
+    for (int j = 0; j < 8; j++) make_qkx1_quants(x + 32 * j, LEVELS - 1, scales[j], mins[j]);
     float max_scale = 0.0f, max_min = 0.0f;
     for (int j = 0; j < 8; j++) max_scale = fmaxf(scales[j], max_scale);
     for (int j = 0; j < 8; j++) max_min = fmaxf(mins[j], max_min);
@@ -134,13 +141,18 @@ __global__ void quantize_q4k(const float *__restrict__ src, int64_t nblocks, uin
             if (d != 0.0f) {
                 const float dm = cq_h2f(dminh) * (float)m;
                 for (int ii = 0; ii < 32; ii++)
-                    dst[ii] = (uint8_t)cq_clampi(cq_nearest_int((x[32 * j + ii] + dm) / d), 0, 15);
+                    dst[ii] = (uint8_t)cq_clampi(cq_nearest_int((x[32 * j + ii] + dm) / d), 0, LEVELS - 1);
             } else {
                 for (int ii = 0; ii < 32; ii++) dst[ii] = 0;
             }
         }
-        for (int l = 0; l < 32; l++) y[16 + 32 * g + l] = (uint8_t)(lo[l] | (hi[l] << 4));
+        for (int l = 0; l < 32; l++) {
+            if (LEVELS == 32) qh[l] |= (uint8_t)(((lo[l] >> 4) << (2 * g)) | ((hi[l] >> 4) << (2 * g + 1)));
+            y[kQs + 32 * g + l] = (uint8_t)((lo[l] & 15) | ((hi[l] & 15) << 4));
+        }
     }
+    if (LEVELS == 32)
+        for (int l = 0; l < 32; l++) y[16 + l] = qh[l];
 }
 
 // utils.rs:61-198 specialised to n = 16, nmax = 32, rmse_type = 1 (weights w = x*x; returns after
@@ -273,7 +285,8 @@ hipError_t cq_launch_quantize_weight(int dtype, const float *src, int64_t nblock
     switch (dtype) {
     case CQ_DTYPE_Q4_0: quantize_q4_0<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q8_0: quantize_q8_0<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
-    case CQ_DTYPE_Q4K: quantize_q4k<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
+    case CQ_DTYPE_Q4K: quantize_q4k<16><<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
+    case CQ_DTYPE_Q5K: quantize_q4k<32><<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q6K: quantize_q6k<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     default: return hipErrorInvalidValue;
     }

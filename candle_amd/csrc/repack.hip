@@ -40,24 +40,11 @@ __global__ void repack_q8_0(const uint8_t *__restrict__ aos, uint8_t *__restrict
     }
 }
 
-// ---- Q4K: 144-byte blocks {f16 d; f16 dmin; u8 scales[12]; u8 qs[128]} ------
-// One thread per 16-byte unit: unit 0 is the header, units 1..8 the nibbles.  The header's twelve
-// bytes of 6-bit fields (utils.rs:49-59 get_scale_min_k4) are unpacked to one byte per field and
-// grouped per 32 qs bytes: record g = {sc[2g], sc[2g+1], mn[2g], mn[2g+1]}; the inverse packs them
-// back (every one of the 96 bits is a field bit, so the round trip is exact).
-__global__ void repack_q4k(const uint8_t *__restrict__ aos, uint8_t *__restrict__ qs, uint8_t *__restrict__ hd,
-                           int64_t nblocks, bool inverse) {
-    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    int64_t b = t / 9;
-    int u = (int)(t - b * 9);
-    if (b >= nblocks) return;
-    uint4 *a = (uint4 *)(aos + b * 144) + u;      // 144 = 9 * 16, base is 256-byte aligned
-    if (u != 0) {
-        uint4 *p = (uint4 *)(qs + b * 128) + (u - 1);
-        if (!inverse) *p = *a; else *a = *p;
-        return;
-    }
-    uint32_t *h = (uint32_t *)(hd + b * CQ_Q4K_HDR);
+// The 16 header bytes {f16 d; f16 dmin; u8 scales[12]} of a Q4K / Q5K block <-> the 20-byte device
+// record: the twelve bytes of 6-bit fields (utils.rs:49-59 get_scale_min_k4) unpacked to one byte
+// per field and grouped per 32 qs bytes, record g = {sc[2g], sc[2g+1], mn[2g], mn[2g+1]}; the
+// inverse packs them back (every one of the 96 bits is a field bit, so the round trip is exact).
+__device__ void k4_header(uint4 *a, uint32_t *h, bool inverse) {
     if (!inverse) {
         const uint4 v = *a;
         h[0] = v.x;
@@ -85,6 +72,74 @@ __global__ void repack_q4k(const uint8_t *__restrict__ aos, uint8_t *__restrict_
         }
         *a = make_uint4(h[0], w[0], w[1], w[2]);
     }
+}
+
+// ---- Q4K: 144-byte blocks {f16 d; f16 dmin; u8 scales[12]; u8 qs[128]} ------
+// One thread per 16-byte unit: unit 0 is the header, units 1..8 the nibbles.
+__global__ void repack_q4k(const uint8_t *__restrict__ aos, uint8_t *__restrict__ qs, uint8_t *__restrict__ hd,
+                           int64_t nblocks, bool inverse) {
+    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t b = t / 9;
+    int u = (int)(t - b * 9);
+    if (b >= nblocks) return;
+    uint4 *a = (uint4 *)(aos + b * 144) + u;      // 144 = 9 * 16, base is 256-byte aligned
+    if (u != 0) {
+        uint4 *p = (uint4 *)(qs + b * 128) + (u - 1);
+        if (!inverse) *p = *a; else *a = *p;
+        return;
+    }
+    k4_header(a, (uint32_t *)(hd + b * CQ_Q4K_HDR), inverse);
+}
+
+// ---- Q5K: 176-byte blocks {f16 d; f16 dmin; u8 scales[12]; u8 qh[32]; u8 qs[128]} ------
+// (k_quants.rs:119-127).  Header and nibbles as Q4K.  Bit j of qh[l] is the fifth bit of element
+// l of sub-block j, i.e. of the low (j even) or high (j odd) nibble of qs byte 32*(j/2) + l.  The
+// device plane holds, per 32 qs bytes g, two words L (sub-block 2g) and H (sub-block 2g+1) with
+//   bit 8c + i  =  fifth bit belonging to byte c of qs word i  (l = 4i + c),
+// so that (W >> i) & 0x01010101 lines the four bits up with the four nibbles of word i.
+// One thread per 16-byte unit of the block: 0 header, 1 the whole qh (32 bytes), 2 idle, 3..10 qs.
+__global__ void repack_q5k(const uint8_t *__restrict__ aos, uint8_t *__restrict__ qs, uint8_t *__restrict__ hd,
+                           uint8_t *__restrict__ qh, int64_t nblocks, bool inverse) {
+    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t b = t / 11;
+    int u = (int)(t - b * 11);
+    if (b >= nblocks) return;
+    uint4 *a = (uint4 *)(aos + b * 176) + u;      // 176 = 11 * 16, base is 256-byte aligned
+    if (u >= 3) {
+        uint4 *p = (uint4 *)(qs + b * 128) + (u - 3);
+        if (!inverse) *p = *a; else *a = *p;
+        return;
+    }
+    if (u == 2) return;
+    if (u == 1) {
+        uint8_t *src = (uint8_t *)aos + b * 176 + 16;   // GGML qh[32]
+        uint32_t *dst = (uint32_t *)(qh + b * 32);      // {L, H} x 4
+        if (!inverse) {
+            for (int g = 0; g < 4; g++) {
+                uint32_t L = 0, H = 0;
+                for (int i = 0; i < 8; i++)
+                    for (int c = 0; c < 4; c++) {
+                        const uint32_t v = src[4 * i + c];
+                        L |= ((v >> (2 * g)) & 1u) << (8 * c + i);
+                        H |= ((v >> (2 * g + 1)) & 1u) << (8 * c + i);
+                    }
+                dst[2 * g] = L;
+                dst[2 * g + 1] = H;
+            }
+        } else {
+            for (int i = 0; i < 8; i++)
+                for (int c = 0; c < 4; c++) {
+                    uint32_t v = 0;
+                    for (int g = 0; g < 4; g++) {
+                        v |= ((dst[2 * g] >> (8 * c + i)) & 1u) << (2 * g);
+                        v |= ((dst[2 * g + 1] >> (8 * c + i)) & 1u) << (2 * g + 1);
+                    }
+                    src[4 * i + c] = (uint8_t)v;
+                }
+        }
+        return;
+    }
+    k4_header(a, (uint32_t *)(hd + b * CQ_Q4K_HDR), inverse);
 }
 
 // ---- Q6K: 210-byte blocks {u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d} -----
@@ -172,6 +227,11 @@ hipError_t launch(const cq_weight *w, uint8_t *aos, bool inverse, hipStream_t s)
     case CQ_DTYPE_Q4K: {
         unsigned grid = (unsigned)((nblocks * 9 + threads - 1) / threads);
         repack_q4k<<<grid, threads, 0, s>>>(aos, w->p0, w->p1, nblocks, inverse);
+        break;
+    }
+    case CQ_DTYPE_Q5K: {
+        unsigned grid = (unsigned)((nblocks * 11 + threads - 1) / threads);
+        repack_q5k<<<grid, threads, 0, s>>>(aos, w->p0, w->p1, w->p2, nblocks, inverse);
         break;
     }
     case CQ_DTYPE_Q6K: {

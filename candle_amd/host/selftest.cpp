@@ -32,6 +32,7 @@ static void host_only() {
     EXPECT(block_size(GgmlDType::Q8_0) == 32 && type_size(GgmlDType::Q8_0) == 34, "Q8_0 sizes");
     EXPECT(block_size(GgmlDType::Q8_1) == 32 && type_size(GgmlDType::Q8_1) == 36, "Q8_1 sizes");
     EXPECT(block_size(GgmlDType::Q4K) == 256 && type_size(GgmlDType::Q4K) == 144, "Q4K sizes");
+    EXPECT(block_size(GgmlDType::Q5K) == 256 && type_size(GgmlDType::Q5K) == 176, "Q5K sizes");
     EXPECT(block_size(GgmlDType::Q6K) == 256 && type_size(GgmlDType::Q6K) == 210, "Q6K sizes");
     EXPECT(block_size(GgmlDType::Q8K) == 256 && type_size(GgmlDType::Q8K) == 292, "Q8K sizes");
     EXPECT(to_u32(ggml_dtype_from_u32(12)) == 12, "dtype id round trip");

@@ -28,13 +28,14 @@ class GgmlDType(enum.IntEnum):
     Q8_0 = 8
     Q8_1 = 9
     Q4K = 12
+    Q5K = 13
     Q6K = 14
     Q8K = 15
 
     @classmethod
     def from_str(cls, name: str) -> "GgmlDType":
         """Names accepted by the reference's Python `Tensor.quantize` (lib.rs:1082-1098)."""
-        table = {"q4_0": cls.Q4_0, "q8_0": cls.Q8_0, "q8_1": cls.Q8_1, "q4k": cls.Q4K, "q6k": cls.Q6K,
+        table = {"q4_0": cls.Q4_0, "q8_0": cls.Q8_0, "q8_1": cls.Q8_1, "q4k": cls.Q4K, "q5k": cls.Q5K, "q6k": cls.Q6K,
                  "q8k": cls.Q8K, "f32": cls.F32, "f16": cls.F16}
         key = name.lower()
         if key not in table:
@@ -60,7 +61,7 @@ class GgmlDType(enum.IntEnum):
         return GgmlDType(qhip.load().cq_vec_dot_type(int(self)))
 
 
-_WEIGHT_TYPES = (GgmlDType.Q4_0, GgmlDType.Q8_0, GgmlDType.Q4K, GgmlDType.Q6K)
+_WEIGHT_TYPES = (GgmlDType.Q4_0, GgmlDType.Q8_0, GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K)
 
 
 class QTensor:

@@ -33,6 +33,7 @@ enum {
     CQ_DTYPE_Q8_0 = 8,
     CQ_DTYPE_Q8_1 = 9,  /* activation format only */
     CQ_DTYPE_Q4K = 12,
+    CQ_DTYPE_Q5K = 13,
     CQ_DTYPE_Q6K = 14,
     CQ_DTYPE_Q8K = 15   /* activation format only */
 };

@@ -264,6 +264,6 @@ def test_load_gguf_to_device_and_matmul(tmp_path):
 @pytest.mark.gpu
 def test_load_gguf_rejects_types_without_device_kernels(tmp_path):
     path = str(tmp_path / "q5.gguf")
-    G.save_gguf(path, {"w": HostQTensor(13, bytes(176), (1, 256))}, {})
-    with pytest.raises(GgufError, match="Q5K tensors are not supported on the device"):
+    G.save_gguf(path, {"w": HostQTensor(11, bytes(110), (1, 256))}, {})
+    with pytest.raises(GgufError, match="Q3K tensors are not supported on the device"):
         G.load_gguf(path)

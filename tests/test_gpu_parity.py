@@ -48,7 +48,7 @@ def make_inputs(seed, m, k, n, wscale=0.02, outliers=False):
     return w, x
 
 
-WEIGHT_DTYPES = [orc.Q4_0, orc.Q8_0, orc.Q4K, orc.Q6K]
+WEIGHT_DTYPES = [orc.Q4_0, orc.Q8_0, orc.Q4K, orc.Q5K, orc.Q6K]
 
 
 # ------------------------------------------------------------ activation quantizers ----
@@ -146,7 +146,7 @@ def test_int_dots_bit_exact(qh, dt, m, k, n):
     acts = np.concatenate([orc.quantize(orc.VEC_DOT_TYPE[dt], x[r]) for r in range(m)])
     wi, wm = orc.block_int_dots(dt, acts, m, blocks, n, k)
     assert np.array_equal(oi.cpu().numpy(), wi)
-    if dt == orc.Q4K:
+    if dt in (orc.Q4K, orc.Q5K):
         assert np.array_equal(om.cpu().numpy(), wm)
 
 
@@ -160,6 +160,10 @@ def test_int_dots_bit_exact(qh, dt, m, k, n):
     (orc.Q8_0, 1, 4096, 4096),
     (orc.Q4_0, 3, 64, 4),          # smallest shapes of the reference's tests
     (orc.Q4K, 5, 256, 3),
+    (orc.Q5K, 1, 4096, 4096),
+    (orc.Q5K, 1, 11008, 512),
+    (orc.Q5K, 6, 512, 40),
+    (orc.Q5K, 20, 1024, 24),       # more rows than one pass of the dot-product kernel takes
 ])
 def test_matvec_matches_oracle(qh, dt, m, k, n):
     w, x = make_inputs(7 * dt + k + n, m, k, n)
@@ -407,7 +411,7 @@ def test_reference_goldens_through_hip(qh, goldens, seeded_inputs):
     # quantized_tests.rs:1051-1151 (seeded m=11, k=512, n=21), weights quantized on the device
     g = goldens["seeded_matmul_m11_k512_n21"]
     lhs, rhs = seeded_inputs
-    for name, dt in (("q4k", orc.Q4K), ("q6k", orc.Q6K)):
+    for name, dt in (("q4k", orc.Q4K), ("q5k", orc.Q5K), ("q6k", orc.Q6K)):
         qw = qh.QWeight.zeros(dt, 21, 512).quantize_(dev(rhs))
         out = qh.qmatmul(qw, dev(lhs)).cpu().numpy().ravel()
         spot = [float(np.round(np.float32(1000.0) * out[i]) / np.float32(1000.0)) for i in g["flat_indices"]]
