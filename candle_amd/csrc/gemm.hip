@@ -49,12 +49,15 @@ constexpr int kThreads = kWaves * 64;
 //   d8   : [BM] f32
 //   minp : [BM][2 pieces][8] f16            d8 * bsum32_j split in two f16 pieces (Q4K)
 //   wgt  : per wave: [4 row groups][8 rows][8 chunks] of the 128-byte qs / ql plane (same swizzle),
-//          Q6K also [2 row groups][16 rows][4 chunks] of the 64-byte qh plane (chunk c at c ^ ((r/2)%4))
+//          Q6K also [2 row groups][16 rows][4 chunks] of the 64-byte qh plane (chunk c at c ^ ((r/2)%4)),
+//          Q5K also [32 rows][32 B] of the fifth-bit plane
+constexpr bool is_k4(int dt) { return dt == CQ_DTYPE_Q4K || dt == CQ_DTYPE_Q5K; }   // types with a min term
+
 template <int DT, int MT> struct Tile {
     static constexpr int kAct = MT * 8 * 1024;
     static constexpr int kD8 = (MT * 32 < 64 ? 64 : MT * 32) * 4;   // filled by whole-wave copies of 64 floats
-    static constexpr int kMin = DT == CQ_DTYPE_Q4K ? MT * 32 * 32 : 0;
-    static constexpr int kWgtWave = DT == CQ_DTYPE_Q4K ? 4096 : 6144;
+    static constexpr int kMin = is_k4(DT) ? MT * 32 * 32 : 0;
+    static constexpr int kWgtWave = DT == CQ_DTYPE_Q4K ? 4096 : DT == CQ_DTYPE_Q5K ? 5120 : 6144;
     static constexpr int oD8 = kAct, oMin = oD8 + kD8;
     static constexpr int kBytes = oMin + kMin;                                  // one activation stage (three of them)
     static constexpr int oWgt = 3 * kBytes;                                     // weights: one buffer per wave
@@ -98,6 +101,7 @@ struct LaneGeo {
     uint32_t act_off;   // copy of 8 rows x 128 B of activations: (l/8)*k + ((l%8) ^ (l/8))*16
     uint32_t wq_off;    // the same over the weights' 128-byte plane: (l/8)*kb*128 + ...
     uint32_t wh_off;    // Q6K qh plane, 16 rows x 64 B: (l/4)*kb*64 + ((l%4) ^ ((l/8)%4))*16
+    uint32_t w5_off;    // Q5K fifth-bit plane, 32 rows x 32 B: (l/2)*kb*32 + (l%2)*16
     uint32_t col[4];    // operand read: byte offset of chunk 2j+h of row l%32 inside a [4][8][8] x 16 B image
     uint32_t qh_col[4]; // Q6K: byte offset of the 8 bytes of unit 2x+h of row l%32 inside the qh image
 };
@@ -110,6 +114,7 @@ __device__ __forceinline__ LaneGeo lane_geo(int lane, int64_t k) {
     g.wq_off = r8 * kb * 128u + ((c8 ^ r8) << 4);
     const uint32_t r16 = lane >> 2, c4 = lane & 3;
     g.wh_off = r16 * kb * 64u + ((c4 ^ ((r16 >> 1) & 3)) << 4);
+    g.w5_off = (uint32_t)(lane >> 1) * kb * 32u + (uint32_t)(lane & 1) * 16u;
     const uint32_t r = lane & 31, h = lane >> 5;
 #pragma unroll
     for (uint32_t j = 0; j < 4; j++) {
@@ -137,7 +142,7 @@ __device__ __forceinline__ void stage_issue(uint8_t *buf, const cq_weight &w, co
     for (int j = 0; j < (MT * 32 + 63) / 64; j++) {
         if (j == wave) dma4(a.dT + b * a.m_stride + m0 + j * 64, lane * 4u, buf + T::oD8 + j * 256);
     }
-    if (DT == CQ_DTYPE_Q4K) {
+    if (is_k4(DT)) {
 #pragma unroll
         for (int j = 0; j < MT; j++) {
             if (j + 4 == wave)
@@ -159,12 +164,14 @@ __device__ __forceinline__ void stage_weights(uint8_t *wl, const cq_weight &w, c
             for (int rg = 0; rg < 2; rg++)
                 dma16(w.p1 + ((n_tile + rg * 16) * kb + b) * 64, g.wh_off, wl + 4096 + rg * 1024);
         }
+        if (DT == CQ_DTYPE_Q5K) dma16(w.p2 + (n_tile * kb + b) * 32, g.w5_off, wl + 4096);
     }
 }
 
 // The small per-block weight fields, loaded straight into registers one block ahead.
 template <int DT> struct WHead;
 template <> struct WHead<CQ_DTYPE_Q4K> { uint32_t dd; uint4 rec; };   // d | dmin << 16; records {sc, sc, mn, mn} per 32 qs bytes
+template <> struct WHead<CQ_DTYPE_Q5K> : WHead<CQ_DTYPE_Q4K> {};     // the same header plane
 template <> struct WHead<CQ_DTYPE_Q6K> { uint4 sc; uint32_t d; };   // re-packed scales (two per unit); d
 __device__ __forceinline__ void load_head(const cq_weight &w, int64_t blk, WHead<CQ_DTYPE_Q4K> &r) {
     const uint32_t *h = (const uint32_t *)(w.p1 + blk * CQ_Q4K_HDR);
@@ -187,7 +194,7 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, 
                                           float dw, v8h wmin, int lane, v16f (&out)[MT]) {
     typedef Tile<DT, MT> T;
     if constexpr (T0 >= T1) return;
-    constexpr bool MINS = DT == CQ_DTYPE_Q4K;
+    constexpr bool MINS = is_k4(DT);
     const int h = lane >> 5, col = lane & 31;
     const uint8_t *d8p = cur + T::oD8 + h * 16;        // rows 8j + 4h + [0,4) of a tile
     const uint8_t *mnp = cur + T::oMin + col * 32;     // this lane's row of min pieces
@@ -270,6 +277,43 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g
             bh[2 * gi][i] = (int)pk_mul_u16(lo4, sh0);
             bl[2 * gi + 1][i] = (int)pk_mul_u16(hi4, sl1);   // sub-block 2g+1
             bh[2 * gi + 1][i] = (int)pk_mul_u16(hi4, sh1);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const float v = -dmin * (float)((rec[j >> 1] >> (16 + 8 * (j & 1))) & 0xff);
+        const _Float16 p1 = (_Float16)v;
+        wmin[j] = h == 0 ? p1 : (_Float16)(v - (float)p1);
+    }
+}
+
+// Q5K: the Q4K nibbles plus a fifth bit per quant (words {L, H} per 32 qs bytes, bit 8c + i for byte c
+// of qs word i); scale times quant has up to 11 bits and is split at bit 7, as for Q6K.
+__device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g, const WHead<CQ_DTYPE_Q5K> &wb,
+                                             int lane, v4i (&bl)[8], v4i (&bh)[8], float &dw, v8h &wmin) {
+    const int h = lane >> 5;
+    const uint32_t row = lane & 31;
+    dw = cq_h2f((uint16_t)(wb.dd & 0xffff));
+    const float dmin = cq_h2f((uint16_t)(wb.dd >> 16));
+    const uint32_t rec[4] = {wb.rec.x, wb.rec.y, wb.rec.z, wb.rec.w};   // {sc[2g], sc[2g+1], mn[2g], mn[2g+1]}
+    const uint4 f0 = *(const uint4 *)(wl + 4096 + row * 32u), f1 = *(const uint4 *)(wl + 4096 + row * 32u + 16u);
+    const uint32_t fl[4] = {f0.x, f0.z, f1.x, f1.z}, fh[4] = {f0.y, f0.w, f1.y, f1.w};
+#pragma unroll
+    for (int gi = 0; gi < 4; gi++) {
+        // qs bytes 32g + 16h + [0,16) = qs words 4h .. 4h+3: low nibbles = K-slice 2g, high nibbles = slice 2g+1
+        const uint4 q = *(const uint4 *)(wl + g.col[gi]);
+        const uint32_t s0 = dup16(rec[gi] & 0xff), s1 = dup16((rec[gi] >> 8) & 0xff);
+        const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t lo5 = (qw[i] & 0x0F0F0F0Fu) | (((fl[gi] >> (4 * h + i)) & 0x01010101u) << 4);
+            const uint32_t hi5 = ((qw[i] >> 4) & 0x0F0F0F0Fu) | (((fh[gi] >> (4 * h + i)) & 0x01010101u) << 4);
+            const uint32_t a02 = pk_mul_u16(lo5 & 0x00FF00FFu, s0), a13 = pk_mul_u16((lo5 >> 8) & 0x00FF00FFu, s0);
+            const uint32_t b02 = pk_mul_u16(hi5 & 0x00FF00FFu, s1), b13 = pk_mul_u16((hi5 >> 8) & 0x00FF00FFu, s1);
+            bl[2 * gi][i] = (int)(__builtin_amdgcn_perm(a13, a02, 0x06020400u) & 0x7F7F7F7Fu);
+            bh[2 * gi][i] = (int)__builtin_amdgcn_perm(pk_ashr7_i16(a13), pk_ashr7_i16(a02), 0x06020400u);
+            bl[2 * gi + 1][i] = (int)(__builtin_amdgcn_perm(b13, b02, 0x06020400u) & 0x7F7F7F7Fu);
+            bh[2 * gi + 1][i] = (int)__builtin_amdgcn_perm(pk_ashr7_i16(b13), pk_ashr7_i16(b02), 0x06020400u);
         }
     }
 #pragma unroll
@@ -543,13 +587,14 @@ hipError_t cq_launch_gemm_grouped(const cq_weight *const *experts, int n_experts
                                   float *y, hipStream_t s) {
     if (a.m_stride < ((int64_t)offsets[n_experts] + 31) / 32 * 32) return hipErrorInvalidValue;
     if (experts[0]->dtype == CQ_DTYPE_Q4K) return launch_grouped<CQ_DTYPE_Q4K>(experts, n_experts, offsets, a, y, s);
+    if (experts[0]->dtype == CQ_DTYPE_Q5K) return launch_grouped<CQ_DTYPE_Q5K>(experts, n_experts, offsets, a, y, s);
     return launch_grouped<CQ_DTYPE_Q6K>(experts, n_experts, offsets, a, y, s);
 }
 
 bool cq_gemm_supported(const cq_weight *w, int64_t m, int act_dtype) {
     (void)m;
     // the copies address rows with 32-bit offsets: 8 rows of activations, 16 rows of a weight plane
-    return (w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q6K) && act_dtype == CQ_DTYPE_Q8K && w->k >= 256 &&
+    return (w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q5K || w->dtype == CQ_DTYPE_Q6K) && act_dtype == CQ_DTYPE_Q8K && w->k >= 256 &&
            w->k <= (1 << 24) && w->n % 32 == 0;
 }
 
@@ -558,5 +603,6 @@ hipError_t cq_launch_gemm(const cq_weight *w, cq_act_view a, int act_dtype, int6
     if (m == 0 || w->n == 0) return hipSuccess;
     if (a.m_stride < (m + 127) / 128 * 128) return hipErrorInvalidValue;   // rows the last tile may read
     if (w->dtype == CQ_DTYPE_Q4K) return launch_dt<CQ_DTYPE_Q4K>(w, a, m, y, s);
+    if (w->dtype == CQ_DTYPE_Q5K) return launch_dt<CQ_DTYPE_Q5K>(w, a, m, y, s);
     return launch_dt<CQ_DTYPE_Q6K>(w, a, m, y, s);
 }

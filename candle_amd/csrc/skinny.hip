@@ -60,14 +60,17 @@ __device__ __forceinline__ void dma4(const void *base, uint32_t off, uint8_t *ld
 
 // Per-wave LDS buffer for RT groups of eight activation rows:
 //   wgt : [2 row groups][8 rows][8 chunks of 16 B] of the 128-byte qs / ql plane, chunk c of row r at c ^ (r%8);
-//         Q6K also [16 rows][4 chunks] of the 64-byte qh plane (chunk c at c ^ ((r/2)%4))
+//         Q6K also [16 rows][4 chunks] of the 64-byte qh plane (chunk c at c ^ ((r/2)%4)),
+//         Q5K also [16 rows][32 B] of the fifth-bit plane
 //   act : [RT row groups][2 K-halves][8 rows][8 chunks], same swizzle
 //   d8  : [8*RT] f32         minp : [8*RT][2 pieces][8] f16 (Q4K)
+constexpr bool is_k4(int dt) { return dt == CQ_DTYPE_Q4K || dt == CQ_DTYPE_Q5K; }   // types with a min term
+
 template <int DT, int RT> struct Buf {
-    static constexpr int kWgt = DT == CQ_DTYPE_Q4K ? 2048 : 3072;
+    static constexpr int kWgt = DT == CQ_DTYPE_Q4K ? 2048 : DT == CQ_DTYPE_Q5K ? 2560 : 3072;
     static constexpr int oAct = kWgt, kAct = RT * 2048;
     static constexpr int oD8 = oAct + kAct, kD8 = RT * 32;
-    static constexpr int oMin = oD8 + kD8, kMin = DT == CQ_DTYPE_Q4K ? RT * 256 : 0;
+    static constexpr int oMin = oD8 + kD8, kMin = is_k4(DT) ? RT * 256 : 0;
     static constexpr int kRaw = oMin + kMin;
     // the buffer also carries the wave's partial results at the end: 1 KiB per 16 activation rows
     static constexpr int kBytes = kRaw < 2048 ? 2048 : kRaw;
@@ -79,6 +82,7 @@ __device__ __forceinline__ uint32_t swz_col(uint32_t r, uint32_t c) {
 
 template <int DT> struct WHead;
 template <> struct WHead<CQ_DTYPE_Q4K> { uint32_t dd; uint4 rec; };   // d | dmin << 16; records {sc, sc, mn, mn} per 32 qs bytes
+template <> struct WHead<CQ_DTYPE_Q5K> : WHead<CQ_DTYPE_Q4K> {};       // the same header plane
 template <> struct WHead<CQ_DTYPE_Q6K> { uint4 sc; uint32_t d; };     // re-packed scales (two per unit); d
 __device__ __forceinline__ void load_head(const cq_weight &w, int64_t blk, WHead<CQ_DTYPE_Q4K> &r) {
     const uint32_t *h = (const uint32_t *)(w.p1 + blk * CQ_Q4K_HDR);
@@ -116,6 +120,38 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, int lane, const 
     }
     // min term operand: 32 K-slots = activation pieces [1,1,2,2] x weight pieces [1,2,1,2] of the
     // eight sub-block values -dmin*min_j
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const float v = -dmin * (float)((rec[j >> 1] >> (16 + 8 * (j & 1))) & 0xff);
+        const _Float16 p1 = (_Float16)v;
+        wmin[j] = (kq & 1) == 0 ? p1 : (_Float16)(v - (float)p1);
+    }
+}
+
+// Q5K: the quants are the Q4K nibbles plus a fifth bit (words {L, H} per 32 qs bytes, bit 8c + i for
+// byte c of qs word i); scale times quant has up to 11 bits and is split at bit 7 like Q6K's.
+__device__ __forceinline__ void block_unpack(const uint8_t *wl, int lane, const WHead<CQ_DTYPE_Q5K> &wb, v4i (&bl)[4],
+                                             v4i (&bh)[4], float &dw, v8h &wmin) {
+    const uint32_t r = lane & 15, kq = lane >> 4;
+    dw = cq_h2f((uint16_t)(wb.dd & 0xffff));
+    const float dmin = cq_h2f((uint16_t)(wb.dd >> 16));
+    const uint32_t rec[4] = {wb.rec.x, wb.rec.y, wb.rec.z, wb.rec.w};
+    const uint32_t hi = kq >> 1, nsh = hi * 4, w0 = 4 * (kq & 1);   // first qs word of the lane's 16 bytes
+    const uint4 f0 = *(const uint4 *)(wl + 2048 + r * 32u), f1 = *(const uint4 *)(wl + 2048 + r * 32u + 16u);
+    const uint32_t fifth[4] = {hi ? f0.y : f0.x, hi ? f0.w : f0.z, hi ? f1.y : f1.x, hi ? f1.w : f1.z};
+#pragma unroll
+    for (int gi = 0; gi < 4; gi++) {
+        const uint4 q = *(const uint4 *)(wl + swz_col(r, 2 * gi + (kq & 1)));
+        const uint32_t sc16 = dup16((rec[gi] >> (8 * hi)) & 0xff);   // scale of sub-block 2g + hi
+        const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t q5 = ((qw[i] >> nsh) & 0x0F0F0F0Fu) | (((fifth[gi] >> (w0 + i)) & 0x01010101u) << 4);
+            const uint32_t p02 = pk_mul_u16(q5 & 0x00FF00FFu, sc16), p13 = pk_mul_u16((q5 >> 8) & 0x00FF00FFu, sc16);
+            bl[gi][i] = (int)(__builtin_amdgcn_perm(p13, p02, 0x06020400u) & 0x7F7F7F7Fu);
+            bh[gi][i] = (int)__builtin_amdgcn_perm(pk_ashr7_i16(p13), pk_ashr7_i16(p02), 0x06020400u);
+        }
+    }
 #pragma unroll
     for (int j = 0; j < 8; j++) {
         const float v = -dmin * (float)((rec[j >> 1] >> (16 + 8 * (j & 1))) & 0xff);
@@ -167,7 +203,7 @@ template <int DT, int RT>
 __global__ void __launch_bounds__(kThreads) skinny_kernel(cq_weight w, cq_act_view a, int64_t m0, int64_t m,
                                                           float *__restrict__ y) {
     typedef Buf<DT, RT> B;
-    constexpr bool MINS = DT == CQ_DTYPE_Q4K;
+    constexpr bool MINS = is_k4(DT);
     constexpr int NT = (RT + 1) / 2;   // 16-row tiles
     constexpr int SHIFT = DT == CQ_DTYPE_Q4K ? 3 : 7;
     extern __shared__ __align__(16) uint8_t smem[];
@@ -184,6 +220,7 @@ __global__ void __launch_bounds__(kThreads) skinny_kernel(cq_weight w, cq_act_vi
     const uint32_t wq_off = r8 * (uint32_t)kb * 128u + ((c8 ^ r8) << 4);
     const uint32_t r16 = lane >> 2, c4 = lane & 3;
     const uint32_t wh_off = r16 * (uint32_t)kb * 64u + ((c4 ^ ((r16 >> 1) & 3)) << 4);
+    const uint32_t w5_off = (lane >> 1) * (uint32_t)kb * 32u + (lane & 1) * 16u;   // Q5K: 16 rows x 32 B, lanes 0..31
     // activation operand reads: row of tile t clamped to the rows held
     uint32_t a_col[NT][2];
 #pragma unroll
@@ -203,6 +240,7 @@ __global__ void __launch_bounds__(kThreads) skinny_kernel(cq_weight w, cq_act_vi
 #pragma unroll
         for (int rg = 0; rg < 2; rg++) dma16(w.p0 + ((n_tile + rg * 8) * kb + b) * 128, wq_off, buf + rg * 1024);
         if (DT == CQ_DTYPE_Q6K) dma16(w.p1 + (n_tile * kb + b) * 64, wh_off, buf + 2048);
+        if (DT == CQ_DTYPE_Q5K && lane < 32) dma16(w.p2 + (n_tile * kb + b) * 32, w5_off, buf + 2048);
 #pragma unroll
         for (int i = 0; i < 2 * RT; i++) {
             const int rg = i >> 1, kh = i & 1;
@@ -446,7 +484,7 @@ hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hip
 
 bool cq_skinny_supported(const cq_weight *w, int act_dtype) {
     // the copies address 8 rows of activations and 16 rows of a weight plane with 32-bit offsets
-    const bool kquant = (w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q6K) && act_dtype == CQ_DTYPE_Q8K;
+    const bool kquant = (w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q5K || w->dtype == CQ_DTYPE_Q6K) && act_dtype == CQ_DTYPE_Q8K;
     const bool q8 = (w->dtype == CQ_DTYPE_Q8_0 || w->dtype == CQ_DTYPE_Q4_0) && act_dtype == CQ_DTYPE_Q8_0 && w->k % 256 == 0;
     return (kquant || q8) && w->k >= 256 && w->k <= (1 << 24) && w->n % 16 == 0 && w->n > 0;
 }
@@ -458,5 +496,6 @@ hipError_t cq_launch_skinny(const cq_weight *w, cq_act_view a, int act_dtype, in
     if (w->dtype == CQ_DTYPE_Q8_0) return launch_blk32<CQ_DTYPE_Q8_0>(w, a, m, y, s);
     if (w->dtype == CQ_DTYPE_Q4_0) return launch_blk32<CQ_DTYPE_Q4_0>(w, a, m, y, s);
     if (w->dtype == CQ_DTYPE_Q4K) return launch_dt<CQ_DTYPE_Q4K>(w, a, m, y, s);
+    if (w->dtype == CQ_DTYPE_Q5K) return launch_dt<CQ_DTYPE_Q5K>(w, a, m, y, s);
     return launch_dt<CQ_DTYPE_Q6K>(w, a, m, y, s);
 }

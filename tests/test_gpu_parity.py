@@ -214,7 +214,7 @@ def test_fused_decode_equals_two_launch_path(qh, dt, k, n):
     assert torch.equal(qh.qmatmul(qw, dev(x)), torch.zeros((1, n), device="cuda"))
 
 
-@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K])
+@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q5K, orc.Q6K])
 def test_fused_decode_sign_of_scale_cases(qh, dt):
     """The Q8K scale takes the sign of the FIRST element with the largest magnitude.  Blocks where
     that magnitude occurs with both signs (negative first, positive first, in the same eight
@@ -279,7 +279,7 @@ def test_ragged_batches_match_oracle(qh, dt, m, k, n):
     check_f32(got, one)
 
 
-@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K])
+@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q5K, orc.Q6K])
 @pytest.mark.parametrize("m,k,n", [(2, 256, 16), (3, 512, 48), (8, 4096, 64), (9, 1024, 32), (16, 2048, 80),
                                    (17, 768, 16), (24, 11008, 32), (32, 4096, 16), (33, 2304, 48), (5, 14336, 16)])
 def test_skinny_matches_oracle(qh, dt, m, k, n):
@@ -321,7 +321,7 @@ def test_skinny_unsupported_shapes_are_refused(qh):
         check_f32(qh.qmatmul(qw, dev(x)).cpu().numpy(), orc.matmul(dt, x, orc.quantize(dt, w), n))
 
 
-@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K])
+@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q5K, orc.Q6K])
 def test_gemm_ragged_rows_large(qh, dt):
     """M = 300 (not a multiple of the 128-row workgroup tile) on a K-split shape: every output row
     of the tile kernel equals the dot-product kernels' result for that row within tolerance."""
@@ -337,7 +337,7 @@ def test_gemm_ragged_rows_large(qh, dt):
     check_f32(got, ref)
 
 
-@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K])
+@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q5K, orc.Q6K])
 @pytest.mark.parametrize("m,k,n", [(9, 256, 32), (33, 512, 96), (64, 1024, 160), (130, 768, 288), (11, 512, 64),
                                    (1, 256, 32), (129, 2048, 416)])
 def test_gemm_matches_oracle_small(qh, dt, m, k, n):
@@ -350,7 +350,7 @@ def test_gemm_matches_oracle_small(qh, dt, m, k, n):
     check_f32(got, orc.matmul(dt, x, blocks, n))
 
 
-@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K])
+@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q5K, orc.Q6K])
 def test_gemm_needs_32_row_multiple(qh, dt):
     """Weight row counts that are not a multiple of 32 take the dot-product kernels: forcing the
     tile kernel is an error, the automatic choice still matches the oracle."""
@@ -363,7 +363,7 @@ def test_gemm_needs_32_row_multiple(qh, dt):
     check_f32(qh.qmatmul(qw, dev(x)).cpu().numpy(), orc.matmul(dt, x, blocks, n))
 
 
-@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K])
+@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q5K, orc.Q6K])
 @pytest.mark.parametrize("m,k,n", [(512, 4096, 14336), (512, 14336, 4096)])
 def test_prefill_gemm_config3(qh, dt, m, k, n):
     """BASELINE config 3 at full size: M = 512 tokens on the Mistral FFN shapes, activations N(0,1)
