@@ -11,6 +11,7 @@
 // into the int8 weights as two digits and the block is contracted with two MFMAs per K-slice:
 //   Q4K:  sc = 8*sh + sl (3-bit digits): operands sh*q4, sl*q4 <= 105;  I = 8*acc_hi + acc_lo
 //   Q6K:  P = sc*(q6-32) (13 bits signed): operands P >> 7, P & 127;    I = 128*acc_hi + acc_lo
+//   Q5K:  as Q4K with 5-bit quants (k_quants.rs:1361-1447): P = sc*q5 (11 bits), split like Q6K's
 // I is the same integer as on the CPU.  The Q4K min term is a small f32 contraction over the
 // eight sub-blocks; it runs on the f16 MFMA with both factors split in two f16 pieces (products
 // exact to ~2^-22) and accumulates straight into the f32 result.

@@ -3,7 +3,7 @@
 // for Q6K) - the small-batch decode and the per-expert shapes of a mixture-of-experts layer, where
 // the weights are still read once and the job stays bound by HBM.  The arithmetic is that of the
 // prefill GEMM (gemm.hip): sub-block scales folded into the int8 weight operands as two digits,
-// exact block integers I = 8*hi + lo (Q4K) / 128*hi + lo (Q6K), the Q4K min term on the f16 MFMA.
+// exact block integers I = 8*hi + lo (Q4K) / 128*hi + lo (Q5K, Q6K), the Q4K / Q5K min term on the f16 MFMA.
 //
 // Work split: with so few activation rows there is no tile to reuse weights over, so the K
 // dimension is split instead.  A workgroup owns 16 weight rows (one 16x16x64 MFMA operand); its

@@ -128,8 +128,8 @@ size_t cq_workspace_bytes(const cq_weight *w, int64_t m, int flags);
 int cq_qmatmul(const cq_weight *w, const float *x_dev, int64_t m, float *y_dev, int flags,
                void *workspace_dev, size_t workspace_bytes, void *stream);
 /* Debug/verification: the per-block integer dot products the f32 result is combined from
- * (k_quants.rs:1221-1241 for Q4K, :1615-1633 for Q6K, :245-250 / :640-645 for Q4_0/Q8_0).
- * out_i[(r*n + c)*kb + b] = I_b; out_mn likewise = sum_j bsums_j*min_j (Q4K only, else NULL). */
+ * (k_quants.rs:1221-1241 for Q4K, :1418-1438 for Q5K, :1615-1633 for Q6K, :245-250 / :640-645 for Q4_0/Q8_0).
+ * out_i[(r*n + c)*kb + b] = I_b; out_mn likewise = sum_j bsums_j*min_j (Q4K and Q5K, else NULL). */
 int cq_qmatmul_int_dots(const cq_weight *w, const float *x_dev, int64_t m, int32_t *out_i_dev,
                         int32_t *out_mn_dev, void *workspace_dev, size_t workspace_bytes,
                         void *stream);
