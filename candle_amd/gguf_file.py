@@ -326,6 +326,19 @@ class Content:
             raise GgufError(f"cannot find tensor info for {name}")
         return info.read(r, self.tensor_data_offset)
 
+    def tensor_view(self, buf, name: str) -> HostQTensor:
+        """The tensor's blocks as a view into `buf`, the whole file as a buffer (an `mmap`, `bytes`):
+        nothing is copied on the host, the upload reads the file's pages directly (what the
+        reference's reader leaves as a TODO, ggml_file.rs:213)."""
+        info = self.tensor_infos.get(name)
+        if info is None:
+            raise GgufError(f"cannot find tensor info for {name}")
+        size = tensor_size_in_bytes(info.ggml_dtype, info.shape)
+        start = self.tensor_data_offset + info.offset
+        if start + size > len(buf):
+            raise GgufError("failed to fill whole buffer")
+        return HostQTensor(info.ggml_dtype, np.frombuffer(buf, dtype=np.uint8, count=size, offset=start), info.shape)
+
     def tensor(self, r: BinaryIO, name: str, dev: int = 0):
         """`Content::tensor` (gguf_file.rs:470-481) with a device: read the blocks, upload, re-pack."""
         return self.tensor_host(r, name).to_device(dev)
@@ -378,9 +391,16 @@ def write(w: BinaryIO, metadata: Iterable[Tuple[str, Any]], tensors: Iterable[Tu
 def load_gguf(path: str, dev: int = 0):
     """`load_gguf(path, device)` of the Python binding (lib.rs:1326-1382): every tensor of the file on
     the device, and the metadata as plain Python objects."""
+    import mmap
     with open(path, "rb") as f:
         content = Content.read(f)
-        tensors = {name: content.tensor(f, name, dev) for name in content.tensor_infos}
+        if not content.tensor_infos:
+            return {}, {k: v.to_python() for k, v in content.metadata.items()}
+        # The tensor bytes go from the page cache to the device without a host copy of our own.  The
+        # mapping is not closed by hand: it goes away with the last view into it (an upload that
+        # raises still holds one in its traceback, and closing under it would be an error of its own).
+        mm = mmap.mmap(f.fileno(), 0, access=mmap.ACCESS_READ)
+        tensors = {name: content.tensor_view(mm, name).to_device(dev) for name in content.tensor_infos}
     return tensors, {k: v.to_python() for k, v in content.metadata.items()}
 
 
