@@ -515,3 +515,60 @@ def test_moe_scatter_add_order_and_shapes(qh, tokens, total, hidden):
     wt_d = dev(wt) if total else torch.zeros((0,), device="cuda")
     got = qh.moe_scatter_add(y_d, rid_d, wt_d, tokens).cpu().numpy()
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_moe_config4_full_size(qh):
+    """BASELINE config 4 at its real shape: 8 experts of w1/w3 [14336 x 4096] Q4K and w2 [4096 x 14336]
+    Q6K, 64 tokens routed top-2.  The oracle would need minutes for all of it, so: every expert's
+    slice of each grouped launch is compared with the plain tile kernel on the same rows (the same
+    workgroup body without the tile table), a sample of weight rows of every expert with the
+    oracle, and the combine with the sequential index_add."""
+    hidden, ffn, n_e, tokens, top_k = 4096, 14336, 8, 64, 2
+    rng = np.random.default_rng(4)
+    gen = torch.Generator(device="cuda")
+    xs = rng.standard_normal((tokens, hidden)).astype(np.float32)
+    logits = rng.standard_normal((tokens, n_e)).astype(np.float32)
+    offsets, row_ids, weights = orc.moe_route(orc.softmax_last_dim(logits), top_k)
+    assert offsets[-1] == tokens * top_k
+
+    def make(dt, n, k, seed):
+        gen.manual_seed(seed)
+        w = torch.randn((n, k), generator=gen, device="cuda", dtype=torch.float32) * 0.02
+        return qh.QWeight.zeros(dt, n, k).quantize_(w)
+
+    q1 = [make(orc.Q4K, ffn, hidden, 100 + e) for e in range(n_e)]
+    q3 = [make(orc.Q4K, ffn, hidden, 200 + e) for e in range(n_e)]
+    q2 = [make(orc.Q6K, hidden, ffn, 300 + e) for e in range(n_e)]
+    x_d, rid_d, wt_d = dev(xs), dev(row_ids), dev(weights)
+    h1 = qh.qmatmul_grouped(q1, x_d, rid_d, offsets)
+    h3 = qh.qmatmul_grouped(q3, x_d, rid_d, offsets)
+    h = qh.silu_mul(h1, h3)
+    y = qh.qmatmul_grouped(q2, h, None, offsets)
+    y_fused = qh.qmatmul_grouped(q2, h1, None, offsets, pre=qh.PRE_SILU_MUL, aux=h3)
+    assert torch.allclose(y, y_fused, rtol=1e-5, atol=1e-5)   # w2 splits K: partial sums are added in any order
+    ys = qh.moe_scatter_add(y, rid_d, wt_d, tokens)
+    hn, yn = h.cpu().numpy(), y.cpu().numpy()
+    sample13 = rng.choice(ffn, 24, replace=False)
+    sample2 = rng.choice(hidden, 24, replace=False)
+    for e in range(n_e):
+        sl = slice(int(offsets[e]), int(offsets[e + 1]))
+        if sl.start == sl.stop:
+            continue
+        cur = xs[row_ids[sl]]
+        cur_d = dev(cur)
+        # grouped launch == plain tile kernel on the expert's rows, up to the order in which the partial
+        # sums of a split K are added (a lone expert's launch splits K to fill the machine)
+        for got, qs, inp in ((h1, q1, cur_d), (h3, q3, cur_d), (y, q2, h[sl].contiguous())):
+            assert torch.allclose(got[sl], qh.qmatmul(qs[e], inp, qh.FLAG_FORCE_GEMM), rtol=1e-5, atol=1e-5), e
+        # sampled weight rows against the oracle (GGML rows are independent: a row's blocks are a matrix of one row)
+        for qs, inp, got, k, rows in ((q1, cur, h1, hidden, sample13), (q3, cur, h3, hidden, sample13),
+                                      (q2, hn[sl], y, ffn, sample2)):
+            blocks = qs[e].to_ggml().reshape(qs[e].shape[0], -1)
+            sub = np.ascontiguousarray(blocks[rows]).ravel()
+            want = orc.matmul(qs[e].dtype, inp, sub, len(rows))
+            have = got[sl].cpu().numpy()[:, rows]
+            assert np.linalg.norm(have - want) <= REL_L2_TOL * np.linalg.norm(want), e
+    acc = np.zeros((tokens, hidden), np.float32)
+    for p in range(offsets[-1]):               # sequential index_add in expert order
+        acc[row_ids[p]] += yn[p] * weights[p]
+    assert np.array_equal(ys.cpu().numpy(), acc)
