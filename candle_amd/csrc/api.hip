@@ -373,8 +373,11 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
     // (the 32-element-block types from 4 rows (Q8_0) or 5 rows (Q4_0) on: below that the batched
     // dot-product kernel is as fast or faster, it has no per-block scaling of MFMA results to do)
     const int64_t skinny_from = w->dtype == CQ_DTYPE_Q8_0 ? 4 : w->dtype == CQ_DTYPE_Q4_0 ? 5 : 2;
+    // Q8_0 / Q4_0 have no tile kernel: the split-K kernel, 32 rows per pass over the weights, stays ahead of
+    // the dot-product kernel (8 rows per pass) at every row count.
+    const bool has_tile_kernel = cq_gemm_supported(w, m, act);
     if (!(flags & (CQ_FLAG_FORCE_GEMM | CQ_FLAG_FORCE_MATVEC)) && m >= skinny_from && cq_skinny_supported(w, act) &&
-        (m <= 32 || (m <= 128 && w->n < 8192))) {
+        (m <= 32 || (m <= 128 && w->n < 8192) || !has_tile_kernel)) {
         CQ_HIP_CHECK(cq_launch_skinny(w, v, act, m, y_dev, s));
         return CQ_OK;
     }

@@ -264,7 +264,7 @@ def test_small_batch_matches_oracle(qh, dt, m, k, n):
 
 @pytest.mark.parametrize("dt", WEIGHT_DTYPES)
 @pytest.mark.parametrize("m,k,n", [(3, 512, 37), (5, 1024, 64), (7, 2048, 9), (9, 256, 130), (12, 11008, 24),
-                                   (2, 256, 8), (8, 14336, 16)])
+                                   (2, 256, 8), (8, 14336, 16), (70, 512, 48), (133, 256, 32)])
 def test_ragged_batches_match_oracle(qh, dt, m, k, n):
     """Row counts that do not fill the 4- and 8-row batches of the dot-product kernels, weight row
     counts that are not a multiple of the waves per workgroup, the shortest rows (one K block) and
