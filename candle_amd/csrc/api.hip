@@ -284,7 +284,8 @@ static size_t act_ws_layout(int act_dtype, int64_t m, int64_t k, uint8_t *base, 
     auto take = [&](size_t bytes) { size_t o = off; off = cq_align_up(off + bytes, 256); return o; };
     // Q8K rows are padded (see cq_act_view::m_stride); the others to whole 32-row groups, which the
     // split-K MFMA kernel copies without looking at the row count
-    const int64_t m_pad = act_dtype == CQ_DTYPE_Q8K ? (m + 63) / 64 * 64 + 256 : (m + 31) / 32 * 32;
+    // (beyond 32 rows to whole 128-row tiles, which the 32-element-block tile kernel reads, scales included)
+    const int64_t m_pad = act_dtype == CQ_DTYPE_Q8K ? (m + 63) / 64 * 64 + 256 : m <= 32 ? (m + 31) / 32 * 32 : (m + 127) / 128 * 128;
     const size_t o_qs = take((size_t)(m_pad * k));
     cq_act_view view{};
     view.m_stride = m_pad;
@@ -299,7 +300,7 @@ static size_t act_ws_layout(int act_dtype, int64_t m, int64_t k, uint8_t *base, 
             view.minp = (uint16_t *)(base + o_mp);
         }
     } else {
-        const size_t o_d = take((size_t)(m * (k / 32)) * 4);
+        const size_t o_d = take((size_t)(m_pad * (k / 32)) * 4);
         const size_t o_s = take((size_t)(m * (k / 32)) * 4);
         const size_t o_h = take((size_t)(m * (k / 32)) * 2);
         if (base) {
@@ -373,8 +374,13 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
     // (the 32-element-block types from 4 rows (Q8_0) or 5 rows (Q4_0) on: below that the batched
     // dot-product kernel is as fast or faster, it has no per-block scaling of MFMA results to do)
     const int64_t skinny_from = w->dtype == CQ_DTYPE_Q8_0 ? 4 : w->dtype == CQ_DTYPE_Q4_0 ? 5 : 2;
-    // Q8_0 / Q4_0 have no tile kernel: the split-K kernel, 32 rows per pass over the weights, stays ahead of
-    // the dot-product kernel (8 rows per pass) at every row count.
+    // Q8_0 / Q4_0 beyond 32 rows: their own tile kernel (whole 256-element K steps, n a multiple of 32)
+    if (!(flags & CQ_FLAG_FORCE_MATVEC) && m > 32 && cq_gemm32_supported(w, act)) {
+        CQ_HIP_CHECK(cq_launch_gemm32(w, v, act, m, y_dev, s));
+        return CQ_OK;
+    }
+    // shapes that kernel does not take: the split-K kernel, 32 rows per pass over the weights, stays ahead of the
+    // dot-product kernel (8 rows per pass) at every row count
     const bool has_tile_kernel = cq_gemm_supported(w, m, act);
     if (!(flags & (CQ_FLAG_FORCE_GEMM | CQ_FLAG_FORCE_MATVEC)) && m >= skinny_from && cq_skinny_supported(w, act) &&
         (m <= 32 || (m <= 128 && w->n < 8192) || !has_tile_kernel)) {

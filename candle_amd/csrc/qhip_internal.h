@@ -122,6 +122,9 @@ hipError_t cq_launch_gemm(const cq_weight *w, cq_act_view a, int act_dtype, int6
 bool cq_gemm_grouped_supported(const cq_weight *const *experts, int n_experts, const int32_t *offsets, int act_dtype);
 hipError_t cq_launch_gemm_grouped(const cq_weight *const *experts, int n_experts, const int32_t *offsets, cq_act_view a,
                                   float *y, hipStream_t s);
+// gemm_blk32.hip: the tile kernel for Q8_0 / Q4_0 weights with Q8_0 activations (K a multiple of 256)
+bool cq_gemm32_supported(const cq_weight *w, int act_dtype);
+hipError_t cq_launch_gemm32(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s);
 // skinny.hip: 2..32 activation rows on the int8 MFMA, K split over the waves of a workgroup
 bool cq_skinny_supported(const cq_weight *w, int act_dtype);
 hipError_t cq_launch_skinny(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s);

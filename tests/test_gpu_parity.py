@@ -572,3 +572,41 @@ def test_moe_config4_full_size(qh):
     for p in range(offsets[-1]):               # sequential index_add in expert order
         acc[row_ids[p]] += yn[p] * weights[p]
     assert np.array_equal(ys.cpu().numpy(), acc)
+
+
+# ------------------------------------- tile kernel of the 32-element-block types (Q8_0, Q4_0) ----
+@pytest.mark.parametrize("dt", [orc.Q8_0, orc.Q4_0])
+@pytest.mark.parametrize("m,k,n", [(33, 256, 32), (64, 512, 64), (70, 1024, 96), (130, 768, 288), (200, 2048, 32),
+                                   (129, 4096, 64)])
+def test_gemm_blk32_matches_oracle(qh, dt, m, k, n):
+    """More than 32 rows of Q8_0 / Q4_0 weights go to their own int8-MFMA tile kernel (one MFMA result per
+    32-element block, scaled by the two block scales): ragged row counts, one and several K steps,
+    split K (few workgroups), against the oracle and against the split-K kernel on the same workspace."""
+    w, x = make_inputs(3 * dt + m + k, m, k, n, outliers=True)
+    blocks = orc.quantize(dt, w)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    got = qh.qmatmul(qw, dev(x))
+    check_f32(got.cpu().numpy(), orc.matmul(dt, x, blocks, n))
+    other = qh.qmatmul(qw, dev(x), qh.FLAG_FORCE_SKINNY)
+    assert torch.allclose(got, other, rtol=2e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("dt", [orc.Q8_0, orc.Q4_0])
+def test_gemm_blk32_full_size(qh, dt):
+    """M = 512 on 4096 x 4096: every output against the split-K kernel (a different kernel, the same
+    integers), 48 sampled weight rows against the oracle, and batch invariance against the decode kernel."""
+    m, k, n = 512, 4096, 4096
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(31 + dt)
+    w = torch.randn((n, k), generator=gen, device="cuda", dtype=torch.float32) * 0.02
+    x = torch.randn((m, k), generator=gen, device="cuda", dtype=torch.float32)
+    qw = qh.QWeight.zeros(dt, n, k).quantize_(w)
+    got = qh.qmatmul(qw, x)
+    other = qh.qmatmul(qw, x, qh.FLAG_FORCE_SKINNY)
+    assert torch.allclose(got, other, rtol=2e-5, atol=2e-5)
+    rows = np.random.default_rng(5).choice(n, 48, replace=False)
+    blocks = qw.to_ggml().reshape(n, -1)
+    want = orc.matmul(dt, x.cpu().numpy(), np.ascontiguousarray(blocks[rows]).ravel(), len(rows))
+    check_f32(got.cpu().numpy()[:, rows], want)
+    one = qh.qmatmul(qw, x[7:8].contiguous())
+    assert torch.allclose(got[7:8], one, rtol=2e-5, atol=2e-5)
