@@ -184,10 +184,14 @@ __global__ void __launch_bounds__(kThreads) gemm32_kernel(cq_weight w, cq_act_vi
                 const int t = q >> 3, s = q & 7;
                 return *(const v4i *)(cur + g.col[s & 3] + (t * 2 + (s >> 2)) * 4096);
             };
-            // activation scale of (row l%32 of tile t, block s) as two f16 pieces in K-slots 0 and 1
-            auto d8frag = [&](int q) -> v8h {
+            // activation scale of (row l%32 of tile t, block s): read two steps ahead, and only turned into
+            // the MFMA operand (two f16 pieces in K-slots 0 and 1) in the step that uses it, so that no step
+            // waits for the read it has just issued
+            auto d8raw = [&](int q) -> float {
                 const int t = q >> 3, s = q & 7;
-                const float v = *(const float *)(cur + T::oD8 + (t * 32 + col) * 32 + s * 4);
+                return *(const float *)(cur + T::oD8 + (t * 32 + col) * 32 + s * 4);
+            };
+            auto d8frag = [&](float v) -> v8h {
                 const _Float16 p1 = (_Float16)v;
                 const _Float16 p2 = (_Float16)(v - (float)p1);
                 v8h r = {p1, p2, 0, 0, 0, 0, 0, 0};
@@ -197,17 +201,17 @@ __global__ void __launch_bounds__(kThreads) gemm32_kernel(cq_weight w, cq_act_vi
             v16i acc[2];
             v16f sc[2];
             v4i av[3];
-            v8h dv[3];
+            float dv[3];
             av[0] = afrag(0); av[1] = afrag(1);
-            dv[0] = d8frag(0); dv[1] = d8frag(1);
+            dv[0] = d8raw(0); dv[1] = d8raw(1);
             const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
             const v16f zerof = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int q = 0; q <= MT * 8; q++) {
-                if (q + 2 < MT * 8) { av[(q + 2) % 3] = afrag(q + 2); dv[(q + 2) % 3] = d8frag(q + 2); }
+                if (q + 2 < MT * 8) { av[(q + 2) % 3] = afrag(q + 2); dv[(q + 2) % 3] = d8raw(q + 2); }
                 if (q < MT * 8) {
                     acc[q & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[q % 3], bw[q & 7], zero, 0, 0, 0);
-                    sc[q & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(dv[q % 3], dw[q & 7], zerof, 0, 0, 0);
+                    sc[q & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(d8frag(dv[q % 3]), dw[q & 7], zerof, 0, 0, 0);
                 }
                 // keeps the MFMAs in front of the scaling below: left alone, the scheduler sinks them to the end
                 // of the step, and the next step then starts by waiting for their results
