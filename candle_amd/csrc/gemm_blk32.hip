@@ -194,9 +194,9 @@ __global__ void __launch_bounds__(kThreads) gemm32_kernel(cq_weight w, cq_act_vi
             auto d8frag = [&](float v) -> v8h {
                 const _Float16 p1 = (_Float16)v;
                 const _Float16 p2 = (_Float16)(v - (float)p1);
+                // lanes 32..63 hold K-slots 8..15, where the weight operand is zero: their (finite) values drop out
                 v8h r = {p1, p2, 0, 0, 0, 0, 0, 0};
-                const v8h z = {0, 0, 0, 0, 0, 0, 0, 0};
-                return h == 0 ? r : z;
+                return r;
             };
             v16i acc[2];
             v16f sc[2];
