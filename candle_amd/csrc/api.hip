@@ -336,6 +336,19 @@ static int check_matmul_args(const cq_weight *w, const float *x, int64_t m, cons
     return CQ_OK;
 }
 
+// The quantizer may clear the matmul's output while it reads the activations only if the two do not
+// overlap (a caller may well compute in place when the launches are separate) and y takes 16-byte stores.
+static bool ranges_overlap(const float *a, int64_t na, const float *b, int64_t nb) {
+    return a && b && (uintptr_t)a < (uintptr_t)(b + nb) && (uintptr_t)b < (uintptr_t)(a + na);
+}
+static bool clear_in_quantizer_ok(const float *y, int64_t ny, const float *x, int64_t nx, cq_pre pre) {
+    if ((uintptr_t)y & 15) return false;
+    if (ranges_overlap(y, ny, x, nx)) return false;
+    // rms_norm: aux is one row of weights; silu_mul: aux has the shape of x
+    if (pre.kind != CQ_PRE_NONE && ranges_overlap(y, ny, pre.aux, nx)) return false;
+    return true;
+}
+
 static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int64_t m, float *y_dev, int flags,
                         void *ws, size_t ws_bytes, void *stream) {
     const size_t need = cq_workspace_bytes(w, m, flags);
@@ -358,47 +371,60 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
         CQ_HIP_CHECK(cq_launch_matvec_fused(w, x_dev, pre, y_dev, s));
         return CQ_OK;
     }
-    cq_act_view v;
-    act_ws_layout(act, m, w->k, (uint8_t *)ws, &v);
-    if (!(flags & CQ_FLAG_REUSE_ACT)) CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, nullptr, m, w->k, pre, v, s));
-    if (flags & CQ_FLAG_FORCE_SKINNY) {
-        if (!cq_skinny_supported(w, act))
-            return cq_set_error(CQ_ERR_UNSUPPORTED, "no split-K MFMA kernel for dtype %d with activation dtype %d and n = %lld",
-                                w->dtype, act, (long long)w->n);
-        CQ_HIP_CHECK(cq_launch_skinny(w, v, act, m, y_dev, s));
-        return CQ_OK;
-    }
+    // Which kernel takes the rows.  Decided before the quantizer runs, because the quantizer clears the
+    // output of a launch that splits K on its way.
+    enum { kSkinny, kGemm32, kGemm, kMatvec } path;
     // Few rows: split K over the waves instead of tiling rows.  Measured faster than the dot-product
     // kernels from 2 rows on and than the tile kernel up to 32 rows (up to 128 rows when n is small
     // and the tile kernel cannot fill the machine).
     // (the 32-element-block types from 4 rows (Q8_0) or 5 rows (Q4_0) on: below that the batched
     // dot-product kernel is as fast or faster, it has no per-block scaling of MFMA results to do)
     const int64_t skinny_from = w->dtype == CQ_DTYPE_Q8_0 ? 4 : w->dtype == CQ_DTYPE_Q4_0 ? 5 : 2;
-    // Q8_0 / Q4_0 beyond 32 rows: their own tile kernel (whole 256-element K steps, n a multiple of 32)
-    if (!(flags & CQ_FLAG_FORCE_MATVEC) && m > 32 && cq_gemm32_supported(w, act)) {
-        CQ_HIP_CHECK(cq_launch_gemm32(w, v, act, m, y_dev, s));
-        return CQ_OK;
-    }
-    // shapes that kernel does not take: the split-K kernel, 32 rows per pass over the weights, stays ahead of the
-    // dot-product kernel (8 rows per pass) at every row count
     const bool has_tile_kernel = cq_gemm_supported(w, m, act);
-    if (!(flags & (CQ_FLAG_FORCE_GEMM | CQ_FLAG_FORCE_MATVEC)) && m >= skinny_from && cq_skinny_supported(w, act) &&
-        (m <= 32 || (m <= 128 && w->n < 8192) || !has_tile_kernel)) {
-        CQ_HIP_CHECK(cq_launch_skinny(w, v, act, m, y_dev, s));
-        return CQ_OK;
+    if (flags & CQ_FLAG_FORCE_SKINNY) {
+        if (!cq_skinny_supported(w, act))
+            return cq_set_error(CQ_ERR_UNSUPPORTED, "no split-K MFMA kernel for dtype %d with activation dtype %d and n = %lld",
+                                w->dtype, act, (long long)w->n);
+        path = kSkinny;
+    } else if (!(flags & CQ_FLAG_FORCE_MATVEC) && m > 32 && cq_gemm32_supported(w, act)) {
+        // Q8_0 / Q4_0 beyond 32 rows: their own tile kernel (whole 256-element K steps, n a multiple of 32)
+        path = kGemm32;
+    } else if (!(flags & (CQ_FLAG_FORCE_GEMM | CQ_FLAG_FORCE_MATVEC)) && m >= skinny_from && cq_skinny_supported(w, act) &&
+               (m <= 32 || (m <= 128 && w->n < 8192) || !has_tile_kernel)) {
+        // (shapes the tile kernels do not take: the split-K kernel, 32 rows per pass over the weights, stays
+        // ahead of the dot-product kernel, 8 rows per pass, at every row count)
+        path = kSkinny;
+    } else {
+        bool use_gemm = false;
+        if (flags & CQ_FLAG_FORCE_GEMM) {
+            if (!has_tile_kernel)
+                return cq_set_error(CQ_ERR_UNSUPPORTED, "no MFMA GEMM for dtype %d with activation dtype %d", w->dtype, act);
+            use_gemm = true;
+        } else if (!(flags & CQ_FLAG_FORCE_MATVEC)) {
+            use_gemm = m > 8 && has_tile_kernel;  // the reference switches kernels at 8 rows (cuda.rs:484-498)
+        }
+        if (act == CQ_DTYPE_Q8_1 && !use_gemm)
+            return cq_set_error(CQ_ERR_UNSUPPORTED, "Q8_1 activations are only handled by the GEMM kernel");
+        path = use_gemm ? kGemm : kMatvec;
     }
-    bool use_gemm = false;
-    if (flags & CQ_FLAG_FORCE_GEMM) {
-        if (!cq_gemm_supported(w, m, act))
-            return cq_set_error(CQ_ERR_UNSUPPORTED, "no MFMA GEMM for dtype %d with activation dtype %d", w->dtype, act);
-        use_gemm = true;
-    } else if (!(flags & CQ_FLAG_FORCE_MATVEC)) {
-        use_gemm = m > 8 && cq_gemm_supported(w, m, act);  // the reference switches kernels at 8 rows (cuda.rs:484-498)
+    cq_act_view v;
+    act_ws_layout(act, m, w->k, (uint8_t *)ws, &v);
+    bool y_cleared = false;
+    if (!(flags & CQ_FLAG_REUSE_ACT)) {
+        cq_clear clear = cq_no_clear();
+        const bool splits = path == kGemm32 ? cq_gemm32_splits_k(w, m) : path == kGemm ? cq_gemm_splits_k(w, m) : false;
+        if (splits && clear_in_quantizer_ok(y_dev, m * w->n, x_dev, m * w->k, pre)) {
+            clear = cq_clear{y_dev, m * w->n};
+            y_cleared = true;
+        }
+        CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, nullptr, m, w->k, pre, v, clear, s));
     }
-    if (act == CQ_DTYPE_Q8_1 && !use_gemm)
-        return cq_set_error(CQ_ERR_UNSUPPORTED, "Q8_1 activations are only handled by the GEMM kernel");
-    if (use_gemm) CQ_HIP_CHECK(cq_launch_gemm(w, v, act, m, y_dev, s));
-    else CQ_HIP_CHECK(cq_launch_matvec(w, v, act, m, y_dev, s));
+    switch (path) {
+        case kSkinny: CQ_HIP_CHECK(cq_launch_skinny(w, v, act, m, y_dev, s)); break;
+        case kGemm32: CQ_HIP_CHECK(cq_launch_gemm32(w, v, act, m, y_dev, y_cleared, s)); break;
+        case kGemm: CQ_HIP_CHECK(cq_launch_gemm(w, v, act, m, y_dev, y_cleared, s)); break;
+        case kMatvec: CQ_HIP_CHECK(cq_launch_matvec(w, v, act, m, y_dev, s)); break;
+    }
     return CQ_OK;
 }
 
@@ -422,7 +448,7 @@ extern "C" int cq_qmatmul_int_dots(const cq_weight *w, const float *x_dev, int64
     hipStream_t s = (hipStream_t)stream;
     cq_act_view v;
     act_ws_layout(act, m, w->k, (uint8_t *)ws, &v);
-    CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, nullptr, m, w->k, cq_no_pre(), v, s));
+    CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, nullptr, m, w->k, cq_no_pre(), v, cq_no_clear(), s));
     CQ_HIP_CHECK(cq_launch_int_dots(w, v, m, out_i, (w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q5K) ? out_mn : nullptr, s));
     return CQ_OK;
 }
@@ -458,16 +484,23 @@ static int grouped_impl(const cq_weight *const *experts, int n_experts, const fl
     hipStream_t s = (hipStream_t)stream;
     cq_act_view v;
     act_ws_layout(act, total, w0->k, (uint8_t *)ws, &v);
-    // gather + quantize every routed row once, then one matmul per non-empty expert over its slice
-    CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, row_ids_dev, total, w0->k, pre, v, s));
     // experts with more than eight rows among them: one tile-kernel launch for all experts
     int64_t most = 0;
     for (int e = 0; e < n_experts; e++) most = offsets[e + 1] - offsets[e] > most ? offsets[e + 1] - offsets[e] : most;
     const bool want_gemm = (flags & CQ_FLAG_FORCE_GEMM) ? true : (flags & CQ_FLAG_FORCE_MATVEC) ? false : most > 8;
-    if (want_gemm && cq_gemm_grouped_supported(experts, n_experts, offsets, act)) {
-        CQ_HIP_CHECK(cq_launch_gemm_grouped(experts, n_experts, offsets, v, y_dev, s));
+    const bool grouped = want_gemm && cq_gemm_grouped_supported(experts, n_experts, offsets, act);
+    // gather + quantize every routed row once (clearing the output on the way if the grouped launch splits K;
+    // with row ids the extent of x is not known here, so nothing is cleared then)
+    cq_clear clear = cq_no_clear();
+    if (grouped && !row_ids_dev && cq_gemm_grouped_splits_k(experts, n_experts, offsets) &&
+        clear_in_quantizer_ok(y_dev, total * w0->n, x_dev, total * w0->k, pre))
+        clear = cq_clear{y_dev, total * w0->n};
+    CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, row_ids_dev, total, w0->k, pre, v, clear, s));
+    if (grouped) {
+        CQ_HIP_CHECK(cq_launch_gemm_grouped(experts, n_experts, offsets, v, y_dev, clear.p != nullptr, s));
         return CQ_OK;
     }
+    // otherwise one matmul per non-empty expert over its slice
     for (int e = 0; e < n_experts; e++) {
         const int64_t r0 = offsets[e], te = offsets[e + 1] - offsets[e];
         if (te == 0) continue;
@@ -486,7 +519,7 @@ static int grouped_impl(const cq_weight *const *experts, int n_experts, const fl
         const bool use_gemm = (flags & CQ_FLAG_FORCE_GEMM) ? true
                               : (flags & CQ_FLAG_FORCE_MATVEC) ? false
                                                                : (te > 8 && cq_gemm_supported(experts[e], te, act));
-        if (use_gemm) CQ_HIP_CHECK(cq_launch_gemm(experts[e], ve, act, te, ye, s));
+        if (use_gemm) CQ_HIP_CHECK(cq_launch_gemm(experts[e], ve, act, te, ye, false, s));
         else CQ_HIP_CHECK(cq_launch_matvec(experts[e], ve, act, te, ye, s));
     }
     return CQ_OK;

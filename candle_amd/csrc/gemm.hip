@@ -518,16 +518,25 @@ int num_cus() {
     return g_cus;
 }
 
+// rows of a workgroup's tile, in units of 32
+int tile_mt(int64_t m) { return m <= 32 ? 1 : m <= 64 ? 2 : 4; }
+
+// Too few workgroups for `slots` of them at once: K is split (at least four blocks per part).
+int pick_ksplit(int64_t tiles, int64_t kb, int64_t slots) {
+    int ksplit = 1;
+    while (tiles * ksplit * 2 <= slots && kb / (ksplit * 2) >= 4 && ksplit < 16) ksplit *= 2;
+    return ksplit;
+}
+
+int64_t n_tiles(const cq_weight *w) { return (w->n + kWaves * 32 - 1) / (kWaves * 32); }
+
 template <int DT, int MT>
-hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
+hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, bool y_cleared, hipStream_t s) {
     const size_t lds = Tile<DT, MT>::kTotal;
     if (hipError_t e = cq_ensure_lds<gemm_kernel<DT, MT>>(w->dev, lds); e != hipSuccess) return e;
-    const int64_t gx = (w->n + kWaves * 32 - 1) / (kWaves * 32), gy = (m + MT * 32 - 1) / (MT * 32);
-    // too few workgroups for the machine: split K (at least four blocks per part)
-    int ksplit = 1;
-    const int64_t kb = w->k >> 8;
-    while (gx * gy * ksplit * 2 <= num_cus() && kb / (ksplit * 2) >= 4 && ksplit < 16) ksplit *= 2;
-    if (ksplit > 1) {
+    const int64_t gx = n_tiles(w), gy = (m + MT * 32 - 1) / (MT * 32);
+    const int ksplit = pick_ksplit(gx * gy, w->k >> 8, num_cus());
+    if (ksplit > 1 && !y_cleared) {
         hipError_t e = cq_launch_fill_zero(y, m * w->n, s);
         if (e != hipSuccess) return e;
     }
@@ -537,15 +546,16 @@ hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hip
 }
 
 template <int DT>
-hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
-    if (m <= 32) return launch_mt<DT, 1>(w, a, m, y, s);
-    if (m <= 64) return launch_mt<DT, 2>(w, a, m, y, s);
-    return launch_mt<DT, 4>(w, a, m, y, s);
+hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, bool y_cleared, hipStream_t s) {
+    const int mt = tile_mt(m);
+    if (mt == 1) return launch_mt<DT, 1>(w, a, m, y, y_cleared, s);
+    if (mt == 2) return launch_mt<DT, 2>(w, a, m, y, y_cleared, s);
+    return launch_mt<DT, 4>(w, a, m, y, y_cleared, s);
 }
 
 template <int DT>
 hipError_t launch_grouped(const cq_weight *const *experts, int n_experts, const int32_t *offsets, cq_act_view a,
-                          float *y, hipStream_t s) {
+                          float *y, bool y_cleared, hipStream_t s) {
     GroupArgs ga;
     int ntiles = 0;
     for (int e = 0; e < n_experts; e++) {
@@ -562,11 +572,9 @@ hipError_t launch_grouped(const cq_weight *const *experts, int n_experts, const 
     const cq_weight *w = experts[0];
     const size_t lds = Tile<DT, 1>::kTotal;
     if (hipError_t e = cq_ensure_lds<gemm_grouped_kernel<DT>>(w->dev, lds); e != hipSuccess) return e;
-    const int64_t gx = (w->n + kWaves * 32 - 1) / (kWaves * 32);
-    int ksplit = 1;
-    const int64_t kb = w->k >> 8;
-    while (gx * ntiles * ksplit * 2 <= 2 * num_cus() && kb / (ksplit * 2) >= 4 && ksplit < 16) ksplit *= 2;
-    if (ksplit > 1) {
+    const int64_t gx = n_tiles(w);
+    const int ksplit = pick_ksplit(gx * ntiles, w->k >> 8, 2 * num_cus());   // two single-tile workgroups per CU
+    if (ksplit > 1 && !y_cleared) {
         hipError_t e = cq_launch_fill_zero(y, (int64_t)offsets[n_experts] * w->n, s);
         if (e != hipSuccess) return e;
     }
@@ -585,11 +593,22 @@ bool cq_gemm_grouped_supported(const cq_weight *const *experts, int n_experts, c
 }
 
 hipError_t cq_launch_gemm_grouped(const cq_weight *const *experts, int n_experts, const int32_t *offsets, cq_act_view a,
-                                  float *y, hipStream_t s) {
+                                  float *y, bool y_cleared, hipStream_t s) {
     if (a.m_stride < ((int64_t)offsets[n_experts] + 31) / 32 * 32) return hipErrorInvalidValue;
-    if (experts[0]->dtype == CQ_DTYPE_Q4K) return launch_grouped<CQ_DTYPE_Q4K>(experts, n_experts, offsets, a, y, s);
-    if (experts[0]->dtype == CQ_DTYPE_Q5K) return launch_grouped<CQ_DTYPE_Q5K>(experts, n_experts, offsets, a, y, s);
-    return launch_grouped<CQ_DTYPE_Q6K>(experts, n_experts, offsets, a, y, s);
+    if (experts[0]->dtype == CQ_DTYPE_Q4K) return launch_grouped<CQ_DTYPE_Q4K>(experts, n_experts, offsets, a, y, y_cleared, s);
+    if (experts[0]->dtype == CQ_DTYPE_Q5K) return launch_grouped<CQ_DTYPE_Q5K>(experts, n_experts, offsets, a, y, y_cleared, s);
+    return launch_grouped<CQ_DTYPE_Q6K>(experts, n_experts, offsets, a, y, y_cleared, s);
+}
+
+bool cq_gemm_grouped_splits_k(const cq_weight *const *experts, int n_experts, const int32_t *offsets) {
+    int64_t tiles = 0;
+    for (int e = 0; e < n_experts; e++) tiles += (offsets[e + 1] - offsets[e] + 31) / 32;
+    return tiles > 0 && pick_ksplit(n_tiles(experts[0]) * tiles, experts[0]->k >> 8, 2 * num_cus()) > 1;
+}
+
+bool cq_gemm_splits_k(const cq_weight *w, int64_t m) {
+    const int mt = tile_mt(m);
+    return m > 0 && pick_ksplit(n_tiles(w) * ((m + mt * 32 - 1) / (mt * 32)), w->k >> 8, num_cus()) > 1;
 }
 
 bool cq_gemm_supported(const cq_weight *w, int64_t m, int act_dtype) {
@@ -599,11 +618,12 @@ bool cq_gemm_supported(const cq_weight *w, int64_t m, int act_dtype) {
            w->k <= (1 << 24) && w->n % 32 == 0;
 }
 
-hipError_t cq_launch_gemm(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s) {
+hipError_t cq_launch_gemm(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, bool y_cleared,
+                          hipStream_t s) {
     if (!cq_gemm_supported(w, m, act_dtype)) return hipErrorNotSupported;
     if (m == 0 || w->n == 0) return hipSuccess;
     if (a.m_stride < (m + 127) / 128 * 128) return hipErrorInvalidValue;   // rows the last tile may read
-    if (w->dtype == CQ_DTYPE_Q4K) return launch_dt<CQ_DTYPE_Q4K>(w, a, m, y, s);
-    if (w->dtype == CQ_DTYPE_Q5K) return launch_dt<CQ_DTYPE_Q5K>(w, a, m, y, s);
-    return launch_dt<CQ_DTYPE_Q6K>(w, a, m, y, s);
+    if (w->dtype == CQ_DTYPE_Q4K) return launch_dt<CQ_DTYPE_Q4K>(w, a, m, y, y_cleared, s);
+    if (w->dtype == CQ_DTYPE_Q5K) return launch_dt<CQ_DTYPE_Q5K>(w, a, m, y, y_cleared, s);
+    return launch_dt<CQ_DTYPE_Q6K>(w, a, m, y, y_cleared, s);
 }

@@ -256,15 +256,25 @@ int num_cus() {
     return g_cus;
 }
 
+// rows of a workgroup's tile, in units of 32
+int tile_mt(int64_t m) { return m <= 64 ? 2 : 4; }
+
+// Too few workgroups for the machine: K is split (at least two 256-element steps per part).
+int pick_ksplit(const cq_weight *w, int64_t m) {
+    const int mt = tile_mt(m);
+    const int64_t tiles = ((w->n + kWaves * 32 - 1) / (kWaves * 32)) * ((m + mt * 32 - 1) / (mt * 32)), ks = w->k >> 8;
+    int ksplit = 1;
+    while (tiles * ksplit * 2 <= num_cus() && ks / (ksplit * 2) >= 2 && ksplit < 16) ksplit *= 2;
+    return ksplit;
+}
+
 template <int DT, int MT>
-hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
+hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, bool y_cleared, hipStream_t s) {
     const size_t lds = Tile<DT, MT>::kTotal;
     if (hipError_t e = cq_ensure_lds<gemm32_kernel<DT, MT>>(w->dev, lds); e != hipSuccess) return e;
     const int64_t gx = (w->n + kWaves * 32 - 1) / (kWaves * 32), gy = (m + MT * 32 - 1) / (MT * 32);
-    int ksplit = 1;
-    const int64_t ks = w->k >> 8;
-    while (gx * gy * ksplit * 2 <= num_cus() && ks / (ksplit * 2) >= 2 && ksplit < 16) ksplit *= 2;
-    if (ksplit > 1) {
+    const int ksplit = pick_ksplit(w, m);
+    if (ksplit > 1 && !y_cleared) {
         hipError_t e = cq_launch_fill_zero(y, m * w->n, s);
         if (e != hipSuccess) return e;
     }
@@ -274,9 +284,9 @@ hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hip
 }
 
 template <int DT>
-hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
-    if (m <= 64) return launch_mt<DT, 2>(w, a, m, y, s);
-    return launch_mt<DT, 4>(w, a, m, y, s);
+hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, bool y_cleared, hipStream_t s) {
+    if (tile_mt(m) == 2) return launch_mt<DT, 2>(w, a, m, y, y_cleared, s);
+    return launch_mt<DT, 4>(w, a, m, y, y_cleared, s);
 }
 
 }  // namespace
@@ -287,10 +297,13 @@ bool cq_gemm32_supported(const cq_weight *w, int act_dtype) {
            w->k % 256 == 0 && w->k <= (1 << 24) && w->n % 32 == 0 && w->n > 0;
 }
 
-hipError_t cq_launch_gemm32(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s) {
+bool cq_gemm32_splits_k(const cq_weight *w, int64_t m) { return m > 0 && pick_ksplit(w, m) > 1; }
+
+hipError_t cq_launch_gemm32(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, bool y_cleared,
+                            hipStream_t s) {
     if (!cq_gemm32_supported(w, act_dtype)) return hipErrorNotSupported;
     if (m == 0) return hipSuccess;
     if (a.m_stride < (m + 127) / 128 * 128) return hipErrorInvalidValue;   // rows the last tile may read
-    if (w->dtype == CQ_DTYPE_Q8_0) return launch_dt<CQ_DTYPE_Q8_0>(w, a, m, y, s);
-    return launch_dt<CQ_DTYPE_Q4_0>(w, a, m, y, s);
+    if (w->dtype == CQ_DTYPE_Q8_0) return launch_dt<CQ_DTYPE_Q8_0>(w, a, m, y, y_cleared, s);
+    return launch_dt<CQ_DTYPE_Q4_0>(w, a, m, y, y_cleared, s);
 }

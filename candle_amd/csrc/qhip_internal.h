@@ -99,12 +99,19 @@ struct cq_pre {
     float eps;
 };
 static inline cq_pre cq_no_pre() { return cq_pre{CQ_PRE_NONE, nullptr, 0.0f}; }
+// Floats the activation quantizer sets to zero on its way: the output of a matmul that splits K and adds
+// its partial sums atomically (the launch it saves costs as much as the clearing).  p == nullptr: nothing.
+struct cq_clear {
+    float *p;
+    int64_t count;
+};
+static inline cq_clear cq_no_clear() { return cq_clear{nullptr, 0}; }
 
 // quantize_act.hip
 hipError_t cq_launch_quantize_act_aos(int act_dtype, const float *x, int64_t m, int64_t k, cq_pre pre, void *dst,
                                       hipStream_t s);
 hipError_t cq_launch_quantize_act_ws(int act_dtype, const float *x, const int32_t *row_ids, int64_t m, int64_t k,
-                                     cq_pre pre, cq_act_view v, hipStream_t s);
+                                     cq_pre pre, cq_act_view v, cq_clear clear, hipStream_t s);
 // quantize_weight.hip
 hipError_t cq_launch_quantize_weight(int dtype, const float *src, int64_t nblocks, uint8_t *aos_dev, hipStream_t s);
 // dequantize.hip
@@ -117,14 +124,21 @@ bool cq_matvec_fused_supported(const cq_weight *w);   // m == 1: quantizer fused
 hipError_t cq_launch_matvec_fused(const cq_weight *w, const float *x, cq_pre pre, float *y, hipStream_t s);
 // gemm.hip
 bool cq_gemm_supported(const cq_weight *w, int64_t m, int act_dtype);
-hipError_t cq_launch_gemm(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s);
+// `y_cleared`: y is already zero (a launch that splits K otherwise clears it first); *_splits_k tell
+// beforehand whether the launch will add its results atomically
+hipError_t cq_launch_gemm(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, bool y_cleared,
+                          hipStream_t s);
+bool cq_gemm_splits_k(const cq_weight *w, int64_t m);
 // all experts of a mixture-of-experts projection in one launch; `a` and `y` cover all routed rows
 bool cq_gemm_grouped_supported(const cq_weight *const *experts, int n_experts, const int32_t *offsets, int act_dtype);
 hipError_t cq_launch_gemm_grouped(const cq_weight *const *experts, int n_experts, const int32_t *offsets, cq_act_view a,
-                                  float *y, hipStream_t s);
+                                  float *y, bool y_cleared, hipStream_t s);
+bool cq_gemm_grouped_splits_k(const cq_weight *const *experts, int n_experts, const int32_t *offsets);
 // gemm_blk32.hip: the tile kernel for Q8_0 / Q4_0 weights with Q8_0 activations (K a multiple of 256)
 bool cq_gemm32_supported(const cq_weight *w, int act_dtype);
-hipError_t cq_launch_gemm32(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s);
+hipError_t cq_launch_gemm32(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, bool y_cleared,
+                            hipStream_t s);
+bool cq_gemm32_splits_k(const cq_weight *w, int64_t m);
 // skinny.hip: 2..32 activation rows on the int8 MFMA, K split over the waves of a workgroup
 bool cq_skinny_supported(const cq_weight *w, int act_dtype);
 hipError_t cq_launch_skinny(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s);

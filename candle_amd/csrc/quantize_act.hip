@@ -30,7 +30,21 @@ struct Sink {
     // GGML struct layout (AOS) or the workspace layout (qhip_internal.h)
     uint8_t *aos;
     cq_act_view v;
+    cq_clear clear;
 };
+
+// The launch's threads share the floats to be cleared, four at a time (clear.p is 16-byte aligned).
+__device__ __forceinline__ void clear_floats(const cq_clear &c) {
+    if (!c.p) return;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x * 4;
+    for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4; i < c.count; i += step) {
+        if (i + 4 <= c.count) {
+            *(float4 *)(c.p + i) = make_float4(0.f, 0.f, 0.f, 0.f);
+        } else {
+            for (int64_t j = i; j < c.count; j++) c.p[j] = 0.0f;
+        }
+    }
+}
 
 __device__ __forceinline__ int8_t round_to_i8(float v) { return cq_as_i8(roundf(v)); }
 
@@ -86,6 +100,7 @@ __global__ void __launch_bounds__(256) quantize_q8_0_kernel(const float *__restr
     const int lane = threadIdx.x & 63;
     const int64_t chunks_per_row = (k + 255) / 256;
     const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    clear_floats(out.clear);
     if (wave >= m * chunks_per_row) return;
     const int64_t row = wave / chunks_per_row;
     const int64_t e0 = (wave - row * chunks_per_row) * 256 + 4 * lane;
@@ -175,6 +190,7 @@ __global__ void __launch_bounds__(256) quantize_q8k_kernel(const float *__restri
     const int lane = threadIdx.x & 63;
     const int64_t kb = k / 256;
     const int64_t blk = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    clear_floats(out.clear);
     if (blk >= m * kb) return;
     const int64_t row = blk / kb;
     const int64_t b_in_row = blk - row * kb;
@@ -207,6 +223,7 @@ __global__ void __launch_bounds__(256) quantize_rms_rows_kernel(const float *__r
     const int64_t src_row = row_ids ? (int64_t)row_ids[row] : row;
     const float *xr = x + src_row * k;
     const int64_t chunks = (k + 255) / 256;
+    clear_floats(out.clear);
     for (int64_t c = wave; c < chunks; c += 4) {
         const int64_t e0 = c * 256 + 4 * lane;
         float t = 0.0f;
@@ -276,8 +293,9 @@ hipError_t cq_launch_quantize_act_aos(int act_dtype, const float *x, int64_t m, 
 }
 
 hipError_t cq_launch_quantize_act_ws(int act_dtype, const float *x, const int32_t *row_ids, int64_t m, int64_t k,
-                                     cq_pre pre, cq_act_view v, hipStream_t s) {
+                                     cq_pre pre, cq_act_view v, cq_clear clear, hipStream_t s) {
     Sink out{};
     out.v = v;
+    out.clear = clear;
     return launch<false>(act_dtype, x, row_ids, m, k, pre, out, s);
 }

@@ -610,3 +610,34 @@ def test_gemm_blk32_full_size(qh, dt):
     check_f32(got.cpu().numpy()[:, rows], want)
     one = qh.qmatmul(qw, x[7:8].contiguous())
     assert torch.allclose(got[7:8], one, rtol=2e-5, atol=2e-5)
+
+
+@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K, orc.Q8_0, orc.Q4_0])
+def test_split_k_output_is_cleared_wherever_it_lives(qh, dt):
+    """Launches that split K add into a zeroed output.  The activation quantizer clears it on its way
+    when the output does not overlap the input and takes 16-byte stores; otherwise a fill launch does.
+    All three ways give the oracle's result on an output that held NaNs: a fresh buffer, one that is
+    not 16-byte aligned, and the input's own memory (n == k, computed in place)."""
+    m, k, n = 48, 2048, 2048            # 8 x 1 tiles on 256 CUs: K is split
+    w, x = make_inputs(40 + dt, m, k, n)
+    blocks = orc.quantize(dt, w)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    want = orc.matmul(dt, x, blocks, n)
+    flags = qh.FLAG_FORCE_GEMM if dt in (orc.Q4K, orc.Q6K) else 0
+    xd = dev(x)
+    y = torch.full((m, n), float("nan"), device="cuda")
+    qh.qmatmul(qw, xd, flags, out=y)
+    check_f32(y.cpu().numpy(), want)
+    buf = torch.full((m * n + 4,), float("nan"), device="cuda")
+    y1 = buf[1:1 + m * n].view(m, n)    # 4 bytes past a 16-byte boundary
+    qh.qmatmul(qw, xd, flags, out=y1)
+    assert torch.allclose(y1, y, rtol=1e-5, atol=1e-6)
+    assert torch.isnan(buf[0]) and torch.isnan(buf[1 + m * n:]).all()
+    xin = xd.clone()
+    qh.qmatmul(qw, xin, flags, out=xin)  # in place
+    assert torch.allclose(xin, y, rtol=1e-5, atol=1e-6)
+    # the rows reused from the workspace: nothing is quantized, so the fill launch clears
+    y2 = torch.full((m, n), float("nan"), device="cuda")
+    qh.qmatmul(qw, xd, flags, out=y)
+    qh.qmatmul(qw, xd, flags | qh.FLAG_REUSE_ACT, out=y2)
+    assert torch.allclose(y2, y, rtol=1e-5, atol=1e-6)
