@@ -375,7 +375,7 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
     // output of a launch that splits K on its way.
     enum { kSkinny, kGemm32, kGemm, kMatvec } path;
     // Few rows: split K over the waves instead of tiling rows.  Measured faster than the dot-product
-    // kernels from 2 rows on and than the tile kernel up to 32 rows (up to 128 rows when n is small
+    // kernels from 2 rows on and than the tile kernel up to 32 rows (up to 64 rows when n is small
     // and the tile kernel cannot fill the machine).
     // (the 32-element-block types from 4 rows (Q8_0) or 5 rows (Q4_0) on: below that the batched
     // dot-product kernel is as fast or faster, it has no per-block scaling of MFMA results to do)
@@ -390,7 +390,7 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
         // Q8_0 / Q4_0 beyond 32 rows: their own tile kernel (whole 256-element K steps, n a multiple of 32)
         path = kGemm32;
     } else if (!(flags & (CQ_FLAG_FORCE_GEMM | CQ_FLAG_FORCE_MATVEC)) && m >= skinny_from && cq_skinny_supported(w, act) &&
-               (m <= 32 || (m <= 128 && w->n < 8192) || !has_tile_kernel)) {
+               (m <= 32 || (m <= 64 && w->n < 8192) || !has_tile_kernel)) {
         // (shapes the tile kernels do not take: the split-K kernel, 32 rows per pass over the weights, stays
         // ahead of the dot-product kernel, 8 rows per pass, at every row count)
         path = kSkinny;

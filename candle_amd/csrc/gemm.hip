@@ -518,9 +518,6 @@ int num_cus() {
     return g_cus;
 }
 
-// rows of a workgroup's tile, in units of 32
-int tile_mt(int64_t m) { return m <= 32 ? 1 : m <= 64 ? 2 : 4; }
-
 // Too few workgroups for `slots` of them at once: K is split (at least four blocks per part).
 int pick_ksplit(int64_t tiles, int64_t kb, int64_t slots) {
     int ksplit = 1;
@@ -530,12 +527,44 @@ int pick_ksplit(int64_t tiles, int64_t kb, int64_t slots) {
 
 int64_t n_tiles(const cq_weight *w) { return (w->n + kWaves * 32 - 1) / (kWaves * 32); }
 
+// Tile height (MT x 32 activation rows per workgroup) and K split of a launch, from a cost model fitted to
+// measurements (Q4K, 256 CUs; unit 1/16 us): a workgroup spends 22 units per K block unpacking its weights
+// and 13.5 per 32-row tile on it, 24 on starting and finishing; workgroups run one per CU, in rounds; a split
+// launch adds every part to the output atomically, which moves about 1.1 TB/s.  Tall tiles amortise
+// the unpacking, short ones fill the machine without splitting K: 4096 x 4096 at 512 rows takes 54 us as
+// 64 tiles of 128 rows split four ways and 42 us as 256 tiles of 32 rows.
+struct Plan {
+    int mt, ksplit;
+};
+Plan pick_plan(const cq_weight *w, int64_t m) {
+    const int64_t gx = n_tiles(w), kb = w->k >> 8, cus = num_cus();
+    const double atomic_pass = (double)m * (double)w->n * 4.0 / 1.1e6 * 16.0;   // bytes / (1.1e6 bytes per us) in units
+    Plan best{1, 1};
+    double best_cost = 0.0;
+    bool first = true;
+    for (int mt = 4; mt >= 1; mt >>= 1) {
+        if (mt > 1 && m <= 16 * mt) continue;   // half the height holds all rows
+        const int64_t tiles = gx * ((m + mt * 32 - 1) / (mt * 32));
+        for (int ks = 1; ks <= 16; ks *= 2) {
+            if (ks > 1 && kb / ks < 4) break;
+            const int64_t rounds = (tiles * ks + cus - 1) / cus;
+            const double cost = (double)rounds * ((double)((kb + ks - 1) / ks) * (22.0 + 13.5 * mt) + 24.0) +
+                                (ks > 1 ? ks * atomic_pass : 0.0);
+            if (first || cost < best_cost) {
+                best = Plan{mt, ks};
+                best_cost = cost;
+                first = false;
+            }
+        }
+    }
+    return best;
+}
+
 template <int DT, int MT>
-hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, bool y_cleared, hipStream_t s) {
+hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, int ksplit, bool y_cleared, hipStream_t s) {
     const size_t lds = Tile<DT, MT>::kTotal;
     if (hipError_t e = cq_ensure_lds<gemm_kernel<DT, MT>>(w->dev, lds); e != hipSuccess) return e;
     const int64_t gx = n_tiles(w), gy = (m + MT * 32 - 1) / (MT * 32);
-    const int ksplit = pick_ksplit(gx * gy, w->k >> 8, num_cus());
     if (ksplit > 1 && !y_cleared) {
         hipError_t e = cq_launch_fill_zero(y, m * w->n, s);
         if (e != hipSuccess) return e;
@@ -547,10 +576,10 @@ hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, boo
 
 template <int DT>
 hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, bool y_cleared, hipStream_t s) {
-    const int mt = tile_mt(m);
-    if (mt == 1) return launch_mt<DT, 1>(w, a, m, y, y_cleared, s);
-    if (mt == 2) return launch_mt<DT, 2>(w, a, m, y, y_cleared, s);
-    return launch_mt<DT, 4>(w, a, m, y, y_cleared, s);
+    const Plan p = pick_plan(w, m);
+    if (p.mt == 1) return launch_mt<DT, 1>(w, a, m, y, p.ksplit, y_cleared, s);
+    if (p.mt == 2) return launch_mt<DT, 2>(w, a, m, y, p.ksplit, y_cleared, s);
+    return launch_mt<DT, 4>(w, a, m, y, p.ksplit, y_cleared, s);
 }
 
 template <int DT>
@@ -606,10 +635,7 @@ bool cq_gemm_grouped_splits_k(const cq_weight *const *experts, int n_experts, co
     return tiles > 0 && pick_ksplit(n_tiles(experts[0]) * tiles, experts[0]->k >> 8, 2 * num_cus()) > 1;
 }
 
-bool cq_gemm_splits_k(const cq_weight *w, int64_t m) {
-    const int mt = tile_mt(m);
-    return m > 0 && pick_ksplit(n_tiles(w) * ((m + mt * 32 - 1) / (mt * 32)), w->k >> 8, num_cus()) > 1;
-}
+bool cq_gemm_splits_k(const cq_weight *w, int64_t m) { return m > 0 && pick_plan(w, m).ksplit > 1; }
 
 bool cq_gemm_supported(const cq_weight *w, int64_t m, int act_dtype) {
     (void)m;

@@ -256,24 +256,42 @@ int num_cus() {
     return g_cus;
 }
 
-// rows of a workgroup's tile, in units of 32
-int tile_mt(int64_t m) { return m <= 64 ? 2 : 4; }
-
-// Too few workgroups for the machine: K is split (at least two 256-element steps per part).
-int pick_ksplit(const cq_weight *w, int64_t m) {
-    const int mt = tile_mt(m);
-    const int64_t tiles = ((w->n + kWaves * 32 - 1) / (kWaves * 32)) * ((m + mt * 32 - 1) / (mt * 32)), ks = w->k >> 8;
-    int ksplit = 1;
-    while (tiles * ksplit * 2 <= num_cus() && ks / (ksplit * 2) >= 2 && ksplit < 16) ksplit *= 2;
-    return ksplit;
+// Tile height (MT x 32 activation rows per workgroup) and K split of a launch, from a cost model fitted to
+// measurements (Q8_0, 256 CUs; unit 1/16 us): a workgroup spends 10 units per 256-element K step on its
+// weights and 23 per 32-row tile on it, 24 on starting and finishing; workgroups run one per CU, in rounds;
+// a split launch adds every part to the output atomically, which moves about 1.1 TB/s.
+struct Plan {
+    int mt, ksplit;
+};
+Plan pick_plan(const cq_weight *w, int64_t m) {
+    const int64_t gx = (w->n + kWaves * 32 - 1) / (kWaves * 32), ks_total = w->k >> 8, cus = num_cus();
+    const double atomic_pass = (double)m * (double)w->n * 4.0 / 1.1e6 * 16.0;   // bytes / (1.1e6 bytes per us) in units
+    Plan best{1, 1};
+    double best_cost = 0.0;
+    bool first = true;
+    for (int mt = 4; mt >= 1; mt >>= 1) {
+        if (mt > 1 && m <= 16 * mt) continue;   // half the height holds all rows
+        const int64_t tiles = gx * ((m + mt * 32 - 1) / (mt * 32));
+        for (int ks = 1; ks <= 16; ks *= 2) {
+            if (ks > 1 && ks_total / ks < 2) break;
+            const int64_t rounds = (tiles * ks + cus - 1) / cus;
+            const double cost = (double)rounds * ((double)((ks_total + ks - 1) / ks) * (10.0 + 23.0 * mt) + 24.0) +
+                                (ks > 1 ? ks * atomic_pass : 0.0);
+            if (first || cost < best_cost) {
+                best = Plan{mt, ks};
+                best_cost = cost;
+                first = false;
+            }
+        }
+    }
+    return best;
 }
 
 template <int DT, int MT>
-hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, bool y_cleared, hipStream_t s) {
+hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, int ksplit, bool y_cleared, hipStream_t s) {
     const size_t lds = Tile<DT, MT>::kTotal;
     if (hipError_t e = cq_ensure_lds<gemm32_kernel<DT, MT>>(w->dev, lds); e != hipSuccess) return e;
     const int64_t gx = (w->n + kWaves * 32 - 1) / (kWaves * 32), gy = (m + MT * 32 - 1) / (MT * 32);
-    const int ksplit = pick_ksplit(w, m);
     if (ksplit > 1 && !y_cleared) {
         hipError_t e = cq_launch_fill_zero(y, m * w->n, s);
         if (e != hipSuccess) return e;
@@ -285,8 +303,10 @@ hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, boo
 
 template <int DT>
 hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, bool y_cleared, hipStream_t s) {
-    if (tile_mt(m) == 2) return launch_mt<DT, 2>(w, a, m, y, y_cleared, s);
-    return launch_mt<DT, 4>(w, a, m, y, y_cleared, s);
+    const Plan p = pick_plan(w, m);
+    if (p.mt == 1) return launch_mt<DT, 1>(w, a, m, y, p.ksplit, y_cleared, s);
+    if (p.mt == 2) return launch_mt<DT, 2>(w, a, m, y, p.ksplit, y_cleared, s);
+    return launch_mt<DT, 4>(w, a, m, y, p.ksplit, y_cleared, s);
 }
 
 }  // namespace
@@ -297,7 +317,7 @@ bool cq_gemm32_supported(const cq_weight *w, int act_dtype) {
            w->k % 256 == 0 && w->k <= (1 << 24) && w->n % 32 == 0 && w->n > 0;
 }
 
-bool cq_gemm32_splits_k(const cq_weight *w, int64_t m) { return m > 0 && pick_ksplit(w, m) > 1; }
+bool cq_gemm32_splits_k(const cq_weight *w, int64_t m) { return m > 0 && pick_plan(w, m).ksplit > 1; }
 
 hipError_t cq_launch_gemm32(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, bool y_cleared,
                             hipStream_t s) {
