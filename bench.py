@@ -231,6 +231,34 @@ def main() -> int:
     gemm_tops = 2.0 * gm * gk * gn / (gemm_avg_us * 1e-6) / 1e12
     del gq, gx, gy, gws
 
+    # whole calls (activation quantizer + GEMM) on both shapes of configs[2] and on the attention shape
+    whole_calls = {}
+    if not args.no_extras:
+        for name, dt, (wn, wk) in (("q4k_14336x4096", qhip.Q4K, (14336, 4096)), ("q4k_4096x14336", qhip.Q4K, (4096, 14336)),
+                                   ("q6k_14336x4096", qhip.Q6K, (14336, 4096)), ("q6k_4096x14336", qhip.Q6K, (4096, 14336)),
+                                   ("q4k_4096x4096", qhip.Q4K, (4096, 4096))):
+            ww = torch.randn((wn, wk), generator=gen, device=dev, dtype=torch.float32) * 0.02
+            wq = qhip.QWeight.zeros(dt, wn, wk).quantize_(ww)
+            del ww
+            wx = torch.randn((gm, wk), generator=gen, device=dev, dtype=torch.float32)
+            wy = torch.empty((gm, wn), device=dev, dtype=torch.float32)
+            wws = torch.empty(wq.workspace_bytes(gm), dtype=torch.uint8, device=dev)
+
+            def whole():
+                qhip.check(L.cq_qmatmul(wq.handle, C.c_void_p(wx.data_ptr()), gm, C.c_void_p(wy.data_ptr()), 0,
+                                        C.c_void_p(wws.data_ptr()), wws.numel(),
+                                        C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+            for _ in range(5):
+                whole()
+            w0, w1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            w0.record()
+            for _ in range(40):
+                whole()
+            w1.record()
+            torch.cuda.synchronize()
+            whole_calls[name] = round(w0.elapsed_time(w1) * 1e3 / 40, 1)
+            del wq, wx, wy, wws
+
     # ---- the same step with the model's neighbours of each matmul (reported beside the headline) ----
     # Per layer rms_norm -> q, k, v; o; rms_norm -> gate, up; silu(gate) * up -> down; final rms_norm
     # -> lm_head (quantized_llama.rs:453-511 without attention and residuals).  "separate": one more
@@ -410,6 +438,7 @@ def main() -> int:
             "tops": round(gemm_tops, 1),
             "peak_tops": 5000.0,
             "frac_of_int8_mfma_peak": round(gemm_tops / 5000.0, 4),
+            "whole_call_us_m512": whole_calls or None,
         },
     }
 
