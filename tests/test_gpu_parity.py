@@ -641,3 +641,29 @@ def test_split_k_output_is_cleared_wherever_it_lives(qh, dt):
     qh.qmatmul(qw, xd, flags, out=y)
     qh.qmatmul(qw, xd, flags | qh.FLAG_REUSE_ACT, out=y2)
     assert torch.allclose(y2, y, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K, orc.Q8_0, orc.Q4_0])
+@pytest.mark.parametrize("m,k,n", [(40, 1024, 1024), (100, 2048, 4096), (300, 1024, 4096), (520, 1024, 2048),
+                                   (130, 4096, 11008), (1000, 512, 8192)])
+def test_tile_plans_agree_with_dot_product_kernels(qh, dt, m, k, n):
+    """The tile kernels pick tile height and K split per shape; whatever they pick, the result equals the
+    dot-product kernels' (which the tests above hold against the oracle) to rounding, and a sample of
+    weight rows is held against the oracle directly."""
+    rng = np.random.default_rng(m + k + n + dt)
+    gen = torch.Generator(device="cuda").manual_seed(m + k + n + dt)
+    wt = torch.randn((n, k), generator=gen, device="cuda") * 0.02
+    qw = qh.QWeight.zeros(dt, n, k).quantize_(wt)
+    del wt
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    xd = dev(x)
+    got = qh.qmatmul(qw, xd)
+    ref = qh.qmatmul(qw, xd, qh.FLAG_FORCE_MATVEC)
+    err = (torch.linalg.norm(got - ref) / torch.linalg.norm(ref)).item()
+    assert err <= 2e-6, err
+    rows = np.sort(rng.choice(n, size=16, replace=False))
+    row_bytes = k // orc.BLOCK_SIZE[dt] * orc.TYPE_SIZE[dt]
+    blocks = qw.to_ggml().reshape(n, row_bytes)[rows].ravel()
+    want = orc.matmul(dt, x, blocks, len(rows))
+    g = got.cpu().numpy()[:, rows].astype(np.float64)
+    assert np.linalg.norm(g - want) / np.linalg.norm(want) <= REL_L2_TOL
