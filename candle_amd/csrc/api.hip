@@ -438,6 +438,38 @@ extern "C" int cq_qmatmul_fused(const cq_weight *w, int pre, const float *x_dev,
     return qmatmul_impl(w, x_dev, cq_pre{pre, aux_dev, eps}, m, y_dev, flags, ws, ws_bytes, stream);
 }
 
+extern "C" int cq_qmatmul_multi(const cq_weight *const *ws, int count, int pre, const float *x_dev, const float *aux_dev,
+                                float eps, int64_t m, float *const *ys_dev, int flags, void *workspace, size_t ws_bytes,
+                                void *stream) {
+    if (!ws || !ys_dev || count < 1) return cq_set_error(CQ_ERR_INVALID, "null argument");
+    for (int i = 0; i < count; i++) {
+        if (!ws[i]) return cq_set_error(CQ_ERR_INVALID, "null weight %d", i);
+        if (ws[i]->dtype != ws[0]->dtype || ws[i]->k != ws[0]->k || ws[i]->dev != ws[0]->dev)
+            return cq_set_error(CQ_ERR_INVALID, "weight %d differs in dtype, row length or device from weight 0", i);
+    }
+    const cq_pre p{pre, aux_dev, eps};
+    // one activation row, two or three weights: one launch over all their rows
+    if (m == 1 && flags == 0 && cq_matvec_fused_multi_supported(ws, count, pre)) {
+        if (!x_dev) return cq_set_error(CQ_ERR_INVALID, "null argument");
+        if ((uintptr_t)x_dev & 15) return cq_set_error(CQ_ERR_INVALID, "x must be 16-byte aligned");
+        for (int i = 0; i < count; i++)
+            if (!ys_dev[i]) return cq_set_error(CQ_ERR_INVALID, "null argument");
+        if (int rc = check_pre(p)) return rc;
+        CQ_HIP_CHECK(hipSetDevice(ws[0]->dev));
+        CQ_HIP_CHECK(cq_launch_matvec_fused_multi(ws, count, x_dev, p, ys_dev, (hipStream_t)stream));
+        return CQ_OK;
+    }
+    // otherwise one matmul per weight; with more than one row the rows are quantized once, by the first
+    const bool share = m > 1 && !(flags & CQ_FLAG_REUSE_ACT);
+    for (int i = 0; i < count; i++) {
+        const bool reuse = share && i > 0;
+        if (int rc = qmatmul_impl(ws[i], x_dev, reuse ? cq_no_pre() : p, m, ys_dev[i], reuse ? flags | CQ_FLAG_REUSE_ACT : flags,
+                                  workspace, ws_bytes, stream))
+            return rc;
+    }
+    return CQ_OK;
+}
+
 extern "C" int cq_qmatmul_int_dots(const cq_weight *w, const float *x_dev, int64_t m, int32_t *out_i, int32_t *out_mn,
                                    void *ws, size_t ws_bytes, void *stream) {
     const size_t need = cq_workspace_bytes(w, m, 0);

@@ -619,16 +619,50 @@ __device__ __forceinline__ float row_dot(const uint8_t *smem, const LdsRow r, ui
 // PRE: the model step computed on the loaded activations before they are quantized (cq_pre):
 // silu(x) * x2 elementwise, or rms_norm, for which the waves first add up the squares of their
 // chunks and exchange the chunk sums through LDS, at the price of one more workgroup barrier.
-template <int DT, int UPL, int NW, int DEPTH, int PRE>
+// The weights behind the first of a launch over several weights: planes, output, first row of the launch.
+template <int NWT> struct FusedMore {
+    uint8_t *p[NWT - 1][4];
+    float *y[NWT - 1];
+    int64_t first[NWT - 1];
+};
+template <> struct FusedMore<1> {};
+
+// NWT > 1: up to NWT weights of the same type and row length take the same activations in one launch
+// (q, k, v of an attention block).  The launch's rows are the weights' rows one after the other;
+// `more` names the planes, outputs and row ranges of the weights behind the first.
+template <int DT, int UPL, int NW, int DEPTH, int PRE, int NWT = 1>
 __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float *x, cq_pre pre,
                                                         float *__restrict__ y, int64_t total_waves,
-                                                        int64_t rows_per_wave, int64_t rows_extra) {
+                                                        int64_t rows_per_wave, int64_t rows_extra, FusedMore<NWT> more) {
     extern __shared__ __align__(16) uint8_t smem[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: scalar loops and branches
     const uint32_t units = (uint32_t)(w.k / Geo<DT>::kElems);
     const int64_t row0 = (int64_t)blockIdx.x * NW + wave;
     const int64_t T = total_waves;
+    // weight, output and local row of a row of the launch (wave-uniform: scalar selects)
+    auto pick = [&](int64_t row, cq_weight &ws, float *&ys) -> int64_t {
+        ws = w;
+        ys = y;
+        int64_t first = 0;
+        if constexpr (NWT > 1) {
+#pragma unroll
+            for (int t = 0; t < NWT - 1; t++) {
+                if (row >= more.first[t]) {
+                    ws.p0 = more.p[t][0]; ws.p1 = more.p[t][1]; ws.p2 = more.p[t][2]; ws.p3 = more.p[t][3];
+                    ys = more.y[t];
+                    first = more.first[t];
+                }
+            }
+        }
+        return row - first;
+    };
+    auto load_launch_row = [&](int64_t row, UnitRaw<DT> (&buf)[UPL]) {
+        cq_weight ws;
+        float *ys;
+        const int64_t lr = pick(row, ws, ys);
+        load_row<DT, UPL>(ws, lr, units, buf);
+    };
     // rows of this wave (>= DEPTH): n / T, plus one for the first n % T waves (both from the host)
     const int64_t cnt = rows_per_wave + (row0 < rows_extra ? 1 : 0);
 
@@ -652,8 +686,8 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     UnitRaw<DT> a[UPL], b[DEPTH == 2 ? UPL : 1];
-    load_row<DT, UPL>(w, row0, units, a);
-    if constexpr (DEPTH == 2) load_row<DT, UPL>(w, row0 + T, units, b);
+    load_launch_row(row0, a);
+    if constexpr (DEPTH == 2) load_launch_row(row0 + T, b);
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     const LdsRow r = lds_row<DT>(w.k, 0);
@@ -727,13 +761,16 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
     if constexpr (kRms && kPairs) yscale = row_scale();
     auto put = [&](int64_t row, float v) {
         if constexpr (kRms && kPairs) v *= yscale;
-        if (lane == 0) y[row] = v;
+        cq_weight ws;
+        float *ys;
+        const int64_t lr = pick(row, ws, ys);
+        if (lane == 0) ys[lr] = v;
     };
 
     if constexpr (DEPTH == 1) {
         for (int64_t i = 0; i < cnt; i++) {
             const float s = row_dot<DT, UPL>(smem, r, units, a);
-            if (i + 1 < cnt) load_row<DT, UPL>(w, row0 + (i + 1) * T, units, a);
+            if (i + 1 < cnt) load_launch_row(row0 + (i + 1) * T, a);
             put(row0 + i * T, s);
         }
     } else {
@@ -747,19 +784,19 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
                 UnitRaw<DT> ta[UPL], tb[UPL];
 #pragma unroll
                 for (int c = 0; c < UPL; c++) ta[c] = a[c];
-                load_row<DT, UPL>(w, row0 + (i + 2) * T, units, a);
+                load_launch_row(row0 + (i + 2) * T, a);
                 __builtin_amdgcn_sched_barrier(0);
                 s0 = row_dot<DT, UPL>(smem, r, units, ta);
 #pragma unroll
                 for (int c = 0; c < UPL; c++) tb[c] = b[c];
-                load_row<DT, UPL>(w, row0 + (i + 3) * T, units, b);
+                load_launch_row(row0 + (i + 3) * T, b);
                 __builtin_amdgcn_sched_barrier(0);
                 s1 = row_dot<DT, UPL>(smem, r, units, tb);
             } else {
                 s0 = row_dot<DT, UPL>(smem, r, units, a);
-                load_row<DT, UPL>(w, row0 + (i + 2) * T, units, a);
+                load_launch_row(row0 + (i + 2) * T, a);
                 s1 = row_dot<DT, UPL>(smem, r, units, b);
-                load_row<DT, UPL>(w, row0 + (i + 3) * T, units, b);
+                load_launch_row(row0 + (i + 3) * T, b);
             }
             put(row0 + i * T, s0);
             put(row0 + (i + 1) * T, s1);
@@ -775,7 +812,7 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
             put(row0 + (i + 1) * T, s1);
         } else {
             const float s0 = row_dot<DT, UPL>(smem, r, units, a);
-            load_row<DT, UPL>(w, row0 + (i + 2) * T, units, a);
+            load_launch_row(row0 + (i + 2) * T, a);
             const float s1 = row_dot<DT, UPL>(smem, r, units, b);
             put(row0 + i * T, s0);
             put(row0 + (i + 1) * T, s1);
@@ -948,8 +985,9 @@ int num_cus() {
 
 // Eight waves per workgroup, one workgroup per CU.  Whole workgroups only, and every wave
 // gets at least `depth` rows: wgs * 8 * depth <= n.
-template <int DT, int UPL, int PRE>
-hipError_t launch_fused_upl(const cq_weight *w, const float *x, cq_pre pre, float *y, hipStream_t s) {
+template <int DT, int UPL, int PRE, int NWT = 1>
+hipError_t launch_fused_upl(const cq_weight *w, int64_t n, FusedMore<NWT> more, const float *x, cq_pre pre, float *y,
+                            hipStream_t s) {
     constexpr int NW = 8;
     constexpr int kXch = (UPL * Geo<DT>::kElems / (Geo<DT>::kActK ? 8 : 4) + NW - 1) / NW;   // as in the kernel
     const size_t lds = PRE == CQ_PRE_RMS_NORM ? fused_red_offset<DT>(w->k) + 4 * (size_t)((Geo<DT>::kActK ? 2 : 1) * kXch * NW)
@@ -958,16 +996,20 @@ hipError_t launch_fused_upl(const cq_weight *w, const float *x, cq_pre pre, floa
     // per CU measured faster than two on every decode shape (11008 x 4096 Q4K: 7.0 us against 7.6 us)
     const int64_t max_wgs = num_cus();
     int depth = UPL <= 2 ? 2 : 1;
-    if (w->n < NW * 2) depth = 1;
-    if (w->n < NW) {  // fewer rows than one workgroup's waves: the two-launch path handles it
+    if (n < NW * 2) depth = 1;
+    if (n < NW) {  // fewer rows than one workgroup's waves: the two-launch path handles it
         return hipErrorInvalidConfiguration;
     }
-    int64_t wgs = w->n / (NW * depth);
+    int64_t wgs = n / (NW * depth);
     if (wgs > max_wgs) wgs = max_wgs;
-    const int64_t tw = wgs * NW, rpw = w->n / tw, extra = w->n % tw;
-    if (depth == 2) CQ_LAUNCH((fused_kernel<DT, UPL, NW, 2, PRE>), (unsigned)wgs, NW * 64, lds, s, *w, x, pre, y, tw, rpw, extra);
-    else CQ_LAUNCH((fused_kernel<DT, UPL, NW, 1, PRE>), (unsigned)wgs, NW * 64, lds, s, *w, x, pre, y, tw, rpw, extra);
+    const int64_t tw = wgs * NW, rpw = n / tw, extra = n % tw;
+    if (depth == 2) CQ_LAUNCH((fused_kernel<DT, UPL, NW, 2, PRE, NWT>), (unsigned)wgs, NW * 64, lds, s, *w, x, pre, y, tw, rpw, extra, more);
+    else CQ_LAUNCH((fused_kernel<DT, UPL, NW, 1, PRE, NWT>), (unsigned)wgs, NW * 64, lds, s, *w, x, pre, y, tw, rpw, extra, more);
     return hipGetLastError();
+}
+template <int DT, int UPL, int PRE>
+hipError_t launch_fused_upl(const cq_weight *w, const float *x, cq_pre pre, float *y, hipStream_t s) {
+    return launch_fused_upl<DT, UPL, PRE, 1>(w, w->n, FusedMore<1>{}, x, pre, y, s);
 }
 
 template <int DT>
@@ -1086,7 +1128,70 @@ hipError_t launch_ints(const cq_weight *w, cq_act_view a, int64_t m, int32_t *oi
     return hipSuccess;
 }
 
+// Two or three weights on the same activations (same type, row length and device; rows of at most 256
+// units): one launch over all their rows.
+constexpr int kMultiMax = 3;
+template <int DT, int PRE>
+hipError_t launch_fused_multi_pre(const cq_weight *const *ws, int count, const float *x, cq_pre pre, float *const *ys,
+                                  hipStream_t s) {
+    FusedMore<kMultiMax> more;
+    int64_t n = ws[0]->n;
+    for (int t = 0; t < kMultiMax - 1; t++) {
+        const int j = t + 1 < count ? t + 1 : count - 1;   // unused slots repeat the last weight with no rows
+        more.p[t][0] = ws[j]->p0; more.p[t][1] = ws[j]->p1; more.p[t][2] = ws[j]->p2; more.p[t][3] = ws[j]->p3;
+        more.y[t] = ys[j];
+        more.first[t] = n;
+        if (t + 1 < count) n += ws[j]->n;
+    }
+    // (a slot that repeats the last weight starts at the end of the launch: no row reaches it)
+    const cq_weight *w = ws[0];
+    const int upl = (int)((w->k / Geo<DT>::kElems + 63) / 64);
+    if (upl <= 1) return launch_fused_upl<DT, 1, PRE, kMultiMax>(w, n, more, x, pre, ys[0], s);
+    if (upl <= 2) return launch_fused_upl<DT, 2, PRE, kMultiMax>(w, n, more, x, pre, ys[0], s);
+    if (upl <= 3) return launch_fused_upl<DT, 3, PRE, kMultiMax>(w, n, more, x, pre, ys[0], s);
+    return launch_fused_upl<DT, 4, PRE, kMultiMax>(w, n, more, x, pre, ys[0], s);
+}
+template <int DT>
+hipError_t launch_fused_multi(const cq_weight *const *ws, int count, const float *x, cq_pre pre, float *const *ys,
+                              hipStream_t s) {
+    switch (pre.kind) {
+    case CQ_PRE_NONE: return launch_fused_multi_pre<DT, CQ_PRE_NONE>(ws, count, x, pre, ys, s);
+    case CQ_PRE_RMS_NORM: return launch_fused_multi_pre<DT, CQ_PRE_RMS_NORM>(ws, count, x, pre, ys, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+
 }  // namespace
+
+bool cq_matvec_fused_multi_supported(const cq_weight *const *ws, int count, int pre_kind) {
+    if (count < 2 || count > kMultiMax || (pre_kind != CQ_PRE_NONE && pre_kind != CQ_PRE_RMS_NORM)) return false;
+    for (int i = 0; i < count; i++) {
+        if (ws[i]->dtype != ws[0]->dtype || ws[i]->k != ws[0]->k || ws[i]->dev != ws[0]->dev || ws[i]->n == 0) return false;
+        if (!cq_matvec_fused_supported(ws[i])) return false;
+    }
+    int64_t units = 0;
+    switch (ws[0]->dtype) {
+    case CQ_DTYPE_Q4_0: units = ws[0]->k / Geo<CQ_DTYPE_Q4_0>::kElems; break;
+    case CQ_DTYPE_Q8_0: units = ws[0]->k / Geo<CQ_DTYPE_Q8_0>::kElems; break;
+    case CQ_DTYPE_Q4K: units = ws[0]->k / Geo<CQ_DTYPE_Q4K>::kElems; break;
+    case CQ_DTYPE_Q5K: units = ws[0]->k / Geo<CQ_DTYPE_Q5K>::kElems; break;
+    case CQ_DTYPE_Q6K: units = ws[0]->k / Geo<CQ_DTYPE_Q6K>::kElems; break;
+    default: return false;
+    }
+    return units <= 256;
+}
+
+hipError_t cq_launch_matvec_fused_multi(const cq_weight *const *ws, int count, const float *x, cq_pre pre,
+                                        float *const *ys, hipStream_t s) {
+    switch (ws[0]->dtype) {
+    case CQ_DTYPE_Q4_0: return launch_fused_multi<CQ_DTYPE_Q4_0>(ws, count, x, pre, ys, s);
+    case CQ_DTYPE_Q8_0: return launch_fused_multi<CQ_DTYPE_Q8_0>(ws, count, x, pre, ys, s);
+    case CQ_DTYPE_Q4K: return launch_fused_multi<CQ_DTYPE_Q4K>(ws, count, x, pre, ys, s);
+    case CQ_DTYPE_Q5K: return launch_fused_multi<CQ_DTYPE_Q5K>(ws, count, x, pre, ys, s);
+    case CQ_DTYPE_Q6K: return launch_fused_multi<CQ_DTYPE_Q6K>(ws, count, x, pre, ys, s);
+    default: return hipErrorInvalidValue;
+    }
+}
 
 bool cq_matvec_fused_supported(const cq_weight *w) {
     switch (w->dtype) {

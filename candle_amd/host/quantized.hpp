@@ -13,6 +13,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdint>
 #include <memory>
 #include <numeric>
@@ -243,6 +244,38 @@ class QMatMul {
     // forward(silu(gate) * up): the feed-forward's w2 (Mlp::forward, quantized_llama.rs:56-63)
     Tensor forward_silu_mul(const Tensor &gate, const Tensor &up, hipStream_t stream = nullptr) const {
         return qtensor_->storage().fwd(qtensor_->shape(), gate, stream, CQ_PRE_SILU_MUL, &up);
+    }
+    // {m.forward(xs) for m in mats} (with alpha: of rms_norm(xs, alpha, eps)) for matrices of one dtype and row
+    // length, as q, k, v (quantized_llama.rs:206-208) or w1, w3 (:60-61): one launch for one activation row,
+    // the rows quantized once otherwise
+    static std::vector<Tensor> forward_multi(const std::vector<const QMatMul *> &mats, const Tensor &xs,
+                                             const Tensor *alpha = nullptr, float eps = 0.0f, hipStream_t stream = nullptr) {
+        if (mats.empty()) throw Error("forward_multi: no matrices");
+        const int64_t k = mats[0]->qtensor_->shape().back();
+        if (xs.rank() < 2) throw Error("input tensor has only one dimension " + to_string(xs.shape));
+        if (alpha && alpha->shape != Shape{k})
+            throw Error("shape mismatch in rms-norm " + to_string(xs.shape) + " " + to_string(alpha->shape));
+        const int64_t m = k ? elem_count(xs.shape) / k : 0;
+        std::vector<const cq_weight *> ws;
+        std::vector<Tensor> ys;
+        std::vector<float *> yp;
+        size_t ws_bytes = 0;
+        for (const QMatMul *mm : mats) {
+            const Shape &sh = mm->qtensor_->shape();
+            if (sh.size() != 2 || xs.shape.back() != sh[1])
+                throw Error("input tensor " + to_string(xs.shape) + " incompatible with " + to_string(sh));
+            Shape out_shape = xs.shape;
+            out_shape.back() = sh[0];
+            ys.push_back(Tensor{out_shape, DeviceBuffer<float>((size_t)(m * sh[0]))});
+            yp.push_back(ys.back().data.get());
+            ws.push_back(mm->qtensor_->storage().raw());
+            ws_bytes = std::max(ws_bytes, cq_workspace_bytes(ws.back(), m, CQ_FLAG_AUTO));
+        }
+        DeviceBuffer<uint8_t> wsp(ws_bytes);
+        check(cq_qmatmul_multi(ws.data(), (int)ws.size(), alpha ? CQ_PRE_RMS_NORM : CQ_PRE_NONE, xs.data.get(),
+                               alpha ? alpha->data.get() : nullptr, eps, m, yp.data(), CQ_FLAG_AUTO, wsp.get(), ws_bytes,
+                               stream), "QMatMul::forward_multi");
+        return ys;
     }
     const QTensor &qtensor() const { return *qtensor_; }
 

@@ -118,6 +118,20 @@ static void fused_neighbours() {
     Tensor short_alpha = Tensor::from_host(std::vector<float>((size_t)(k - 1), 1.f), {k - 1});
     EXPECT(throws([&] { mm.forward_rms_norm(xt, short_alpha, eps); }), "alpha of the wrong length must be an error");
     EXPECT(throws([&] { mm.forward_silu_mul(xt, one); }), "operands of different shapes must be an error");
+    // forward_multi: every output equals the matrix's own forward(), one row (one launch) and several
+    std::vector<float> w2((size_t)(2 * n * k));
+    for (size_t i = 0; i < w2.size(); i++) w2[i] = 0.02f * std::cos(0.23f * (float)i);
+    QMatMul mm2 = QMatMul::from_qtensor(QTensor::quantize(Tensor::from_host(w2, {2 * n, k}), GgmlDType::Q4K));
+    for (const Tensor *in : {&one, &xt}) {
+        std::vector<Tensor> ys = QMatMul::forward_multi({&mm, &mm2}, *in);
+        EXPECT(ys.size() == 2 && ys[1].shape.back() == 2 * n, "forward_multi: output shapes");
+        close(ys[0].to_host(), mm.forward(*in).to_host(), "forward_multi, first matrix");
+        close(ys[1].to_host(), mm2.forward(*in).to_host(), "forward_multi, second matrix");
+        std::vector<Tensor> yn = QMatMul::forward_multi({&mm, &mm2}, *in, &at, eps);
+        close(yn[1].to_host(), mm2.forward_rms_norm(*in, at, eps).to_host(), "forward_multi with rms_norm");
+    }
+    QMatMul other = QMatMul::from_qtensor(QTensor::quantize(Tensor::from_host(w, {n, k}), GgmlDType::Q6K));
+    EXPECT(throws([&] { QMatMul::forward_multi({&mm, &other}, xt); }), "matrices of different dtypes must be an error");
 }
 
 int main(int argc, char **argv) {

@@ -26,7 +26,7 @@ EXPORTS = [
     "cq_weight_device", "cq_weight_shape", "cq_weight_destroy", "cq_act_bytes", "cq_quantize_act",
     "cq_workspace_bytes", "cq_qmatmul", "cq_qmatmul_int_dots", "cq_grouped_workspace_bytes",
     "cq_qmatmul_grouped", "cq_silu_mul", "cq_moe_scatter_add", "cq_timing_arm", "cq_timing_elapsed_us",
-    "cq_selfcheck_round", "cq_quantize_act_fused", "cq_qmatmul_fused", "cq_qmatmul_grouped_fused",
+    "cq_selfcheck_round", "cq_quantize_act_fused", "cq_qmatmul_fused", "cq_qmatmul_grouped_fused", "cq_qmatmul_multi",
 ]
 
 
@@ -80,6 +80,7 @@ def load():
     L.cq_qmatmul_fused.argtypes = [vp, ci, vp, vp, C.c_float, i64, vp, ci, vp, sz, vp]
     L.cq_qmatmul_grouped_fused.argtypes = [C.POINTER(vp), ci, ci, vp, vp, C.c_float, vp, C.POINTER(C.c_int32), vp, ci,
                                            vp, sz, vp]
+    L.cq_qmatmul_multi.argtypes = [C.POINTER(vp), ci, ci, vp, vp, C.c_float, i64, C.POINTER(vp), ci, vp, sz, vp]
     _lib = L
     return L
 
@@ -276,6 +277,34 @@ def qmatmul(w: QWeight, x, flags: int = 0, out=None, workspace: Workspace | None
                                  C.c_void_p(out.data_ptr()), flags, C.c_void_p(ws.data_ptr()), ws.numel(),
                                  _stream_ptr()))
     return out
+
+
+def qmatmul_multi(ws, x, flags: int = 0, workspace: Workspace | None = None, pre: int = PRE_NONE, aux=None,
+                  eps: float = 0.0):
+    """[x . W^T for W in ws]: several weights (same dtype and row length) on the same activations, one
+    launch for one activation row, rows quantized once otherwise (cq_qmatmul_multi)."""
+    torch = _torch()
+    L = load()
+    _require_f32_cuda(x)
+    _check_pre(pre, x, aux)
+    ws = list(ws)
+    if not ws:
+        raise QHipError("no weights")
+    k = ws[0].shape[1]
+    if x.dim() < 2:
+        raise QHipError(f"input tensor has only one dimension {tuple(x.shape)}")
+    if x.shape[-1] != k:
+        raise QHipError(f"input tensor {tuple(x.shape)} incompatible with {ws[0].shape}")
+    m = x.numel() // k if k else 0
+    outs = [torch.empty(tuple(x.shape[:-1]) + (w.shape[0],), dtype=torch.float32, device=x.device) for w in ws]
+    need = max(L.cq_workspace_bytes(w.handle, m, flags) for w in ws)
+    wsp = (workspace or _default_ws).get(need, x.device)
+    vp = C.c_void_p
+    handles = (vp * len(ws))(*[w.handle for w in ws])
+    ys = (vp * len(ws))(*[o.data_ptr() for o in outs])
+    check(L.cq_qmatmul_multi(handles, len(ws), pre, vp(x.data_ptr()), vp(aux.data_ptr()) if aux is not None else None,
+                             eps, m, ys, flags, vp(wsp.data_ptr()), wsp.numel(), _stream_ptr()))
+    return outs
 
 
 def qmatmul_int_dots(w: QWeight, x):

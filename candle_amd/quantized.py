@@ -185,5 +185,14 @@ class QMatMul:
         (Mlp::forward, quantized_llama.rs:56-63)."""
         return qhip.qmatmul(self.qtensor.weight, gate, workspace=self._ws, pre=qhip.PRE_SILU_MUL, aux=up)
 
+    @staticmethod
+    def forward_multi(mats, xs, alpha=None, eps: float = 0.0):
+        """`[m.forward(xs) for m in mats]` (with `alpha`: of rms_norm(xs, alpha, eps)) for matrices of one
+        dtype and row length, as the q, k, v projections (quantized_llama.rs:206-208) or w1 and w3
+        (:60-61): one launch for one activation row, the rows quantized once otherwise."""
+        mats = list(mats)
+        pre = qhip.PRE_NONE if alpha is None else qhip.PRE_RMS_NORM
+        return qhip.qmatmul_multi([m.qtensor.weight for m in mats], xs, workspace=mats[0]._ws, pre=pre, aux=alpha, eps=eps)
+
     def dequantize_f16(self):
         return self.qtensor.dequantize_f16()

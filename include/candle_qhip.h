@@ -171,6 +171,19 @@ int cq_quantize_act_fused(int dev, int act_dtype, int pre, const float *x_dev, c
                           int64_t m, int64_t k, void *dst_blocks_dev, void *stream);
 int cq_qmatmul_fused(const cq_weight *w, int pre, const float *x_dev, const float *aux_dev, float eps, int64_t m,
                      float *y_dev, int flags, void *workspace_dev, size_t workspace_bytes, void *stream);
+/* Several weights on the same activations: ys[i] = x . ws[i]^T, i < count (the q, k, v projections of an
+ * attention block, quantized_llama.rs:206-208; w1 and w3 of the feed-forward block, :60-61), with the step
+ * `pre` in front as in cq_qmatmul_fused (CQ_PRE_NONE for none).  The weights share dtype, row length k and
+ * device; their row counts may differ.  One activation row and two or three weights with rows of at most
+ * 256 lane units (k <= 16384 for Q4K/Q5K, 8192 for Q6K/Q4_0, 4096 for Q8_0), flags == 0: a single launch
+ * for all of them, each output bit-identical to its own cq_qmatmul_fused call.  More rows: the rows are
+ * quantized once and every weight takes its matmul from the shared workspace (size: the largest
+ * cq_workspace_bytes among the weights).  Anything else: one call per weight.  The reference has no
+ * counterpart, it calls QMatMul::forward once per weight; a `Hip` arm can offer it to the model code beside
+ * forward(). */
+int cq_qmatmul_multi(const cq_weight *const *ws, int count, int pre, const float *x_dev, const float *aux_dev, float eps,
+                     int64_t m, float *const *ys_dev, int flags, void *workspace_dev, size_t workspace_bytes,
+                     void *stream);
 /* cq_qmatmul_grouped with the same step applied to the gathered rows (row p reads x and aux at
  * row_ids[p], or p when row_ids is NULL). */
 int cq_qmatmul_grouped_fused(const cq_weight *const *experts, int n_experts, int pre, const float *x_dev,
