@@ -21,7 +21,8 @@ def test_graph_replays_match_eager():
     dev = torch.device("cuda:0")
     rng = np.random.default_rng(21)
     # one call per kernel family: one-launch decode, decode with a fused rms_norm, split-K MFMA (4 rows),
-    # dot-product kernel (2 rows of Q8_0), tile kernel with split K (zero fill + atomic adds), grouped experts
+    # dot-product kernel (2 rows of Q8_0), tile kernel with split K (zero fill + atomic adds), grouped experts,
+    # two weights in one decode launch
     cases = [("decode", orc.Q4K, 1, 4096, 512), ("rms", orc.Q6K, 1, 2048, 256), ("skinny", orc.Q4K, 4, 1024, 64),
              ("batched", orc.Q8_0, 2, 512, 40), ("gemm", orc.Q6K, 40, 2048, 64)]
     weights, xs, ys, wss = {}, {}, {}, {}
@@ -41,8 +42,16 @@ def test_graph_replays_match_eager():
     arr = (C.c_void_p * n_e)(*[e.handle.value for e in experts])
     gws = torch.empty(L.cq_grouped_workspace_bytes(arr, n_e, 30, 0), dtype=torch.uint8, device=dev)
 
+    # two weights on the decode case's input in one launch
+    pair = [weights["decode"], qhip.QWeight.from_ggml(orc.Q4K, orc.quantize(orc.Q4K, make_inputs(77, 1, 4096, 128)[0]), 128, 4096)]
+    pair_y = [torch.empty((1, 512), dtype=torch.float32, device=dev), torch.empty((1, 128), dtype=torch.float32, device=dev)]
+    pair_w = (C.c_void_p * 2)(*[w.handle for w in pair])
+    pair_o = (C.c_void_p * 2)(*[t.data_ptr() for t in pair_y])
+
     def step():
         s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        qhip.check(L.cq_qmatmul_multi(pair_w, 2, qhip.PRE_NONE, C.c_void_p(xs["decode"].data_ptr()), None, 0.0, 1, pair_o, 0,
+                                      C.c_void_p(wss["decode"].data_ptr()), wss["decode"].numel(), s))
         for name, dt, m, k, n in cases:
             args = (C.c_void_p(xs[name].data_ptr()), m, C.c_void_p(ys[name].data_ptr()), 0,
                     C.c_void_p(wss[name].data_ptr()), wss[name].numel(), s)
@@ -74,7 +83,8 @@ def test_graph_replays_match_eager():
             torch.cuda.synchronize()
             want = {k: v.clone() for k, v in ys.items()}
             want_g = gy.clone()
-            for t in list(ys.values()) + [gy]:
+            want_p = [t.clone() for t in pair_y]
+            for t in list(ys.values()) + [gy] + pair_y:
                 t.fill_(float("nan"))                # eager work between the replays; also proves the replay writes
             torch.cuda.synchronize()
             graph.replay()
@@ -85,3 +95,5 @@ def test_graph_replays_match_eager():
                 else:
                     assert torch.equal(ys[name], want[name]), (seed, name)
             assert torch.allclose(gy, want_g, rtol=1e-5, atol=1e-6), seed
+            assert torch.equal(pair_y[0], want_p[0]) and torch.equal(pair_y[1], want_p[1]), seed
+            assert torch.equal(pair_y[0], ys["decode"]), seed   # the same rows as the weight's own call
