@@ -281,12 +281,23 @@ def main() -> int:
             qhip.check(L.cq_qmatmul(calls[i][0].handle, C.c_void_p(x.data_ptr()), 1, C.c_void_p(outputs[i].data_ptr()),
                                     0, C.c_void_p(ws.data_ptr()), ws.numel(), s))
 
+        def multi_call(first, count, x, s):   # rms_norm -> `count` projections, one launch
+            hs = (C.c_void_p * count)(*[calls[first + t][0].handle for t in range(count)])
+            ys = (C.c_void_p * count)(*[outputs[first + t].data_ptr() for t in range(count)])
+            qhip.check(L.cq_qmatmul_multi(hs, count, qhip.PRE_RMS_NORM, C.c_void_p(x.data_ptr()), C.c_void_p(alpha.data_ptr()),
+                                          eps, 1, ys, 0, C.c_void_p(ws.data_ptr()), ws.numel(), s))
+
         def chain(fused):
             s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
             norm = lambda x: torch.nn.functional.rms_norm(x, (HIDDEN,), alpha, eps)
             for layer in range(args.layers):
                 b = layer * len(LAYER_SHAPES)
-                if fused:
+                if fused == "shared":
+                    multi_call(b, 3, inputs["x_attn"], s)
+                    plain_call(b + 3, inputs["x_o"], s)
+                    multi_call(b + 4, 2, outputs[b + 3], s)
+                    fused_call(b + 6, qhip.PRE_SILU_MUL, outputs[b + 4], outputs[b + 5], s)
+                elif fused:
                     for j in range(3):
                         fused_call(b + j, qhip.PRE_RMS_NORM, inputs["x_attn"], alpha, s)
                     plain_call(b + 3, inputs["x_o"], s)
@@ -312,7 +323,7 @@ def main() -> int:
 
         times = {}
         with torch.cuda.stream(side):
-            for name, fused in (("separate", False), ("fused", True)):
+            for name, fused in (("separate", False), ("fused", True), ("shared", "shared")):
                 chain(fused)
                 torch.cuda.synchronize()
                 gn_ = torch.cuda.CUDAGraph()
@@ -333,6 +344,7 @@ def main() -> int:
             "matmuls_only_ms": round(ms_per_step, 4),
             "separate_launches_ms": round(times["separate"], 4),
             "fused_ms": round(times["fused"], 4),
+            "fused_shared_input_ms": round(times["shared"], 4),   # q, k, v and gate, up each in one cq_qmatmul_multi launch
         }
     except Exception as e:  # reported beside the headline only: never fails the bench line
         if not (args.no_extras or args.no_graph):
