@@ -645,7 +645,7 @@ def test_split_k_output_is_cleared_wherever_it_lives(qh, dt):
 
 @pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K, orc.Q8_0, orc.Q4_0])
 @pytest.mark.parametrize("m,k,n", [(40, 1024, 1024), (100, 2048, 4096), (300, 1024, 4096), (520, 1024, 2048),
-                                   (130, 4096, 11008), (1000, 512, 8192)])
+                                   (130, 4096, 11008), (1000, 512, 8192), (4100, 1024, 1024), (48, 512, 40000)])
 def test_tile_plans_agree_with_dot_product_kernels(qh, dt, m, k, n):
     """The tile kernels pick tile height and K split per shape; whatever they pick, the result equals the
     dot-product kernels' (which the tests above hold against the oracle) to rounding, and a sample of
