@@ -407,6 +407,12 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
             return cq_set_error(CQ_ERR_UNSUPPORTED, "Q8_1 activations are only handled by the GEMM kernel");
         path = use_gemm ? kGemm : kMatvec;
     }
+    // two to four rows of short enough weight rows: the one-launch kernel again, every unpacked weight unit
+    // contracted with each activation row
+    if (flags == 0 && pre.kind == CQ_PRE_NONE && cq_matvec_fused_rows_supported(w, m)) {
+        CQ_HIP_CHECK(cq_launch_matvec_fused_rows(w, x_dev, m, y_dev, s));
+        return CQ_OK;
+    }
     cq_act_view v;
     act_ws_layout(act, m, w->k, (uint8_t *)ws, &v);
     bool y_cleared = false;
@@ -460,7 +466,9 @@ extern "C" int cq_qmatmul_multi(const cq_weight *const *ws, int count, int pre, 
         return CQ_OK;
     }
     // otherwise one matmul per weight; with more than one row the rows are quantized once, by the first
-    const bool share = m > 1 && !(flags & CQ_FLAG_REUSE_ACT);
+    // (two to four rows that the one-launch kernel takes need no quantizer launch to share)
+    const bool share = m > 1 && !(flags & CQ_FLAG_REUSE_ACT) &&
+                       !(flags == 0 && pre == CQ_PRE_NONE && cq_matvec_fused_rows_supported(ws[0], m));
     for (int i = 0; i < count; i++) {
         const bool reuse = share && i > 0;
         if (int rc = qmatmul_impl(ws[i], x_dev, reuse ? cq_no_pre() : p, m, ys_dev[i], reuse ? flags | CQ_FLAG_REUSE_ACT : flags,

@@ -609,6 +609,36 @@ __device__ __forceinline__ float row_dot(const uint8_t *smem, const LdsRow r, ui
     return wave_sum(acc);
 }
 
+// The same for MB activation rows in LDS: the unit is unpacked once, every row's sum is added up in the
+// order of the single-row function.
+template <int MB> struct Sums {
+    float v[MB];
+};
+template <int DT, int UPL, int MB>
+__device__ __forceinline__ Sums<MB> row_dot_rows(const uint8_t *smem, const LdsRow (&r)[MB], uint32_t units,
+                                               const UnitRaw<DT> (&buf)[UPL]) {
+    const uint32_t lane = threadIdx.x & 63;
+    constexpr uint32_t kB = Geo<DT>::kUnitsPerBlock;
+    Sums<MB> acc;
+#pragma unroll
+    for (int m = 0; m < MB; m++) acc.v[m] = 0.0f;
+#pragma unroll
+    for (int c = 0; c < UPL; c++) {
+        const uint32_t u = c * 64 + lane;
+        const uint32_t uc = u < units ? u : (units - kB + (lane & (kB - 1)));
+        UnitW<DT> uw;
+        decode_unit<DT>(buf[c], lane & 7, uw);
+#pragma unroll
+        for (int m = 0; m < MB; m++) {
+            const float v = unit_value<DT>(smem, uw, r[m], uc, units);
+            acc.v[m] += u < units ? v : 0.0f;
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MB; m++) acc.v[m] = wave_sum(acc.v[m]);
+    return acc;
+}
+
 // Wave g of `total_waves` handles rows g, g + total_waves, ...  The launcher guarantees that every
 // wave has at least DEPTH rows, so the prologue loads are unconditional: the compiler can then
 // count outstanding loads exactly and waits for the activation chunk only (issued first; loads
@@ -630,7 +660,9 @@ template <> struct FusedMore<1> {};
 // NWT > 1: up to NWT weights of the same type and row length take the same activations in one launch
 // (q, k, v of an attention block).  The launch's rows are the weights' rows one after the other;
 // `more` names the planes, outputs and row ranges of the weights behind the first.
-template <int DT, int UPL, int NW, int DEPTH, int PRE, int NWT = 1>
+// MB > 1 (with PRE none and one weight): MB activation rows x[MB][k], outputs y[MB][n]; every weight row is
+// unpacked once and contracted with each of them.
+template <int DT, int UPL, int NW, int DEPTH, int PRE, int NWT = 1, int MB = 1>
 __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float *x, cq_pre pre,
                                                         float *__restrict__ y, int64_t total_waves,
                                                         int64_t rows_per_wave, int64_t rows_extra, FusedMore<NWT> more) {
@@ -670,10 +702,15 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
     // per step for Q8_0 activations, two for Q8K
     constexpr bool kPairs = Geo<DT>::kActK;
     constexpr int XCH = (UPL * Geo<DT>::kElems / (kPairs ? 8 : 4) + NW - 1) / NW;
-    float4 fx[kPairs ? 1 : XCH];
-    X8 fx8[kPairs ? XCH : 1];
-    if constexpr (kPairs) load_x_pairs<XCH, NW>(x, w.k, wave, fx8);
-    else load_x_chunks<XCH, NW>(x, w.k, wave, fx);
+    float4 fxa[MB][kPairs ? 1 : XCH];
+    X8 fx8a[MB][kPairs ? XCH : 1];
+#pragma unroll
+    for (int m = 0; m < MB; m++) {
+        if constexpr (kPairs) load_x_pairs<XCH, NW>(x + m * w.k, w.k, wave, fx8a[m]);
+        else load_x_chunks<XCH, NW>(x + m * w.k, w.k, wave, fxa[m]);
+    }
+    auto &fx = fxa[0];
+    auto &fx8 = fx8a[0];
     float4 gx[(PRE != CQ_PRE_NONE && !kPairs) ? XCH : 1];   // the second operand, at the same elements
     X8 gx8[(PRE != CQ_PRE_NONE && kPairs) ? XCH : 1];
     if constexpr (PRE != CQ_PRE_NONE) {
@@ -756,20 +793,32 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
     }
     if constexpr (kPairs) quantize_pairs_to_lds<DT, XCH, NW>(smem, w.k, wave, r, fx8);
     else quantize_row_to_lds<DT, XCH, NW>(smem, w.k, wave, r, fx);
+    LdsRow rm[MB];
+    rm[0] = r;
+#pragma unroll
+    for (int m = 1; m < MB; m++) {
+        rm[m] = lds_row<DT>(w.k, m);
+        if constexpr (kPairs) quantize_pairs_to_lds<DT, XCH, NW>(smem, w.k, wave, rm[m], fx8a[m]);
+        else quantize_row_to_lds<DT, XCH, NW>(smem, w.k, wave, rm[m], fxa[m]);
+    }
     __syncthreads();
     float yscale = 1.0f;
     if constexpr (kRms && kPairs) yscale = row_scale();
-    auto put = [&](int64_t row, float v) {
-        if constexpr (kRms && kPairs) v *= yscale;
+    auto put = [&](int64_t row, Sums<MB> v) {
         cq_weight ws;
         float *ys;
         const int64_t lr = pick(row, ws, ys);
-        if (lane == 0) ys[lr] = v;
+#pragma unroll
+        for (int m = 0; m < MB; m++) {
+            float t = v.v[m];
+            if constexpr (kRms && kPairs) t *= yscale;
+            if (lane == 0) ys[m * w.n + lr] = t;
+        }
     };
 
     if constexpr (DEPTH == 1) {
         for (int64_t i = 0; i < cnt; i++) {
-            const float s = row_dot<DT, UPL>(smem, r, units, a);
+            const Sums<MB> s = row_dot_rows<DT, UPL, MB>(smem, rm, units, a);
             if (i + 1 < cnt) load_launch_row(row0 + (i + 1) * T, a);
             put(row0 + i * T, s);
         }
@@ -779,23 +828,23 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
         for (; i + 3 < cnt; i += 2) {
             // the refill of a buffer is issued before the arithmetic on its old contents (which move
             // to other registers), so a wave keeps up to three rows in flight
-            float s0, s1;
+            Sums<MB> s0, s1;
             if constexpr (UPL <= 2) {
                 UnitRaw<DT> ta[UPL], tb[UPL];
 #pragma unroll
                 for (int c = 0; c < UPL; c++) ta[c] = a[c];
                 load_launch_row(row0 + (i + 2) * T, a);
                 __builtin_amdgcn_sched_barrier(0);
-                s0 = row_dot<DT, UPL>(smem, r, units, ta);
+                s0 = row_dot_rows<DT, UPL, MB>(smem, rm, units, ta);
 #pragma unroll
                 for (int c = 0; c < UPL; c++) tb[c] = b[c];
                 load_launch_row(row0 + (i + 3) * T, b);
                 __builtin_amdgcn_sched_barrier(0);
-                s1 = row_dot<DT, UPL>(smem, r, units, tb);
+                s1 = row_dot_rows<DT, UPL, MB>(smem, rm, units, tb);
             } else {
-                s0 = row_dot<DT, UPL>(smem, r, units, a);
+                s0 = row_dot_rows<DT, UPL, MB>(smem, rm, units, a);
                 load_launch_row(row0 + (i + 2) * T, a);
-                s1 = row_dot<DT, UPL>(smem, r, units, b);
+                s1 = row_dot_rows<DT, UPL, MB>(smem, rm, units, b);
                 load_launch_row(row0 + (i + 3) * T, b);
             }
             put(row0 + i * T, s0);
@@ -806,17 +855,17 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
         if (!third) {
             // two rows in one stretch of straight-line code: their dependent chains (dot products,
             // wave reductions) interleave
-            const float s0 = row_dot<DT, UPL>(smem, r, units, a);
-            const float s1 = row_dot<DT, UPL>(smem, r, units, b);
+            const Sums<MB> s0 = row_dot_rows<DT, UPL, MB>(smem, rm, units, a);
+            const Sums<MB> s1 = row_dot_rows<DT, UPL, MB>(smem, rm, units, b);
             put(row0 + i * T, s0);
             put(row0 + (i + 1) * T, s1);
         } else {
-            const float s0 = row_dot<DT, UPL>(smem, r, units, a);
+            const Sums<MB> s0 = row_dot_rows<DT, UPL, MB>(smem, rm, units, a);
             load_launch_row(row0 + (i + 2) * T, a);
-            const float s1 = row_dot<DT, UPL>(smem, r, units, b);
+            const Sums<MB> s1 = row_dot_rows<DT, UPL, MB>(smem, rm, units, b);
             put(row0 + i * T, s0);
             put(row0 + (i + 1) * T, s1);
-            const float s2 = row_dot<DT, UPL>(smem, r, units, a);
+            const Sums<MB> s2 = row_dot_rows<DT, UPL, MB>(smem, rm, units, a);
             put(row0 + (i + 2) * T, s2);
         }
     }
@@ -985,13 +1034,13 @@ int num_cus() {
 
 // Eight waves per workgroup, one workgroup per CU.  Whole workgroups only, and every wave
 // gets at least `depth` rows: wgs * 8 * depth <= n.
-template <int DT, int UPL, int PRE, int NWT = 1>
+template <int DT, int UPL, int PRE, int NWT = 1, int MB = 1>
 hipError_t launch_fused_upl(const cq_weight *w, int64_t n, FusedMore<NWT> more, const float *x, cq_pre pre, float *y,
                             hipStream_t s) {
     constexpr int NW = 8;
     constexpr int kXch = (UPL * Geo<DT>::kElems / (Geo<DT>::kActK ? 8 : 4) + NW - 1) / NW;   // as in the kernel
     const size_t lds = PRE == CQ_PRE_RMS_NORM ? fused_red_offset<DT>(w->k) + 4 * (size_t)((Geo<DT>::kActK ? 2 : 1) * kXch * NW)
-                                              : lds_row_bytes<DT>(w->k);
+                                              : lds_row_bytes<DT>(w->k) * MB;
     // every workgroup quantizes the whole activation row, so fewer, longer-lived workgroups win: one
     // per CU measured faster than two on every decode shape (11008 x 4096 Q4K: 7.0 us against 7.6 us)
     const int64_t max_wgs = num_cus();
@@ -1003,8 +1052,8 @@ hipError_t launch_fused_upl(const cq_weight *w, int64_t n, FusedMore<NWT> more, 
     int64_t wgs = n / (NW * depth);
     if (wgs > max_wgs) wgs = max_wgs;
     const int64_t tw = wgs * NW, rpw = n / tw, extra = n % tw;
-    if (depth == 2) CQ_LAUNCH((fused_kernel<DT, UPL, NW, 2, PRE, NWT>), (unsigned)wgs, NW * 64, lds, s, *w, x, pre, y, tw, rpw, extra, more);
-    else CQ_LAUNCH((fused_kernel<DT, UPL, NW, 1, PRE, NWT>), (unsigned)wgs, NW * 64, lds, s, *w, x, pre, y, tw, rpw, extra, more);
+    if (depth == 2) CQ_LAUNCH((fused_kernel<DT, UPL, NW, 2, PRE, NWT, MB>), (unsigned)wgs, NW * 64, lds, s, *w, x, pre, y, tw, rpw, extra, more);
+    else CQ_LAUNCH((fused_kernel<DT, UPL, NW, 1, PRE, NWT, MB>), (unsigned)wgs, NW * 64, lds, s, *w, x, pre, y, tw, rpw, extra, more);
     return hipGetLastError();
 }
 template <int DT, int UPL, int PRE>
@@ -1128,6 +1177,22 @@ hipError_t launch_ints(const cq_weight *w, cq_act_view a, int64_t m, int32_t *oi
     return hipSuccess;
 }
 
+// Two to four activation rows in the one-launch kernel (rows of at most 256 units).
+template <int DT, int MB>
+hipError_t launch_fused_rows_mb(const cq_weight *w, const float *x, float *y, hipStream_t s) {
+    const int upl = (int)((w->k / Geo<DT>::kElems + 63) / 64);
+    if (upl <= 1) return launch_fused_upl<DT, 1, CQ_PRE_NONE, 1, MB>(w, w->n, FusedMore<1>{}, x, cq_no_pre(), y, s);
+    if (upl <= 2) return launch_fused_upl<DT, 2, CQ_PRE_NONE, 1, MB>(w, w->n, FusedMore<1>{}, x, cq_no_pre(), y, s);
+    if (upl <= 3) return launch_fused_upl<DT, 3, CQ_PRE_NONE, 1, MB>(w, w->n, FusedMore<1>{}, x, cq_no_pre(), y, s);
+    return launch_fused_upl<DT, 4, CQ_PRE_NONE, 1, MB>(w, w->n, FusedMore<1>{}, x, cq_no_pre(), y, s);
+}
+template <int DT>
+hipError_t launch_fused_rows(const cq_weight *w, const float *x, int64_t m, float *y, hipStream_t s) {
+    if (m == 2) return launch_fused_rows_mb<DT, 2>(w, x, y, s);
+    if (m == 3) return launch_fused_rows_mb<DT, 3>(w, x, y, s);
+    return launch_fused_rows_mb<DT, 4>(w, x, y, s);
+}
+
 // Two or three weights on the same activations (same type, row length and device; rows of at most 256
 // units): one launch over all their rows.
 constexpr int kMultiMax = 3;
@@ -1162,6 +1227,41 @@ hipError_t launch_fused_multi(const cq_weight *const *ws, int count, const float
 }
 
 }  // namespace
+
+// Measured against the quantizer launch + split-K MFMA kernel (us per call, 2 / 3 / 4 rows): Q4K 4096 x 4096
+// 5.0 / 6.2 / 7.2 against 8.9; 11008 x 4096 8.4 / 10.1 / 11.7 against 13.5; Q8_0 4096 x 4096 6.8 / 7.7 / 8.9
+// against 10.5.  Every further row costs the dot products of one more row per unpacked unit, so the longer
+// the rows (elements per lane), the fewer rows pay off: K = 8192 Q4K 8.7 / 10.5 / 13.9 against 12.5,
+// K = 14336 Q4K 13.8 / 43 (registers spill) against 17.6.
+bool cq_matvec_fused_rows_supported(const cq_weight *w, int64_t m) {
+    if (m < 2 || m > 4 || !cq_matvec_fused_supported(w)) return false;
+    int64_t units = 0, elems = 0;
+    size_t row_bytes = 0;
+    switch (w->dtype) {
+    case CQ_DTYPE_Q4_0: elems = Geo<CQ_DTYPE_Q4_0>::kElems; row_bytes = lds_row_bytes<CQ_DTYPE_Q4_0>(w->k); break;
+    case CQ_DTYPE_Q8_0: elems = Geo<CQ_DTYPE_Q8_0>::kElems; row_bytes = lds_row_bytes<CQ_DTYPE_Q8_0>(w->k); break;
+    case CQ_DTYPE_Q4K: elems = Geo<CQ_DTYPE_Q4K>::kElems; row_bytes = lds_row_bytes<CQ_DTYPE_Q4K>(w->k); break;
+    case CQ_DTYPE_Q5K: elems = Geo<CQ_DTYPE_Q5K>::kElems; row_bytes = lds_row_bytes<CQ_DTYPE_Q5K>(w->k); break;
+    case CQ_DTYPE_Q6K: elems = Geo<CQ_DTYPE_Q6K>::kElems; row_bytes = lds_row_bytes<CQ_DTYPE_Q6K>(w->k); break;
+    default: return false;
+    }
+    units = w->k / elems;
+    if (units > 256 || row_bytes * (size_t)m > 64 * 1024 - 1024) return false;
+    const int64_t per_lane = (units + 63) / 64 * elems;   // elements of a row per lane
+    return per_lane <= 64 ? true : per_lane <= 128 ? m <= 3 : m <= 2;
+}
+
+hipError_t cq_launch_matvec_fused_rows(const cq_weight *w, const float *x, int64_t m, float *y, hipStream_t s) {
+    if (w->n == 0) return hipSuccess;
+    switch (w->dtype) {
+    case CQ_DTYPE_Q4_0: return launch_fused_rows<CQ_DTYPE_Q4_0>(w, x, m, y, s);
+    case CQ_DTYPE_Q8_0: return launch_fused_rows<CQ_DTYPE_Q8_0>(w, x, m, y, s);
+    case CQ_DTYPE_Q4K: return launch_fused_rows<CQ_DTYPE_Q4K>(w, x, m, y, s);
+    case CQ_DTYPE_Q5K: return launch_fused_rows<CQ_DTYPE_Q5K>(w, x, m, y, s);
+    case CQ_DTYPE_Q6K: return launch_fused_rows<CQ_DTYPE_Q6K>(w, x, m, y, s);
+    default: return hipErrorInvalidValue;
+    }
+}
 
 bool cq_matvec_fused_multi_supported(const cq_weight *const *ws, int count, int pre_kind) {
     if (count < 2 || count > kMultiMax || (pre_kind != CQ_PRE_NONE && pre_kind != CQ_PRE_RMS_NORM)) return false;

@@ -122,6 +122,9 @@ hipError_t cq_launch_int_dots(const cq_weight *w, cq_act_view a, int64_t m, int3
                               hipStream_t s);
 bool cq_matvec_fused_supported(const cq_weight *w);   // m == 1: quantizer fused into the matvec launch
 hipError_t cq_launch_matvec_fused(const cq_weight *w, const float *x, cq_pre pre, float *y, hipStream_t s);
+// 2 <= m <= 4 rows in the one-launch kernel (short rows only)
+bool cq_matvec_fused_rows_supported(const cq_weight *w, int64_t m);
+hipError_t cq_launch_matvec_fused_rows(const cq_weight *w, const float *x, int64_t m, float *y, hipStream_t s);
 // m == 1, several weights on the same activations in one launch (same dtype, k, device; 2 or 3 of them)
 bool cq_matvec_fused_multi_supported(const cq_weight *const *ws, int count, int pre_kind);
 hipError_t cq_launch_matvec_fused_multi(const cq_weight *const *ws, int count, const float *x, cq_pre pre,

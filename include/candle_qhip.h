@@ -58,7 +58,7 @@ enum {
                                  same m, k and activation format (q/k/v or gate/up share their input): skip the
                                  quantizer launch.  No counterpart in the reference, which re-quantizes per call.     */
     CQ_FLAG_FORCE_SKINNY = 32, /* the split-K MFMA kernel for few rows whatever m is (A/B runs)                                */
-    CQ_FLAG_STAGED_ACT = 16   /* m == 1 only: run the stand-alone quantizer into the workspace and the plain matvec
+    CQ_FLAG_STAGED_ACT = 16   /* up to four rows: run the stand-alone quantizer into the workspace and a matmul kernel
                                  (two launches, as cuda.rs:249-293 does) instead of the single fused launch           */
 };
 

@@ -667,3 +667,26 @@ def test_tile_plans_agree_with_dot_product_kernels(qh, dt, m, k, n):
     want = orc.matmul(dt, x, blocks, len(rows))
     g = got.cpu().numpy()[:, rows].astype(np.float64)
     assert np.linalg.norm(g - want) / np.linalg.norm(want) <= REL_L2_TOL
+
+
+@pytest.mark.parametrize("dt", WEIGHT_DTYPES)
+@pytest.mark.parametrize("m,k,n", [(2, 4096, 264), (3, 2048, 77), (4, 1024, 4096), (2, 8192, 64), (3, 8192, 40)])
+def test_few_rows_one_launch_equals_single_rows(qh, dt, m, k, n):
+    """Two to four activation rows on short enough weight rows go through the one-launch decode kernel:
+    every output row has the bits of its own one-row call (same order of operations per row), and the
+    two-launch path (quantizer + matmul kernel) agrees to rounding; longer rows stay on the two-launch path
+    and still match."""
+    w, x = make_inputs(7 * dt + m + k + n, m, k, n, outliers=True)
+    blocks = orc.quantize(dt, w)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    xd = dev(x)
+    got = qh.qmatmul(qw, xd)
+    elems = {orc.Q4_0: 32, orc.Q8_0: 16, orc.Q4K: 64, orc.Q5K: 64, orc.Q6K: 32}[dt]   # weights per 16-byte lane unit
+    units = k // elems
+    per_lane = -(-units // 64) * elems
+    if units <= 256 and (per_lane <= 64 or (per_lane <= 128 and m <= 3) or m <= 2):   # the library's rule
+        for r in range(m):
+            assert torch.equal(got[r:r + 1], qh.qmatmul(qw, xd[r:r + 1].contiguous())), r
+    two = qh.qmatmul(qw, xd, qh.FLAG_STAGED_ACT)
+    assert (torch.linalg.norm(got - two) / torch.linalg.norm(two)).item() <= 2e-6
+    check_f32(got.cpu().numpy(), orc.matmul(dt, x, blocks, n))
