@@ -1177,14 +1177,16 @@ hipError_t launch_ints(const cq_weight *w, cq_act_view a, int64_t m, int32_t *oi
     return hipSuccess;
 }
 
-// Two to four activation rows in the one-launch kernel (rows of at most 256 units).
+// Two to four activation rows in the one-launch kernel (rows of at most 256 units; 384 for two rows).
 template <int DT, int MB>
 hipError_t launch_fused_rows_mb(const cq_weight *w, const float *x, float *y, hipStream_t s) {
     const int upl = (int)((w->k / Geo<DT>::kElems + 63) / 64);
     if (upl <= 1) return launch_fused_upl<DT, 1, CQ_PRE_NONE, 1, MB>(w, w->n, FusedMore<1>{}, x, cq_no_pre(), y, s);
     if (upl <= 2) return launch_fused_upl<DT, 2, CQ_PRE_NONE, 1, MB>(w, w->n, FusedMore<1>{}, x, cq_no_pre(), y, s);
     if (upl <= 3) return launch_fused_upl<DT, 3, CQ_PRE_NONE, 1, MB>(w, w->n, FusedMore<1>{}, x, cq_no_pre(), y, s);
-    return launch_fused_upl<DT, 4, CQ_PRE_NONE, 1, MB>(w, w->n, FusedMore<1>{}, x, cq_no_pre(), y, s);
+    if (upl <= 4) return launch_fused_upl<DT, 4, CQ_PRE_NONE, 1, MB>(w, w->n, FusedMore<1>{}, x, cq_no_pre(), y, s);
+    if constexpr (MB == 2) return launch_fused_upl<DT, 6, CQ_PRE_NONE, 1, MB>(w, w->n, FusedMore<1>{}, x, cq_no_pre(), y, s);
+    return hipErrorInvalidConfiguration;
 }
 template <int DT>
 hipError_t launch_fused_rows(const cq_weight *w, const float *x, int64_t m, float *y, hipStream_t s) {
@@ -1246,7 +1248,7 @@ bool cq_matvec_fused_rows_supported(const cq_weight *w, int64_t m) {
     default: return false;
     }
     units = w->k / elems;
-    if (units > 256 || row_bytes * (size_t)m > 64 * 1024 - 1024) return false;
+    if (units > (m == 2 ? 384 : 256) || row_bytes * (size_t)m > 64 * 1024 - 1024) return false;
     const int64_t per_lane = (units + 63) / 64 * elems;   // elements of a row per lane
     return per_lane <= 64 ? true : per_lane <= 128 ? m <= 3 : m <= 2;
 }

@@ -670,7 +670,8 @@ def test_tile_plans_agree_with_dot_product_kernels(qh, dt, m, k, n):
 
 
 @pytest.mark.parametrize("dt", WEIGHT_DTYPES)
-@pytest.mark.parametrize("m,k,n", [(2, 4096, 264), (3, 2048, 77), (4, 1024, 4096), (2, 8192, 64), (3, 8192, 40)])
+@pytest.mark.parametrize("m,k,n", [(2, 4096, 264), (3, 2048, 77), (4, 1024, 4096), (2, 8192, 64), (3, 8192, 40), (2, 11008, 72),
+                                   (3, 11008, 72)])
 def test_few_rows_one_launch_equals_single_rows(qh, dt, m, k, n):
     """Two to four activation rows on short enough weight rows go through the one-launch decode kernel:
     every output row has the bits of its own one-row call (same order of operations per row), and the
@@ -684,7 +685,7 @@ def test_few_rows_one_launch_equals_single_rows(qh, dt, m, k, n):
     elems = {orc.Q4_0: 32, orc.Q8_0: 16, orc.Q4K: 64, orc.Q5K: 64, orc.Q6K: 32}[dt]   # weights per 16-byte lane unit
     units = k // elems
     per_lane = -(-units // 64) * elems
-    if units <= 256 and (per_lane <= 64 or (per_lane <= 128 and m <= 3) or m <= 2):   # the library's rule
+    if units <= (384 if m == 2 else 256) and (per_lane <= 64 or (per_lane <= 128 and m <= 3) or m <= 2):   # the library's rule
         for r in range(m):
             assert torch.equal(got[r:r + 1], qh.qmatmul(qw, xd[r:r + 1].contiguous())), r
     two = qh.qmatmul(qw, xd, qh.FLAG_STAGED_ACT)
