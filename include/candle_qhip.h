@@ -56,7 +56,10 @@ enum {
                                  instead of the CPU formulation's Q8K; not bit-comparable with the CPU QMatMul        */
     CQ_FLAG_REUSE_ACT = 8,    /* the workspace already holds this x, quantized by an earlier cq_qmatmul call with the
                                  same m, k and activation format (q/k/v or gate/up share their input): skip the
-                                 quantizer launch.  No counterpart in the reference, which re-quantizes per call.     */
+                                 quantizer launch.  The earlier call must have gone through the workspace: more than
+                                 four rows, or CQ_FLAG_STAGED_ACT (calls of up to four rows may quantize inside their
+                                 single launch and leave the workspace alone); cq_qmatmul_multi takes care of this
+                                 by itself.  No counterpart in the reference, which re-quantizes per call.            */
     CQ_FLAG_FORCE_SKINNY = 32, /* the split-K MFMA kernel for few rows whatever m is (A/B runs)                                */
     CQ_FLAG_STAGED_ACT = 16   /* up to four rows: run the stand-alone quantizer into the workspace and a matmul kernel
                                  (two launches, as cuda.rs:249-293 does) instead of the single fused launch           */
