@@ -404,6 +404,49 @@ def main() -> int:
         if not (args.no_extras or args.no_graph):
             print(f"bench.py: merged-projection step not measured ({e})", file=sys.stderr)
 
+    # ---- configs[2]-style small batches on the headline's weights (reported beside the headline) --------
+    # Whole calls (quantizer launch included where there is one), graph replay over the 32 layers' attn_q
+    # [4096 x 4096] and ffn_gate [11008 x 4096] weights, so every call streams its weights from HBM.
+    small_batch = None
+    try:
+        if args.no_extras or args.no_graph or args.layers < 8:
+            raise RuntimeError("skipped by --no-extras / --no-graph / --layers")
+        small_batch = {}
+        for label, idx in (("q4k_4096x4096", 0), ("q4k_11008x4096", 4)):
+            picks = [calls[layer * len(LAYER_SHAPES) + idx] for layer in range(args.layers)]
+            n_out = picks[0][3]
+            for mb in (2, 4, 8, 16):
+                xb = torch.randn((mb, HIDDEN), generator=gen, device=dev, dtype=torch.float32)
+                yb = torch.empty((mb, n_out), device=dev, dtype=torch.float32)
+                wsb = torch.empty(max(picks[0][0].workspace_bytes(mb), 256), dtype=torch.uint8, device=dev)
+
+                def b_step():
+                    s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+                    for (qw, *_r) in picks:
+                        qhip.check(L.cq_qmatmul(qw.handle, C.c_void_p(xb.data_ptr()), mb, C.c_void_p(yb.data_ptr()), 0,
+                                                C.c_void_p(wsb.data_ptr()), wsb.numel(), s))
+
+                with torch.cuda.stream(side):
+                    b_step()
+                    torch.cuda.synchronize()
+                    gb_ = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(gb_, stream=side):
+                        b_step()
+                    gb_.replay()
+                    torch.cuda.synchronize()
+                    b0, b1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    b0.record()
+                    for _ in range(10):
+                        gb_.replay()
+                    b1.record()
+                    torch.cuda.synchronize()
+                small_batch["%s_m%d_us" % (label, mb)] = round(b0.elapsed_time(b1) * 1e3 / (10 * len(picks)), 2)
+                del gb_, xb, yb, wsb
+    except Exception as e:  # reported beside the headline only: never fails the bench line
+        small_batch = None
+        if not (args.no_extras or args.no_graph):
+            print(f"bench.py: small batches not measured ({e})", file=sys.stderr)
+
     # ---- the headline's own weights, q/k/v and gate/up each through one cq_qmatmul_multi call ---------
     # (same weights, inputs and bytes as the headline step; 129 launches instead of 225)
     shared = None
@@ -511,6 +554,8 @@ def main() -> int:
         result["merged_projections"] = merged
     if shared is not None:
         result["shared_input_launches"] = shared
+    if small_batch is not None:
+        result["small_batch"] = small_batch
 
     # ---- CPU baseline: restated candle CPU QMatMul (AVX2 + threads) on a bounded sample ----
     if not args.no_cpu:
