@@ -23,8 +23,9 @@ def test_graph_replays_match_eager():
     # one call per kernel family: one-launch decode, decode with a fused rms_norm, split-K MFMA (4 rows),
     # dot-product kernel (2 rows of Q8_0), tile kernel with split K (zero fill + atomic adds), grouped experts,
     # two weights in one decode launch
-    cases = [("decode", orc.Q4K, 1, 4096, 512), ("rms", orc.Q6K, 1, 2048, 256), ("skinny", orc.Q4K, 4, 1024, 64),
-             ("batched", orc.Q8_0, 2, 512, 40), ("gemm", orc.Q6K, 40, 2048, 64)]
+    # (three rows of short weight rows take the one-launch kernel again: "rows")
+    cases = [("decode", orc.Q4K, 1, 4096, 512), ("rms", orc.Q6K, 1, 2048, 256), ("rows", orc.Q4K, 3, 1024, 64),
+             ("skinny", orc.Q4K, 6, 1024, 64), ("batched", orc.Q8_0, 2, 8192, 40), ("gemm", orc.Q6K, 40, 2048, 64)]
     weights, xs, ys, wss = {}, {}, {}, {}
     for name, dt, m, k, n in cases:
         w, _ = make_inputs(len(name) + k, m, k, n)
