@@ -454,15 +454,15 @@ extern "C" int cq_qmatmul_multi(const cq_weight *const *ws, int count, int pre, 
             return cq_set_error(CQ_ERR_INVALID, "weight %d differs in dtype, row length or device from weight 0", i);
     }
     const cq_pre p{pre, aux_dev, eps};
-    // one activation row, two or three weights: one launch over all their rows
-    if (m == 1 && flags == 0 && cq_matvec_fused_multi_supported(ws, count, pre)) {
+    // one activation row (or up to four of short weight rows), two or three weights: one launch over all their rows
+    if (m >= 1 && m <= 4 && flags == 0 && cq_matvec_fused_multi_supported(ws, count, pre, m)) {
         if (!x_dev) return cq_set_error(CQ_ERR_INVALID, "null argument");
         if ((uintptr_t)x_dev & 15) return cq_set_error(CQ_ERR_INVALID, "x must be 16-byte aligned");
         for (int i = 0; i < count; i++)
             if (!ys_dev[i]) return cq_set_error(CQ_ERR_INVALID, "null argument");
         if (int rc = check_pre(p)) return rc;
         CQ_HIP_CHECK(hipSetDevice(ws[0]->dev));
-        CQ_HIP_CHECK(cq_launch_matvec_fused_multi(ws, count, x_dev, p, ys_dev, (hipStream_t)stream));
+        CQ_HIP_CHECK(cq_launch_matvec_fused_multi(ws, count, x_dev, p, m, ys_dev, (hipStream_t)stream));
         return CQ_OK;
     }
     // otherwise one matmul per weight; with more than one row the rows are quantized once, by the first

@@ -654,6 +654,7 @@ template <int NWT> struct FusedMore {
     uint8_t *p[NWT - 1][4];
     float *y[NWT - 1];
     int64_t first[NWT - 1];
+    int64_t n[NWT - 1];   // rows of the weight (the stride between the output rows of two activation rows)
 };
 template <> struct FusedMore<1> {};
 
@@ -682,6 +683,7 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
             for (int t = 0; t < NWT - 1; t++) {
                 if (row >= more.first[t]) {
                     ws.p0 = more.p[t][0]; ws.p1 = more.p[t][1]; ws.p2 = more.p[t][2]; ws.p3 = more.p[t][3];
+                    ws.n = more.n[t];
                     ys = more.y[t];
                     first = more.first[t];
                 }
@@ -812,7 +814,7 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
         for (int m = 0; m < MB; m++) {
             float t = v.v[m];
             if constexpr (kRms && kPairs) t *= yscale;
-            if (lane == 0) ys[m * w.n + lr] = t;
+            if (lane == 0) ys[m * ws.n + lr] = t;
         }
     };
 
@@ -1198,7 +1200,7 @@ hipError_t launch_fused_rows(const cq_weight *w, const float *x, int64_t m, floa
 // Two or three weights on the same activations (same type, row length and device; rows of at most 256
 // units): one launch over all their rows.
 constexpr int kMultiMax = 3;
-template <int DT, int PRE>
+template <int DT, int PRE, int MB = 1>
 hipError_t launch_fused_multi_pre(const cq_weight *const *ws, int count, const float *x, cq_pre pre, float *const *ys,
                                   hipStream_t s) {
     FusedMore<kMultiMax> more;
@@ -1207,20 +1209,24 @@ hipError_t launch_fused_multi_pre(const cq_weight *const *ws, int count, const f
         const int j = t + 1 < count ? t + 1 : count - 1;   // unused slots repeat the last weight with no rows
         more.p[t][0] = ws[j]->p0; more.p[t][1] = ws[j]->p1; more.p[t][2] = ws[j]->p2; more.p[t][3] = ws[j]->p3;
         more.y[t] = ys[j];
+        more.n[t] = ws[j]->n;
         more.first[t] = n;
         if (t + 1 < count) n += ws[j]->n;
     }
     // (a slot that repeats the last weight starts at the end of the launch: no row reaches it)
     const cq_weight *w = ws[0];
     const int upl = (int)((w->k / Geo<DT>::kElems + 63) / 64);
-    if (upl <= 1) return launch_fused_upl<DT, 1, PRE, kMultiMax>(w, n, more, x, pre, ys[0], s);
-    if (upl <= 2) return launch_fused_upl<DT, 2, PRE, kMultiMax>(w, n, more, x, pre, ys[0], s);
-    if (upl <= 3) return launch_fused_upl<DT, 3, PRE, kMultiMax>(w, n, more, x, pre, ys[0], s);
-    return launch_fused_upl<DT, 4, PRE, kMultiMax>(w, n, more, x, pre, ys[0], s);
+    if (upl <= 1) return launch_fused_upl<DT, 1, PRE, kMultiMax, MB>(w, n, more, x, pre, ys[0], s);
+    if (upl <= 2) return launch_fused_upl<DT, 2, PRE, kMultiMax, MB>(w, n, more, x, pre, ys[0], s);
+    if (upl <= 3) return launch_fused_upl<DT, 3, PRE, kMultiMax, MB>(w, n, more, x, pre, ys[0], s);
+    return launch_fused_upl<DT, 4, PRE, kMultiMax, MB>(w, n, more, x, pre, ys[0], s);
 }
 template <int DT>
-hipError_t launch_fused_multi(const cq_weight *const *ws, int count, const float *x, cq_pre pre, float *const *ys,
-                              hipStream_t s) {
+hipError_t launch_fused_multi(const cq_weight *const *ws, int count, const float *x, cq_pre pre, int64_t m,
+                              float *const *ys, hipStream_t s) {
+    if (m == 2) return launch_fused_multi_pre<DT, CQ_PRE_NONE, 2>(ws, count, x, pre, ys, s);
+    if (m == 3) return launch_fused_multi_pre<DT, CQ_PRE_NONE, 3>(ws, count, x, pre, ys, s);
+    if (m == 4) return launch_fused_multi_pre<DT, CQ_PRE_NONE, 4>(ws, count, x, pre, ys, s);
     switch (pre.kind) {
     case CQ_PRE_NONE: return launch_fused_multi_pre<DT, CQ_PRE_NONE>(ws, count, x, pre, ys, s);
     case CQ_PRE_RMS_NORM: return launch_fused_multi_pre<DT, CQ_PRE_RMS_NORM>(ws, count, x, pre, ys, s);
@@ -1265,8 +1271,9 @@ hipError_t cq_launch_matvec_fused_rows(const cq_weight *w, const float *x, int64
     }
 }
 
-bool cq_matvec_fused_multi_supported(const cq_weight *const *ws, int count, int pre_kind) {
+bool cq_matvec_fused_multi_supported(const cq_weight *const *ws, int count, int pre_kind, int64_t m) {
     if (count < 2 || count > kMultiMax || (pre_kind != CQ_PRE_NONE && pre_kind != CQ_PRE_RMS_NORM)) return false;
+    if (m != 1 && (pre_kind != CQ_PRE_NONE || !cq_matvec_fused_rows_supported(ws[0], m))) return false;
     for (int i = 0; i < count; i++) {
         if (ws[i]->dtype != ws[0]->dtype || ws[i]->k != ws[0]->k || ws[i]->dev != ws[0]->dev || ws[i]->n == 0) return false;
         if (!cq_matvec_fused_supported(ws[i])) return false;
@@ -1283,14 +1290,14 @@ bool cq_matvec_fused_multi_supported(const cq_weight *const *ws, int count, int 
     return units <= 256;
 }
 
-hipError_t cq_launch_matvec_fused_multi(const cq_weight *const *ws, int count, const float *x, cq_pre pre,
+hipError_t cq_launch_matvec_fused_multi(const cq_weight *const *ws, int count, const float *x, cq_pre pre, int64_t m,
                                         float *const *ys, hipStream_t s) {
     switch (ws[0]->dtype) {
-    case CQ_DTYPE_Q4_0: return launch_fused_multi<CQ_DTYPE_Q4_0>(ws, count, x, pre, ys, s);
-    case CQ_DTYPE_Q8_0: return launch_fused_multi<CQ_DTYPE_Q8_0>(ws, count, x, pre, ys, s);
-    case CQ_DTYPE_Q4K: return launch_fused_multi<CQ_DTYPE_Q4K>(ws, count, x, pre, ys, s);
-    case CQ_DTYPE_Q5K: return launch_fused_multi<CQ_DTYPE_Q5K>(ws, count, x, pre, ys, s);
-    case CQ_DTYPE_Q6K: return launch_fused_multi<CQ_DTYPE_Q6K>(ws, count, x, pre, ys, s);
+    case CQ_DTYPE_Q4_0: return launch_fused_multi<CQ_DTYPE_Q4_0>(ws, count, x, pre, m, ys, s);
+    case CQ_DTYPE_Q8_0: return launch_fused_multi<CQ_DTYPE_Q8_0>(ws, count, x, pre, m, ys, s);
+    case CQ_DTYPE_Q4K: return launch_fused_multi<CQ_DTYPE_Q4K>(ws, count, x, pre, m, ys, s);
+    case CQ_DTYPE_Q5K: return launch_fused_multi<CQ_DTYPE_Q5K>(ws, count, x, pre, m, ys, s);
+    case CQ_DTYPE_Q6K: return launch_fused_multi<CQ_DTYPE_Q6K>(ws, count, x, pre, m, ys, s);
     default: return hipErrorInvalidValue;
     }
 }

@@ -125,9 +125,10 @@ hipError_t cq_launch_matvec_fused(const cq_weight *w, const float *x, cq_pre pre
 // 2 <= m <= 4 rows in the one-launch kernel (short rows only)
 bool cq_matvec_fused_rows_supported(const cq_weight *w, int64_t m);
 hipError_t cq_launch_matvec_fused_rows(const cq_weight *w, const float *x, int64_t m, float *y, hipStream_t s);
-// m == 1, several weights on the same activations in one launch (same dtype, k, device; 2 or 3 of them)
-bool cq_matvec_fused_multi_supported(const cq_weight *const *ws, int count, int pre_kind);
-hipError_t cq_launch_matvec_fused_multi(const cq_weight *const *ws, int count, const float *x, cq_pre pre,
+// several weights on the same activations in one launch (same dtype, k, device; 2 or 3 of them): one row, or
+// as many rows as cq_matvec_fused_rows_supported allows (then without a fused step)
+bool cq_matvec_fused_multi_supported(const cq_weight *const *ws, int count, int pre_kind, int64_t m);
+hipError_t cq_launch_matvec_fused_multi(const cq_weight *const *ws, int count, const float *x, cq_pre pre, int64_t m,
                                         float *const *ys, hipStream_t s);
 // gemm.hip
 bool cq_gemm_supported(const cq_weight *w, int64_t m, int act_dtype);

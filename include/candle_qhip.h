@@ -179,9 +179,10 @@ int cq_qmatmul_fused(const cq_weight *w, int pre, const float *x_dev, const floa
  * `pre` in front as in cq_qmatmul_fused (CQ_PRE_NONE for none).  The weights share dtype, row length k and
  * device; their row counts may differ.  One activation row and two or three weights with rows of at most
  * 256 lane units (k <= 16384 for Q4K/Q5K, 8192 for Q6K/Q4_0, 4096 for Q8_0), flags == 0: a single launch
- * for all of them, each output bit-identical to its own cq_qmatmul_fused call.  More rows: the rows are
- * quantized once and every weight takes its matmul from the shared workspace (size: the largest
- * cq_workspace_bytes among the weights).  Anything else: one call per weight.  The reference has no
+ * for all of them, each output bit-identical to its own cq_qmatmul_fused call; the same for two to four
+ * rows without a step in front when the weight rows are short enough for the one-launch kernel (k <= 4096
+ * always).  More rows: the rows are quantized once and every weight takes its matmul from the shared
+ * workspace (size: the largest cq_workspace_bytes among the weights).  Anything else: one call per weight.  The reference has no
  * counterpart, it calls QMatMul::forward once per weight; a `Hip` arm can offer it to the model code beside
  * forward(). */
 int cq_qmatmul_multi(const cq_weight *const *ws, int count, int pre, const float *x_dev, const float *aux_dev, float eps,

@@ -70,6 +70,21 @@ def test_more_rows_share_the_quantized_rows(qh, dt, m):
                 check_f32(y.cpu().numpy(), orc.matmul(dt, x, blocks, w.shape[0]))
 
 
+@pytest.mark.parametrize("dt", WEIGHT_DTYPES)
+@pytest.mark.parametrize("m", [2, 3, 4])
+def test_few_rows_one_launch_equals_separate_calls(qh, dt, m):
+    """Two to four activation rows of short weight rows: still one launch over all weights, every output
+    bit-identical to the weight's own call (which takes the same kernel for one weight)."""
+    k, ns = 2048, (264, 40, 96)
+    ws = _weights(qh, dt, k, ns, 400 + dt + m)
+    x = np.random.default_rng(m * 7 + dt).standard_normal((m, k)).astype(np.float32)
+    xd = dev(x)
+    outs = qh.qmatmul_multi([w for w, _ in ws], xd)
+    for (w, blocks), y in zip(ws, outs):
+        assert torch.equal(y, qh.qmatmul(w, xd))
+        check_f32(y.cpu().numpy(), orc.matmul(dt, x, blocks, w.shape[0]))
+
+
 def test_single_weight_four_weights_and_errors(qh):
     dt, k = orc.Q4K, 512
     ws = _weights(qh, dt, k, (32, 32, 64, 32), 300)
