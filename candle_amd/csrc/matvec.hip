@@ -1054,8 +1054,13 @@ hipError_t launch_fused_upl(const cq_weight *w, int64_t n, FusedMore<NWT> more, 
     int64_t wgs = n / (NW * depth);
     if (wgs > max_wgs) wgs = max_wgs;
     const int64_t tw = wgs * NW, rpw = n / tw, extra = n % tw;
-    if (depth == 2) CQ_LAUNCH((fused_kernel<DT, UPL, NW, 2, PRE, NWT, MB>), (unsigned)wgs, NW * 64, lds, s, *w, x, pre, y, tw, rpw, extra, more);
-    else CQ_LAUNCH((fused_kernel<DT, UPL, NW, 1, PRE, NWT, MB>), (unsigned)wgs, NW * 64, lds, s, *w, x, pre, y, tw, rpw, extra, more);
+    if constexpr (UPL <= 2) {   // (longer rows never run two deep: no instance of that)
+        if (depth == 2) {
+            CQ_LAUNCH((fused_kernel<DT, UPL, NW, 2, PRE, NWT, MB>), (unsigned)wgs, NW * 64, lds, s, *w, x, pre, y, tw, rpw, extra, more);
+            return hipGetLastError();
+        }
+    }
+    CQ_LAUNCH((fused_kernel<DT, UPL, NW, 1, PRE, NWT, MB>), (unsigned)wgs, NW * 64, lds, s, *w, x, pre, y, tw, rpw, extra, more);
     return hipGetLastError();
 }
 template <int DT, int UPL, int PRE>
