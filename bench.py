@@ -44,7 +44,8 @@ LAYER_SHAPES = [
 
 
 def ggml_bytes(dtype: str, n: int, k: int) -> int:
-    return n * k // 256 * {"q4k": 144, "q6k": 210}[dtype]
+    blk, size = {"q4k": (256, 144), "q6k": (256, 210), "q4_0": (32, 18), "q8_0": (32, 34)}[dtype]
+    return n * k // blk * size
 
 
 def main() -> int:
@@ -205,7 +206,7 @@ def main() -> int:
     small_gbs = (sum(b for _, b in small) / sum(d for d, _ in small) / 1e9) if small else None
 
     # ---- the other half of the metric: Q4_K prefill GEMM, M = 512 on the Mistral FFN shape ----
-    # (BASELINE.json configs[2]; reported beside the headline, not as `value`)
+    # (BASELINE.json configs[3]; reported beside the headline, not as `value`)
     gm, gk, gn = 512, 4096, 14336
     gen.manual_seed(4242)
     gw = torch.randn((gn, gk), generator=gen, device=dev, dtype=torch.float32) * 0.02
@@ -231,7 +232,7 @@ def main() -> int:
     gemm_tops = 2.0 * gm * gk * gn / (gemm_avg_us * 1e-6) / 1e12
     del gq, gx, gy, gws
 
-    # whole calls (activation quantizer + GEMM) on both shapes of configs[2] and on the attention shape
+    # whole calls (activation quantizer + GEMM) on both shapes of configs[3] and on the attention shape
     whole_calls = {}
     if not args.no_extras:
         for name, dt, (wn, wk) in (("q4k_14336x4096", qhip.Q4K, (14336, 4096)), ("q4k_4096x14336", qhip.Q4K, (4096, 14336)),
@@ -447,6 +448,111 @@ def main() -> int:
         if not (args.no_extras or args.no_graph):
             print(f"bench.py: small batches not measured ({e})", file=sys.stderr)
 
+    # ---- the other configurations' shapes, whole calls in a graph replay (reported beside the headline) ------
+    # configs[0]: one Q4_0 [4096 x 4096] matvec (Q8_0 activations); configs[2]'s Q8_0 half: 2-16 rows on
+    # Q8_0 weights of both decode shapes; configs[4]: the Mixtral-shaped expert FFN (8 experts, 64 tokens,
+    # top-2: two grouped launches on the routed rows, silu * mul on the way into the grouped w2 launch,
+    # weighted scatter-add).  Sixteen distinct weights per shape take turns so that each call streams from HBM.
+    other = None
+    try:
+        if args.no_extras or args.no_graph or args.layers < 8:
+            raise RuntimeError("skipped by --no-extras / --no-graph / --layers")
+        other = {}
+
+        def replay_us(fn, calls_per_replay, reps=10):
+            with torch.cuda.stream(side):
+                fn()
+                torch.cuda.synchronize()
+                g_ = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g_, stream=side):
+                    fn()
+                g_.replay()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(reps):
+                    g_.replay()
+                e1.record()
+                torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / (reps * calls_per_replay)
+            del g_
+            return us
+
+        def make_weights(dt, n, k, count, seed0):
+            out = []
+            for t in range(count):
+                gen.manual_seed(seed0 + t)
+                w_ = torch.randn((n, k), generator=gen, device=dev, dtype=torch.float32) * 0.02
+                out.append(qhip.QWeight.zeros(dt, n, k).quantize_(w_))
+                del w_
+            return out
+
+        def calls_on(weights, xb, yb, wsb, mb):
+            def fn():
+                s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+                for qw in weights:
+                    qhip.check(L.cq_qmatmul(qw.handle, C.c_void_p(xb.data_ptr()), mb, C.c_void_p(yb.data_ptr()), 0,
+                                            C.c_void_p(wsb.data_ptr()), wsb.numel(), s))
+            return fn
+
+        for label, dt, dtname, n_out in (("q4_0_4096x4096", qhip.Q4_0, "q4_0", HIDDEN), ("q8_0_4096x4096", qhip.Q8_0, "q8_0", HIDDEN),
+                                         ("q8_0_11008x4096", qhip.Q8_0, "q8_0", FFN)):
+            weights = make_weights(dt, n_out, HIDDEN, 16, 50_000 + n_out + dt)
+            for mb in ((1,) if dt == qhip.Q4_0 else (1, 2, 4, 8, 16)):
+                xb = torch.randn((mb, HIDDEN), generator=gen, device=dev, dtype=torch.float32)
+                yb = torch.empty((mb, n_out), device=dev, dtype=torch.float32)
+                wsb = torch.empty(max(weights[0].workspace_bytes(mb), 256), dtype=torch.uint8, device=dev)
+                us = replay_us(calls_on(weights, xb, yb, wsb, mb), len(weights))
+                other["%s_m%d_us" % (label, mb)] = round(us, 2)
+                if mb == 1:
+                    other["%s_m1_GBs" % label] = round(ggml_bytes(dtname, n_out, HIDDEN) / us / 1e3, 1)
+                del xb, yb, wsb
+            del weights
+
+        n_e, tokens, ffn_moe = 8, 64, 14336
+        w1 = make_weights(qhip.Q4K, ffn_moe, HIDDEN, n_e, 60_000)
+        w3 = make_weights(qhip.Q4K, ffn_moe, HIDDEN, n_e, 60_100)
+        w2 = make_weights(qhip.Q6K, HIDDEN, ffn_moe, n_e, 60_200)
+        gen.manual_seed(60_300)
+        xs = torch.randn((tokens, HIDDEN), generator=gen, device=dev, dtype=torch.float32)
+        probs = torch.softmax(torch.randn((tokens, n_e), generator=gen, device=dev, dtype=torch.float32), dim=-1).cpu().numpy()
+        top = np.argsort(-probs, axis=1, kind="stable")[:, :2]
+        topw = np.take_along_axis(probs, top, axis=1)
+        topw = topw / topw.sum(axis=1, keepdims=True)
+        rid, wts, offs = [], [], [0]
+        for e in range(n_e):
+            tok, slot = np.nonzero(top == e)
+            rid.extend(tok.tolist())
+            wts.extend(topw[tok, slot].tolist())
+            offs.append(len(rid))
+        rid_d = torch.tensor(rid, dtype=torch.int32, device=dev)
+        wts_d = torch.tensor(wts, dtype=torch.float32, device=dev)
+        offs = np.asarray(offs, dtype=np.int32)
+        moe_ws = qhip.Workspace()
+
+        def moe_ffn():
+            h1 = qhip.qmatmul_grouped(w1, xs, rid_d, offs, workspace=moe_ws)
+            h3 = qhip.qmatmul_grouped(w3, xs, rid_d, offs, workspace=moe_ws)
+            y_ = qhip.qmatmul_grouped(w2, h1, None, offs, workspace=moe_ws, pre=qhip.PRE_SILU_MUL, aux=h3)
+            return qhip.moe_scatter_add(y_, rid_d, wts_d, tokens)
+
+        moe_us = replay_us(moe_ffn, 1, reps=20)
+        moe_bytes = n_e * (2 * ggml_bytes("q4k", ffn_moe, HIDDEN) + ggml_bytes("q6k", HIDDEN, ffn_moe))
+        other["moe_ffn"] = {
+            "workload": "configs[4]: 8 experts (w1, w3 [14336x4096] Q4_K, w2 [4096x14336] Q6_K), 64 tokens, top-2: "
+                        "3 grouped launches + quantizers + scatter-add, cold weights not forced (914 MB > caches)",
+            "us_per_ffn": round(moe_us, 1),
+            "weight_bytes": moe_bytes,
+            "GBs": round(moe_bytes / moe_us / 1e3, 1),
+            "frac_of_hbm_peak": round(moe_bytes / moe_us / 1e3 / 8000.0, 4),
+            "rows_per_expert": [int(offs[e + 1] - offs[e]) for e in range(n_e)],
+        }
+        del w1, w2, w3
+    except Exception as e:  # reported beside the headline only: never fails the bench line
+        other = None
+        if not (args.no_extras or args.no_graph):
+            print(f"bench.py: other configurations not measured ({e})", file=sys.stderr)
+
     # ---- the headline's own weights, q/k/v and gate/up each through one cq_qmatmul_multi call ---------
     # (same weights, inputs and bytes as the headline step; 129 launches instead of 225)
     shared = None
@@ -538,7 +644,7 @@ def main() -> int:
             "per_kernel_events_attn_4096x4096_GBs": round(small_gbs, 1) if small_gbs else None,
         },
         "prefill_gemm": {
-            "workload": "configs[2]: Q4_K [14336x4096] x Q8_K activations, M=512 (Mistral-7B FFN up/gate)",
+            "workload": "configs[3]: Q4_K [14336x4096] x Q8_K activations, M=512 (Mistral-7B FFN up/gate)",
             "kernel": "gemm_kernel<Q4K> (int8 MFMA, quantizer launch not included)",
             "avg_launch_us": round(gemm_avg_us, 2),
             "tops": round(gemm_tops, 1),
@@ -556,6 +662,8 @@ def main() -> int:
         result["shared_input_launches"] = shared
     if small_batch is not None:
         result["small_batch"] = small_batch
+    if other is not None:
+        result["other_configs"] = other
 
     # ---- CPU baseline: restated candle CPU QMatMul (AVX2 + threads) on a bounded sample ----
     if not args.no_cpu:
