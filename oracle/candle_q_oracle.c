@@ -27,9 +27,14 @@
  *   silu_mul (op.rs:607-609, quantized_llama.rs:60-62) : closed form in float64 (no reference
  *        golden prints silu of known inputs on this path; PARITY UNPINNED beyond that: the last
  *        bits depend on the platform's expf)
- *   q8_1 quantize (k_quants.rs:665-691)         : PARITY UNPINNED by any reference
- *        golden (no reference test inspects its output); checked only against
- *        the closed form "q8_0 plus s = f16(f16(sum q) * d)".
+ *   q4_1 quantize, dequant, q4_1 x q8_1 dot (k_quants.rs:257-350; oracle only, the
+ *        product has no Q4_1 weights)            : :256-287 (128 round-trip values), :393-434
+ *        (RMSE bound), :795 + :866 (dot-product error <= 0.008 on cos vectors, x2 on ramps)
+ *   q8_1 quantize (k_quants.rs:665-691)         : d and qs by the q8_0 goldens (same
+ *        arithmetic); the `s` field by the reference's q4_1 x q8_1 dot-product bounds above
+ *        (the result is sum_i*d*d8 + m*s, so a dropped, mis-signed or unscaled s leaves the
+ *        bound by orders of magnitude: tests/test_oracle_golden.py shows each such mutant
+ *        failing) and by the invariant |s - d*sum(q)| <= one f16 ulp of s.
  *   q4k x q8_1 and q6k x q8_1 dot formulas      : PARITY UNPINNED on CPU (they
  *        exist only in the reference's CUDA kernels, quantized.cu:2141-2166,
  *        :2258-2281); checked by float64 brute force on dequantized operands.
@@ -52,6 +57,7 @@ enum {
 /* Block layouts, k_quants.rs:42-155 (#[repr(C)], little endian). */
 #pragma pack(push, 1)
 typedef struct { uint16_t d; uint8_t qs[16]; } block_q4_0;                      /* 18  */
+typedef struct { uint16_t d; uint16_t m; uint8_t qs[16]; } block_q4_1;          /* 20  */
 typedef struct { uint16_t d; int8_t qs[32]; } block_q8_0;                       /* 34  */
 typedef struct { uint16_t d; uint16_t s; int8_t qs[32]; } block_q8_1;           /* 36  */
 typedef struct { uint16_t d; uint16_t dmin; uint8_t scales[K_SCALE_SIZE]; uint8_t qs[QK_K / 2]; } block_q4k; /* 144 */
@@ -60,6 +66,7 @@ typedef struct { float d; int8_t qs[QK_K]; int16_t bsums[QK_K / 16]; } block_q8k
 #pragma pack(pop)
 
 _Static_assert(sizeof(block_q4_0) == 18, "q4_0");
+_Static_assert(sizeof(block_q4_1) == 20, "q4_1");
 _Static_assert(sizeof(block_q8_0) == 34, "q8_0");
 _Static_assert(sizeof(block_q8_1) == 36, "q8_1");
 typedef struct { uint16_t d; uint16_t dmin; uint8_t scales[K_SCALE_SIZE]; uint8_t qh[QK_K / 8]; uint8_t qs[QK_K / 2]; } block_q5k; /* 176, k_quants.rs:119-127 */
@@ -211,6 +218,48 @@ static float vec_dot_q4_0_q8_0(int64_t n, const block_q4_0 *xs, const block_q8_0
     return sumf;
 }
 
+/* --------------------------------------------------------------- Q4_1 ---- */
+/* Oracle only: the reference's own Q4_1 vectors are what pins BlockQ8_1::from_float's `s`.
+ * k_quants.rs:296-326 (from_float; f32::min / f32::max ignore a NaN operand like fminf / fmaxf) */
+int orc_quantize_q4_1(const float *xs, void *out, int64_t k) {
+    if (k % 32 != 0) return -1;
+    block_q4_1 *ys = (block_q4_1 *)out;
+    for (int64_t i = 0; i < k / 32; i++) {
+        const float *x = xs + i * 32;
+        float min = INFINITY, max = -INFINITY;
+        for (int j = 0; j < 32; j++) {
+            min = fminf(x[j], min);
+            max = fmaxf(x[j], max);
+        }
+        float d = (max - min) / 15.0f;
+        float id = d != 0.0f ? 1.0f / d : 0.0f;
+        ys[i].d = orc_f32_to_f16(d);
+        ys[i].m = orc_f32_to_f16(min);
+        for (int j = 0; j < 16; j++) {
+            float x0 = (x[j] - min) * id;
+            float x1 = (x[16 + j] - min) * id;
+            uint8_t xi0 = as_u8(x0 + 0.5f); if (xi0 > 15) xi0 = 15;
+            uint8_t xi1 = as_u8(x1 + 0.5f); if (xi1 > 15) xi1 = 15;
+            ys[i].qs[j] = (uint8_t)(xi0 | (xi1 << 4));
+        }
+    }
+    return 0;
+}
+
+/* k_quants.rs:329-349 */
+int orc_dequantize_q4_1(const void *in, float *ys, int64_t k) {
+    if (k % 32 != 0) return -1;
+    const block_q4_1 *xs = (const block_q4_1 *)in;
+    for (int64_t i = 0; i < k / 32; i++) {
+        float d = orc_f16_to_f32(xs[i].d), m = orc_f16_to_f32(xs[i].m);
+        for (int j = 0; j < 16; j++) {
+            ys[i * 32 + j] = (float)(xs[i].qs[j] & 0x0F) * d + m;
+            ys[i * 32 + j + 16] = (float)(xs[i].qs[j] >> 4) * d + m;
+        }
+    }
+    return 0;
+}
+
 /* --------------------------------------------------------------- Q8_0 ---- */
 /* k_quants.rs:586-615 */
 int orc_quantize_q8_0(const float *xs, void *out, int64_t k) {
@@ -278,6 +327,25 @@ int orc_quantize_q8_1(const float *xs, void *out, int64_t k) {
         uint16_t hs = orc_f32_to_f16((float)sum);
         ys[i].s = orc_f32_to_f16(orc_f16_to_f32(hs) * orc_f16_to_f32(ys[i].d));
     }
+    return 0;
+}
+
+/* k_quants.rs:267-294 (vec_dot_unopt of Q4_1 x Q8_1; the block count must be even) */
+static int vec_dot_q4_1_q8_1(int64_t n, const block_q4_1 *xs, const block_q8_1 *ys, float *out) {
+    int64_t nb = n / 32;
+    if (nb % 2 != 0) return -1;
+    float sumf = 0.0f;
+    for (int64_t i = 0; i < nb; i++) {
+        int32_t sumi = 0;
+        for (int j = 0; j < 16; j++) {
+            int32_t v0 = xs[i].qs[j] & 0x0F;
+            int32_t v1 = xs[i].qs[j] >> 4;
+            sumi += v0 * (int32_t)ys[i].qs[j] + v1 * (int32_t)ys[i].qs[j + 16];
+        }
+        sumf += (float)sumi * orc_f16_to_f32(xs[i].d) * orc_f16_to_f32(ys[i].d) +
+                orc_f16_to_f32(xs[i].m) * orc_f16_to_f32(ys[i].s);
+    }
+    *out = sumf;
     return 0;
 }
 
@@ -879,14 +947,14 @@ static inline int32_t int_q6k_q8k(const block_q6k *x, const block_q8k *y) {
 /* -------------------------------------------------------- type dispatch ---- */
 int64_t orc_block_size(int dtype) {
     switch (dtype) {
-    case ORC_Q4_0: case ORC_Q8_0: case ORC_Q8_1: return 32;
+    case ORC_Q4_0: case ORC_Q4_1: case ORC_Q8_0: case ORC_Q8_1: return 32;
     case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return QK_K;
     default: return 0;
     }
 }
 int64_t orc_type_size(int dtype) {
     switch (dtype) {
-    case ORC_Q4_0: return 18; case ORC_Q8_0: return 34; case ORC_Q8_1: return 36;
+    case ORC_Q4_0: return 18; case ORC_Q4_1: return 20; case ORC_Q8_0: return 34; case ORC_Q8_1: return 36;
     case ORC_Q4K: return 144; case ORC_Q5K: return 176; case ORC_Q6K: return 210; case ORC_Q8K: return 292;
     default: return 0;
     }
@@ -896,6 +964,7 @@ int64_t orc_type_size(int dtype) {
 int orc_vec_dot_type(int dtype) {
     switch (dtype) {
     case ORC_Q4_0: case ORC_Q8_0: return ORC_Q8_0;
+    case ORC_Q4_1: return ORC_Q8_1;   /* k_quants.rs:260 */
     case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return ORC_Q8K;
     default: return -1;
     }
@@ -904,6 +973,7 @@ int orc_vec_dot_type(int dtype) {
 int orc_quantize(int dtype, const float *xs, void *out, int64_t k) {
     switch (dtype) {
     case ORC_Q4_0: return orc_quantize_q4_0(xs, out, k);
+    case ORC_Q4_1: return orc_quantize_q4_1(xs, out, k);
     case ORC_Q8_0: return orc_quantize_q8_0(xs, out, k);
     case ORC_Q8_1: return orc_quantize_q8_1(xs, out, k);
     case ORC_Q4K: return orc_quantize_q4k(xs, out, k);
@@ -917,6 +987,7 @@ int orc_quantize(int dtype, const float *xs, void *out, int64_t k) {
 int orc_dequantize(int dtype, const void *in, float *ys, int64_t k) {
     switch (dtype) {
     case ORC_Q4_0: return orc_dequantize_q4_0(in, ys, k);
+    case ORC_Q4_1: return orc_dequantize_q4_1(in, ys, k);
     case ORC_Q8_0: return orc_dequantize_q8_0(in, ys, k);
     case ORC_Q4K: return orc_dequantize_q4k(in, ys, k);
     case ORC_Q5K: return orc_dequantize_q5k(in, ys, k);
@@ -932,6 +1003,7 @@ int orc_vec_dot(int dtype, int64_t n, const void *xs, const void *ys, float *out
     if (bs == 0 || n % bs != 0) return -1;
     switch (dtype) {
     case ORC_Q4_0: *out = vec_dot_q4_0_q8_0(n, xs, ys); return 0;
+    case ORC_Q4_1: return vec_dot_q4_1_q8_1(n, xs, ys, out);
     case ORC_Q8_0: *out = vec_dot_q8_0_q8_0(n, xs, ys); return 0;
     case ORC_Q4K: *out = vec_dot_q4k_q8k(n, xs, ys); return 0;
     case ORC_Q5K: *out = vec_dot_q5k_q8k(n, xs, ys); return 0;

@@ -6,7 +6,7 @@ import pytest
 
 from oracle import cpu_oracle as orc
 
-DT = {"q4_0": orc.Q4_0, "q8_0": orc.Q8_0, "q4k": orc.Q4K, "q5k": orc.Q5K, "q6k": orc.Q6K, "q8k": orc.Q8K}
+DT = {"q4_0": orc.Q4_0, "q4_1": orc.Q4_1, "q8_0": orc.Q8_0, "q4k": orc.Q4K, "q5k": orc.Q5K, "q6k": orc.Q6K, "q8k": orc.Q8K}
 
 
 # ---------------------------------------------------------------- f16 ----
@@ -100,7 +100,7 @@ def _ggml_like(offset):
     return (np.float32(0.1) + np.float32(2.0) * np.cos(i + np.float32(offset), dtype=np.float32)).astype(np.float32)
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q4k", "q5k", "q6k", "q8k", "q8_0"])
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q4k", "q5k", "q6k", "q8k", "q8_0"])
 def test_quantization_total_error(goldens, name):
     src = _ggml_like(0.0)
     dst = orc.dequantize(DT[name], orc.quantize(DT[name], src))
@@ -256,8 +256,10 @@ def test_q8_0_closed_form():
 
 
 def test_q8_1_is_q8_0_plus_s():
-    """BlockQ8_1::from_float (k_quants.rs:665-691) has no reference golden: parity unpinned.
-    Checked against its closed form: same d and qs as Q8_0, s = f16(f16(sum q) * d)."""
+    """BlockQ8_1::from_float (k_quants.rs:665-691): d and qs are BlockQ8_0::from_float's (pinned by the Q4_0 /
+    Q8_0 goldens); `s` against the closed form f16(f16(sum q) * d) and the looser invariant that it is d * sum(q)
+    to within one f16 unit in the last place.  What pins `s` independently of this reading is the reference's
+    Q4_1 x Q8_1 dot-product test below."""
     rng = np.random.default_rng(7)
     x = (rng.standard_normal(4096) * 3).astype(np.float32)
     b0 = orc.quantize(orc.Q8_0, x).reshape(-1, 34)
@@ -268,6 +270,111 @@ def test_q8_1_is_q8_0_plus_s():
     s = b1[:, 2:4].copy().view(np.float16)[:, 0]
     want = (qs.sum(1).astype(np.float32).astype(np.float16).astype(np.float32) * d.astype(np.float32)).astype(np.float16)
     assert np.array_equal(s.view(np.uint16), want.view(np.uint16))
+    exact = d.astype(np.float64) * qs.sum(1)
+    ulp = np.spacing(np.abs(s).astype(np.float16)).astype(np.float64)
+    assert (np.abs(s.astype(np.float64) - exact) <= ulp).all()
+
+
+# ---- Q4_1 (oracle only): the reference vectors that depend on the `s` field of Q8_1 blocks ----
+def test_q4_1_roundtrip_golden(goldens):
+    """quantize_q4_1 (quantized_tests.rs:256-287): ramp 0..127 through Q4_1 and back, 3 decimals."""
+    g = goldens["q4_1_roundtrip_ramp128"]
+    src = np.arange(128, dtype=np.float32)
+    blocks = orc.quantize(orc.Q4_1, src)
+    assert blocks.size == 4 * 20
+    dst = orc.dequantize(orc.Q4_1, blocks)
+    # round_vector: (1000 * x).round() / 1000 in f32, half away from zero (no value is near a tie)
+    t = np.float32(1000.0) * dst
+    rounded = (np.sign(t) * np.floor(np.abs(t) + np.float32(0.5))).astype(np.float32) / np.float32(1000.0)
+    assert rounded.tolist() == [float(np.float32(v)) for v in g["dst_rounded_3"]]
+
+
+def _seq_dot_f32(a, b):
+    """vec_dot_reference (quantized_tests.rs:781-783): f32 products added one by one."""
+    acc = np.float32(0.0)
+    for p in (a * b).astype(np.float32):
+        acc = np.float32(acc + p)
+    return float(acc)
+
+
+def _q4_1_cases():
+    ramp = (np.arange(4096, dtype=np.float32) / np.float32(4096))
+    return ((_ggml_like(0.0), _ggml_like(1.0), 1.0), (ramp, ramp, 2.0))
+
+
+def _q4_1_dot_error(a, b, mutate=None):
+    aq = orc.quantize(orc.Q4_1, a)
+    bq = orc.quantize(orc.Q8_1, b).reshape(-1, 36).copy()
+    if mutate is not None:
+        d = bq[:, :2].copy().view(np.float16)[:, 0].astype(np.float32)
+        s = bq[:, 2:4].copy().view(np.float16)[:, 0].astype(np.float32)
+        sumq = bq[:, 4:].copy().view(np.int8).astype(np.int32).sum(1).astype(np.float32)
+        with np.errstate(over="ignore"):
+            bq[:, 2:4] = mutate(d, s, sumq).astype(np.float16).reshape(-1, 1).view(np.uint8)
+    res = orc.vec_dot(orc.Q4_1, a.size, aq, bq.ravel())
+    return abs(res - _seq_dot_f32(a, b)) / a.size
+
+
+def test_q4_1_dot_product_error_pins_q8_1_s(goldens):
+    """ggml_matmul_error_test::<BlockQ4_1> (quantized_tests.rs:795, :866): Q4_1 weights against Q8_1 activations
+    on the cos vectors (bound 0.008) and the ramps (x2).  The result is sum_i * d * d8 + m * s per block, so this
+    is the reference-held check of BlockQ8_1::from_float's `s`."""
+    g = goldens["dot_product_error"]
+    for a, b, err_m in _q4_1_cases():
+        err = _q4_1_dot_error(a, b)
+        assert np.isfinite(err) and err <= g["max_dot_product_error"]
+        assert err - g["leniency"] <= g["ggml_error"]["q4_1"] * err_m, err
+
+
+@pytest.mark.parametrize("mutant", ["dropped", "negated", "unscaled_sum", "scale_only", "halved", "one_percent_low"])
+def test_q4_1_dot_product_bound_rejects_wrong_s(goldens, mutant):
+    """The bound above is sharp enough: each plausible mistake in `s` fails it on at least one of the two inputs."""
+    g = goldens["dot_product_error"]
+    mutate = {
+        "dropped": lambda d, s, sumq: np.zeros_like(s),
+        "negated": lambda d, s, sumq: -s,
+        "unscaled_sum": lambda d, s, sumq: sumq,
+        "scale_only": lambda d, s, sumq: d,
+        "halved": lambda d, s, sumq: s * np.float32(0.5),
+        # the reference's bound sits 1.1 % above the correct result on the cos vectors, so even this fails it
+        "one_percent_low": lambda d, s, sumq: s * np.float32(0.99),
+    }[mutant]
+    failed = False
+    for a, b, err_m in _q4_1_cases():
+        err = _q4_1_dot_error(a, b, mutate)
+        if not np.isfinite(err) or err > g["max_dot_product_error"] or err - g["leniency"] > g["ggml_error"]["q4_1"] * err_m:
+            failed = True
+    assert failed, mutant
+
+
+def test_q4_1_closed_form_and_matmul_driver():
+    """Q4_1 from_float / to_float / dot against an independent numpy evaluation (float64 for the combine), and the
+    matmul driver with Q8_1 as the VecDotType (k_quants.rs:260, :1842-1883)."""
+    rng = np.random.default_rng(21)
+    m, k, n = 3, 256, 5
+    lhs = rng.standard_normal((m, k)).astype(np.float32)
+    rhs = (rng.standard_normal((n, k)) * 0.02 + 0.01).astype(np.float32)
+    w = orc.quantize(orc.Q4_1, rhs).reshape(n, k // 32, 20)
+    d = w[..., :2].copy().view(np.float16)[..., 0]
+    mn = w[..., 2:4].copy().view(np.float16)[..., 0]
+    q = np.concatenate([w[..., 4:] & 15, w[..., 4:] >> 4], axis=-1).astype(np.int64)   # elements j, then j + 16
+    xb = rhs.reshape(n, k // 32, 32)
+    assert np.array_equal(mn, xb.min(-1).astype(np.float16))
+    assert np.array_equal(d, ((xb.max(-1) - xb.min(-1)) / np.float32(15.0)).astype(np.float16))
+    deq = orc.dequantize(orc.Q4_1, w.ravel()).reshape(n, k // 32, 32)
+    assert np.array_equal(deq, q.astype(np.float32) * d.astype(np.float32)[..., None] + mn.astype(np.float32)[..., None])
+    assert np.abs(deq - xb).max() <= (xb.max(-1) - xb.min(-1)).max() / 15 * 0.5 + 1e-4
+    a = np.stack([orc.quantize(orc.Q8_1, lhs[r]) for r in range(m)]).reshape(m, k // 32, 36)
+    d8 = a[..., :2].copy().view(np.float16)[..., 0].astype(np.float64)
+    s8 = a[..., 2:4].copy().view(np.float16)[..., 0].astype(np.float64)
+    q8 = a[..., 4:].copy().view(np.int8).astype(np.int64)
+    sumi = np.einsum("nbl,mbl->mnb", q, q8)
+    ref = (sumi * d.astype(np.float64)[None] * d8[:, None] + mn.astype(np.float64)[None] * s8[:, None]).sum(-1)
+    out = orc.matmul(orc.Q4_1, lhs, w.ravel(), n)
+    assert np.abs(out - ref).max() <= 1e-5 * np.abs(ref).max() + 1e-6
+    # odd block counts are refused like the reference (k_quants.rs:274-276)
+    with pytest.raises(ValueError):
+        orc.vec_dot(orc.Q4_1, 32, w.ravel()[:20], a.ravel()[:36])
 
 
 @pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4k", "q5k", "q6k", "q8k"])
