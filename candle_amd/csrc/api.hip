@@ -166,6 +166,54 @@ extern "C" int cq_weight_create(int dev, int dt, const void *host_blocks, size_t
     return CQ_OK;
 }
 
+// QCudaStorage::zeros / load_quantized know an element count only (cuda.rs:368-381, :591-612): the storage is
+// a flat run of blocks, and any [n, k] with n * k elements and k a multiple of the block size is a way of
+// reading it (the planes are ordered by flat block index).  Until a shape is given it reads as one block per row.
+extern "C" int cq_weight_zeros_flat(int dev, int dt, int64_t elem_count, cq_weight **out) {
+    const int64_t bs = cq_block_size(dt);
+    if (!out) return cq_set_error(CQ_ERR_INVALID, "out is null");
+    *out = nullptr;
+    if (bs == 0 || !is_weight_dtype(dt)) return cq_set_error(CQ_ERR_UNSUPPORTED, "unsupported weight dtype %d", dt);
+    if (elem_count < 0 || elem_count % bs != 0)
+        return cq_set_error(CQ_ERR_INVALID, "element count %lld is not a multiple of the block size %lld",
+                            (long long)elem_count, (long long)bs);
+    return cq_weight_zeros(dev, dt, elem_count / bs, bs, out);
+}
+
+extern "C" int cq_weight_create_flat(int dev, int dt, const void *host_blocks, size_t nbytes, cq_weight **out) {
+    const int64_t bs = cq_block_size(dt), ts = cq_type_size(dt);
+    if (!out) return cq_set_error(CQ_ERR_INVALID, "out is null");
+    *out = nullptr;
+    if (bs == 0 || !is_weight_dtype(dt)) return cq_set_error(CQ_ERR_UNSUPPORTED, "unsupported weight dtype %d", dt);
+    if (nbytes % (size_t)ts != 0)
+        return cq_set_error(CQ_ERR_INVALID, "%zu bytes are not a whole number of %lld-byte blocks", nbytes, (long long)ts);
+    return cq_weight_create(dev, dt, host_blocks, nbytes, (int64_t)(nbytes / (size_t)ts), bs, out);
+}
+
+// check_shape (mod.rs:304-316) plus the element count of the storage
+static int check_view_shape(const cq_weight *w, int64_t n, int64_t k) {
+    if (!w) return cq_set_error(CQ_ERR_INVALID, "null weight");
+    const int64_t bs = cq_block_size(w->dtype);
+    if (n < 0 || k < 0) return cq_set_error(CQ_ERR_INVALID, "negative shape [%lld, %lld]", (long long)n, (long long)k);
+    if (k % bs != 0)
+        return cq_set_error(CQ_ERR_INVALID,
+                            "quantized tensor must have their last dim divisible by block size [%lld, %lld] %lld",
+                            (long long)n, (long long)k, (long long)bs);
+    if (n * k != w->n * w->k)
+        return cq_set_error(CQ_ERR_INVALID, "shape [%lld, %lld] does not cover the %lld elements of the storage",
+                            (long long)n, (long long)k, (long long)(w->n * w->k));
+    return CQ_OK;
+}
+
+extern "C" int64_t cq_weight_elem_count(const cq_weight *w) { return w ? w->n * w->k : 0; }
+
+extern "C" int cq_weight_set_shape(cq_weight *w, int64_t n, int64_t k) {
+    if (int rc = check_view_shape(w, n, k)) return rc;
+    w->n = n;
+    w->k = k;
+    return CQ_OK;
+}
+
 extern "C" int cq_weight_quantize(cq_weight *w, const float *src_dev, void *stream) {
     if (!w || !src_dev) return cq_set_error(CQ_ERR_INVALID, "null argument");
     if (w->ggml_bytes == 0) return CQ_OK;
@@ -365,8 +413,14 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
     const int act = act_dtype_for(w, flags);
     CQ_HIP_CHECK(hipSetDevice(w->dev));
     hipStream_t s = (hipStream_t)stream;
+    // In the one-launch kernels every workgroup reads x (and aux) in its prologue while others already store y:
+    // an output that overlaps an input goes through the quantizer launch instead, which has read all of x
+    // before the matmul kernel writes anything.
+    const bool in_place = ranges_overlap(y_dev, m * w->n, x_dev, m * w->k) ||
+                          (pre.kind != CQ_PRE_NONE &&
+                           ranges_overlap(y_dev, m * w->n, pre.aux, pre.kind == CQ_PRE_RMS_NORM ? w->k : m * w->k));
     // decode (one activation row): a single launch that quantizes x in its prologue
-    if (m == 1 && !(flags & (CQ_FLAG_REUSE_ACT | CQ_FLAG_FORCE_GEMM | CQ_FLAG_STAGED_ACT | CQ_FLAG_ACT_Q8_1)) &&
+    if (m == 1 && !in_place && !(flags & (CQ_FLAG_REUSE_ACT | CQ_FLAG_FORCE_GEMM | CQ_FLAG_STAGED_ACT | CQ_FLAG_ACT_Q8_1)) &&
         cq_matvec_fused_supported(w)) {
         CQ_HIP_CHECK(cq_launch_matvec_fused(w, x_dev, pre, y_dev, s));
         return CQ_OK;
@@ -407,9 +461,14 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
             return cq_set_error(CQ_ERR_UNSUPPORTED, "Q8_1 activations are only handled by the GEMM kernel");
         path = use_gemm ? kGemm : kMatvec;
     }
+    if (path == kMatvec && !cq_matvec_row_fits(w))
+        return cq_set_error(CQ_ERR_UNSUPPORTED,
+                            "rows of %lld elements are too long for the dot-product kernels, which keep one quantized row "
+                            "in the 160 KiB of LDS (about 150000 elements for Q4K/Q5K/Q6K, 139000 for Q8_0/Q4_0)",
+                            (long long)w->k);
     // two to four rows of short enough weight rows: the one-launch kernel again, every unpacked weight unit
     // contracted with each activation row
-    if (flags == 0 && pre.kind == CQ_PRE_NONE && cq_matvec_fused_rows_supported(w, m)) {
+    if (flags == 0 && pre.kind == CQ_PRE_NONE && !in_place && cq_matvec_fused_rows_supported(w, m)) {
         CQ_HIP_CHECK(cq_launch_matvec_fused_rows(w, x_dev, m, y_dev, s));
         return CQ_OK;
     }
@@ -439,6 +498,20 @@ extern "C" int cq_qmatmul(const cq_weight *w, const float *x_dev, int64_t m, flo
     return qmatmul_impl(w, x_dev, cq_no_pre(), m, y_dev, flags, ws, ws_bytes, stream);
 }
 
+extern "C" size_t cq_workspace_bytes_shaped(const cq_weight *w, int64_t n, int64_t k, int64_t m, int flags) {
+    if (!w || m <= 0 || check_view_shape(w, n, k) != CQ_OK) return 0;
+    return act_ws_layout(act_dtype_for(w, flags), m, k, nullptr, nullptr);
+}
+
+extern "C" int cq_qmatmul_shaped(const cq_weight *w, int64_t n, int64_t k, const float *x_dev, int64_t m, float *y_dev,
+                                 int flags, void *ws, size_t ws_bytes, void *stream) {
+    if (int rc = check_view_shape(w, n, k)) return rc;
+    cq_weight view = *w;   // the kernels take the descriptor by value; nothing keeps a pointer to it
+    view.n = n;
+    view.k = k;
+    return qmatmul_impl(&view, x_dev, cq_no_pre(), m, y_dev, flags, ws, ws_bytes, stream);
+}
+
 extern "C" int cq_qmatmul_fused(const cq_weight *w, int pre, const float *x_dev, const float *aux_dev, float eps,
                                 int64_t m, float *y_dev, int flags, void *ws, size_t ws_bytes, void *stream) {
     return qmatmul_impl(w, x_dev, cq_pre{pre, aux_dev, eps}, m, y_dev, flags, ws, ws_bytes, stream);
@@ -454,6 +527,12 @@ extern "C" int cq_qmatmul_multi(const cq_weight *const *ws, int count, int pre, 
             return cq_set_error(CQ_ERR_INVALID, "weight %d differs in dtype, row length or device from weight 0", i);
     }
     const cq_pre p{pre, aux_dev, eps};
+    // every weight reads the same x (and aux): an output on top of them would be read back by the weights behind it
+    for (int i = 0; i < count && m > 0; i++) {
+        if (ranges_overlap(ys_dev[i], m * ws[i]->n, x_dev, m * ws[0]->k) ||
+            (pre != CQ_PRE_NONE && ranges_overlap(ys_dev[i], m * ws[i]->n, aux_dev, pre == CQ_PRE_RMS_NORM ? ws[0]->k : m * ws[0]->k)))
+            return cq_set_error(CQ_ERR_INVALID, "output %d overlaps the activations: cq_qmatmul_multi does not work in place", i);
+    }
     // one activation row (or up to four of short weight rows), two or three weights: one launch over all their rows
     if (m >= 1 && m <= 4 && flags == 0 && cq_matvec_fused_multi_supported(ws, count, pre, m)) {
         if (!x_dev) return cq_set_error(CQ_ERR_INVALID, "null argument");
@@ -484,6 +563,7 @@ extern "C" int cq_qmatmul_int_dots(const cq_weight *w, const float *x_dev, int64
     int rc = check_matmul_args(w, x_dev, m, out_i, ws, ws_bytes, need);
     if (rc || m == 0 || w->n == 0 || w->k == 0) return rc;
     const int act = cq_vec_dot_type(w->dtype);
+    if (!cq_matvec_row_fits(w)) return cq_set_error(CQ_ERR_UNSUPPORTED, "rows of %lld elements do not fit the LDS", (long long)w->k);
     CQ_HIP_CHECK(hipSetDevice(w->dev));
     hipStream_t s = (hipStream_t)stream;
     cq_act_view v;

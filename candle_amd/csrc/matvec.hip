@@ -943,6 +943,8 @@ __global__ void __launch_bounds__(NW * 64) batched_kernel(cq_weight w, cq_act_vi
 
 // ------------------------------------------------------------ staged kernel (m <= 4 rows) ----
 constexpr int kStagedThreads = 256;
+// The dot-product kernels keep one whole quantized activation row in LDS: a workgroup can have 160 KiB.
+constexpr size_t kMaxRowLds = 160 * 1024;
 
 template <int DT, int MB>
 __global__ void __launch_bounds__(kStagedThreads) staged_kernel(cq_weight w, cq_act_view a, int64_t m0,
@@ -1159,10 +1161,17 @@ hipError_t launch_staged(const cq_weight *w, cq_act_view a, int64_t m, float *y,
         int mb = left >= 4 ? 4 : (left >= 2 ? 2 : 1);
         while (mb > 1 && lds_row_bytes<DT>(w->k) * mb > 64 * 1024) mb >>= 1;
         const size_t lds = lds_row_bytes<DT>(w->k) * mb;
-        if (lds > 64 * 1024) return hipErrorInvalidValue;
-        if (mb == 4) CQ_LAUNCH((staged_kernel<DT, 4>), grid, kStagedThreads, lds, s, *w, a, m0, rpw, y);
-        else if (mb == 2) CQ_LAUNCH((staged_kernel<DT, 2>), grid, kStagedThreads, lds, s, *w, a, m0, rpw, y);
-        else CQ_LAUNCH((staged_kernel<DT, 1>), grid, kStagedThreads, lds, s, *w, a, m0, rpw, y);
+        if (lds > kMaxRowLds) return hipErrorInvalidValue;   // (cq_matvec_row_fits tells beforehand)
+        if (mb == 4) {
+            if (hipError_t e = cq_ensure_lds<staged_kernel<DT, 4>>(w->dev, lds); e != hipSuccess) return e;
+            CQ_LAUNCH((staged_kernel<DT, 4>), grid, kStagedThreads, lds, s, *w, a, m0, rpw, y);
+        } else if (mb == 2) {
+            if (hipError_t e = cq_ensure_lds<staged_kernel<DT, 2>>(w->dev, lds); e != hipSuccess) return e;
+            CQ_LAUNCH((staged_kernel<DT, 2>), grid, kStagedThreads, lds, s, *w, a, m0, rpw, y);
+        } else {
+            if (hipError_t e = cq_ensure_lds<staged_kernel<DT, 1>>(w->dev, lds); e != hipSuccess) return e;
+            CQ_LAUNCH((staged_kernel<DT, 1>), grid, kStagedThreads, lds, s, *w, a, m0, rpw, y);
+        }
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         m0 += mb;
@@ -1173,7 +1182,8 @@ hipError_t launch_staged(const cq_weight *w, cq_act_view a, int64_t m, float *y,
 template <int DT>
 hipError_t launch_ints(const cq_weight *w, cq_act_view a, int64_t m, int32_t *oi, int32_t *omn, hipStream_t s) {
     const size_t lds = lds_row_bytes<DT>(w->k);
-    if (lds > 64 * 1024) return hipErrorInvalidValue;
+    if (lds > kMaxRowLds) return hipErrorInvalidValue;
+    if (hipError_t e = cq_ensure_lds<int_dots_kernel<DT>>(w->dev, lds); e != hipSuccess) return e;
     const int rpw = 8;
     const unsigned grid = (unsigned)((w->n + rpw - 1) / rpw);
     for (int64_t m0 = 0; m0 < m; m0++) {
@@ -1304,6 +1314,19 @@ hipError_t cq_launch_matvec_fused_multi(const cq_weight *const *ws, int count, c
     case CQ_DTYPE_Q5K: return launch_fused_multi<CQ_DTYPE_Q5K>(ws, count, x, pre, m, ys, s);
     case CQ_DTYPE_Q6K: return launch_fused_multi<CQ_DTYPE_Q6K>(ws, count, x, pre, m, ys, s);
     default: return hipErrorInvalidValue;
+    }
+}
+
+// Whether one quantized activation row of this weight's K fits the LDS of a workgroup, which every
+// dot-product kernel needs (K up to about 150 000 for the K-quants, 139 000 for Q8_0 / Q4_0).
+bool cq_matvec_row_fits(const cq_weight *w) {
+    switch (w->dtype) {
+    case CQ_DTYPE_Q4_0: return lds_row_bytes<CQ_DTYPE_Q4_0>(w->k) <= kMaxRowLds;
+    case CQ_DTYPE_Q8_0: return lds_row_bytes<CQ_DTYPE_Q8_0>(w->k) <= kMaxRowLds;
+    case CQ_DTYPE_Q4K: return lds_row_bytes<CQ_DTYPE_Q4K>(w->k) <= kMaxRowLds;
+    case CQ_DTYPE_Q5K: return lds_row_bytes<CQ_DTYPE_Q5K>(w->k) <= kMaxRowLds;
+    case CQ_DTYPE_Q6K: return lds_row_bytes<CQ_DTYPE_Q6K>(w->k) <= kMaxRowLds;
+    default: return false;
     }
 }
 

@@ -105,17 +105,16 @@ struct Tensor {
 // ---- QHipStorage: what QCudaStorage offers (cuda.rs:367-500) ----------------------------------
 class QHipStorage {
   public:
-    // cuda.rs:368-380 `zeros(device, elem_count, dtype)`; the [n, k] split comes from the tensor shape
-    static QHipStorage zeros(int device, int64_t n, int64_t k, GgmlDType dtype) {
+    // cuda.rs:368-381 `zeros(device, elem_count, dtype)`: the storage knows an element count, no shape
+    static QHipStorage zeros(int device, int64_t elem_count, GgmlDType dtype) {
         cq_weight *w = nullptr;
-        check(cq_weight_zeros(device, (int)to_u32(dtype), n, k, &w), "QHipStorage::zeros");
+        check(cq_weight_zeros_flat(device, (int)to_u32(dtype), elem_count, &w), "QHipStorage::zeros");
         return QHipStorage(w);
     }
-    // cuda.rs:591-612 `load_quantized`: host GGML blocks -> device, re-packed on upload
-    static QHipStorage load_quantized(int device, GgmlDType dtype, const void *blocks, size_t nbytes, int64_t n,
-                                      int64_t k) {
+    // cuda.rs:591-612 `load_quantized(device, data: &[T])`: host GGML blocks -> device, re-packed on upload
+    static QHipStorage load_quantized(int device, GgmlDType dtype, const void *blocks, size_t nbytes) {
         cq_weight *w = nullptr;
-        check(cq_weight_create(device, (int)to_u32(dtype), blocks, nbytes, n, k, &w), "load_quantized");
+        check(cq_weight_create_flat(device, (int)to_u32(dtype), blocks, nbytes, &w), "load_quantized");
         return QHipStorage(w);
     }
     ~QHipStorage() { if (w_) cq_weight_destroy(w_); }
@@ -130,21 +129,23 @@ class QHipStorage {
     GgmlDType dtype() const { return ggml_dtype_from_u32((uint32_t)cq_weight_dtype(w_)); }   // cuda.rs:382-384
     int device() const { return cq_weight_device(w_); }                                       // cuda.rs:386-388
     size_t storage_size_in_bytes() const { return cq_weight_size_in_bytes(w_); }              // cuda.rs:474-476
+    int64_t elem_count() const { return cq_weight_elem_count(w_); }
+    // The [n, k] the entry points without a shape argument read the storage as (QTensor::new fixes it).
     std::pair<int64_t, int64_t> dims() const {
         int64_t n = 0, k = 0;
         check(cq_weight_shape(w_, &n, &k), "QHipStorage::dims");
         return {n, k};
     }
+    void set_dims(int64_t n, int64_t k) { check(cq_weight_set_shape(w_, n, k), "QHipStorage::set_dims"); }
     // cuda.rs:390-446
     Tensor dequantize(const Shape &shape, hipStream_t stream = nullptr) const {
-        Tensor t{shape, DeviceBuffer<float>((size_t)elem_count(shape))};
+        Tensor t{shape, DeviceBuffer<float>((size_t)candle_hip::elem_count(shape))};
         check(cq_weight_dequantize(w_, t.data.get(), stream), "QHipStorage::dequantize");
         return t;
     }
     // cuda.rs:448-472: f32 source on the same device; quantized on the device
     void quantize(const Tensor &src, hipStream_t stream = nullptr) {
-        auto [n, k] = dims();
-        if (elem_count(src.shape) != n * k) throw Error("QHipStorage::quantize: size mismatch");
+        if (candle_hip::elem_count(src.shape) != elem_count()) throw Error("QHipStorage::quantize: size mismatch");
         check(cq_weight_quantize(w_, src.data.get(), stream), "QHipStorage::quantize");
     }
     std::vector<uint8_t> data() const {   // host GGML blocks (inverse re-pack)
@@ -169,17 +170,23 @@ class QHipStorage {
             throw Error("shape mismatch in rms-norm " + to_string(x.shape) + " " + (aux ? to_string(aux->shape) : "none"));  // ops.rs:644-650
         if (pre == CQ_PRE_SILU_MUL && (!aux || aux->shape != x.shape))
             throw Error("shape mismatch in silu-mul " + to_string(x.shape) + " " + (aux ? to_string(aux->shape) : "none"));
-        const int64_t m = k ? elem_count(x.shape) / k : 0;
+        const int64_t m = k ? candle_hip::elem_count(x.shape) / k : 0;
         Shape out_shape = x.shape;
         out_shape.back() = n;
         Tensor y{out_shape, DeviceBuffer<float>((size_t)(m * n))};
-        const size_t ws_bytes = cq_workspace_bytes(w_, m, CQ_FLAG_AUTO);
+        // the shape arrives with the call, as in the reference: the storage is read as [n, k] for this launch
+        const size_t ws_bytes = cq_workspace_bytes_shaped(w_, n, k, m, CQ_FLAG_AUTO);
+        if (m > 0 && n * k != elem_count()) throw Error("QHipStorage::fwd: " + to_string(self_shape) + " does not cover the storage");
         DeviceBuffer<uint8_t> ws(ws_bytes);   // per call, like the reference's quantized-activation buffer (cuda.rs:249-252)
-        if (pre == CQ_PRE_NONE)
-            check(cq_qmatmul(w_, x.data.get(), m, y.data.get(), CQ_FLAG_AUTO, ws.get(), ws_bytes, stream), "QHipStorage::fwd");
-        else
+        if (pre == CQ_PRE_NONE) {
+            check(cq_qmatmul_shaped(w_, n, k, x.data.get(), m, y.data.get(), CQ_FLAG_AUTO, ws.get(), ws_bytes, stream),
+                  "QHipStorage::fwd");
+        } else {
+            // the fused entry points read the shape QTensor::new fixed
+            if (dims() != std::pair<int64_t, int64_t>{n, k}) throw Error("QHipStorage::fwd: fused steps need the tensor's own shape");
             check(cq_qmatmul_fused(w_, pre, x.data.get(), aux->data.get(), eps, m, y.data.get(), CQ_FLAG_AUTO, ws.get(),
                                    ws_bytes, stream), "QHipStorage::fwd");
+        }
         // the workspace is freed when this returns; hipFree waits for the device, as dropping a
         // CudaSlice synchronises with its stream
         return y;
@@ -203,12 +210,13 @@ class QTensor {
   public:
     QTensor(QHipStorage storage, Shape shape) : storage_(std::move(storage)), shape_(std::move(shape)) {
         check_shape(shape_, block_size(storage_.dtype()));                                   // mod.rs:319-323 `new`
+        const int64_t k = shape_.back();
+        storage_.set_dims(k ? elem_count(shape_) / k : 0, k);   // leading dims flattened into rows
     }
     // mod.rs:325-343
     static QTensor quantize(const Tensor &src, GgmlDType dtype, int device = 0) {
         check_shape(src.shape, block_size(dtype));
-        const int64_t k = src.shape.back(), n = k ? elem_count(src.shape) / k : 0;
-        QHipStorage s = QHipStorage::zeros(device, n, k, dtype);
+        QHipStorage s = QHipStorage::zeros(device, elem_count(src.shape), dtype);   // Device::qzeros, mod.rs:40-57
         s.quantize(src);
         return QTensor(std::move(s), src.shape);
     }

@@ -85,6 +85,20 @@ static void roundtrip() {
     float worst = 0.f;
     for (size_t i = 0; i < src.size(); i++) worst = std::fmax(worst, std::fabs(back[i] - src[i]));
     EXPECT(worst < 0.017f, "Q4K round-trip max error %f", worst);
+    // load_quantized(device, blocks) knows no shape (cuda.rs:591-612): the tensor's shape arrives with QTensor::new
+    // and reaches the kernel with the call (fwd(self_shape, ..), cuda.rs:478-499)
+    std::vector<uint8_t> blocks = q.data();
+    QHipStorage st = QHipStorage::load_quantized(0, GgmlDType::Q4K, blocks.data(), blocks.size());
+    EXPECT(st.elem_count() == n * k && st.storage_size_in_bytes() == blocks.size(), "flat storage size");
+    std::vector<float> x((size_t)k);
+    for (int i = 0; i < k; i++) x[(size_t)i] = std::cos(0.3f * (float)i);
+    Tensor xt = Tensor::from_host(x, {1, k});
+    std::vector<float> direct = st.fwd({n, k}, xt).to_host();
+    QMatMul mm = QMatMul::from_qtensor(QTensor(std::move(st), {n, k}));
+    EXPECT(mm.forward(xt).to_host() == direct, "flat storage: forward through QTensor differs from fwd(self_shape)");
+    EXPECT(QMatMul::from_qtensor(std::move(q)).forward(xt).to_host() == direct, "flat storage: differs from the quantized tensor");
+    EXPECT(throws([&] { QHipStorage::zeros(0, 100, GgmlDType::Q4K); }), "element count that is no whole number of blocks");
+    EXPECT(throws([&] { QTensor(QHipStorage::zeros(0, 512, GgmlDType::Q4K), {3, 256}); }), "shape that does not cover the storage");
 }
 
 static void fused_neighbours() {

@@ -27,6 +27,8 @@ EXPORTS = [
     "cq_workspace_bytes", "cq_qmatmul", "cq_qmatmul_int_dots", "cq_grouped_workspace_bytes",
     "cq_qmatmul_grouped", "cq_silu_mul", "cq_moe_scatter_add", "cq_timing_arm", "cq_timing_elapsed_us",
     "cq_selfcheck_round", "cq_quantize_act_fused", "cq_qmatmul_fused", "cq_qmatmul_grouped_fused", "cq_qmatmul_multi",
+    "cq_weight_zeros_flat", "cq_weight_create_flat", "cq_weight_elem_count", "cq_weight_set_shape",
+    "cq_workspace_bytes_shaped", "cq_qmatmul_shaped",
 ]
 
 
@@ -81,6 +83,12 @@ def load():
     L.cq_qmatmul_grouped_fused.argtypes = [C.POINTER(vp), ci, ci, vp, vp, C.c_float, vp, C.POINTER(C.c_int32), vp, ci,
                                            vp, sz, vp]
     L.cq_qmatmul_multi.argtypes = [C.POINTER(vp), ci, ci, vp, vp, C.c_float, i64, C.POINTER(vp), ci, vp, sz, vp]
+    L.cq_weight_zeros_flat.argtypes = [ci, ci, i64, C.POINTER(vp)]
+    L.cq_weight_create_flat.argtypes = [ci, ci, vp, sz, C.POINTER(vp)]
+    L.cq_weight_elem_count.restype = i64; L.cq_weight_elem_count.argtypes = [vp]
+    L.cq_weight_set_shape.argtypes = [vp, i64, i64]
+    L.cq_workspace_bytes_shaped.restype = sz; L.cq_workspace_bytes_shaped.argtypes = [vp, i64, i64, i64, ci]
+    L.cq_qmatmul_shaped.argtypes = [vp, i64, i64, vp, i64, vp, ci, vp, sz, vp]
     _lib = L
     return L
 
@@ -150,6 +158,29 @@ class QWeight:
         h = C.c_void_p()
         check(L.cq_weight_zeros(dev, dtype, n, k, C.byref(h)))
         return cls(h.value, dev)
+
+    @classmethod
+    def zeros_flat(cls, dtype: int, elem_count: int, dev: int = 0) -> "QWeight":
+        """QCudaStorage::zeros(device, el_count, dtype) (cuda.rs:368-381): storage without a shape."""
+        h = C.c_void_p()
+        check(load().cq_weight_zeros_flat(dev, dtype, elem_count, C.byref(h)))
+        return cls(h.value, dev)
+
+    @classmethod
+    def from_ggml_flat(cls, dtype: int, blocks: np.ndarray, dev: int = 0) -> "QWeight":
+        """load_quantized(device, data) (cuda.rs:591-612): blocks only, the shape comes with the call."""
+        blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+        h = C.c_void_p()
+        check(load().cq_weight_create_flat(dev, dtype, blocks.ctypes.data, blocks.size, C.byref(h)))
+        return cls(h.value, dev)
+
+    def set_shape(self, n: int, k: int) -> "QWeight":
+        check(load().cq_weight_set_shape(self._h, n, k))
+        return self
+
+    @property
+    def elem_count(self) -> int:
+        return load().cq_weight_elem_count(self._h)
 
     def __del__(self):
         try:
@@ -276,6 +307,27 @@ def qmatmul(w: QWeight, x, flags: int = 0, out=None, workspace: Workspace | None
         check(L.cq_qmatmul_fused(w.handle, pre, C.c_void_p(x.data_ptr()), C.c_void_p(aux.data_ptr()), eps, m,
                                  C.c_void_p(out.data_ptr()), flags, C.c_void_p(ws.data_ptr()), ws.numel(),
                                  _stream_ptr()))
+    return out
+
+
+def qmatmul_shaped(w: QWeight, shape, x, flags: int = 0, out=None, workspace: Workspace | None = None):
+    """QCudaStorage::fwd(&self, self_shape, x, layout) (cuda.rs:478-499): the weight's [n, k] arrives with the
+    call; the storage only knows its element count."""
+    torch = _torch()
+    L = load()
+    _require_f32_cuda(x)
+    n, k = (int(v) for v in shape)
+    if x.dim() < 2:
+        raise QHipError(f"input tensor has only one dimension {tuple(x.shape)}")
+    if x.shape[-1] != k:
+        raise QHipError(f"input tensor {tuple(x.shape)} incompatible with {(n, k)}")
+    m = x.numel() // k if k else 0
+    if out is None:
+        out = torch.empty(tuple(x.shape[:-1]) + (n,), dtype=torch.float32, device=x.device)
+    need = L.cq_workspace_bytes_shaped(w.handle, n, k, m, flags)
+    ws = (workspace or _default_ws).get(need, x.device)
+    check(L.cq_qmatmul_shaped(w.handle, n, k, C.c_void_p(x.data_ptr()), m, C.c_void_p(out.data_ptr()), flags,
+                              C.c_void_p(ws.data_ptr()), ws.numel(), _stream_ptr()))
     return out
 
 

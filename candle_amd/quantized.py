@@ -69,8 +69,13 @@ class QTensor:
     tensors; higher ranks are kept as their shape with the leading dims flattened into `n`."""
 
     def __init__(self, weight: qhip.QWeight, shape):
+        """`QTensor::new(storage, shape)` (mod.rs:318-323): the shape is checked against the block size and
+        the storage's element count, and becomes the [rows, k] the matmul entry points read the storage as."""
         self._w = weight
         self._shape = tuple(int(s) for s in shape)
+        _check_shape(self._shape, qhip.load().cq_block_size(weight.dtype))
+        k = self._shape[-1]
+        weight.set_shape(int(np.prod(self._shape[:-1])) if len(self._shape) > 1 else 1, k)
 
     # ---- constructors ---------------------------------------------------------------------
     @classmethod
@@ -82,9 +87,8 @@ class QTensor:
             raise qhip.QHipError(f"quantize: unsupported dtype {dtype.name}")
         shape = tuple(src.shape)
         _check_shape(shape, dtype.block_size())
-        k = shape[-1]
-        n = int(np.prod(shape[:-1])) if len(shape) > 1 else 1
-        w = qhip.QWeight.zeros(int(dtype), n, k, dev=src.device.index or 0)
+        # Device::qzeros(elem_count, dtype) then QStorage::quantize (mod.rs:331-338): the storage has no shape
+        w = qhip.QWeight.zeros_flat(int(dtype), int(np.prod(shape)), dev=src.device.index or 0)
         w.quantize_(src.contiguous() if not src.is_contiguous() else src)
         return cls(w, shape)
 
@@ -94,9 +98,7 @@ class QTensor:
         dtype = GgmlDType(dtype)
         shape = tuple(int(s) for s in shape)
         _check_shape(shape, dtype.block_size())
-        k = shape[-1]
-        n = int(np.prod(shape[:-1])) if len(shape) > 1 else 1
-        return cls(qhip.QWeight.from_ggml(int(dtype), blocks, n, k, dev), shape)
+        return cls(qhip.QWeight.from_ggml_flat(int(dtype), blocks, dev), shape)
 
     # ---- getters (mod.rs:345-359; lib.rs:1214-1240) ---------------------------------------------
     @property
@@ -151,28 +153,52 @@ def _check_shape(shape, block_size: int):
                              f"{tuple(shape)} {block_size}")
 
 
-class QMatMul:
-    """`QMatMul::QTensor` arm (mod.rs:394-462): y = x . W^T with W quantized, computed by the
-    device kernels without dequantizing W."""
+def _env_switch(name: str) -> bool:
+    """mod.rs:400-420: set and neither empty nor "0"."""
+    import os
+    v = os.environ.get(name)
+    return v is not None and v != "" and v != "0"
 
-    def __init__(self, qtensor: QTensor):
+
+class QMatMul:
+    """`QMatMul` (mod.rs:394-462): y = x . W^T.  The `QTensor` arm keeps W quantized and runs the device
+    kernels; `from_arc` picks the `Tensor` / `TensorF16` arms (W dequantized once, then the host
+    framework's dense matmul: torch here, candle's own on the Rust side) when `CANDLE_DEQUANTIZE_ALL` /
+    `CANDLE_DEQUANTIZE_ALL_F16` ask for it (mod.rs:423-438)."""
+
+    def __init__(self, qtensor: QTensor, arm: str = "QTensor", dense=None):
         if qtensor.rank() != 2:
             raise qhip.QHipError(f"QMatMul needs a rank-2 weight, got {qtensor.shape}")
         self.qtensor = qtensor
+        self.arm = arm          # "QTensor" | "Tensor" | "TensorF16"
+        self.dense = dense      # the dequantized weight of the two dense arms
         self._ws = qhip.Workspace()
 
     @classmethod
     def from_qtensor(cls, qtensor: QTensor) -> "QMatMul":
-        return cls(qtensor)
+        return cls.from_arc(qtensor)
 
     @classmethod
     def from_arc(cls, qtensor: QTensor) -> "QMatMul":
+        if _env_switch("CANDLE_DEQUANTIZE_ALL"):
+            return cls(qtensor, "Tensor", qtensor.dequantize())
+        if _env_switch("CANDLE_DEQUANTIZE_ALL_F16"):
+            return cls(qtensor, "TensorF16", qtensor.dequantize_f16())
         return cls(qtensor)
 
     def forward(self, xs):
         """mod.rs:528-550 -> `cpu_fwd` semantics (mod.rs:469-500): xs f32, contiguous, rank >= 2,
         last dim == k; result has xs' shape with the last dim replaced by n."""
+        if self.arm == "Tensor":        # mod.rs:531-538
+            return xs.matmul(self.dense.t())
+        if self.arm == "TensorF16":     # mod.rs:539-547
+            return xs.to(self.dense.dtype).matmul(self.dense.t()).to(xs.dtype)
         return qhip.qmatmul(self.qtensor.weight, xs, workspace=self._ws)
+
+    def forward_via_f16(self, xs):
+        """mod.rs:452-461."""
+        w = self.dequantize_f16()
+        return xs.to(w.dtype).matmul(w.t()).to(xs.dtype)
 
     def forward_rms_norm(self, xs, alpha, eps: float):
         """`self.forward(rms_norm(xs, alpha, eps))` (RmsNorm::forward, candle-transformers/src/
@@ -195,4 +221,9 @@ class QMatMul:
         return qhip.qmatmul_multi([m.qtensor.weight for m in mats], xs, workspace=mats[0]._ws, pre=pre, aux=alpha, eps=eps)
 
     def dequantize_f16(self):
+        """mod.rs:444-450."""
+        if self.arm == "Tensor":
+            return self.dense.half()
+        if self.arm == "TensorF16":
+            return self.dense
         return self.qtensor.dequantize_f16()

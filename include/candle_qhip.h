@@ -15,6 +15,12 @@
  *    synchronisation, like the reference's CUDA arm (cuda.rs:478-499).
  *  - the device layout of a cq_weight is private (re-packed planes), as
  *    QStorage::data() is "not implemented" for device arms (mod.rs:126-128).
+ *  - aliasing: cq_qmatmul / cq_qmatmul_fused / cq_qmatmul_shaped may be called in place (y on top of
+ *    x or aux): such a call goes through the separate quantizer launch, which has read every input
+ *    before the matmul kernel stores anything.  cq_qmatmul_multi and the grouped calls refuse /
+ *    do not support outputs that overlap their inputs.  The workspace never overlaps anything.
+ *  - every matmul call needs its workspace (size from cq_workspace_bytes*), also the calls that
+ *    usually finish in one launch without touching it: which kernels run is the library's choice.
  *  - no C++ exception or abort crosses this boundary.
  */
 #ifndef CANDLE_QHIP_H
@@ -95,6 +101,18 @@ int cq_weight_create(int dev, int ggml_dtype, const void *host_ggml_blocks, size
                      int64_t n, int64_t k, cq_weight **out);
 /* QCudaStorage::zeros (cuda.rs:368-381): zero-filled storage for n*k elements. */
 int cq_weight_zeros(int dev, int ggml_dtype, int64_t n, int64_t k, cq_weight **out);
+/* The same two constructors with the reference's own signatures, which know an element count and no
+ * shape: QCudaStorage::zeros(device, el_count, dtype) (cuda.rs:368-381; Device::qzeros, mod.rs:40-57) and
+ * load_quantized(device, data: &[T]) (cuda.rs:591-612).  The storage is a flat run of blocks (the device
+ * planes are ordered by flat block index), so it can be read as any [n, k] with n * k == elem_count and
+ * k % block_size == 0; until told otherwise it reads as [elem_count / block_size, block_size].  The shape
+ * arrives with the call (cq_qmatmul_shaped, as QCudaStorage::fwd takes self_shape, cuda.rs:478-499) or is
+ * fixed once with cq_weight_set_shape (QTensor::new, mod.rs:318-323), which the entry points without a
+ * shape argument then use. */
+int cq_weight_zeros_flat(int dev, int ggml_dtype, int64_t elem_count, cq_weight **out);
+int cq_weight_create_flat(int dev, int ggml_dtype, const void *host_ggml_blocks, size_t nbytes, cq_weight **out);
+int64_t cq_weight_elem_count(const cq_weight *w);                /* QTensor::shape().elem_count() */
+int cq_weight_set_shape(cq_weight *w, int64_t n, int64_t k);     /* check_shape, mod.rs:304-316   */
 /* QCudaStorage::quantize (cuda.rs:448-472): f32 [n*k] on the device -> this storage.  The
  * reference copies to the host and runs T::from_float there; here the same arithmetic runs in
  * a HIP kernel and yields the same bytes. */
@@ -130,6 +148,11 @@ size_t cq_workspace_bytes(const cq_weight *w, int64_t m, int flags);
  * x contiguous f32; m = product of the leading dims of the input tensor. */
 int cq_qmatmul(const cq_weight *w, const float *x_dev, int64_t m, float *y_dev, int flags,
                void *workspace_dev, size_t workspace_bytes, void *stream);
+/* The same with the weight's shape given at the call, exactly as QCudaStorage::fwd(&self, self_shape, ..)
+ * receives it (cuda.rs:478-499): [n, k] must cover the storage's elements, k % block_size == 0. */
+size_t cq_workspace_bytes_shaped(const cq_weight *w, int64_t n, int64_t k, int64_t m, int flags);
+int cq_qmatmul_shaped(const cq_weight *w, int64_t n, int64_t k, const float *x_dev, int64_t m, float *y_dev,
+                      int flags, void *workspace_dev, size_t workspace_bytes, void *stream);
 /* Debug/verification: the per-block integer dot products the f32 result is combined from
  * (k_quants.rs:1221-1241 for Q4K, :1418-1438 for Q5K, :1615-1633 for Q6K, :245-250 / :640-645 for Q4_0/Q8_0).
  * out_i[(r*n + c)*kb + b] = I_b; out_mn likewise = sum_j bsums_j*min_j (Q4K and Q5K, else NULL). */

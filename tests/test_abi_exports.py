@@ -18,6 +18,56 @@ def declared_functions():
     return sorted(set(names))
 
 
+def c_declarations():
+    """[(return type, name, [(type, name), ...])] of every function the header declares."""
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"^\s*#.*$", "", text, flags=re.M)
+    out = []
+    for ret, name, args in re.findall(r"([A-Za-z_][\w ]*?[\s\*]+)(cq_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", text, flags=re.S):
+        params = []
+        for a in " ".join(args.split()).split(","):
+            a = a.strip()
+            if a == "void" or not a:
+                continue
+            m = re.match(r"(.*?)(\w+)$", a)
+            params.append((m.group(1).strip(), m.group(2)))
+        out.append((" ".join(ret.split()), name, params))
+    return out
+
+
+_RUST_TYPES = {
+    "int": "c_int", "int64_t": "i64", "size_t": "usize", "float": "f32", "void": "()",
+    "const char *": "*const c_char", "const void *": "*const c_void", "void *": "*mut c_void",
+    "const float *": "*const f32", "float *": "*mut f32", "float *const *": "*const *mut f32",
+    "const int32_t *": "*const i32", "int32_t *": "*mut i32", "int64_t *": "*mut i64", "uint16_t *": "*mut u16",
+    "uint64_t *": "*mut u64", "double *": "*mut f64",
+    "cq_weight *": "*mut CqWeight", "const cq_weight *": "*const CqWeight", "cq_weight **": "*mut *mut CqWeight",
+    "const cq_weight *const *": "*const *const CqWeight",
+}
+
+
+def rust_signature(decl):
+    """The `pub fn` line a Rust sys-crate declares for one C declaration."""
+    ret, name, params = decl
+    args = ", ".join(f"{n}: {_RUST_TYPES[t]}" for t, n in params)
+    tail = "" if ret == "void" else f" -> {_RUST_TYPES[ret]}"
+    return f"pub fn {name}({args}){tail};"
+
+
+def test_integration_doc_binds_every_declared_symbol():
+    """The integration guide's `extern "C"` block (the sys-crate a maintainer adds) lists every entry point of
+    the header with the header's argument names and the matching Rust types."""
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    block = re.search(r'extern "C" \{(.*?)\n\}', text, flags=re.S).group(1)
+    got = {re.match(r"pub fn (cq_\w+)", " ".join(f.split())).group(1): " ".join(f.split()).replace("( ", "(")
+           for f in re.findall(r"pub fn cq_[^;]*;", block, flags=re.S)}
+    want = {d[1]: rust_signature(d) for d in c_declarations()}
+    assert sorted(got) == sorted(want)
+    for name in want:
+        assert got[name] == want[name], (got[name], want[name])
+
+
 @pytest.fixture(scope="module")
 def lib():
     from candle_amd import qhip
