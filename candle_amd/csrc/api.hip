@@ -123,6 +123,10 @@ static int weight_alloc(int dev, int dt, int64_t n, int64_t k, cq_weight **out) 
     w->p1 = (uint8_t *)w->base + o1;
     w->p2 = (uint8_t *)w->base + o2;
     w->p3 = (uint8_t *)w->base + o3;
+    // creating a weight is the set-up call every user of a device goes through: the scratch array of
+    // cq_qmatmul_static is looked up here, so that the first matmul on the device has nothing left to set up
+    // (a failure is reported by cq_qmatmul_static itself, which looks again)
+    (void)cq_static_scratch_ptr(dev);
     *out = w;
     return CQ_OK;
 }

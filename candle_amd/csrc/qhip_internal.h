@@ -158,6 +158,11 @@ hipError_t cq_launch_scatter_add(const float *y, const int32_t *row_ids, const f
 
 hipError_t cq_launch_fill_zero(float *p, int64_t count, hipStream_t s);
 
+// no_alloc.hip: device address of the static scratch array of cq_qmatmul_static on `dev` (the current
+// device); looked up once per device.  Weight creation calls it so that the first matmul on a device finds
+// the address cached.
+uint8_t *cq_static_scratch_ptr(int dev);
+
 #if defined(__HIPCC__)
 #include <hip/hip_ext.h>
 #include <atomic>

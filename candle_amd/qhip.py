@@ -28,7 +28,7 @@ EXPORTS = [
     "cq_qmatmul_grouped", "cq_silu_mul", "cq_moe_scatter_add", "cq_timing_arm", "cq_timing_elapsed_us",
     "cq_selfcheck_round", "cq_quantize_act_fused", "cq_qmatmul_fused", "cq_qmatmul_grouped_fused", "cq_qmatmul_multi",
     "cq_weight_zeros_flat", "cq_weight_create_flat", "cq_weight_elem_count", "cq_weight_set_shape",
-    "cq_workspace_bytes_shaped", "cq_qmatmul_shaped",
+    "cq_workspace_bytes_shaped", "cq_qmatmul_shaped", "cq_qmatmul_static",
 ]
 
 
@@ -89,6 +89,7 @@ def load():
     L.cq_weight_set_shape.argtypes = [vp, i64, i64]
     L.cq_workspace_bytes_shaped.restype = sz; L.cq_workspace_bytes_shaped.argtypes = [vp, i64, i64, i64, ci]
     L.cq_qmatmul_shaped.argtypes = [vp, i64, i64, vp, i64, vp, ci, vp, sz, vp]
+    L.cq_qmatmul_static.argtypes = [vp, vp, i64, vp, ci, vp]
     _lib = L
     return L
 

@@ -153,6 +153,17 @@ int cq_qmatmul(const cq_weight *w, const float *x_dev, int64_t m, float *y_dev, 
 size_t cq_workspace_bytes_shaped(const cq_weight *w, int64_t n, int64_t k, int64_t m, int flags);
 int cq_qmatmul_shaped(const cq_weight *w, int64_t n, int64_t k, const float *x_dev, int64_t m, float *y_dev,
                       int flags, void *workspace_dev, size_t workspace_bytes, void *stream);
+/* cq_qmatmul for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  No counterpart in the reference (which allocates its quantized
+ * activations per call, cuda.rs:249-252).  Same arguments and results as cq_qmatmul without the workspace:
+ * the quantized activations go to an array of CQ_STATIC_SCRATCH_BYTES that is part of the library's device
+ * code, so every GPU the library runs on holds that much until the process ends.  Calls that need more
+ * (cq_workspace_bytes(w, m, flags) > CQ_STATIC_SCRATCH_BYTES) fail with CQ_ERR_WORKSPACE.  The call itself
+ * allocates and frees nothing; the array's address is looked up when the first weight is created on a device.
+ * All calls on one GPU share the array: calls that overlap in time on one GPU (two streams, two host threads)
+ * race on it; calls in stream order do not. */
+#define CQ_STATIC_SCRATCH_BYTES (16u << 20)
+int cq_qmatmul_static(const cq_weight *w, const float *x_dev, int64_t m, float *y_dev, int flags, void *stream);
 /* Debug/verification: the per-block integer dot products the f32 result is combined from
  * (k_quants.rs:1221-1241 for Q4K, :1418-1438 for Q5K, :1615-1633 for Q6K, :245-250 / :640-645 for Q4_0/Q8_0).
  * out_i[(r*n + c)*kb + b] = I_b; out_mn likewise = sum_j bsums_j*min_j (Q4K and Q5K, else NULL). */
