@@ -48,6 +48,83 @@ def ggml_bytes(dtype: str, n: int, k: int) -> int:
     return n * k // blk * size
 
 
+def envelope() -> int:
+    """What one launch can reach on this device: an empty kernel (the fixed cost of a launch) and a pure
+    streaming read (16 bytes per lane and step, four steps in flight, nothing else) of the byte counts of the
+    decode launches, back to back eagerly and as a chain of 225 graph nodes like the decode step.  Every
+    launch of a chain reads a buffer of its own (4 GB in rotation: HBM, not the 256 MB Infinity Cache)."""
+    import ctypes as C
+
+    import torch
+
+    from candle_amd import build as qbuild
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    P = C.CDLL(qbuild.PROBE_LIB_PATH)
+    vp = C.c_void_p
+    P.cqp_empty.argtypes = [C.c_int, C.c_int, C.c_int, vp, vp]
+    P.cqp_stream_read.argtypes = [vp, C.c_size_t, C.c_int, C.c_int, C.c_int, vp, vp]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    pool = torch.full(((4 << 30) // 4,), 1, dtype=torch.int32, device=dev)
+    NODES = 225
+
+    def timed(launch, graph: bool):
+        """µs per launch of NODES launches, eagerly or as one graph replay (median of 7)."""
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            s = vp(side.cuda_stream)
+            for i in range(NODES):
+                launch(i, s)
+            torch.cuda.synchronize()
+            g = None
+            if graph:
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=side):
+                    for i in range(NODES):
+                        launch(i, s)
+            times = []
+            for _ in range(7):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                if g is not None:
+                    g.replay()
+                else:
+                    for i in range(NODES):
+                        launch(i, s)
+                e1.record()
+                torch.cuda.synchronize()
+                times.append(e0.elapsed_time(e1) * 1e3 / NODES)
+        return sorted(times)[len(times) // 2]
+
+    out = {"nodes_per_chain": NODES, "empty_kernel_us": {}, "stream_read": {}}
+    for grid, block, lds in ((256, 512, 0), (256, 512, 20480), (256, 256, 0), (256, 64, 0), (1, 64, 0), (2048, 256, 0)):
+        def launch(i, s, grid=grid, block=block, lds=lds):
+            P.cqp_empty(grid, block, lds, vp(sink.data_ptr()), s)
+        out["empty_kernel_us"][f"grid{grid}_block{block}_lds{lds}"] = {
+            "eager": round(timed(launch, False), 3), "graph": round(timed(launch, True), 3)}
+    # the byte counts of the decode launches: Q4_K 4096x4096, Q4_K 11008x4096, Q6_K 4096x11008, Q6_K 32000x4096
+    for name, nbytes in (("q4k_4096x4096", 9437184), ("q4k_11008x4096", 25362432), ("q6k_4096x11008", 36986880),
+                         ("q6k_32000x4096", 107520000)):
+        span = (nbytes + 4095) // 4096 * 4096
+        slots = pool.numel() * 4 // span
+        row = {"bytes": nbytes}
+        for grid, block, unroll in ((2048, 256, 4), (1024, 512, 4), (256, 512, 8)):
+            def launch(i, s, grid=grid, block=block, unroll=unroll):
+                P.cqp_stream_read(vp(pool.data_ptr() + (i % slots) * span), nbytes, grid, block, unroll,
+                                  vp(sink.data_ptr()), s)
+            for mode, graph in (("eager", False), ("graph", True)):
+                us = timed(launch, graph)
+                row[f"grid{grid}_block{block}_u{unroll}_{mode}_us"] = round(us, 3)
+                row[f"grid{grid}_block{block}_u{unroll}_{mode}_GBs"] = round(nbytes / us / 1e3, 1)
+        out["stream_read"][name] = row
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -62,7 +139,13 @@ def main() -> int:
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain device copy of 256 MiB three times (a kernel of known HBM traffic, to "
                          "calibrate FETCH_SIZE / WRITE_SIZE counters in a profiler run)")
+    ap.add_argument("--envelope", action="store_true",
+                    help="instead of the bench: time an empty kernel and a pure 16-byte-per-lane streaming read of the "
+                         "decode launches' sizes, eagerly and as a 225-node graph chain (what a single launch can reach "
+                         "on this device), and print that as one JSON line")
     args = ap.parse_args()
+    if args.envelope:
+        return envelope()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (one process, one MI355X); --gpus must be 1", file=sys.stderr)
         return 2

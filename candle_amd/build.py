@@ -35,13 +35,21 @@ def _compile(src: str) -> str:
     return obj
 
 
+# Measurement aid (bench.py --envelope): empty and streaming-read reference kernels, a library of its own.
+PROBE_SOURCE = "probe.hip"
+PROBE_LIB_PATH = os.path.join(LIB_DIR, "libcandle_qhip_probe.so")
+
+
 def build(verbose: bool = True) -> str:
     os.makedirs(LIB_DIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
-        objs = list(ex.map(_compile, SOURCES))
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES) + 1)) as ex:
+        objs = list(ex.map(_compile, SOURCES + [PROBE_SOURCE]))
+    probe_obj = objs.pop()
     subprocess.check_call(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs])
+    subprocess.check_call(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PROBE_LIB_PATH, probe_obj])
     if verbose:
         print("built", LIB_PATH)
+        print("built", PROBE_LIB_PATH)
     return LIB_PATH
 
 

@@ -27,6 +27,7 @@ typedef void __attribute__((address_space(3))) *lptr_t;
 
 constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
+constexpr int kMaxLds = 160 * 1024;   // LDS of a CU, which a single workgroup may take
 
 __device__ __forceinline__ uint32_t pk_mul_u16(uint32_t a, uint32_t b) {
     const us2 r = __builtin_bit_cast(us2, a) * __builtin_bit_cast(us2, b);
@@ -85,9 +86,12 @@ template <> struct WHead<CQ_DTYPE_Q4K> { uint32_t dd; uint4 rec; };   // d | dmi
 template <> struct WHead<CQ_DTYPE_Q5K> : WHead<CQ_DTYPE_Q4K> {};       // the same header plane
 template <> struct WHead<CQ_DTYPE_Q6K> { uint4 sc; uint32_t d; };     // re-packed scales (two per unit); d
 __device__ __forceinline__ void load_head(const cq_weight &w, int64_t blk, WHead<CQ_DTYPE_Q4K> &r) {
-    const uint32_t *h = (const uint32_t *)(w.p1 + blk * CQ_Q4K_HDR);
-    r.dd = h[0];
-    r.rec = make_uint4(h[1], h[2], h[3], h[4]);
+    // two loads (16 + 4 bytes; the 20-byte records are 4-byte aligned, which is all a global load needs)
+    typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+    const uint8_t *h = w.p1 + blk * CQ_Q4K_HDR;
+    const u32x4_a4 v = *(const u32x4_a4 *)h;
+    r.dd = v.x;
+    r.rec = make_uint4(v.y, v.z, v.w, *(const uint32_t *)(h + 16));
 }
 __device__ __forceinline__ void load_head(const cq_weight &w, int64_t blk, WHead<CQ_DTYPE_Q6K> &r) {
     r.sc = *(const uint4 *)(w.p2 + blk * 16);
@@ -300,6 +304,214 @@ __global__ void __launch_bounds__(kThreads) skinny_kernel(cq_weight w, cq_act_vi
     }
 }
 
+// ------------------------------------------------------------ resident-activation variant ----
+// The kernel above re-reads the activations once per 16 weight rows: with 16 activation rows that is more
+// bytes (from L2) than the weights themselves (16 K against 9 K per workgroup for Q4K), and the launch is bound
+// by it.  When the quantized activations of the call fit the LDS beside the weight buffers (4096 columns x 16
+// rows: 75 KiB) a launch of at most one workgroup per CU copies them once, each wave the K blocks it owns (sixteen
+// waves: one block each for 4096 columns, a single memory round trip), and then walks its share of the 16-row
+// weight tiles (tile t of workgroup g: g + t * G) streaming weights only.  The launcher takes it where every
+// workgroup has one tile (n <= 16 x the number of CUs); with more tiles per workgroup it measured no faster than
+// the kernel above, also with the next tile's weights copied ahead into a second buffer (NBUF == 2).
+//   per K block b  : act [RT][2 K-halves][8 rows][8 chunks] | d8 [8*RT] f32 | minp [8*RT][2][8] f16 (k4 types)
+//   per wave, block: weights of one tile (kWgt bytes), twice when NBUF == 2; a wave's first buffer of a tile also
+//                    carries its partial results of that tile (1 KiB per 16 activation rows)
+template <int DT, int RT> struct Res {
+    static constexpr int kWgt = Buf<DT, RT>::kWgt;
+    static constexpr int kActBlk = RT * 2048 + RT * 32 + (is_k4(DT) ? RT * 256 : 0);
+    static constexpr int oD8 = RT * 2048, oMin = oD8 + RT * 32;
+    static size_t bytes(int64_t kb, int nbuf) { return (size_t)kb * kActBlk + (size_t)kb * nbuf * kWgt; }
+};
+
+// Copies with one descriptor per plane, built once, and the position inside the plane as a 32-bit scalar offset
+// (the planes of a tensor this kernel takes are far below 4 GiB): two scalar instructions per copy instead of
+// rebuilding a descriptor from a 64-bit address for each.
+struct ResPlanes {
+    __amdgpu_buffer_rsrc_t wq, wh, w5, aq, ad, am;
+};
+__device__ __forceinline__ void dma16s(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff, uint8_t *lds) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lptr_t)lds, 16, (int)voff, (int)soff, 0, 0);
+}
+__device__ __forceinline__ void dma4s(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff, uint8_t *lds) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lptr_t)lds, 4, (int)voff, (int)soff, 0, 0);
+}
+
+// Issues the copies of the weights of the tile starting at row n_tile for K block b into `wl`.
+template <int DT>
+__device__ __forceinline__ void res_issue_weights(uint8_t *__restrict__ wl, const ResPlanes &pl, uint32_t n_tile, uint32_t b,
+                                                  uint32_t kb, uint32_t wq_off, uint32_t wh_off, uint32_t w5_off, int lane) {
+    const uint32_t blk = n_tile * kb + b;
+    dma16s(pl.wq, wq_off, blk * 128u, wl);
+    dma16s(pl.wq, wq_off, blk * 128u + kb * 1024u, wl + 1024);
+    if (DT == CQ_DTYPE_Q6K) dma16s(pl.wh, wh_off, blk * 64u, wl + 2048);
+    if (DT == CQ_DTYPE_Q5K && lane < 32) dma16s(pl.w5, w5_off, blk * 32u, wl + 2048);
+}
+
+// One K block of one tile: unpack the weights in `wl`, contract with the resident activation slice `act`.
+template <int DT, int RT, int NT>
+__device__ __forceinline__ void res_block(const uint8_t *__restrict__ wl, const uint8_t *__restrict__ act, int lane,
+                                          const WHead<DT> &head, const uint32_t (&a_col)[NT][2], v4f (&out)[NT]) {
+    typedef Res<DT, RT> R;
+    constexpr bool MINS = is_k4(DT);
+    constexpr int SHIFT = DT == CQ_DTYPE_Q4K ? 3 : 7;
+    const uint32_t r = lane & 15, kq = lane >> 4;
+    v4i bl[4], bh[4];
+    float dw;
+    v8h wmin;
+    block_unpack(wl, lane, head, bl, bh, dw, wmin);
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const v4f d8 = *(const v4f *)(act + R::oD8 + (t * 16 + 4 * kq < 8u * RT ? t * 16 + 4 * kq : 0) * 4);
+        if (MINS) {
+            const uint32_t row = t * 16 + r < 8u * RT ? t * 16 + r : 8u * RT - 1;
+            const v8h ma = *(const v8h *)(act + R::oMin + row * 32 + (kq >> 1) * 16);
+            out[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ma, wmin, out[t], 0, 0, 0);
+        }
+        v4i acc_lo = {0, 0, 0, 0}, acc_hi = {0, 0, 0, 0};
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            const v4i av = *(const v4i *)(act + a_col[t][s & 1] + (s >> 1) * 1024);
+            acc_lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bl[s], acc_lo, 0, 0, 0);
+            acc_hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bh[s], acc_hi, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int I = (acc_hi[i] << SHIFT) + acc_lo[i];
+            out[t][i] = __builtin_fmaf((float)I * dw, d8[i], out[t][i]);
+        }
+    }
+}
+
+// m <= 8 * RT activation rows (the workspace pads rows, so whole groups are copied); n % 16 == 0; at most
+// kMaxBpw K blocks per wave.  `tiles` = n / 16, dealt to the gridDim.x workgroups in turn.
+constexpr int kMaxBpw = 4;
+template <int DT, int RT, int kWaves, int NBUF>
+__global__ void __launch_bounds__(kWaves * 64) skinny_resident_kernel(cq_weight w, cq_act_view a, int64_t m,
+                                                                      float *__restrict__ y) {
+    typedef Res<DT, RT> R;
+    constexpr bool MINS = is_k4(DT);
+    constexpr int NT = (RT + 1) / 2;   // 16-row tiles of activation rows
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t r = lane & 15, kq = lane >> 4;
+    const int64_t k = w.k, kb = w.k >> 8;
+    const int64_t tiles = w.n / 16;
+    uint8_t *wgt_base = smem + kb * R::kActBlk;
+
+    const uint32_t r8 = lane >> 3, c8 = lane & 7;
+    const uint32_t act_off = r8 * (uint32_t)k + ((c8 ^ r8) << 4);
+    const uint32_t wq_off = r8 * (uint32_t)kb * 128u + ((c8 ^ r8) << 4);
+    const uint32_t r16 = lane >> 2, c4 = lane & 3;
+    const uint32_t wh_off = r16 * (uint32_t)kb * 64u + ((c4 ^ ((r16 >> 1) & 3)) << 4);
+    const uint32_t w5_off = (lane >> 1) * (uint32_t)kb * 32u + (lane & 1) * 16u;
+    uint32_t a_col[NT][2];
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const uint32_t row = t * 16 + r < 8u * RT ? t * 16 + r : 8u * RT - 1;
+#pragma unroll
+        for (uint32_t e = 0; e < 2; e++)
+            a_col[t][e] = (row >> 3) * 2048u + (row & 7) * 128u + (((4 * e + kq) ^ (row & 7)) << 4);
+    }
+    ResPlanes pl;
+    pl.wq = wave_rsrc(w.p0);
+    pl.wh = wave_rsrc(w.p1);
+    pl.w5 = wave_rsrc(w.p2);
+    pl.aq = wave_rsrc(a.qs);
+    pl.ad = wave_rsrc(a.dT);
+    pl.am = wave_rsrc(a.minp);
+    const uint32_t kb32 = (uint32_t)kb, k32 = (uint32_t)k, mstr = (uint32_t)a.m_stride;
+    // ---- the wave's K blocks: the small fields of the first tile's weights (registers; requested first, they are
+    // what the unpacking starts with), activation slices once, weights of the first tile
+    int64_t tile = blockIdx.x;
+    WHead<DT> head[kMaxBpw];
+#pragma unroll
+    for (int j = 0; j < kMaxBpw; j++) {
+        const int64_t b = wave + (int64_t)j * kWaves;
+        if (b < kb && tile < tiles) load_head(w, (tile * 16 + r) * kb + b, head[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < kMaxBpw; j++) {
+        const uint32_t b = (uint32_t)wave + (uint32_t)j * kWaves;
+        if (b < kb32) {
+            uint8_t *act = smem + b * R::kActBlk;
+#pragma unroll
+            for (int i = 0; i < 2 * RT; i++) {
+                const uint32_t rg = i >> 1, kh = i & 1;
+                dma16s(pl.aq, act_off, rg * 8u * k32 + b * 256u + kh * 128u, act + i * 1024);
+            }
+            if (lane < 8 * RT) dma4s(pl.ad, lane * 4u, b * mstr * 4u, act + R::oD8);
+            if (MINS && lane < 16 * RT) dma16s(pl.am, lane * 16u, b * mstr * 32u, act + R::oMin);
+            if (tile < tiles)
+                res_issue_weights<DT>(wgt_base + (b * NBUF) * R::kWgt, pl, (uint32_t)tile * 16u, b, kb32, wq_off, wh_off, w5_off, lane);
+        }
+    }
+    int par = 0;
+    for (; tile < tiles; tile += gridDim.x) {
+        const int64_t n_tile = tile * 16, next = tile + gridDim.x;
+        __builtin_amdgcn_s_waitcnt(0);   // this tile's weights (and, the first time, the activations) have landed
+        if (NBUF == 2 && next < tiles) {
+#pragma unroll
+            for (int j = 0; j < kMaxBpw; j++) {
+                const int64_t b = wave + (int64_t)j * kWaves;
+                if (b < kb)
+                    res_issue_weights<DT>(wgt_base + (b * NBUF + (par ^ 1)) * R::kWgt, pl, (uint32_t)next * 16u, (uint32_t)b, kb32,
+                                          wq_off, wh_off, w5_off, lane);
+            }
+        }
+        v4f out[NT];
+#pragma unroll
+        for (int t = 0; t < NT; t++) out[t] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int j = 0; j < kMaxBpw; j++) {
+            const int64_t b = wave + (int64_t)j * kWaves;
+            if (b < kb)
+                res_block<DT, RT, NT>(wgt_base + (b * NBUF + (NBUF == 2 ? par : 0)) * R::kWgt, smem + b * R::kActBlk, lane,
+                                      head[j], a_col, out);
+        }
+        // ---- sum the waves' partial tiles in wave order (through the wave's first weight buffer of this tile)
+        uint8_t *part = wgt_base + ((int64_t)wave * NBUF + (NBUF == 2 ? par : 0)) * R::kWgt;
+        if (wave < kb) {   // (a wave without a K block has no buffer and nothing to add)
+#pragma unroll
+            for (int t = 0; t < NT; t++) *(v4f *)(part + t * 1024 + lane * 16) = out[t];
+        }
+        __syncthreads();
+        if (wave < NT) {
+            v4f s = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+            const int64_t nw = kb < kWaves ? kb : kWaves;   // waves that own a block
+            for (int64_t o = 0; o < nw; o++) {
+                const v4f p = *(const v4f *)(wgt_base + (o * NBUF + (NBUF == 2 ? par : 0)) * R::kWgt + wave * 1024 + lane * 16);
+                s += p;
+            }
+            const int64_t col = n_tile + r;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int64_t row = wave * 16 + kq * 4 + i;
+                if (row < m) y[row * w.n + col] = s[i];
+            }
+        }
+        if (NBUF == 1 && next < tiles) {
+            __syncthreads();   // the partial results have been read: the buffers take the next tile's weights
+#pragma unroll
+            for (int j = 0; j < kMaxBpw; j++) {
+                const int64_t b = wave + (int64_t)j * kWaves;
+                if (b < kb)
+                    res_issue_weights<DT>(wgt_base + b * R::kWgt, pl, (uint32_t)next * 16u, (uint32_t)b, kb32, wq_off, wh_off, w5_off, lane);
+            }
+        } else if (NBUF == 2) {
+            __syncthreads();   // ... before the tile after the next one is copied over them
+        }
+        if (next < tiles) {
+#pragma unroll
+            for (int j = 0; j < kMaxBpw; j++) {
+                const int64_t b = wave + (int64_t)j * kWaves;
+                if (b < kb) load_head(w, (next * 16 + r) * kb + b, head[j]);
+            }
+        }
+        par ^= 1;
+    }
+}
+
 // ---------------------------------------------------- Q8_0 / Q4_0 weights x Q8_0 activations ----
 // The same work split for 32-element blocks (k_quants.rs:618-649, :224-254: sumf += sumi * d_w *
 // d_x per block).  Q8_0 weights are int8 already and Q4_0 weights are one mask away from it, so the
@@ -480,6 +692,45 @@ hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hip
     return hipSuccess;
 }
 
+
+// The resident-activation kernel where the call's activations and the weight buffers fit the LDS (see above).
+template <int DT, int RT, int NW, int NBUF>
+hipError_t launch_res_inst(const cq_weight *w, cq_act_view a, int64_t m, float *y, size_t lds, unsigned grid, hipStream_t s) {
+    if (hipError_t e = cq_ensure_lds<skinny_resident_kernel<DT, RT, NW, NBUF>>(w->dev, lds); e != hipSuccess) return e;
+    CQ_LAUNCH((skinny_resident_kernel<DT, RT, NW, NBUF>), grid, NW * 64, lds, s, *w, a, m, y);
+    return hipGetLastError();
+}
+template <int DT, int RT>
+bool launch_res_rt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s, hipError_t *err) {
+    const int64_t kb = w->k >> 8, tiles = w->n / 16;
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (cus <= 0) cus = 256;
+    const unsigned grid = (unsigned)(tiles < cus ? tiles : cus);
+    const bool sixteen = kb > 8;
+    if (kb > (sixteen ? 16 : 8) * kMaxBpw) return false;
+    // the copies address every plane with 32-bit byte offsets
+    if ((uint64_t)w->n * (uint64_t)kb * 128u >= (1ull << 32) || (uint64_t)a.m_stride * (uint64_t)w->k >= (1ull << 32)) return false;
+    // Measured (Q4K, 16 rows, matmul kernel alone): 4096 x 4096, one tile per workgroup, 5.95 us against 6.5 us for the
+    // kernel that copies activations per block; 11008 x 4096, two or three tiles per workgroup, 12.7 against 12.5 us
+    // (also with the next tile's weights copied ahead into a second buffer): taken where every workgroup has one tile.
+    if (tiles > grid) return false;
+    const size_t one = Res<DT, RT>::bytes(kb, 1);
+    if (one <= (size_t)kMaxLds) {
+        *err = sixteen ? launch_res_inst<DT, RT, 16, 1>(w, a, m, y, one, grid, s) : launch_res_inst<DT, RT, 8, 1>(w, a, m, y, one, grid, s);
+        return true;
+    }
+    return false;
+}
+template <int DT>
+bool launch_res(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s, hipError_t *err) {
+    if (m <= 8) return launch_res_rt<DT, 1>(w, a, m, y, s, err);
+    if (m <= 16) return launch_res_rt<DT, 2>(w, a, m, y, s, err);
+    if (m <= 24) return launch_res_rt<DT, 3>(w, a, m, y, s, err);
+    if (m <= 32) return launch_res_rt<DT, 4>(w, a, m, y, s, err);
+    return false;
+}
+
 }  // namespace
 
 bool cq_skinny_supported(const cq_weight *w, int act_dtype) {
@@ -495,6 +746,12 @@ hipError_t cq_launch_skinny(const cq_weight *w, cq_act_view a, int act_dtype, in
     if (a.m_stride < (m + 31) / 32 * 32) return hipErrorInvalidValue;   // whole 8-row groups are copied
     if (w->dtype == CQ_DTYPE_Q8_0) return launch_blk32<CQ_DTYPE_Q8_0>(w, a, m, y, s);
     if (w->dtype == CQ_DTYPE_Q4_0) return launch_blk32<CQ_DTYPE_Q4_0>(w, a, m, y, s);
+    hipError_t e = hipSuccess;
+#ifndef CQ_EXP_NO_RESIDENT
+    if (w->dtype == CQ_DTYPE_Q4K && launch_res<CQ_DTYPE_Q4K>(w, a, m, y, s, &e)) return e;
+    if (w->dtype == CQ_DTYPE_Q5K && launch_res<CQ_DTYPE_Q5K>(w, a, m, y, s, &e)) return e;
+    if (w->dtype == CQ_DTYPE_Q6K && launch_res<CQ_DTYPE_Q6K>(w, a, m, y, s, &e)) return e;
+#endif
     if (w->dtype == CQ_DTYPE_Q4K) return launch_dt<CQ_DTYPE_Q4K>(w, a, m, y, s);
     if (w->dtype == CQ_DTYPE_Q5K) return launch_dt<CQ_DTYPE_Q5K>(w, a, m, y, s);
     return launch_dt<CQ_DTYPE_Q6K>(w, a, m, y, s);
