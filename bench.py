@@ -317,6 +317,7 @@ def main() -> int:
 
     # whole calls (activation quantizer + GEMM) on both shapes of configs[3] and on the attention shape
     whole_calls = {}
+    gemm_cases = {}
     if not args.no_extras:
         for name, dt, (wn, wk) in (("q4k_14336x4096", qhip.Q4K, (14336, 4096)), ("q4k_4096x14336", qhip.Q4K, (4096, 14336)),
                                    ("q6k_14336x4096", qhip.Q6K, (14336, 4096)), ("q6k_4096x14336", qhip.Q6K, (4096, 14336)),
@@ -341,6 +342,30 @@ def main() -> int:
             w1.record()
             torch.cuda.synchronize()
             whole_calls[name] = round(w0.elapsed_time(w1) * 1e3 / 40, 1)
+            if name != "q4k_4096x4096":
+                # the matmul kernel alone (library event pair), as TOPS and as a fraction of the int8 MFMA peak
+                k_us = sorted(qhip.timed_kernel_us(whole) for _ in range(5))[2]
+                case = {"kernel_us": round(k_us, 2), "tops": round(2.0 * gm * wk * wn / (k_us * 1e-6) / 1e12, 1)}
+                case["frac_of_int8_mfma_peak"] = round(case["tops"] / 5000.0, 4)
+                # the same product with the activations quantized to Q8_1 (the reference's CUDA formulation): its cost and
+                # its distance from the CPU formulation's result
+                q81_ws = torch.empty(L.cq_workspace_bytes(wq.handle, gm, qhip.FLAG_ACT_Q8_1), dtype=torch.uint8, device=dev)
+                y81 = torch.empty_like(wy)
+
+                def whole81():
+                    qhip.check(L.cq_qmatmul(wq.handle, C.c_void_p(wx.data_ptr()), gm, C.c_void_p(y81.data_ptr()),
+                                            qhip.FLAG_ACT_Q8_1, C.c_void_p(q81_ws.data_ptr()), q81_ws.numel(),
+                                            C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+                whole81()
+                w0.record()
+                for _ in range(3):
+                    whole81()
+                w1.record()
+                torch.cuda.synchronize()
+                case["q8_1_variant_us"] = round(w0.elapsed_time(w1) * 1e3 / 3, 1)
+                case["q8_1_variant_rel_l2_vs_q8k"] = float(f"{float((y81 - wy).norm() / wy.norm()):.3e}")
+                gemm_cases[name] = case
+                del q81_ws, y81
             del wq, wx, wy, wws
 
     # ---- the same step with the model's neighbours of each matmul (reported beside the headline) ----
@@ -734,6 +759,7 @@ def main() -> int:
             "peak_tops": 5000.0,
             "frac_of_int8_mfma_peak": round(gemm_tops / 5000.0, 4),
             "whole_call_us_m512": whole_calls or None,
+            "configs3_cases": gemm_cases or None,
         },
     }
 

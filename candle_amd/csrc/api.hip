@@ -417,6 +417,20 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
     const int act = act_dtype_for(w, flags);
     CQ_HIP_CHECK(hipSetDevice(w->dev));
     hipStream_t s = (hipStream_t)stream;
+    if (flags & CQ_FLAG_ACT_Q8_1) {
+        // the reference's CUDA formulation (cuda.rs:298-365): activations to Q8_1, one dot-product kernel for every row count
+        if (act != CQ_DTYPE_Q8_1 || !cq_matmul_q8_1_supported(w))
+            return cq_set_error(CQ_ERR_UNSUPPORTED, "Q8_1 activations are for Q4K and Q6K weights with rows that fit the LDS (dtype %d, k = %lld)",
+                                w->dtype, (long long)w->k);
+        if (flags & ~(CQ_FLAG_ACT_Q8_1 | CQ_FLAG_REUSE_ACT))
+            return cq_set_error(CQ_ERR_INVALID, "CQ_FLAG_ACT_Q8_1 combines with CQ_FLAG_REUSE_ACT only");
+        cq_act_view v;
+        act_ws_layout(act, m, w->k, (uint8_t *)ws, &v);
+        if (!(flags & CQ_FLAG_REUSE_ACT))
+            CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, nullptr, m, w->k, pre, v, cq_no_clear(), s));
+        CQ_HIP_CHECK(cq_launch_matmul_q8_1(w, v, m, y_dev, s));
+        return CQ_OK;
+    }
     // In the one-launch kernels every workgroup reads x (and aux) in its prologue while others already store y:
     // an output that overlaps an input goes through the quantizer launch instead, which has read all of x
     // before the matmul kernel writes anything.

@@ -982,6 +982,109 @@ __global__ void __launch_bounds__(kStagedThreads) staged_kernel(cq_weight w, cq_
     }
 }
 
+// ------------------------------------------------- K-quant weights x Q8_1 activations ----
+// The formulation of the reference's CUDA arm (mul_mat_via_q8_1, quantized/cuda.rs:298-365; dot bodies
+// candle-kernels/src/quantized.cu:2141-2166 for Q4K and :2258-2281 for Q6K) with the activations quantized by the CPU
+// rule of BlockQ8_1::from_float (k_quants.rs:665-691):
+//   Q4K: per block  d * sum_j d8_j * float(sc_j * dot_j)  -  dmin * sum_j s8_j * float(m_j)      (j: 32-element sub-blocks)
+//   Q6K: per block  d * sum_j float(sc_j) * (d8_{j/2} * float(dot_j))                            (j: 16-element groups)
+// with d8 / s8 the scale and the `s` field of the activation's 32-element Q8_1 block.  The integers (dot_j, sc_j * dot_j)
+// are exact; the f32 sums run per lane and then over the wave, not in the reference's block order.
+// LDS image of one activation row: the int8 planes of the Q8K image (piece_off), then per unit the two block
+// scales {d8, d8'} and, for Q4K, the two `s` values, as f32.
+template <int DT> __host__ __device__ constexpr size_t q81_row_bytes(int64_t k) {
+    return (size_t)k + (size_t)(k / Geo<DT>::kElems) * (DT == CQ_DTYPE_Q4K ? 16 : 8);
+}
+
+template <int DT, int MB>
+__global__ void __launch_bounds__(kStagedThreads) q81_kernel(cq_weight w, cq_act_view a, int64_t m0, int64_t m,
+                                                             int rows_per_wg, float *__restrict__ y) {
+    static_assert(DT == CQ_DTYPE_Q4K || DT == CQ_DTYPE_Q6K, "Q4K and Q6K only");
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int64_t k = w.k;
+    const uint32_t units = (uint32_t)(k / Geo<DT>::kElems);
+    const uint32_t row_bytes = (uint32_t)q81_row_bytes<DT>(k);
+    const int64_t nb32 = k / 32;
+    // ---- stage MB quantized rows (rows past the last one repeat it; their results are not stored)
+    for (int i = 0; i < MB; i++) {
+        const int64_t src = m0 + i < m ? m0 + i : m - 1;
+        LdsRow r;
+        r.lo = i * row_bytes;
+        r.hi = r.lo + units * 16;
+        const int4 *q = (const int4 *)(a.qs + src * k);
+        for (int piece = threadIdx.x; piece < (int)(k / 16); piece += kStagedThreads)
+            lds_put<int4>(smem, piece_off<DT>(r, piece, units), q[piece]);
+        const uint32_t sc_off = i * row_bytes + (uint32_t)k;
+        for (uint32_t u = threadIdx.x; u < units; u += kStagedThreads) {
+            if (DT == CQ_DTYPE_Q4K) {
+                // unit u = sub-blocks 2u and 2u + 1 = Q8_1 blocks 2u, 2u + 1
+                const float2 d = *(const float2 *)(a.d + src * nb32 + 2 * u);
+                const uint32_t s2 = *(const uint32_t *)(a.s16 + src * nb32 + 2 * u);
+                lds_put<float4>(smem, sc_off + 16 * u, make_float4(d.x, d.y, cq_h2f((uint16_t)(s2 & 0xffff)), cq_h2f((uint16_t)(s2 >> 16))));
+            } else {
+                // unit p = 4h + 2t + i of a weight block: the low nibbles are elements 128h + 32t + 16i + [0, 16) of the
+                // block, the high nibbles those 64 further on: Q8_1 blocks 4h + t and 4h + t + 2 of the block's eight
+                const uint32_t blk = u >> 3, p = u & 7, q = 4 * (p >> 2) + ((p >> 1) & 1);
+                const float *d = a.d + src * nb32 + 8 * blk + q;
+                lds_put<float2>(smem, sc_off + 8 * u, make_float2(d[0], d[2]));
+            }
+        }
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t row_begin = (int64_t)blockIdx.x * rows_per_wg;
+    const int64_t row_end = row_begin + rows_per_wg < w.n ? row_begin + rows_per_wg : w.n;
+    for (int64_t row = row_begin + wave; row < row_end; row += kStagedThreads / 64) {
+        float acc[MB];
+#pragma unroll
+        for (int i = 0; i < MB; i++) acc[i] = 0.0f;
+        for (uint32_t u = lane; u < units; u += 64) {
+            UnitRaw<DT> raw;
+            load_unit<DT>(w, row, units, u, raw);
+            UnitW<DT> uw;
+            decode_unit<DT>(raw, lane & 7, uw);
+            if (DT == CQ_DTYPE_Q6K) {
+                // quants 0..63 -> q - 32 as int8, byte-wise (no carry between bytes: q + 0x60 < 0x100)
+#pragma unroll
+                for (int x = 0; x < 4; x++) {
+                    uw.lo[x] = (uw.lo[x] + 0x60606060u) ^ 0x80808080u;
+                    uw.hi[x] = (uw.hi[x] + 0x60606060u) ^ 0x80808080u;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < MB; i++) {
+                const uint32_t base = i * row_bytes;
+                if (DT == CQ_DTYPE_Q4K) {
+                    const uint32_t plane = units * 16, at = base + u * 16;
+                    const int4 a0 = lds_get<int4>(smem, at), a1 = lds_get<int4>(smem, at + plane);
+                    const int4 a2 = lds_get<int4>(smem, at + 2 * plane), a3 = lds_get<int4>(smem, at + 3 * plane);
+                    const int dlo = dot16(uw.lo, a0) + dot16(uw.lo + 4, a1);
+                    const int dhi = dot16(uw.hi, a2) + dot16(uw.hi + 4, a3);
+                    const float4 sc = lds_get<float4>(smem, base + (uint32_t)k + 16 * u);   // {d8, d8', s8, s8'}
+                    float sd = sc.x * (float)(dlo * uw.sc_lo);
+                    sd += sc.y * (float)(dhi * uw.sc_hi);
+                    float sm = sc.z * (float)uw.mn_lo;
+                    sm += sc.w * (float)uw.mn_hi;
+                    acc[i] += uw.dw * sd - uw.dmin * sm;
+                } else {
+                    const int4 alo = lds_get<int4>(smem, base + u * 16);
+                    const int4 ahi = lds_get<int4>(smem, base + units * 16 + u * 16);
+                    const int dlo = dot16(uw.lo, alo), dhi = dot16(uw.hi, ahi);
+                    const float2 d8 = lds_get<float2>(smem, base + (uint32_t)k + 8 * u);
+                    float sd = (float)uw.sc_lo * (d8.x * (float)dlo);
+                    sd += (float)uw.sc_hi * (d8.y * (float)dhi);
+                    acc[i] += uw.dw * sd;
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < MB; i++) {
+            const float sum = wave_sum(acc[i]);
+            if (lane == 0 && m0 + i < m) y[(m0 + i) * w.n + row] = sum;
+        }
+    }
+}
+
 // Per-block integer dots for verification: same unit arithmetic as the kernels above.
 template <int DT>
 __global__ void __launch_bounds__(kStagedThreads) int_dots_kernel(cq_weight w, cq_act_view a, int64_t m0,
@@ -1364,6 +1467,47 @@ hipError_t cq_launch_matvec(const cq_weight *w, cq_act_view a, int act_dtype, in
     case CQ_DTYPE_Q6K: return launch_staged<CQ_DTYPE_Q6K>(w, a, m, y, s);
     default: return hipErrorInvalidValue;
     }
+}
+
+namespace {
+template <int DT, int MB>
+hipError_t launch_q81_mb(const cq_weight *w, cq_act_view a, int64_t m0, int64_t m, float *y, hipStream_t s) {
+    const size_t lds = q81_row_bytes<DT>(w->k) * MB;
+    if (hipError_t e = cq_ensure_lds<q81_kernel<DT, MB>>(w->dev, lds); e != hipSuccess) return e;
+    const int rpw = pick_rows_per_wg(w->n);
+    const unsigned grid = (unsigned)((w->n + rpw - 1) / rpw);
+    CQ_LAUNCH((q81_kernel<DT, MB>), grid, kStagedThreads, lds, s, *w, a, m0, m, rpw, y);
+    return hipGetLastError();
+}
+template <int DT> hipError_t launch_q81(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
+    // eight activation rows per pass over the weights when their images fit the LDS, else four, two, one
+    int mb = 8;
+    while (mb > 1 && q81_row_bytes<DT>(w->k) * mb > kMaxRowLds) mb >>= 1;
+    if (q81_row_bytes<DT>(w->k) > kMaxRowLds) return hipErrorInvalidValue;
+    for (int64_t m0 = 0; m0 < m; m0 += mb) {
+        const int64_t left = m - m0;
+        hipError_t e;
+        if (mb == 8 && left > 4) e = launch_q81_mb<DT, 8>(w, a, m0, m, y, s);
+        else if (mb >= 4 && left > 2) e = launch_q81_mb<DT, 4>(w, a, m0, m, y, s);
+        else if (mb >= 2 && left > 1) e = launch_q81_mb<DT, 2>(w, a, m0, m, y, s);
+        else e = launch_q81_mb<DT, 1>(w, a, m0, m, y, s);
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+}  // namespace
+
+bool cq_matmul_q8_1_supported(const cq_weight *w) {
+    if (w->dtype == CQ_DTYPE_Q4K) return q81_row_bytes<CQ_DTYPE_Q4K>(w->k) <= kMaxRowLds;
+    if (w->dtype == CQ_DTYPE_Q6K) return q81_row_bytes<CQ_DTYPE_Q6K>(w->k) <= kMaxRowLds;
+    return false;
+}
+
+hipError_t cq_launch_matmul_q8_1(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
+    if (m == 0 || w->n == 0) return hipSuccess;
+    if (w->dtype == CQ_DTYPE_Q4K) return launch_q81<CQ_DTYPE_Q4K>(w, a, m, y, s);
+    if (w->dtype == CQ_DTYPE_Q6K) return launch_q81<CQ_DTYPE_Q6K>(w, a, m, y, s);
+    return hipErrorInvalidValue;
 }
 
 hipError_t cq_launch_int_dots(const cq_weight *w, cq_act_view a, int64_t m, int32_t *out_i, int32_t *out_mn,

@@ -121,6 +121,9 @@ hipError_t cq_launch_matvec(const cq_weight *w, cq_act_view a, int act_dtype, in
 hipError_t cq_launch_int_dots(const cq_weight *w, cq_act_view a, int64_t m, int32_t *out_i, int32_t *out_mn,
                               hipStream_t s);
 bool cq_matvec_row_fits(const cq_weight *w);          // K small enough for the dot-product kernels (one quantized row in LDS)
+// Q4K / Q6K weights with Q8_1 activations (the reference's CUDA formulation), any number of rows
+bool cq_matmul_q8_1_supported(const cq_weight *w);
+hipError_t cq_launch_matmul_q8_1(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s);
 bool cq_matvec_fused_supported(const cq_weight *w);   // m == 1: quantizer fused into the matvec launch
 hipError_t cq_launch_matvec_fused(const cq_weight *w, const float *x, cq_pre pre, float *y, hipStream_t s);
 // 2 <= m <= 4 rows in the one-launch kernel (short rows only)
