@@ -591,6 +591,31 @@ extern "C" int cq_qmatmul_int_dots(const cq_weight *w, const float *x_dev, int64
     return CQ_OK;
 }
 
+extern "C" int cq_qmatmul_int_dots_mfma(const cq_weight *w, const float *x_dev, int64_t m, int kernel, int32_t *out_i,
+                                        float *out_mn, void *ws, size_t ws_bytes, void *stream) {
+    const size_t need = cq_workspace_bytes(w, m, 0);
+    int rc = check_matmul_args(w, x_dev, m, out_i, ws, ws_bytes, need);
+    if (rc || m == 0 || w->n == 0 || w->k == 0) return rc;
+    const int act = cq_vec_dot_type(w->dtype);
+    const bool kquant = w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q5K || w->dtype == CQ_DTYPE_Q6K;
+    bool ok = false;
+    if (kernel == CQ_MFMA_SKINNY) ok = cq_skinny_supported(w, act);
+    else if (kernel == CQ_MFMA_TILE) ok = kquant ? cq_gemm_supported(w, m, act) : m > 32 && cq_gemm32_supported(w, act);   // as cq_qmatmul
+    else return cq_set_error(CQ_ERR_INVALID, "kernel must be CQ_MFMA_SKINNY or CQ_MFMA_TILE");
+    if (!ok) return cq_set_error(CQ_ERR_UNSUPPORTED, "that kernel does not take this weight (dtype %d, %lld x %lld) with %lld rows", w->dtype,
+                                 (long long)w->n, (long long)w->k, (long long)m);
+    CQ_HIP_CHECK(hipSetDevice(w->dev));
+    hipStream_t s = (hipStream_t)stream;
+    cq_act_view v;
+    act_ws_layout(act, m, w->k, (uint8_t *)ws, &v);
+    CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, nullptr, m, w->k, cq_no_pre(), v, cq_no_clear(), s));
+    const cq_mfma_dump d{out_i, (w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q5K) ? out_mn : nullptr};
+    if (kernel == CQ_MFMA_SKINNY) CQ_HIP_CHECK(cq_launch_skinny_dump(w, v, act, m, d, s));
+    else if (kquant) CQ_HIP_CHECK(cq_launch_gemm_dump(w, v, act, m, d, s));
+    else CQ_HIP_CHECK(cq_launch_gemm32_dump(w, v, act, m, d, s));
+    return CQ_OK;
+}
+
 // ------------------------------------------------------------------- MoE ----
 extern "C" size_t cq_grouped_workspace_bytes(const cq_weight *const *experts, int n_experts, int64_t total_rows,
                                              int flags) {

@@ -184,15 +184,25 @@ __device__ __forceinline__ void load_head(const cq_weight &w, int64_t blk, WHead
     r.d = ((const uint16_t *)w.p3)[blk];
 }
 
+// Verification build (DUMP): where a lane's integers of the current block go, and how many of the tile rows exist.
+struct DumpLane {
+    int32_t *i;     // element (row m0, the lane's weight row, block b) of cq_mfma_dump::i
+    float *mn;      // the same of cq_mfma_dump::mn, or null
+    int64_t rs;     // elements between two activation rows
+    int64_t rows;   // rows m0 .. m0 + rows - 1 exist
+};
+
 // One block for this wave's 32 weight rows against the MT activation tiles in `cur`, as a
 // hand-laid software pipeline of 8*(MT+1) steps.  Step (t, s) issues the two int8 MFMAs of tile t,
 // K-slice s, and, in their shadow, the scaling of two of the sixteen integers of tile t-1 (VALU);
 // LDS reads run two steps ahead.  The accumulator pair alternates between two register sets.  A
 // scheduling barrier after every step keeps the compiler from hoisting all MFMAs to the front,
 // which would need MT accumulator sets at once.
-template <int DT, int MT, int T0, int T1, int SHIFT, bool HALF>
+// DUMP: instead of scaling them into `out`, the block integers I (and the min term as the f16 MFMA delivers
+// it, from a zero accumulator) are stored through `dl`.
+template <int DT, int MT, int T0, int T1, int SHIFT, bool HALF, bool DUMP>
 __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, const v4i (&bl)[8], const v4i (&bh)[8],
-                                          float dw, v8h wmin, int lane, v16f (&out)[MT]) {
+                                          float dw, v8h wmin, int lane, v16f (&out)[MT], const DumpLane &dl) {
     typedef Tile<DT, MT> T;
     if constexpr (T0 >= T1) return;
     constexpr bool MINS = is_k4(DT);
@@ -220,12 +230,22 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, 
         if (q + 2 < T1 * 8) a[(q + 2) % 3] = afrag(q + 2);
         if (t < T1) {
             if (s == 0) {
-                if (MINS) {
+                if (MINS && !DUMP) {
                     // min term: out -= sum_j (dmin*min_j) * (d8*bsum32_j).  K-slots 0..7 carry piece 1
                     // of the weight factor, slots 8..15 piece 2; the activation operand carries one of
                     // its pieces in both halves.
                     out[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma1, wmin, out[t], 0, 0, 0);
                     out[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma2, wmin, out[t], 0, 0, 0);
+                }
+                if (MINS && DUMP && dl.mn) {
+                    v16f mn = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                    mn = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma1, wmin, mn, 0, 0, 0);
+                    mn = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma2, wmin, mn, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        const int64_t row = t * 32 + (i >> 2) * 8 + h * 4 + (i & 3);
+                        if (row < dl.rows) dl.mn[row * dl.rs] = mn[i];
+                    }
                 }
                 const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                 acc_lo[t & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[q % 3], bl[0], zero, 0, 0, 0);
@@ -247,6 +267,11 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, 
             for (int i = 2 * s; i < 2 * s + 2; i++) {
                 if (HALF && i >= 8) continue;   // rows 16..31 of the tile are not wanted
                 const int I = (acc_hi[p][i] << SHIFT) + acc_lo[p][i];
+                if (DUMP) {
+                    const int64_t row = (t - 1) * 32 + (i >> 2) * 8 + h * 4 + (i & 3);
+                    if (row < dl.rows) dl.i[row * dl.rs] = I;
+                    continue;
+                }
                 float o = __builtin_fmaf((float)I * dw, dreg[(i >> 2) & 1][i & 3], out[t - 1][i]);
                 asm volatile("" : "+v"(o));   // pins the scaling to this step (pure ops float otherwise)
                 out[t - 1][i] = o;
@@ -377,11 +402,11 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g
 // which is refilled for block b+1 as soon as they are in registers.  The LDS regions are distinct
 // (`__restrict__`): without that knowledge the compiler makes every LDS read wait for all copies in
 // flight, which would serialise the pipeline.
-template <int DT, int MT, bool TRAIL, bool HALF>
+template <int DT, int MT, bool TRAIL, bool HALF, bool DUMP>
 __device__ __forceinline__ void block_step(const uint8_t *__restrict__ cur, uint8_t *__restrict__ nxt,
                                            uint8_t *__restrict__ wl, const cq_weight &w, const cq_act_view &a,
                                            const LaneGeo &g, int64_t m0, int64_t n_tile, bool n_ok, bool more, int64_t b,
-                                           int wave, int lane, const WHead<DT> &hcur, v16f (&out)[MT]) {
+                                           int wave, int lane, const WHead<DT> &hcur, v16f (&out)[MT], const DumpLane &dl) {
     constexpr int SHIFT = DT == CQ_DTYPE_Q4K ? 3 : 7;
     constexpr int SPLIT = TRAIL ? MT / 2 : MT;   // tiles [SPLIT, MT) follow the barrier
     v4i bl[8], bh[8];
@@ -391,20 +416,20 @@ __device__ __forceinline__ void block_step(const uint8_t *__restrict__ cur, uint
     if (n_ok) {
         block_unpack(wl, g, hcur, lane, bl, bh, dw, wmin);
         if (more) stage_weights<DT>(wl, w, g, n_tile, b + 1);
-        tiles_mac<DT, MT, 0, SPLIT, SHIFT, HALF>(cur, g, bl, bh, dw, wmin, lane, out);
+        tiles_mac<DT, MT, 0, SPLIT, SHIFT, HALF, DUMP>(cur, g, bl, bh, dw, wmin, lane, out, dl);
     }
     __builtin_amdgcn_s_waitcnt(0);   // the next stage and the wave's next weights have landed in LDS
     __syncthreads();
-    if (TRAIL && n_ok) tiles_mac<DT, MT, SPLIT, MT, SHIFT, HALF>(cur, g, bl, bh, dw, wmin, lane, out);
+    if (TRAIL && n_ok) tiles_mac<DT, MT, SPLIT, MT, SHIFT, HALF, DUMP>(cur, g, bl, bh, dw, wmin, lane, out, dl);
 }
 
 // ------------------------------------------------------------------ kernel ----
 // Requires n % 32 == 0 and an activation workspace with padded rows (cq_act_view::m_stride).
 // One workgroup: activation rows [m0, m0 + 32*MT) (stored up to row m - 1) x the 256 weight rows of
 // blockIdx.x, K blocks of part blockIdx.z.
-template <int DT, int MT>
+template <int DT, int MT, bool DUMP = false>
 __device__ __forceinline__ void gemm_body(const cq_weight &w, const cq_act_view &a, int64_t m0, int64_t m,
-                                          float *__restrict__ y, int ksplit) {
+                                          float *__restrict__ y, int ksplit, cq_mfma_dump dump = cq_mfma_dump{nullptr, nullptr}) {
     typedef Tile<DT, MT> T;
     extern __shared__ __align__(16) uint8_t smem[];
     const int lane = threadIdx.x & 63;
@@ -446,9 +471,14 @@ __device__ __forceinline__ void gemm_body(const cq_weight &w, const cq_act_view 
         for (int64_t b = b0; b < b1; b++) {
             const bool more = b + 1 < b1;
             if (more) load_head(w, nc * kb + b + 1, hnxt);
-            block_step<DT, MT, decltype(trail)::value, decltype(half)::value>(smem + ic * T::kBytes, smem + in * T::kBytes, wl, w,
-                                                                              a, g, m0, n_tile, n_ok, more, b, wave, lane,
-                                                                              hcur, out);
+            DumpLane dl{nullptr, nullptr, 0, 0};
+            if (DUMP) {
+                const int64_t at = (m0 * w.n + nc) * kb + b;
+                dl = DumpLane{dump.i + at, dump.mn ? dump.mn + at : nullptr, w.n * kb, m - m0};
+            }
+            block_step<DT, MT, decltype(trail)::value, decltype(half)::value, DUMP>(smem + ic * T::kBytes, smem + in * T::kBytes,
+                                                                                    wl, w, a, g, m0, n_tile, n_ok, more, b, wave,
+                                                                                    lane, hcur, out, dl);
             hcur = hnxt;
             rotate();
         }
@@ -466,7 +496,7 @@ __device__ __forceinline__ void gemm_body(const cq_weight &w, const cq_act_view 
         else run(T_{}, F_{});
     }
 
-    if (n_ok) {
+    if (n_ok && !DUMP) {
 #pragma unroll
         for (int t = 0; t < MT; t++) {
 #pragma unroll
@@ -485,6 +515,13 @@ template <int DT, int MT>
 __global__ void __launch_bounds__(kThreads) gemm_kernel(cq_weight w, cq_act_view a, int64_t m, float *__restrict__ y,
                                                         int ksplit) {
     gemm_body<DT, MT>(w, a, (int64_t)blockIdx.y * (MT * 32), m, y, ksplit);
+}
+
+// The same launch with the block integers stored instead of the result (verification).
+template <int DT, int MT>
+__global__ void __launch_bounds__(kThreads) gemm_dump_kernel(cq_weight w, cq_act_view a, int64_t m, int ksplit,
+                                                             cq_mfma_dump dump) {
+    gemm_body<DT, MT, true>(w, a, (int64_t)blockIdx.y * (MT * 32), m, nullptr, ksplit, dump);
 }
 
 // Grouped (mixture-of-experts) variant: one launch for every expert.  blockIdx.y walks a table of
@@ -582,6 +619,23 @@ hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, boo
     return launch_mt<DT, 4>(w, a, m, y, p.ksplit, y_cleared, s);
 }
 
+// The launch cq_launch_gemm would make (same tile height, same K split), storing the block integers.
+template <int DT, int MT>
+hipError_t launch_dump_mt(const cq_weight *w, cq_act_view a, int64_t m, int ksplit, cq_mfma_dump d, hipStream_t s) {
+    const size_t lds = Tile<DT, MT>::kTotal;
+    if (hipError_t e = cq_ensure_lds<gemm_dump_kernel<DT, MT>>(w->dev, lds); e != hipSuccess) return e;
+    dim3 grid((unsigned)n_tiles(w), (unsigned)((m + MT * 32 - 1) / (MT * 32)), (unsigned)ksplit);
+    CQ_LAUNCH((gemm_dump_kernel<DT, MT>), grid, kThreads, lds, s, *w, a, m, ksplit, d);
+    return hipGetLastError();
+}
+template <int DT>
+hipError_t launch_dump_dt(const cq_weight *w, cq_act_view a, int64_t m, cq_mfma_dump d, hipStream_t s) {
+    const Plan p = pick_plan(w, m);
+    if (p.mt == 1) return launch_dump_mt<DT, 1>(w, a, m, p.ksplit, d, s);
+    if (p.mt == 2) return launch_dump_mt<DT, 2>(w, a, m, p.ksplit, d, s);
+    return launch_dump_mt<DT, 4>(w, a, m, p.ksplit, d, s);
+}
+
 template <int DT>
 hipError_t launch_grouped(const cq_weight *const *experts, int n_experts, const int32_t *offsets, cq_act_view a,
                           float *y, bool y_cleared, hipStream_t s) {
@@ -627,6 +681,15 @@ hipError_t cq_launch_gemm_grouped(const cq_weight *const *experts, int n_experts
     if (experts[0]->dtype == CQ_DTYPE_Q4K) return launch_grouped<CQ_DTYPE_Q4K>(experts, n_experts, offsets, a, y, y_cleared, s);
     if (experts[0]->dtype == CQ_DTYPE_Q5K) return launch_grouped<CQ_DTYPE_Q5K>(experts, n_experts, offsets, a, y, y_cleared, s);
     return launch_grouped<CQ_DTYPE_Q6K>(experts, n_experts, offsets, a, y, y_cleared, s);
+}
+
+hipError_t cq_launch_gemm_dump(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, cq_mfma_dump d, hipStream_t s) {
+    if (!cq_gemm_supported(w, m, act_dtype)) return hipErrorNotSupported;
+    if (m == 0 || w->n == 0) return hipSuccess;
+    if (a.m_stride < (m + 127) / 128 * 128) return hipErrorInvalidValue;
+    if (w->dtype == CQ_DTYPE_Q4K) return launch_dump_dt<CQ_DTYPE_Q4K>(w, a, m, d, s);
+    if (w->dtype == CQ_DTYPE_Q5K) return launch_dump_dt<CQ_DTYPE_Q5K>(w, a, m, d, s);
+    return launch_dump_dt<CQ_DTYPE_Q6K>(w, a, m, d, s);
 }
 
 bool cq_gemm_grouped_splits_k(const cq_weight *const *experts, int n_experts, const int32_t *offsets) {

@@ -7,10 +7,11 @@
 // A 32-element block is exactly one K-slice of v_mfma_i32_32x32x32_i8, so the integer of every
 // (activation row, weight row, block) is one MFMA result element, I (Q4_0 nibbles go in as q - 8, so
 // no correction term is left).  Its scale d8[row, block] * dw[col, block] is an outer product: a
-// second MFMA lays it out in the accumulator layout (v_mfma_f32_32x32x16_f16 with two non-zero K-slots:
-// dw is an f16 already, d8 goes in as two f16 pieces, so the product is exact to about 2^-22; the f32
-// MFMA with one K-slot gives the exactly rounded product but holds the matrix pipe twice as long),
-// and the VALU work per element is one conversion and one fma.
+// second MFMA lays it out in the accumulator layout (v_mfma_f32_32x32x16_bf16 with six non-zero K-slots:
+// d8 goes in as three bf16 pieces and dw, an f16, as two, all exact, so the six products are the exact
+// product whatever the magnitude of the activations - f16 pieces would lose d8 below 2^-14 - and the result is
+// d8 * dw to f32 rounding; the f32 MFMA with one K-slot holds the matrix pipe twice as long), and the VALU
+// work per element is one conversion and one fma.
 //
 // Work split as in the K-quant tile kernel (gemm.hip): a workgroup of eight waves covers 32*MT
 // activation rows x 256 weight rows, a wave owns 32 weight rows; per 256-element step of K the
@@ -25,7 +26,7 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
-typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef uint32_t v4u __attribute__((ext_vector_type(4)));
 typedef void __attribute__((address_space(3))) *lptr_t;
 
@@ -110,9 +111,10 @@ __device__ __forceinline__ void stage_weights(uint8_t *wl, const cq_weight &w, c
     }
 }
 
-template <int DT, int MT>
+// DUMP (verification): the block integers are stored through `dump` instead of the result through `y`.
+template <int DT, int MT, bool DUMP>
 __global__ void __launch_bounds__(kThreads) gemm32_kernel(cq_weight w, cq_act_view a, int64_t m, float *__restrict__ y,
-                                                          int ksplit) {
+                                                          int ksplit, cq_mfma_dump dump) {
     typedef Tile<DT, MT> T;
     extern __shared__ __align__(16) uint8_t smem[];
     const int lane = threadIdx.x & 63;
@@ -169,14 +171,18 @@ __global__ void __launch_bounds__(kThreads) gemm32_kernel(cq_weight w, cq_act_vi
                 stage_weights<DT>(wl, w, g, n_tile, b + 1);
                 dnext = *(const uint4 *)(dplane + nc * (k >> 5) + (b + 1) * 8);
             }
-            // scale operand of block s: K-slots 0 and 1 both carry dw (an f16 already), the other slots zero
+            // scale operand of block s: dw = b1 + b2 (bf16 pieces, exact: an f16 has 11 significant bits); lanes
+            // 0..31 carry b1 in K-slots 0..2, lanes 32..63 carry b2 in K-slots 8..10, the other slots zero
             const uint32_t dwords[4] = {dcur.x, dcur.y, dcur.z, dcur.w};
-            v8h dw[8];
+            v8bf dw[8];
 #pragma unroll
             for (int s = 0; s < 8; s++) {
-                const uint32_t bits = (dwords[s >> 1] >> (16 * (s & 1))) & 0xffffu;
-                const v4u pk = {h == 0 ? bits | (bits << 16) : 0u, 0u, 0u, 0u};
-                dw[s] = __builtin_bit_cast(v8h, pk);
+                const float f = cq_h2f((uint16_t)((dwords[s >> 1] >> (16 * (s & 1))) & 0xffffu));
+                const uint32_t fb = __float_as_uint(f);
+                const float b2 = f - __uint_as_float(fb & 0xffff0000u);
+                const uint32_t piece = h == 0 ? fb >> 16 : __float_as_uint(b2) >> 16;
+                const v4u pk = {piece | (piece << 16), piece, 0u, 0u};
+                dw[s] = __builtin_bit_cast(v8bf, pk);
             }
 
             // steps q = (tile t, block s): the two MFMAs of step q, and in their shadow the scaling of step q-1
@@ -185,18 +191,21 @@ __global__ void __launch_bounds__(kThreads) gemm32_kernel(cq_weight w, cq_act_vi
                 return *(const v4i *)(cur + g.col[s & 3] + (t * 2 + (s >> 2)) * 4096);
             };
             // activation scale of (row l%32 of tile t, block s): read two steps ahead, and only turned into
-            // the MFMA operand (two f16 pieces in K-slots 0 and 1) in the step that uses it, so that no step
+            // the MFMA operand (three bf16 pieces) in the step that uses it, so that no step
             // waits for the read it has just issued
             auto d8raw = [&](int q) -> float {
                 const int t = q >> 3, s = q & 7;
                 return *(const float *)(cur + T::oD8 + (t * 32 + col) * 32 + s * 4);
             };
-            auto d8frag = [&](float v) -> v8h {
-                const _Float16 p1 = (_Float16)v;
-                const _Float16 p2 = (_Float16)(v - (float)p1);
-                // lanes 32..63 hold K-slots 8..15, where the weight operand is zero: their (finite) values drop out
-                v8h r = {p1, p2, 0, 0, 0, 0, 0, 0};
-                return r;
+            auto d8frag = [&](float v) -> v8bf {
+                // v = a1 + a2 + a3, each the leading eight bits of what the pieces before it leave (exact);
+                // K-slots 0..2 of both lane halves
+                const uint32_t vb = __float_as_uint(v);
+                const float r1 = v - __uint_as_float(vb & 0xffff0000u);
+                const uint32_t rb = __float_as_uint(r1);
+                const float a3 = r1 - __uint_as_float(rb & 0xffff0000u);
+                const v4u pk = {__builtin_amdgcn_perm(rb, vb, 0x07060302u), __float_as_uint(a3) >> 16, 0u, 0u};
+                return __builtin_bit_cast(v8bf, pk);
             };
             v16i acc[2];
             v16f sc[2];
@@ -211,7 +220,7 @@ __global__ void __launch_bounds__(kThreads) gemm32_kernel(cq_weight w, cq_act_vi
                 if (q + 2 < MT * 8) { av[(q + 2) % 3] = afrag(q + 2); dv[(q + 2) % 3] = d8raw(q + 2); }
                 if (q < MT * 8) {
                     acc[q & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[q % 3], bw[q & 7], zero, 0, 0, 0);
-                    sc[q & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(d8frag(dv[q % 3]), dw[q & 7], zerof, 0, 0, 0);
+                    sc[q & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(d8frag(dv[q % 3]), dw[q & 7], zerof, 0, 0, 0);
                 }
                 // keeps the MFMAs in front of the scaling below: left alone, the scheduler sinks them to the end
                 // of the step, and the next step then starts by waiting for their results
@@ -219,7 +228,14 @@ __global__ void __launch_bounds__(kThreads) gemm32_kernel(cq_weight w, cq_act_vi
                 if (q > 0) {
                     const int p = (q - 1) & 1, t = (q - 1) >> 3;
 #pragma unroll
-                    for (int i = 0; i < 16; i++) out[t][i] = __builtin_fmaf((float)acc[p][i], sc[p][i], out[t][i]);
+                    for (int i = 0; i < 16; i++) {
+                        if (DUMP) {
+                            const int64_t row = m0 + t * 32 + (i >> 2) * 8 + h * 4 + (i & 3);
+                            if (row < m) dump.i[(row * w.n + n) * (k >> 5) + b * 8 + ((q - 1) & 7)] = acc[p][i];
+                        } else {
+                            out[t][i] = __builtin_fmaf((float)acc[p][i], sc[p][i], out[t][i]);
+                        }
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -228,7 +244,7 @@ __global__ void __launch_bounds__(kThreads) gemm32_kernel(cq_weight w, cq_act_vi
         __syncthreads();
     }
 
-    if (n_ok) {
+    if (n_ok && !DUMP) {
 #pragma unroll
         for (int t = 0; t < MT; t++) {
 #pragma unroll
@@ -287,26 +303,28 @@ Plan pick_plan(const cq_weight *w, int64_t m) {
     return best;
 }
 
-template <int DT, int MT>
-hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, int ksplit, bool y_cleared, hipStream_t s) {
+// DUMP: the same launch (tile height, K split) storing the block integers through `d`; y is not touched.
+template <int DT, int MT, bool DUMP>
+hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, int ksplit, bool y_cleared, cq_mfma_dump d,
+                     hipStream_t s) {
     const size_t lds = Tile<DT, MT>::kTotal;
-    if (hipError_t e = cq_ensure_lds<gemm32_kernel<DT, MT>>(w->dev, lds); e != hipSuccess) return e;
+    if (hipError_t e = cq_ensure_lds<gemm32_kernel<DT, MT, DUMP>>(w->dev, lds); e != hipSuccess) return e;
     const int64_t gx = (w->n + kWaves * 32 - 1) / (kWaves * 32), gy = (m + MT * 32 - 1) / (MT * 32);
-    if (ksplit > 1 && !y_cleared) {
+    if (!DUMP && ksplit > 1 && !y_cleared) {
         hipError_t e = cq_launch_fill_zero(y, m * w->n, s);
         if (e != hipSuccess) return e;
     }
     dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)ksplit);
-    CQ_LAUNCH((gemm32_kernel<DT, MT>), grid, kThreads, lds, s, *w, a, m, y, ksplit);
+    CQ_LAUNCH((gemm32_kernel<DT, MT, DUMP>), grid, kThreads, lds, s, *w, a, m, y, ksplit, d);
     return hipGetLastError();
 }
 
-template <int DT>
-hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, bool y_cleared, hipStream_t s) {
+template <int DT, bool DUMP>
+hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, bool y_cleared, cq_mfma_dump d, hipStream_t s) {
     const Plan p = pick_plan(w, m);
-    if (p.mt == 1) return launch_mt<DT, 1>(w, a, m, y, p.ksplit, y_cleared, s);
-    if (p.mt == 2) return launch_mt<DT, 2>(w, a, m, y, p.ksplit, y_cleared, s);
-    return launch_mt<DT, 4>(w, a, m, y, p.ksplit, y_cleared, s);
+    if (p.mt == 1) return launch_mt<DT, 1, DUMP>(w, a, m, y, p.ksplit, y_cleared, d, s);
+    if (p.mt == 2) return launch_mt<DT, 2, DUMP>(w, a, m, y, p.ksplit, y_cleared, d, s);
+    return launch_mt<DT, 4, DUMP>(w, a, m, y, p.ksplit, y_cleared, d, s);
 }
 
 }  // namespace
@@ -324,6 +342,15 @@ hipError_t cq_launch_gemm32(const cq_weight *w, cq_act_view a, int act_dtype, in
     if (!cq_gemm32_supported(w, act_dtype)) return hipErrorNotSupported;
     if (m == 0) return hipSuccess;
     if (a.m_stride < (m + 127) / 128 * 128) return hipErrorInvalidValue;   // rows the last tile may read
-    if (w->dtype == CQ_DTYPE_Q8_0) return launch_dt<CQ_DTYPE_Q8_0>(w, a, m, y, y_cleared, s);
-    return launch_dt<CQ_DTYPE_Q4_0>(w, a, m, y, y_cleared, s);
+    const cq_mfma_dump none{nullptr, nullptr};
+    if (w->dtype == CQ_DTYPE_Q8_0) return launch_dt<CQ_DTYPE_Q8_0, false>(w, a, m, y, y_cleared, none, s);
+    return launch_dt<CQ_DTYPE_Q4_0, false>(w, a, m, y, y_cleared, none, s);
+}
+
+hipError_t cq_launch_gemm32_dump(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, cq_mfma_dump d, hipStream_t s) {
+    if (!cq_gemm32_supported(w, act_dtype)) return hipErrorNotSupported;
+    if (m == 0) return hipSuccess;
+    if (a.m_stride < (m + 127) / 128 * 128) return hipErrorInvalidValue;
+    if (w->dtype == CQ_DTYPE_Q8_0) return launch_dt<CQ_DTYPE_Q8_0, true>(w, a, m, nullptr, true, d, s);
+    return launch_dt<CQ_DTYPE_Q4_0, true>(w, a, m, nullptr, true, d, s);
 }

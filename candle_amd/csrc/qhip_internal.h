@@ -134,6 +134,18 @@ hipError_t cq_launch_matvec_fused_rows(const cq_weight *w, const float *x, int64
 bool cq_matvec_fused_multi_supported(const cq_weight *const *ws, int count, int pre_kind, int64_t m);
 hipError_t cq_launch_matvec_fused_multi(const cq_weight *const *ws, int count, const float *x, cq_pre pre, int64_t m,
                                         float *const *ys, hipStream_t s);
+// Verification output of the MFMA kernels (gemm.hip, gemm_blk32.hip, skinny.hip): what the f32 result is combined
+// from, per activation row r, weight row c and block b, at [(r*n + c)*blocks + b].
+//   i  : the block's integer dot product, the number the dot-product kernels and the CPU form
+//   mn : types with a min term (Q4K, Q5K; else null): -(dmin*d8) * sum_j min_j*bsum32_j as the f16 MFMA delivers
+//        it from a zero accumulator - a float, the kernels never hold this term as an integer
+struct cq_mfma_dump {
+    int32_t *i;
+    float *mn;
+};
+hipError_t cq_launch_gemm_dump(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, cq_mfma_dump d, hipStream_t s);
+hipError_t cq_launch_gemm32_dump(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, cq_mfma_dump d, hipStream_t s);
+hipError_t cq_launch_skinny_dump(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, cq_mfma_dump d, hipStream_t s);
 // gemm.hip
 bool cq_gemm_supported(const cq_weight *w, int64_t m, int act_dtype);
 // `y_cleared`: y is already zero (a launch that splits K otherwise clears it first); *_splits_k tell

@@ -203,9 +203,11 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, int lane, const 
 
 // RT = groups of eight activation rows held (rows m0 .. m0 + 8*RT - 1; the workspace pads rows, so
 // whole groups can be copied); results are stored for rows < m.  Requires n % 16 == 0.
-template <int DT, int RT>
+// DUMP (verification): the block integers, and the min term as the f16 MFMA delivers it from a zero accumulator,
+// are stored through `dump` instead of the result through `y`.
+template <int DT, int RT, bool DUMP>
 __global__ void __launch_bounds__(kThreads) skinny_kernel(cq_weight w, cq_act_view a, int64_t m0, int64_t m,
-                                                          float *__restrict__ y) {
+                                                          float *__restrict__ y, cq_mfma_dump dump) {
     typedef Buf<DT, RT> B;
     constexpr bool MINS = is_k4(DT);
     constexpr int NT = (RT + 1) / 2;   // 16-row tiles
@@ -267,7 +269,15 @@ __global__ void __launch_bounds__(kThreads) skinny_kernel(cq_weight w, cq_act_vi
             if (MINS) {
                 const uint32_t row = t * 16 + r < 8u * RT ? t * 16 + r : 8u * RT - 1;
                 const v8h ma = *(const v8h *)(buf + B::oMin + row * 32 + (kq >> 1) * 16);
-                out[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ma, wmin, out[t], 0, 0, 0);
+                if (!DUMP) out[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ma, wmin, out[t], 0, 0, 0);
+                if (DUMP && dump.mn) {
+                    const v4f mn = __builtin_amdgcn_mfma_f32_16x16x32_f16(ma, wmin, (v4f){0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int64_t orow = m0 + t * 16 + kq * 4 + i;
+                        if (orow < m) dump.mn[(orow * w.n + n_tile + r) * kb + b] = mn[i];
+                    }
+                }
             }
             v4i acc_lo = {0, 0, 0, 0}, acc_hi = {0, 0, 0, 0};
 #pragma unroll
@@ -279,10 +289,16 @@ __global__ void __launch_bounds__(kThreads) skinny_kernel(cq_weight w, cq_act_vi
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const int I = (acc_hi[i] << SHIFT) + acc_lo[i];
-                out[t][i] = __builtin_fmaf((float)I * dw, d8[i], out[t][i]);
+                if (DUMP) {
+                    const int64_t orow = m0 + t * 16 + kq * 4 + i;
+                    if (orow < m) dump.i[(orow * w.n + n_tile + r) * kb + b] = I;
+                } else {
+                    out[t][i] = __builtin_fmaf((float)I * dw, d8[i], out[t][i]);
+                }
             }
         }
     }
+    if (DUMP) return;
 
     // ---- sum the eight waves' partial tiles in wave order
 #pragma unroll
@@ -348,9 +364,11 @@ __device__ __forceinline__ void res_issue_weights(uint8_t *__restrict__ wl, cons
 }
 
 // One K block of one tile: unpack the weights in `wl`, contract with the resident activation slice `act`.
-template <int DT, int RT, int NT>
+// DUMP: the integers go to dump.i / dump.mn at `at` + row * `rs` (rows < m) instead of into `out`.
+template <int DT, int RT, int NT, bool DUMP>
 __device__ __forceinline__ void res_block(const uint8_t *__restrict__ wl, const uint8_t *__restrict__ act, int lane,
-                                          const WHead<DT> &head, const uint32_t (&a_col)[NT][2], v4f (&out)[NT]) {
+                                          const WHead<DT> &head, const uint32_t (&a_col)[NT][2], v4f (&out)[NT],
+                                          const cq_mfma_dump &dump, int64_t at, int64_t rs, int64_t m) {
     typedef Res<DT, RT> R;
     constexpr bool MINS = is_k4(DT);
     constexpr int SHIFT = DT == CQ_DTYPE_Q4K ? 3 : 7;
@@ -365,7 +383,15 @@ __device__ __forceinline__ void res_block(const uint8_t *__restrict__ wl, const 
         if (MINS) {
             const uint32_t row = t * 16 + r < 8u * RT ? t * 16 + r : 8u * RT - 1;
             const v8h ma = *(const v8h *)(act + R::oMin + row * 32 + (kq >> 1) * 16);
-            out[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ma, wmin, out[t], 0, 0, 0);
+            if (!DUMP) out[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ma, wmin, out[t], 0, 0, 0);
+            if (DUMP && dump.mn) {
+                const v4f mn = __builtin_amdgcn_mfma_f32_16x16x32_f16(ma, wmin, (v4f){0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int64_t orow = t * 16 + kq * 4 + i;
+                    if (orow < m) dump.mn[at + orow * rs] = mn[i];
+                }
+            }
         }
         v4i acc_lo = {0, 0, 0, 0}, acc_hi = {0, 0, 0, 0};
 #pragma unroll
@@ -377,7 +403,12 @@ __device__ __forceinline__ void res_block(const uint8_t *__restrict__ wl, const 
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int I = (acc_hi[i] << SHIFT) + acc_lo[i];
-            out[t][i] = __builtin_fmaf((float)I * dw, d8[i], out[t][i]);
+            if (DUMP) {
+                const int64_t orow = t * 16 + kq * 4 + i;
+                if (orow < m) dump.i[at + orow * rs] = I;
+            } else {
+                out[t][i] = __builtin_fmaf((float)I * dw, d8[i], out[t][i]);
+            }
         }
     }
 }
@@ -385,9 +416,9 @@ __device__ __forceinline__ void res_block(const uint8_t *__restrict__ wl, const 
 // m <= 8 * RT activation rows (the workspace pads rows, so whole groups are copied); n % 16 == 0; at most
 // kMaxBpw K blocks per wave.  `tiles` = n / 16, dealt to the gridDim.x workgroups in turn.
 constexpr int kMaxBpw = 4;
-template <int DT, int RT, int kWaves, int NBUF>
+template <int DT, int RT, int kWaves, int NBUF, bool DUMP>
 __global__ void __launch_bounds__(kWaves * 64) skinny_resident_kernel(cq_weight w, cq_act_view a, int64_t m,
-                                                                      float *__restrict__ y) {
+                                                                      float *__restrict__ y, cq_mfma_dump dump) {
     typedef Res<DT, RT> R;
     constexpr bool MINS = is_k4(DT);
     constexpr int NT = (RT + 1) / 2;   // 16-row tiles of activation rows
@@ -466,8 +497,8 @@ __global__ void __launch_bounds__(kWaves * 64) skinny_resident_kernel(cq_weight 
         for (int j = 0; j < kMaxBpw; j++) {
             const int64_t b = wave + (int64_t)j * kWaves;
             if (b < kb)
-                res_block<DT, RT, NT>(wgt_base + (b * NBUF + (NBUF == 2 ? par : 0)) * R::kWgt, smem + b * R::kActBlk, lane,
-                                      head[j], a_col, out);
+                res_block<DT, RT, NT, DUMP>(wgt_base + (b * NBUF + (NBUF == 2 ? par : 0)) * R::kWgt, smem + b * R::kActBlk, lane,
+                                            head[j], a_col, out, dump, (n_tile + r) * kb + b, w.n * kb, m);
         }
         // ---- sum the waves' partial tiles in wave order (through the wave's first weight buffer of this tile)
         uint8_t *part = wgt_base + ((int64_t)wave * NBUF + (NBUF == 2 ? par : 0)) * R::kWgt;
@@ -476,7 +507,7 @@ __global__ void __launch_bounds__(kWaves * 64) skinny_resident_kernel(cq_weight 
             for (int t = 0; t < NT; t++) *(v4f *)(part + t * 1024 + lane * 16) = out[t];
         }
         __syncthreads();
-        if (wave < NT) {
+        if (wave < NT && !DUMP) {
             v4f s = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
             const int64_t nw = kb < kWaves ? kb : kWaves;   // waves that own a block
             for (int64_t o = 0; o < nw; o++) {
@@ -527,9 +558,9 @@ template <int RT> struct BufQ8 {
     static constexpr int kBytes = kRaw;   // >= 2 KiB of partial results
 };
 
-template <int DT, int RT>
+template <int DT, int RT, bool DUMP>
 __global__ void __launch_bounds__(kThreads) skinny_blk32_kernel(cq_weight w, cq_act_view a, int64_t m0, int64_t m,
-                                                                float *__restrict__ y) {
+                                                                float *__restrict__ y, cq_mfma_dump dump) {
     typedef BufQ8<RT> B;
     constexpr bool Q4 = DT == CQ_DTYPE_Q4_0;
     constexpr int NT = (RT + 1) / 2;   // 16-row tiles
@@ -623,11 +654,17 @@ __global__ void __launch_bounds__(kThreads) skinny_blk32_kernel(cq_weight w, cq_
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const int I = Q4 ? acc[i] - 8 * bs[Q4 ? t : 0][i][b >> 2][b & 3] : acc[i];
-                    out[t][i] = __builtin_fmaf((float)I * dw, da[t][i][b >> 2][b & 3], out[t][i]);
+                    if (DUMP) {
+                        const int64_t orow = m0 + t * 16 + kq * 4 + i;
+                        if (orow < m) dump.i[(orow * w.n + n_tile + r) * kb + g * 8 + b] = I;
+                    } else {
+                        out[t][i] = __builtin_fmaf((float)I * dw, da[t][i][b >> 2][b & 3], out[t][i]);
+                    }
                 }
             }
         }
     }
+    if (DUMP) return;
 
     // ---- sum the eight waves' partial tiles in wave order
 #pragma unroll
@@ -649,44 +686,46 @@ __global__ void __launch_bounds__(kThreads) skinny_blk32_kernel(cq_weight w, cq_
     }
 }
 
-template <int DT, int RT>
-hipError_t launch_blk32_rt(const cq_weight *w, cq_act_view a, int64_t m0, int64_t m, float *y, hipStream_t s) {
+// DUMP (all launchers below): the launch cq_launch_skinny would make, storing the block integers through `d`.
+template <int DT, int RT, bool DUMP>
+hipError_t launch_blk32_rt(const cq_weight *w, cq_act_view a, int64_t m0, int64_t m, float *y, cq_mfma_dump d, hipStream_t s) {
     const size_t lds = (size_t)BufQ8<RT>::kBytes * kWaves;
-    if (hipError_t e = cq_ensure_lds<skinny_blk32_kernel<DT, RT>>(w->dev, lds); e != hipSuccess) return e;
-    CQ_LAUNCH((skinny_blk32_kernel<DT, RT>), (unsigned)(w->n / 16), kThreads, lds, s, *w, a, m0, m, y);
+    if (hipError_t e = cq_ensure_lds<skinny_blk32_kernel<DT, RT, DUMP>>(w->dev, lds); e != hipSuccess) return e;
+    CQ_LAUNCH((skinny_blk32_kernel<DT, RT, DUMP>), (unsigned)(w->n / 16), kThreads, lds, s, *w, a, m0, m, y, d);
     return hipGetLastError();
 }
 
-template <int DT> hipError_t launch_blk32(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
+template <int DT, bool DUMP>
+hipError_t launch_blk32(const cq_weight *w, cq_act_view a, int64_t m, float *y, cq_mfma_dump d, hipStream_t s) {
     for (int64_t m0 = 0; m0 < m; m0 += 32) {
         const int64_t left = m - m0;
         hipError_t e;
-        if (left <= 8) e = launch_blk32_rt<DT, 1>(w, a, m0, m, y, s);
-        else if (left <= 16) e = launch_blk32_rt<DT, 2>(w, a, m0, m, y, s);
-        else if (left <= 24) e = launch_blk32_rt<DT, 3>(w, a, m0, m, y, s);
-        else e = launch_blk32_rt<DT, 4>(w, a, m0, m, y, s);
+        if (left <= 8) e = launch_blk32_rt<DT, 1, DUMP>(w, a, m0, m, y, d, s);
+        else if (left <= 16) e = launch_blk32_rt<DT, 2, DUMP>(w, a, m0, m, y, d, s);
+        else if (left <= 24) e = launch_blk32_rt<DT, 3, DUMP>(w, a, m0, m, y, d, s);
+        else e = launch_blk32_rt<DT, 4, DUMP>(w, a, m0, m, y, d, s);
         if (e != hipSuccess) return e;
     }
     return hipSuccess;
 }
 
-template <int DT, int RT>
-hipError_t launch_rt(const cq_weight *w, cq_act_view a, int64_t m0, int64_t m, float *y, hipStream_t s) {
+template <int DT, int RT, bool DUMP>
+hipError_t launch_rt(const cq_weight *w, cq_act_view a, int64_t m0, int64_t m, float *y, cq_mfma_dump d, hipStream_t s) {
     const size_t lds = (size_t)Buf<DT, RT>::kBytes * kWaves;
-    if (hipError_t e = cq_ensure_lds<skinny_kernel<DT, RT>>(w->dev, lds); e != hipSuccess) return e;
-    CQ_LAUNCH((skinny_kernel<DT, RT>), (unsigned)(w->n / 16), kThreads, lds, s, *w, a, m0, m, y);
+    if (hipError_t e = cq_ensure_lds<skinny_kernel<DT, RT, DUMP>>(w->dev, lds); e != hipSuccess) return e;
+    CQ_LAUNCH((skinny_kernel<DT, RT, DUMP>), (unsigned)(w->n / 16), kThreads, lds, s, *w, a, m0, m, y, d);
     return hipGetLastError();
 }
 
-template <int DT>
-hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
+template <int DT, bool DUMP>
+hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, cq_mfma_dump d, hipStream_t s) {
     for (int64_t m0 = 0; m0 < m; m0 += 32) {
         const int64_t left = m - m0;
         hipError_t e;
-        if (left <= 8) e = launch_rt<DT, 1>(w, a, m0, m, y, s);
-        else if (left <= 16) e = launch_rt<DT, 2>(w, a, m0, m, y, s);
-        else if (left <= 24) e = launch_rt<DT, 3>(w, a, m0, m, y, s);
-        else e = launch_rt<DT, 4>(w, a, m0, m, y, s);
+        if (left <= 8) e = launch_rt<DT, 1, DUMP>(w, a, m0, m, y, d, s);
+        else if (left <= 16) e = launch_rt<DT, 2, DUMP>(w, a, m0, m, y, d, s);
+        else if (left <= 24) e = launch_rt<DT, 3, DUMP>(w, a, m0, m, y, d, s);
+        else e = launch_rt<DT, 4, DUMP>(w, a, m0, m, y, d, s);
         if (e != hipSuccess) return e;
     }
     return hipSuccess;
@@ -694,14 +733,15 @@ hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hip
 
 
 // The resident-activation kernel where the call's activations and the weight buffers fit the LDS (see above).
-template <int DT, int RT, int NW, int NBUF>
-hipError_t launch_res_inst(const cq_weight *w, cq_act_view a, int64_t m, float *y, size_t lds, unsigned grid, hipStream_t s) {
-    if (hipError_t e = cq_ensure_lds<skinny_resident_kernel<DT, RT, NW, NBUF>>(w->dev, lds); e != hipSuccess) return e;
-    CQ_LAUNCH((skinny_resident_kernel<DT, RT, NW, NBUF>), grid, NW * 64, lds, s, *w, a, m, y);
+template <int DT, int RT, int NW, int NBUF, bool DUMP>
+hipError_t launch_res_inst(const cq_weight *w, cq_act_view a, int64_t m, float *y, size_t lds, unsigned grid, cq_mfma_dump d,
+                           hipStream_t s) {
+    if (hipError_t e = cq_ensure_lds<skinny_resident_kernel<DT, RT, NW, NBUF, DUMP>>(w->dev, lds); e != hipSuccess) return e;
+    CQ_LAUNCH((skinny_resident_kernel<DT, RT, NW, NBUF, DUMP>), grid, NW * 64, lds, s, *w, a, m, y, d);
     return hipGetLastError();
 }
-template <int DT, int RT>
-bool launch_res_rt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s, hipError_t *err) {
+template <int DT, int RT, bool DUMP>
+bool launch_res_rt(const cq_weight *w, cq_act_view a, int64_t m, float *y, cq_mfma_dump d, hipStream_t s, hipError_t *err) {
     const int64_t kb = w->k >> 8, tiles = w->n / 16;
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
@@ -717,18 +757,37 @@ bool launch_res_rt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipSt
     if (tiles > grid) return false;
     const size_t one = Res<DT, RT>::bytes(kb, 1);
     if (one <= (size_t)kMaxLds) {
-        *err = sixteen ? launch_res_inst<DT, RT, 16, 1>(w, a, m, y, one, grid, s) : launch_res_inst<DT, RT, 8, 1>(w, a, m, y, one, grid, s);
+        *err = sixteen ? launch_res_inst<DT, RT, 16, 1, DUMP>(w, a, m, y, one, grid, d, s)
+                       : launch_res_inst<DT, RT, 8, 1, DUMP>(w, a, m, y, one, grid, d, s);
         return true;
     }
     return false;
 }
-template <int DT>
-bool launch_res(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s, hipError_t *err) {
-    if (m <= 8) return launch_res_rt<DT, 1>(w, a, m, y, s, err);
-    if (m <= 16) return launch_res_rt<DT, 2>(w, a, m, y, s, err);
-    if (m <= 24) return launch_res_rt<DT, 3>(w, a, m, y, s, err);
-    if (m <= 32) return launch_res_rt<DT, 4>(w, a, m, y, s, err);
+template <int DT, bool DUMP>
+bool launch_res(const cq_weight *w, cq_act_view a, int64_t m, float *y, cq_mfma_dump d, hipStream_t s, hipError_t *err) {
+    if (m <= 8) return launch_res_rt<DT, 1, DUMP>(w, a, m, y, d, s, err);
+    if (m <= 16) return launch_res_rt<DT, 2, DUMP>(w, a, m, y, d, s, err);
+    if (m <= 24) return launch_res_rt<DT, 3, DUMP>(w, a, m, y, d, s, err);
+    if (m <= 32) return launch_res_rt<DT, 4, DUMP>(w, a, m, y, d, s, err);
     return false;
+}
+
+template <bool DUMP>
+hipError_t launch_any(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, cq_mfma_dump d, hipStream_t s) {
+    if (!cq_skinny_supported(w, act_dtype)) return hipErrorNotSupported;
+    if (m == 0) return hipSuccess;
+    if (a.m_stride < (m + 31) / 32 * 32) return hipErrorInvalidValue;   // whole 8-row groups are copied
+    if (w->dtype == CQ_DTYPE_Q8_0) return launch_blk32<CQ_DTYPE_Q8_0, DUMP>(w, a, m, y, d, s);
+    if (w->dtype == CQ_DTYPE_Q4_0) return launch_blk32<CQ_DTYPE_Q4_0, DUMP>(w, a, m, y, d, s);
+    hipError_t e = hipSuccess;
+#ifndef CQ_EXP_NO_RESIDENT
+    if (w->dtype == CQ_DTYPE_Q4K && launch_res<CQ_DTYPE_Q4K, DUMP>(w, a, m, y, d, s, &e)) return e;
+    if (w->dtype == CQ_DTYPE_Q5K && launch_res<CQ_DTYPE_Q5K, DUMP>(w, a, m, y, d, s, &e)) return e;
+    if (w->dtype == CQ_DTYPE_Q6K && launch_res<CQ_DTYPE_Q6K, DUMP>(w, a, m, y, d, s, &e)) return e;
+#endif
+    if (w->dtype == CQ_DTYPE_Q4K) return launch_dt<CQ_DTYPE_Q4K, DUMP>(w, a, m, y, d, s);
+    if (w->dtype == CQ_DTYPE_Q5K) return launch_dt<CQ_DTYPE_Q5K, DUMP>(w, a, m, y, d, s);
+    return launch_dt<CQ_DTYPE_Q6K, DUMP>(w, a, m, y, d, s);
 }
 
 }  // namespace
@@ -741,18 +800,9 @@ bool cq_skinny_supported(const cq_weight *w, int act_dtype) {
 }
 
 hipError_t cq_launch_skinny(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s) {
-    if (!cq_skinny_supported(w, act_dtype)) return hipErrorNotSupported;
-    if (m == 0) return hipSuccess;
-    if (a.m_stride < (m + 31) / 32 * 32) return hipErrorInvalidValue;   // whole 8-row groups are copied
-    if (w->dtype == CQ_DTYPE_Q8_0) return launch_blk32<CQ_DTYPE_Q8_0>(w, a, m, y, s);
-    if (w->dtype == CQ_DTYPE_Q4_0) return launch_blk32<CQ_DTYPE_Q4_0>(w, a, m, y, s);
-    hipError_t e = hipSuccess;
-#ifndef CQ_EXP_NO_RESIDENT
-    if (w->dtype == CQ_DTYPE_Q4K && launch_res<CQ_DTYPE_Q4K>(w, a, m, y, s, &e)) return e;
-    if (w->dtype == CQ_DTYPE_Q5K && launch_res<CQ_DTYPE_Q5K>(w, a, m, y, s, &e)) return e;
-    if (w->dtype == CQ_DTYPE_Q6K && launch_res<CQ_DTYPE_Q6K>(w, a, m, y, s, &e)) return e;
-#endif
-    if (w->dtype == CQ_DTYPE_Q4K) return launch_dt<CQ_DTYPE_Q4K>(w, a, m, y, s);
-    if (w->dtype == CQ_DTYPE_Q5K) return launch_dt<CQ_DTYPE_Q5K>(w, a, m, y, s);
-    return launch_dt<CQ_DTYPE_Q6K>(w, a, m, y, s);
+    return launch_any<false>(w, a, act_dtype, m, y, cq_mfma_dump{nullptr, nullptr}, s);
+}
+
+hipError_t cq_launch_skinny_dump(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, cq_mfma_dump d, hipStream_t s) {
+    return launch_any<true>(w, a, act_dtype, m, nullptr, d, s);
 }

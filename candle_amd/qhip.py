@@ -24,7 +24,7 @@ EXPORTS = [
     "cq_weight_create", "cq_weight_zeros", "cq_weight_quantize", "cq_weight_dequantize",
     "cq_weight_dequantize_f16", "cq_weight_to_ggml", "cq_weight_size_in_bytes", "cq_weight_dtype",
     "cq_weight_device", "cq_weight_shape", "cq_weight_destroy", "cq_act_bytes", "cq_quantize_act",
-    "cq_workspace_bytes", "cq_qmatmul", "cq_qmatmul_int_dots", "cq_grouped_workspace_bytes",
+    "cq_workspace_bytes", "cq_qmatmul", "cq_qmatmul_int_dots", "cq_qmatmul_int_dots_mfma", "cq_grouped_workspace_bytes",
     "cq_qmatmul_grouped", "cq_silu_mul", "cq_moe_scatter_add", "cq_timing_arm", "cq_timing_elapsed_us",
     "cq_selfcheck_round", "cq_quantize_act_fused", "cq_qmatmul_fused", "cq_qmatmul_grouped_fused", "cq_qmatmul_multi",
     "cq_weight_zeros_flat", "cq_weight_create_flat", "cq_weight_elem_count", "cq_weight_set_shape",
@@ -70,6 +70,7 @@ def load():
     L.cq_workspace_bytes.restype = sz; L.cq_workspace_bytes.argtypes = [vp, i64, ci]
     L.cq_qmatmul.argtypes = [vp, vp, i64, vp, ci, vp, sz, vp]
     L.cq_qmatmul_int_dots.argtypes = [vp, vp, i64, vp, vp, vp, sz, vp]
+    L.cq_qmatmul_int_dots_mfma.argtypes = [vp, vp, i64, C.c_int, vp, vp, vp, sz, vp]
     L.cq_grouped_workspace_bytes.restype = sz
     L.cq_grouped_workspace_bytes.argtypes = [C.POINTER(vp), ci, i64, ci]
     L.cq_qmatmul_grouped.argtypes = [C.POINTER(vp), ci, vp, vp, C.POINTER(C.c_int32), vp, ci, vp, sz, vp]
@@ -374,6 +375,27 @@ def qmatmul_int_dots(w: QWeight, x):
     check(L.cq_qmatmul_int_dots(w.handle, C.c_void_p(x.data_ptr()), m, C.c_void_p(oi.data_ptr()),
                                 C.c_void_p(om.data_ptr()) if om is not None else None,
                                 C.c_void_p(ws.data_ptr()), ws.numel(), _stream_ptr()))
+    return oi, om
+
+
+MFMA_SKINNY, MFMA_TILE = 1, 2
+
+
+def qmatmul_int_dots_mfma(w: QWeight, x, kernel: int):
+    """The block integers out of the matrix-core kernels: (int32 [m, n, blocks], float32 min term or None)."""
+    torch = _torch()
+    L = load()
+    _require_f32_cuda(x)
+    n, k = w.shape
+    m = x.shape[0]
+    kb = k // L.cq_block_size(w.dtype)
+    oi = torch.full((m, n, kb), -(2 ** 31), dtype=torch.int32, device=x.device)
+    om = torch.full((m, n, kb), float("nan"), dtype=torch.float32, device=x.device) if w.dtype in (Q4K, Q5K) else None
+    need = L.cq_workspace_bytes(w.handle, m, 0)
+    ws = _default_ws.get(need, x.device)
+    check(L.cq_qmatmul_int_dots_mfma(w.handle, C.c_void_p(x.data_ptr()), m, kernel, C.c_void_p(oi.data_ptr()),
+                                     C.c_void_p(om.data_ptr()) if om is not None else None,
+                                     C.c_void_p(ws.data_ptr()), ws.numel(), _stream_ptr()))
     return oi, om
 
 

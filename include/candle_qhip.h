@@ -175,6 +175,18 @@ int cq_qmatmul_int_dots(const cq_weight *w, const float *x_dev, int64_t m, int32
                         int32_t *out_mn_dev, void *workspace_dev, size_t workspace_bytes,
                         void *stream);
 
+/* The same integers out of the matrix-core kernels (the verification above runs the dot-product kernels): `kernel`
+ * picks the small-batch kernel (CQ_MFMA_SKINNY: the launch cq_qmatmul makes for 2..32 rows, whatever m is here) or
+ * the tile kernel of the prefill path (CQ_MFMA_TILE, with the tile height and K split cq_qmatmul picks for m;
+ * Q8_0 and Q4_0 weights: more than 32 rows, as in cq_qmatmul).
+ * out_i as above.  out_mn (Q4K, Q5K; else NULL) is a float: those kernels contract the min term on the f16 matrix
+ * core, -(dmin*d8) * sum_j min_j*bsum32_j from operands split in two f16 pieces each, and never hold the integer
+ * sum; it is stored as that contraction delivers it for one block.  No counterpart in the reference. */
+#define CQ_MFMA_SKINNY 1
+#define CQ_MFMA_TILE 2
+int cq_qmatmul_int_dots_mfma(const cq_weight *w, const float *x_dev, int64_t m, int kernel, int32_t *out_i_dev,
+                             float *out_mn_dev, void *workspace_dev, size_t workspace_bytes, void *stream);
+
 /* ---- grouped experts (MoE FFN) ------------------------------------------- */
 /* One QMatMul per expert over gathered rows, as MlpOrMoe::forward does sequentially
  * (candle-transformers/src/models/quantized_llama.rs:117-135): for expert e and p in

@@ -368,8 +368,10 @@ def test_gemm_needs_32_row_multiple(qh, dt):
 def test_prefill_gemm_config3(qh, dt, m, k, n):
     """BASELINE config 3 at full size: M = 512 tokens on the Mistral FFN shapes, activations N(0,1)
     with 1% outliers at +-8 sigma.  Weights are quantized on the device (bit-identical to the CPU
-    quantizer, checked above); the oracle evaluates a sample of 96 weight rows over all 512 tokens,
-    and the whole output is checked for batch invariance against the decode kernel on 4 rows."""
+    quantizer, checked above).  The oracle evaluates, over all 512 tokens, 96 weight rows: the first and the last
+    row of the first, a middle and the last workgroup tile (256 weight rows each), of a wave's 32-row tile inside
+    them, and random rows for the rest.  The whole 512 x n output is compared with the dot-product kernels
+    (oracle-checked row by row above), so that no tile of the launch goes unseen."""
     rng = np.random.default_rng(k + dt)
     gen = torch.Generator(device="cuda").manual_seed(k + dt)
     wt = torch.randn((n, k), generator=gen, device="cuda") * 0.02
@@ -379,20 +381,30 @@ def test_prefill_gemm_config3(qh, dt, m, k, n):
     idx = rng.choice(x.size, size=x.size // 100, replace=False)
     x.ravel()[idx] = np.where(rng.random(idx.size) < 0.5, -8.0, 8.0).astype(np.float32)
     xd = dev(x)
-    got = qh.qmatmul(qw, xd).cpu().numpy()                      # m > 8: MFMA kernel
-    rows = np.sort(rng.choice(n, size=96, replace=False))
+    got_d = qh.qmatmul(qw, xd)                                  # m > 32: the tile kernel
+    got = got_d.cpu().numpy()
+    tiles = n // 256
+    edge = []
+    for t in (0, tiles // 2, tiles - 1):
+        edge += [256 * t, 256 * t + 31, 256 * t + 32, 256 * t + 224, 256 * t + 255]
+    rest = rng.choice(n, size=96 - len(edge), replace=False)
+    rows = np.unique(np.concatenate([np.array(edge), rest]))
     row_bytes = k // 256 * orc.TYPE_SIZE[dt]
     blocks = qw.to_ggml().reshape(n, row_bytes)[rows].ravel()
     want = orc.matmul(dt, x, blocks, len(rows))
     g = got[:, rows].astype(np.float64)
     err = np.linalg.norm(g - want) / np.linalg.norm(want)
     assert err <= REL_L2_TOL, err
-    for r in range(0, m, 37):
+    for r in list(range(0, m, 37)) + [127, 128, m - 1]:          # with the edges of the 128-row activation tiles
         # max-abs bar, with ||row||_2 scaled from the sampled columns to the full row
         nrm = np.linalg.norm(want[r]) * np.sqrt(n / len(rows))
         assert np.abs(g[r] - want[r]).max() <= MAX_ABS_FACTOR * nrm
-    mv = qh.qmatmul(qw, xd[:4].contiguous(), qh.FLAG_FORCE_MATVEC).cpu().numpy()
-    assert np.linalg.norm(got[:4] - mv) / np.linalg.norm(mv) <= 1e-5
+    # every element against the dot-product kernels: same integers, f32 sums in another order
+    mv = qh.qmatmul(qw, xd, qh.FLAG_FORCE_MATVEC)
+    diff = (got_d - mv).double()
+    row_norm = mv.double().norm(dim=1)
+    assert float((diff.norm(dim=1) / row_norm).max()) <= 1e-5
+    assert float((diff.abs().amax(dim=1) / row_norm).max()) <= 1e-5
 
 
 def test_reference_goldens_through_hip(qh, goldens, seeded_inputs):
