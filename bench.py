@@ -125,6 +125,65 @@ def envelope() -> int:
     return 0
 
 
+def small_batch_probe(rounds: int, copy_probe: bool = False) -> int:
+    """configs[2] alone, for a profiler run: whole cq_qmatmul calls with 2, 8 and 16 activation rows on Q4_K and
+    Q8_0 weights of both decode shapes, launched eagerly `rounds` times over sixteen distinct weights per shape
+    (each call streams its weights from HBM), and the same timed with HIP events.  One JSON line."""
+    import ctypes as C
+
+    import torch
+
+    from candle_amd import qhip
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    L = qhip.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    gen = torch.Generator(device=dev)
+    vp = C.c_void_p
+    out = {"rounds": rounds, "weights_per_shape": 16, "whole_call_us": {}}
+    if copy_probe:   # a kernel of known HBM traffic, to calibrate FETCH_SIZE / WRITE_SIZE
+        src = torch.full((64 * 1024 * 1024,), 1.0, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    for dtname, dt in (("q4k", qhip.Q4K), ("q8_0", qhip.Q8_0)):
+        for n_out in (HIDDEN, FFN):
+            weights = []
+            for t in range(16):
+                gen.manual_seed(70_000 + 100 * dt + n_out + t)
+                w_ = torch.randn((n_out, HIDDEN), generator=gen, device=dev, dtype=torch.float32) * 0.02
+                weights.append(qhip.QWeight.zeros(dt, n_out, HIDDEN).quantize_(w_))
+                del w_
+            for mb in (2, 8, 16):
+                xb = torch.randn((mb, HIDDEN), generator=gen, device=dev, dtype=torch.float32)
+                yb = torch.empty((mb, n_out), device=dev, dtype=torch.float32)
+                wsb = torch.empty(max(weights[0].workspace_bytes(mb), 256), dtype=torch.uint8, device=dev)
+                s = vp(torch.cuda.current_stream().cuda_stream)
+
+                def sweep():
+                    for qw in weights:
+                        qhip.check(L.cq_qmatmul(qw.handle, vp(xb.data_ptr()), mb, vp(yb.data_ptr()), 0, vp(wsb.data_ptr()),
+                                                wsb.numel(), s))
+                sweep()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(rounds):
+                    sweep()
+                e1.record()
+                torch.cuda.synchronize()
+                out["whole_call_us"]["%s_%dx%d_m%d_eager" % (dtname, n_out, HIDDEN, mb)] = round(
+                    e0.elapsed_time(e1) * 1e3 / (rounds * len(weights)), 2)
+            del weights
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -143,9 +202,14 @@ def main() -> int:
                     help="instead of the bench: time an empty kernel and a pure 16-byte-per-lane streaming read of the "
                          "decode launches' sizes, eagerly and as a 225-node graph chain (what a single launch can reach "
                          "on this device), and print that as one JSON line")
+    ap.add_argument("--small-batch", type=int, default=0, metavar="ROUNDS",
+                    help="instead of the bench: only the small-batch calls (2, 8, 16 rows; Q4_K and Q8_0; both decode "
+                         "shapes), launched eagerly ROUNDS times, for a profiler run; prints one JSON line")
     args = ap.parse_args()
     if args.envelope:
         return envelope()
+    if args.small_batch > 0:
+        return small_batch_probe(args.small_batch, args.copy_probe)
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (one process, one MI355X); --gpus must be 1", file=sys.stderr)
         return 2
