@@ -287,7 +287,6 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g
                                              int lane, v4i (&bl)[8], v4i (&bh)[8], float &dw, v8h &wmin) {
     const int h = lane >> 5;
     dw = cq_h2f((uint16_t)(wb.dd & 0xffff));
-    const float dmin = cq_h2f((uint16_t)(wb.dd >> 16));
     const uint32_t rec[4] = {wb.rec.x, wb.rec.y, wb.rec.z, wb.rec.w};   // {sc[2g], sc[2g+1], mn[2g], mn[2g+1]}
 #pragma unroll
     for (int gi = 0; gi < 4; gi++) {
@@ -305,12 +304,7 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g
             bh[2 * gi + 1][i] = (int)pk_mul_u16(hi4, sh1);
         }
     }
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-        const float v = -dmin * (float)((rec[j >> 1] >> (16 + 8 * (j & 1))) & 0xff);
-        const _Float16 p1 = (_Float16)v;
-        wmin[j] = h == 0 ? p1 : (_Float16)(v - (float)p1);
-    }
+    wmin = __builtin_bit_cast(v8h, cq_min_term_operand(wb.dd, rec, h != 0));
 }
 
 // Q5K: the Q4K nibbles plus a fifth bit per quant (words {L, H} per 32 qs bytes, bit 8c + i for byte c
@@ -320,7 +314,6 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g
     const int h = lane >> 5;
     const uint32_t row = lane & 31;
     dw = cq_h2f((uint16_t)(wb.dd & 0xffff));
-    const float dmin = cq_h2f((uint16_t)(wb.dd >> 16));
     const uint32_t rec[4] = {wb.rec.x, wb.rec.y, wb.rec.z, wb.rec.w};   // {sc[2g], sc[2g+1], mn[2g], mn[2g+1]}
     const uint4 f0 = *(const uint4 *)(wl + 4096 + row * 32u), f1 = *(const uint4 *)(wl + 4096 + row * 32u + 16u);
     const uint32_t fl[4] = {f0.x, f0.z, f1.x, f1.z}, fh[4] = {f0.y, f0.w, f1.y, f1.w};
@@ -342,12 +335,7 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g
             bh[2 * gi + 1][i] = (int)__builtin_amdgcn_perm(pk_ashr7_i16(b13), pk_ashr7_i16(b02), 0x06020400u);
         }
     }
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-        const float v = -dmin * (float)((rec[j >> 1] >> (16 + 8 * (j & 1))) & 0xff);
-        const _Float16 p1 = (_Float16)v;
-        wmin[j] = h == 0 ? p1 : (_Float16)(v - (float)p1);
-    }
+    wmin = __builtin_bit_cast(v8h, cq_min_term_operand(wb.dd, rec, h != 0));
 }
 
 __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g, const WHead<CQ_DTYPE_Q6K> &wb,

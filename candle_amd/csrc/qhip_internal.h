@@ -223,6 +223,30 @@ __device__ __forceinline__ uint16_t cq_f2h(float f) {  // round-to-nearest-even
     __builtin_memcpy(&h, &v, 2);
     return h;
 }
+// Operand of the Q4K / Q5K min term on the f16 matrix core: the eight values -dmin * min_j of a block, each split in
+// two f16 pieces p1 = f16(v), p2 = f16(v - p1) (v has 17 significant bits; p1 + p2 == v).  Done in packed f16
+// arithmetic: the f16 product IS p1 (correctly rounded), and the f16 fma dmin * min - p1 is the product's rounding
+// error, exactly.  `dd` = d | dmin << 16 (f16 bits), `rec` = the block's four records {sc, sc, mn[2g], mn[2g+1]};
+// `second` picks the piece this lane carries.  Returns the eight halves as four words.
+typedef _Float16 cq_half2 __attribute__((ext_vector_type(2)));
+typedef uint32_t cq_u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ cq_u32x4 cq_min_term_operand(uint32_t dd, const uint32_t (&rec)[4], bool second) {
+    const uint32_t nd = (dd >> 16) ^ 0x8000u;   // -dmin
+    const cq_half2 ndmin = __builtin_bit_cast(cq_half2, nd | (nd << 16));
+    const cq_half2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+    cq_u32x4 out;
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        // the two min bytes as f16: 0x6400 | n is 1024 + n
+        const uint32_t n2 = __builtin_amdgcn_perm(rec[g], 0u, 0x0c070c06u) | 0x64006400u;
+        const cq_half2 mn = __builtin_bit_cast(cq_half2, n2) - k1024;
+        const cq_half2 p1 = ndmin * mn;
+        const cq_half2 p2 = __builtin_elementwise_fma(ndmin, mn, -p1);
+        out[g] = second ? __builtin_bit_cast(uint32_t, p2) : __builtin_bit_cast(uint32_t, p1);
+    }
+    return out;
+}
+
 // Rust `as i8` / `as u8` / `as i32` on f32: truncate toward zero, saturate, NaN -> 0.  That is
 // what the hardware conversions do for the 32-bit range (v_cvt_i32_f32 / v_cvt_u32_f32 round toward
 // zero, clamp, and turn NaN into 0), so the narrow types only add an integer clamp; no branches.

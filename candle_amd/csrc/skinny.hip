@@ -104,7 +104,6 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, int lane, const 
                                              v4i (&bh)[4], float &dw, v8h &wmin) {
     const uint32_t r = lane & 15, kq = lane >> 4;
     dw = cq_h2f((uint16_t)(wb.dd & 0xffff));
-    const float dmin = cq_h2f((uint16_t)(wb.dd >> 16));
     const uint32_t rec[4] = {wb.rec.x, wb.rec.y, wb.rec.z, wb.rec.w};
     // K-slice g = elements 64g..64g+63 = qs bytes 32g..32g+31, low nibbles for the first 32 elements
     // (quarters 0,1: sub-block 2g), high nibbles for the last 32 (quarters 2,3: sub-block 2g+1)
@@ -124,12 +123,7 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, int lane, const 
     }
     // min term operand: 32 K-slots = activation pieces [1,1,2,2] x weight pieces [1,2,1,2] of the
     // eight sub-block values -dmin*min_j
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-        const float v = -dmin * (float)((rec[j >> 1] >> (16 + 8 * (j & 1))) & 0xff);
-        const _Float16 p1 = (_Float16)v;
-        wmin[j] = (kq & 1) == 0 ? p1 : (_Float16)(v - (float)p1);
-    }
+    wmin = __builtin_bit_cast(v8h, cq_min_term_operand(wb.dd, rec, (kq & 1) != 0));
 }
 
 // Q5K: the quants are the Q4K nibbles plus a fifth bit (words {L, H} per 32 qs bytes, bit 8c + i for
@@ -138,7 +132,6 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, int lane, const 
                                              v4i (&bh)[4], float &dw, v8h &wmin) {
     const uint32_t r = lane & 15, kq = lane >> 4;
     dw = cq_h2f((uint16_t)(wb.dd & 0xffff));
-    const float dmin = cq_h2f((uint16_t)(wb.dd >> 16));
     const uint32_t rec[4] = {wb.rec.x, wb.rec.y, wb.rec.z, wb.rec.w};
     const uint32_t hi = kq >> 1, nsh = hi * 4, w0 = 4 * (kq & 1);   // first qs word of the lane's 16 bytes
     const uint4 f0 = *(const uint4 *)(wl + 2048 + r * 32u), f1 = *(const uint4 *)(wl + 2048 + r * 32u + 16u);
@@ -156,12 +149,7 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, int lane, const 
             bh[gi][i] = (int)__builtin_amdgcn_perm(pk_ashr7_i16(p13), pk_ashr7_i16(p02), 0x06020400u);
         }
     }
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-        const float v = -dmin * (float)((rec[j >> 1] >> (16 + 8 * (j & 1))) & 0xff);
-        const _Float16 p1 = (_Float16)v;
-        wmin[j] = (kq & 1) == 0 ? p1 : (_Float16)(v - (float)p1);
-    }
+    wmin = __builtin_bit_cast(v8h, cq_min_term_operand(wb.dd, rec, (kq & 1) != 0));
 }
 
 __device__ __forceinline__ void block_unpack(const uint8_t *wl, int lane, const WHead<CQ_DTYPE_Q6K> &wb, v4i (&bl)[4],
