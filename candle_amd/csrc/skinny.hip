@@ -674,6 +674,186 @@ __global__ void __launch_bounds__(kThreads) skinny_blk32_kernel(cq_weight w, cq_
     }
 }
 
+// ------------------------------------------- the same with everything of a workgroup in flight at once ----
+// The kernel above has one 256-element step per wave in flight and spends most of its life waiting (56 % at
+// s_waitcnt, the vector units 18 % busy).  Where every workgroup has one 16-row weight tile (n <= 16 x the number of
+// compute units) and the call's quantized rows fit the LDS beside the weights, every wave requests all it will need -
+// the activation slices, scales and weights of the K groups it owns (wave w: groups w, w + kWaves, ...) - right away,
+// a single memory round trip, and the arithmetic follows as the data lands.
+//   per K group g : act [RT][2 K-halves][8 rows][8 chunks], swizzled as above | d [8*RT rows][8] f32 |
+//                   Q4_0: bs [8*RT rows][8] i32 (sums of the activation blocks)
+//   then, per group: the 16 weight rows (Q8_0 4 KiB, Q4_0 2 KiB); a wave's first weight buffer also carries its
+//                   partial results (1 KiB per 16 activation rows)
+template <int DT, int RT> struct ResQ8 {
+    static constexpr bool Q4 = DT == CQ_DTYPE_Q4_0;
+    static constexpr int kWgt = Q4 ? 2048 : 4096;
+    static constexpr int oD = RT * 2048, oBs = oD + RT * 256;
+    static constexpr int kActGrp = oBs + (Q4 ? RT * 256 : 0);
+    static size_t bytes(int64_t kg) { return (size_t)kg * (kActGrp + kWgt); }
+};
+
+// m <= 8 * RT rows; n % 16 == 0, one tile per workgroup (gridDim.x == n / 16); at most kMaxBpw K groups per wave.
+template <int DT, int RT, int kWaves, bool DUMP>
+__global__ void __launch_bounds__(kWaves * 64) skinny_blk32_resident_kernel(cq_weight w, cq_act_view a, int64_t m,
+                                                                            float *__restrict__ y, cq_mfma_dump dump) {
+    typedef ResQ8<DT, RT> R;
+    constexpr bool Q4 = R::Q4;
+    constexpr int NT = (RT + 1) / 2;   // 16-row tiles
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t r = lane & 15, kq = lane >> 4;
+    const int64_t k = w.k, kg = w.k >> 8, kb = w.k >> 5;
+    const int64_t n_tile = (int64_t)blockIdx.x * 16;
+    uint8_t *wgt_base = smem + kg * R::kActGrp;
+
+    const uint32_t r8 = lane >> 3, c8 = lane & 7;
+    const uint32_t row_off = r8 * (uint32_t)k + ((c8 ^ r8) << 4);
+    const uint32_t q4_off = r8 * (uint32_t)(k >> 1) + ((c8 ^ r8) << 4);
+    // the scales (and block sums) of row l / 2, half l % 2 of its eight blocks; rows past the last one repeat it
+    // (their planes are not padded)
+    const int64_t srow = (int64_t)(lane >> 1) < m ? (lane >> 1) : m - 1;
+    const uint32_t sc_off = (uint32_t)(srow * kb * 4) + (lane & 1) * 16u;
+    const uint32_t w4_col = (r >> 3) * 1024u + (r & 7) * 128u + (kq & 1) * 8u, w4_shift = 4 * (kq >> 1);
+    uint32_t w_col[4], a_col[NT][4];
+#pragma unroll
+    for (uint32_t c = 0; c < 4; c++) w_col[c] = (r >> 3) * 2048u + (r & 7) * 128u + (((2 * c + (kq >> 1)) ^ (r & 7)) << 4) + (kq & 1) * 8u;
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const uint32_t row = t * 16 + r < 8u * RT ? t * 16 + r : 8u * RT - 1;
+#pragma unroll
+        for (uint32_t c = 0; c < 4; c++)
+            a_col[t][c] = (row >> 3) * 2048u + (row & 7) * 128u + (((2 * c + (kq >> 1)) ^ (row & 7)) << 4) + (kq & 1) * 8u;
+    }
+
+    // ---- everything this wave will need, requested at once
+    uint4 dwv[kMaxBpw];
+#pragma unroll
+    for (int j = 0; j < kMaxBpw; j++) {
+        const int64_t g = wave + (int64_t)j * kWaves;
+        if (g < kg) dwv[j] = *(const uint4 *)(w.p1 + ((n_tile + r) * kb + g * 8) * 2);
+    }
+#pragma unroll
+    for (int j = 0; j < kMaxBpw; j++) {
+        const int64_t g = wave + (int64_t)j * kWaves;
+        if (g < kg) {
+            uint8_t *act = smem + g * R::kActGrp, *wl = wgt_base + g * R::kWgt;
+#pragma unroll
+            for (int i = 0; i < 2 * RT; i++) {
+                const int rg = i >> 1, kh = i & 1;
+                dma16(a.qs + (int64_t)(rg * 8) * k + g * 256 + kh * 128, row_off, act + i * 1024);
+            }
+            if (lane < 16 * RT) dma16((const uint8_t *)(a.d + g * 8), sc_off, act + R::oD);
+            if (Q4 && lane < 16 * RT) dma16((const uint8_t *)(a.bsum32 + g * 8), sc_off, act + R::oBs);
+            if (Q4) {
+#pragma unroll
+                for (int rg = 0; rg < 2; rg++) dma16(w.p0 + (n_tile + rg * 8) * (k >> 1) + g * 128, q4_off, wl + rg * 1024);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int rg = i >> 1, kh = i & 1;
+                    dma16(w.p0 + (n_tile + rg * 8) * k + g * 256 + kh * 128, row_off, wl + i * 1024);
+                }
+            }
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0);   // everything above has landed
+
+    v4f out[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) out[t] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < kMaxBpw; j++) {
+        const int64_t g = wave + (int64_t)j * kWaves;
+        if (g < kg) {
+            const uint8_t *act = smem + g * R::kActGrp, *wl = wgt_base + g * R::kWgt;
+            const uint32_t dww[4] = {dwv[j].x, dwv[j].y, dwv[j].z, dwv[j].w};
+#pragma unroll
+            for (int b = 0; b < 8; b++) {
+                const float dw = cq_h2f((uint16_t)(dww[b >> 1] >> (16 * (b & 1))));
+                long wv;
+                if (Q4) {
+                    const uint2 raw = *(const uint2 *)(wl + w4_col + (((uint32_t)b ^ (r & 7)) << 4));
+                    const uint32_t lo = (raw.x >> w4_shift) & 0x0F0F0F0Fu, hi = (raw.y >> w4_shift) & 0x0F0F0F0Fu;
+                    wv = (long)(((uint64_t)hi << 32) | lo);
+                } else {
+                    wv = *(const long *)(wl + w_col[b & 3] + (b >> 2) * 1024);
+                }
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+                    const long av = *(const long *)(act + a_col[t][b & 3] + (b >> 2) * 1024);
+                    const v4i acc = __builtin_amdgcn_mfma_i32_16x16x32_i8(av, wv, (v4i){0, 0, 0, 0}, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        // scales of result row 4kq + i of tile t (rows past the held groups: the last one, not stored)
+                        const uint32_t srow_i = t * 16 + 4 * kq + i < 8u * RT ? t * 16 + 4 * kq + i : 8u * RT - 1;
+                        const float da = *(const float *)(act + R::oD + srow_i * 32 + b * 4);
+                        const int I = Q4 ? acc[i] - 8 * *(const int32_t *)(act + R::oBs + srow_i * 32 + b * 4) : acc[i];
+                        if (DUMP) {
+                            const int64_t orow = t * 16 + kq * 4 + i;
+                            if (orow < m) dump.i[(orow * w.n + n_tile + r) * kb + g * 8 + b] = I;
+                        } else {
+                            out[t][i] = __builtin_fmaf((float)I * dw, da, out[t][i]);
+                        }
+                    }
+                }
+            }
+        }
+    }
+    if (DUMP) return;
+
+    // ---- sum the waves' partial tiles in wave order (through each wave's first weight buffer)
+    if (wave < kg) {
+#pragma unroll
+        for (int t = 0; t < NT; t++) *(v4f *)(wgt_base + (int64_t)wave * R::kWgt + t * 1024 + lane * 16) = out[t];
+    }
+    __syncthreads();
+    if (wave < NT) {
+        v4f s = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+        const int64_t nw = kg < kWaves ? kg : kWaves;   // waves that own a group
+        for (int64_t o = 0; o < nw; o++) {
+            const v4f p = *(const v4f *)(wgt_base + o * R::kWgt + wave * 1024 + lane * 16);
+            s += p;
+        }
+        const int64_t col = n_tile + r;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int64_t row = wave * 16 + kq * 4 + i;
+            if (row < m) y[row * w.n + col] = s[i];
+        }
+    }
+}
+
+template <int DT, int RT, int NW, bool DUMP>
+hipError_t launch_blk32_res_inst(const cq_weight *w, cq_act_view a, int64_t m, float *y, size_t lds, cq_mfma_dump d, hipStream_t s) {
+    if (hipError_t e = cq_ensure_lds<skinny_blk32_resident_kernel<DT, RT, NW, DUMP>>(w->dev, lds); e != hipSuccess) return e;
+    CQ_LAUNCH((skinny_blk32_resident_kernel<DT, RT, NW, DUMP>), (unsigned)(w->n / 16), NW * 64, lds, s, *w, a, m, y, d);
+    return hipGetLastError();
+}
+// Takes the launch (true) where the resident kernel applies: one tile per workgroup, all operands in the LDS.
+template <int DT, int RT, bool DUMP>
+bool launch_blk32_res_rt(const cq_weight *w, cq_act_view a, int64_t m, float *y, cq_mfma_dump d, hipStream_t s, hipError_t *err) {
+    const int64_t kg = w->k >> 8, tiles = w->n / 16;
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (cus <= 0) cus = 256;
+    if (tiles > cus) return false;
+    const bool sixteen = kg > 8;
+    if (kg > (sixteen ? 16 : 8) * kMaxBpw) return false;
+    const size_t lds = ResQ8<DT, RT>::bytes(kg);
+    if (lds > (size_t)kMaxLds) return false;
+    *err = sixteen ? launch_blk32_res_inst<DT, RT, 16, DUMP>(w, a, m, y, lds, d, s) : launch_blk32_res_inst<DT, RT, 8, DUMP>(w, a, m, y, lds, d, s);
+    return true;
+}
+template <int DT, bool DUMP>
+bool launch_blk32_res(const cq_weight *w, cq_act_view a, int64_t m, float *y, cq_mfma_dump d, hipStream_t s, hipError_t *err) {
+    if (m <= 8) return launch_blk32_res_rt<DT, 1, DUMP>(w, a, m, y, d, s, err);
+    if (m <= 16) return launch_blk32_res_rt<DT, 2, DUMP>(w, a, m, y, d, s, err);
+    if (m <= 24) return launch_blk32_res_rt<DT, 3, DUMP>(w, a, m, y, d, s, err);
+    if (m <= 32) return launch_blk32_res_rt<DT, 4, DUMP>(w, a, m, y, d, s, err);
+    return false;
+}
+
 // DUMP (all launchers below): the launch cq_launch_skinny would make, storing the block integers through `d`.
 template <int DT, int RT, bool DUMP>
 hipError_t launch_blk32_rt(const cq_weight *w, cq_act_view a, int64_t m0, int64_t m, float *y, cq_mfma_dump d, hipStream_t s) {
@@ -765,9 +945,13 @@ hipError_t launch_any(const cq_weight *w, cq_act_view a, int act_dtype, int64_t 
     if (!cq_skinny_supported(w, act_dtype)) return hipErrorNotSupported;
     if (m == 0) return hipSuccess;
     if (a.m_stride < (m + 31) / 32 * 32) return hipErrorInvalidValue;   // whole 8-row groups are copied
+    hipError_t e = hipSuccess;
+#ifndef CQ_EXP_NO_RESIDENT
+    if (w->dtype == CQ_DTYPE_Q8_0 && launch_blk32_res<CQ_DTYPE_Q8_0, DUMP>(w, a, m, y, d, s, &e)) return e;
+    if (w->dtype == CQ_DTYPE_Q4_0 && launch_blk32_res<CQ_DTYPE_Q4_0, DUMP>(w, a, m, y, d, s, &e)) return e;
+#endif
     if (w->dtype == CQ_DTYPE_Q8_0) return launch_blk32<CQ_DTYPE_Q8_0, DUMP>(w, a, m, y, d, s);
     if (w->dtype == CQ_DTYPE_Q4_0) return launch_blk32<CQ_DTYPE_Q4_0, DUMP>(w, a, m, y, d, s);
-    hipError_t e = hipSuccess;
 #ifndef CQ_EXP_NO_RESIDENT
     if (w->dtype == CQ_DTYPE_Q4K && launch_res<CQ_DTYPE_Q4K, DUMP>(w, a, m, y, d, s, &e)) return e;
     if (w->dtype == CQ_DTYPE_Q5K && launch_res<CQ_DTYPE_Q5K, DUMP>(w, a, m, y, d, s, &e)) return e;
