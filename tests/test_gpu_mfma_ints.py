@@ -109,14 +109,40 @@ def test_tile_kernel_integers(qh, dt, m, k, n):
     check_dump(qh, dt, qh.MFMA_TILE, m, k, n, 13 * dt + m + k + n)
 
 
-@pytest.mark.parametrize("x_scale", [1e-2, 30.0])
+@pytest.mark.parametrize("x_scale", [1e-2, 1.0, 30.0, 500.0])
 @pytest.mark.parametrize("kernel", ["skinny", "tile"])
 def test_min_term_error_bound_across_magnitudes(qh, kernel, x_scale):
-    """The split-f16 min term keeps its bound for activations a hundred times smaller and thirty times larger than
-    unit variance (|d8 * bsum32| stays inside the f16 range up to activations of about 2000)."""
+    """The split-f16 min term keeps its bound for activations from a hundred times smaller to five hundred times
+    larger than unit variance (|d8 * bsum32| leaves the f16 range for activations beyond about 2000 throughout a
+    sub-block, and the pieces lose bits below about 1e-3: the documented range of the matrix-core kernels)."""
     kid = qh.MFMA_SKINNY if kernel == "skinny" else qh.MFMA_TILE
     m = 16 if kernel == "skinny" else 70
     check_dump(qh, orc.Q4K, kid, m, 1024, 64, 5, x_scale)
+
+
+@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q5K, orc.Q6K])
+@pytest.mark.parametrize("m,k,n", [(16, 2048, 64), (70, 1024, 96), (512, 512, 64)])
+def test_rows_of_different_magnitudes(qh, dt, m, k, n):
+    """One batch whose rows span five orders of magnitude (0.01 .. 1000), one row with a block a thousand times the
+    others and one all-zero row: every row against the oracle at the usual bars, on both matrix-core kernels."""
+    rng = np.random.default_rng(m + k + n + int(dt))
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    scales = np.float32(10.0) ** rng.integers(-2, 4, size=m).astype(np.float32)
+    scales[2] = 1.0
+    x *= scales[:, None]
+    x[1] = 0.0
+    x[2, 256:512] *= np.float32(1e3)          # one block dwarfs the others of its row
+    blocks = orc.quantize(dt, w)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    want = orc.matmul(dt, x, blocks, n).astype(np.float64)
+    for flags in (qh.FLAG_FORCE_SKINNY, qh.FLAG_FORCE_GEMM):
+        got = qh.qmatmul(qw, dev(x), flags).cpu().numpy().astype(np.float64)
+        assert np.all(np.isfinite(got))
+        for r in range(m):
+            nrm = np.linalg.norm(want[r])
+            assert np.linalg.norm(got[r] - want[r]) <= 1e-4 * nrm + 1e-38, (flags, r, float(scales[r]))
+            assert np.abs(got[r] - want[r]).max() <= 1e-3 * nrm + 1e-38, (flags, r)
 
 
 @pytest.mark.parametrize("dt,k,n", [(orc.Q4K, 4096, 14336), (orc.Q6K, 14336, 4096)])
