@@ -946,17 +946,13 @@ hipError_t launch_any(const cq_weight *w, cq_act_view a, int act_dtype, int64_t 
     if (m == 0) return hipSuccess;
     if (a.m_stride < (m + 31) / 32 * 32) return hipErrorInvalidValue;   // whole 8-row groups are copied
     hipError_t e = hipSuccess;
-#ifndef CQ_EXP_NO_RESIDENT
     if (w->dtype == CQ_DTYPE_Q8_0 && launch_blk32_res<CQ_DTYPE_Q8_0, DUMP>(w, a, m, y, d, s, &e)) return e;
     if (w->dtype == CQ_DTYPE_Q4_0 && launch_blk32_res<CQ_DTYPE_Q4_0, DUMP>(w, a, m, y, d, s, &e)) return e;
-#endif
     if (w->dtype == CQ_DTYPE_Q8_0) return launch_blk32<CQ_DTYPE_Q8_0, DUMP>(w, a, m, y, d, s);
     if (w->dtype == CQ_DTYPE_Q4_0) return launch_blk32<CQ_DTYPE_Q4_0, DUMP>(w, a, m, y, d, s);
-#ifndef CQ_EXP_NO_RESIDENT
     if (w->dtype == CQ_DTYPE_Q4K && launch_res<CQ_DTYPE_Q4K, DUMP>(w, a, m, y, d, s, &e)) return e;
     if (w->dtype == CQ_DTYPE_Q5K && launch_res<CQ_DTYPE_Q5K, DUMP>(w, a, m, y, d, s, &e)) return e;
     if (w->dtype == CQ_DTYPE_Q6K && launch_res<CQ_DTYPE_Q6K, DUMP>(w, a, m, y, d, s, &e)) return e;
-#endif
     if (w->dtype == CQ_DTYPE_Q4K) return launch_dt<CQ_DTYPE_Q4K, DUMP>(w, a, m, y, d, s);
     if (w->dtype == CQ_DTYPE_Q5K) return launch_dt<CQ_DTYPE_Q5K, DUMP>(w, a, m, y, d, s);
     return launch_dt<CQ_DTYPE_Q6K, DUMP>(w, a, m, y, d, s);

@@ -703,3 +703,27 @@ def test_few_rows_one_launch_equals_single_rows(qh, dt, m, k, n):
     two = qh.qmatmul(qw, xd, qh.FLAG_STAGED_ACT)
     assert (torch.linalg.norm(got - two) / torch.linalg.norm(two)).item() <= 2e-6
     check_f32(got.cpu().numpy(), orc.matmul(dt, x, blocks, n))
+
+
+# ------------------------------------------------------------- seeded random shapes ----
+def _random_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(count):
+        dt = int(rng.choice(WEIGHT_DTYPES))
+        blk = 32 if dt in (orc.Q4_0, orc.Q8_0) else 256
+        k = blk * int(rng.integers(1, (2048 // blk) + 1))
+        m = int(rng.choice([1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 31, 32, 33, 40, 64, 65, 70]))
+        n = int(rng.choice([1, 2, 7, 8, 15, 16, 17, 31, 32, 33, 48, 63, 64, 96, 100, 128, 255, 256, 257, 300]))
+        cases.append((dt, m, k, n))
+    return cases
+
+
+@pytest.mark.parametrize("dt,m,k,n", _random_cases(96, 20240611))
+def test_random_shapes_match_oracle(qh, dt, m, k, n):
+    """Whatever kernel the automatic choice lands on for a shape (one-launch decode, several rows in one launch,
+    split-K, tile, dot-product fallbacks for ragged n and k): every row against the oracle at the usual bars."""
+    w, x = make_inputs(dt * 1000003 + m * 10007 + k * 101 + n, m, k, n, outliers=True)
+    blocks = orc.quantize(dt, w)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    check_f32(qh.qmatmul(qw, dev(x)).cpu().numpy(), orc.matmul(dt, x, blocks, n))
