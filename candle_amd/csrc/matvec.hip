@@ -82,45 +82,6 @@ template <int DT> __device__ __forceinline__ uint32_t piece_off(const LdsRow r, 
     return (o >= 4 ? r.hi : r.lo) + (uint32_t)(8 * b + 4 * h + (o & 3)) * 16;
 }
 
-// ------------------------------------------------------------------ wave reductions (DPP) ----
-template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
-}
-template <int CTRL> __device__ __forceinline__ int dpp_i(int v) {
-    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
-}
-constexpr int kQuadSwap1 = 0xB1;   // quad_perm [1,0,3,2]
-constexpr int kQuadSwap2 = 0x4E;   // quad_perm [2,3,0,1]
-constexpr int kHalfMirror = 0x141; // lanes i <-> 7-i inside each 8
-constexpr int kRowMirror = 0x140;  // lanes i <-> 15-i inside each 16
-
-__device__ __forceinline__ float readlane_f(float v, int l) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
-}
-// Sum over the 64 lanes, valid in every lane.
-__device__ __forceinline__ float wave_sum(float v) {
-    v += dpp_f<kQuadSwap1>(v);
-    v += dpp_f<kQuadSwap2>(v);
-    v += dpp_f<kHalfMirror>(v);
-    v += dpp_f<kRowMirror>(v);
-    return readlane_f(v, 0) + readlane_f(v, 16) + readlane_f(v, 32) + readlane_f(v, 48);
-}
-__device__ __forceinline__ float wave_max(float v) {
-    v = fmaxf(v, dpp_f<kQuadSwap1>(v));
-    v = fmaxf(v, dpp_f<kQuadSwap2>(v));
-    v = fmaxf(v, dpp_f<kHalfMirror>(v));
-    v = fmaxf(v, dpp_f<kRowMirror>(v));
-    return fmaxf(fmaxf(readlane_f(v, 0), readlane_f(v, 16)), fmaxf(readlane_f(v, 32), readlane_f(v, 48)));
-}
-__device__ __forceinline__ int wave_min_i(int v) {
-    v = min(v, dpp_i<kQuadSwap1>(v));
-    v = min(v, dpp_i<kQuadSwap2>(v));
-    v = min(v, dpp_i<kHalfMirror>(v));
-    v = min(v, dpp_i<kRowMirror>(v));
-    return min(min(__builtin_amdgcn_readlane(v, 0), __builtin_amdgcn_readlane(v, 16)),
-               min(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
-}
-
 // ------------------------------------------------ activation quantizer inside the matvec ----
 __device__ __forceinline__ uint32_t pack4(int8_t a, int8_t b, int8_t c, int8_t d) {
     return (uint32_t)(uint8_t)a | ((uint32_t)(uint8_t)b << 8) | ((uint32_t)(uint8_t)c << 16) | ((uint32_t)(uint8_t)d << 24);

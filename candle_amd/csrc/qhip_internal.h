@@ -223,6 +223,45 @@ __device__ __forceinline__ uint16_t cq_f2h(float f) {  // round-to-nearest-even
     __builtin_memcpy(&h, &v, 2);
     return h;
 }
+// ------------------------------------------------------------------ wave reductions (DPP) ----
+template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+template <int CTRL> __device__ __forceinline__ int dpp_i(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
+}
+constexpr int kQuadSwap1 = 0xB1;   // quad_perm [1,0,3,2]
+constexpr int kQuadSwap2 = 0x4E;   // quad_perm [2,3,0,1]
+constexpr int kHalfMirror = 0x141; // lanes i <-> 7-i inside each 8
+constexpr int kRowMirror = 0x140;  // lanes i <-> 15-i inside each 16
+
+__device__ __forceinline__ float readlane_f(float v, int l) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+}
+// Sum over the 64 lanes, valid in every lane.
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_f<kQuadSwap1>(v);
+    v += dpp_f<kQuadSwap2>(v);
+    v += dpp_f<kHalfMirror>(v);
+    v += dpp_f<kRowMirror>(v);
+    return readlane_f(v, 0) + readlane_f(v, 16) + readlane_f(v, 32) + readlane_f(v, 48);
+}
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, dpp_f<kQuadSwap1>(v));
+    v = fmaxf(v, dpp_f<kQuadSwap2>(v));
+    v = fmaxf(v, dpp_f<kHalfMirror>(v));
+    v = fmaxf(v, dpp_f<kRowMirror>(v));
+    return fmaxf(fmaxf(readlane_f(v, 0), readlane_f(v, 16)), fmaxf(readlane_f(v, 32), readlane_f(v, 48)));
+}
+__device__ __forceinline__ int wave_min_i(int v) {
+    v = min(v, dpp_i<kQuadSwap1>(v));
+    v = min(v, dpp_i<kQuadSwap2>(v));
+    v = min(v, dpp_i<kHalfMirror>(v));
+    v = min(v, dpp_i<kRowMirror>(v));
+    return min(min(__builtin_amdgcn_readlane(v, 0), __builtin_amdgcn_readlane(v, 16)),
+               min(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
+}
+
 // Operand of the Q4K / Q5K min term on the f16 matrix core: the eight values -dmin * min_j of a block, each split in
 // two f16 pieces p1 = f16(v), p2 = f16(v - p1) (v has 17 significant bits; p1 + p2 == v).  Done in packed f16
 // arithmetic: the f16 product IS p1 (correctly rounded), and the f16 fma dmin * min - p1 is the product's rounding

@@ -53,17 +53,17 @@ __device__ __forceinline__ int8_t round_to_i8(float v) { return cq_as_i8(roundf(
 template <bool AOS, bool Q8_1>
 __device__ __forceinline__ void q8_0_chunk(const float4 f, bool active, int64_t row, int64_t e0, int64_t k, const Sink &out) {
     float amax = fmaxf(fmaxf(fmaxf(fmaxf(0.0f, fabsf(f.x)), fabsf(f.y)), fabsf(f.z)), fabsf(f.w));
-    amax = fmaxf(amax, __shfl_xor(amax, 1));
-    amax = fmaxf(amax, __shfl_xor(amax, 2));
-    amax = fmaxf(amax, __shfl_xor(amax, 4));
+    amax = fmaxf(amax, dpp_f<kQuadSwap1>(amax));
+    amax = fmaxf(amax, dpp_f<kQuadSwap2>(amax));
+    amax = fmaxf(amax, dpp_f<kHalfMirror>(amax));  // quads hold one value each: the mirror pairs them
     const float d = amax / 127.0f;
     const float id = d != 0.0f ? 1.0f / d : 0.0f;
     const int8_t q0 = round_to_i8(f.x * id), q1 = round_to_i8(f.y * id), q2 = round_to_i8(f.z * id),
                  q3 = round_to_i8(f.w * id);
     int sum = (int)q0 + (int)q1 + (int)q2 + (int)q3;
-    sum += __shfl_xor(sum, 1);
-    sum += __shfl_xor(sum, 2);
-    sum += __shfl_xor(sum, 4);
+    sum += dpp_i<kQuadSwap1>(sum);
+    sum += dpp_i<kQuadSwap2>(sum);
+    sum += dpp_i<kHalfMirror>(sum);
     if (!active) return;
     const uint32_t packed = (uint32_t)(uint8_t)q0 | ((uint32_t)(uint8_t)q1 << 8) | ((uint32_t)(uint8_t)q2 << 16) |
                             ((uint32_t)(uint8_t)q3 << 24);
@@ -123,23 +123,19 @@ __device__ __forceinline__ void q8k_chunk(const float4 f, int64_t row, int64_t b
     const int lane = threadIdx.x & 63;
     const int64_t blk = row * (k / 256) + b_in_row;
 
-    // first index with the largest |x| (strict `<` in the reference keeps the earliest)
-    float amax = 0.0f, max = 0.0f;
+    // The first element whose |x| equals the block maximum decides the sign of the scale (strict
+    // `<` in the reference keeps the earliest).  Reductions run on DPP operands, not through LDS.
+    const float a0 = fabsf(f.x), a1 = fabsf(f.y), a2 = fabsf(f.z), a3 = fabsf(f.w);
+    const float amax = wave_max(fmaxf(fmaxf(fmaxf(fmaxf(0.0f, a0), a1), a2), a3));
     int idx = 0x7fffffff;
-    {
-        const float v[4] = {f.x, f.y, f.z, f.w};
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            if (amax < fabsf(v[i])) { amax = fabsf(v[i]); max = v[i]; idx = 4 * lane + i; }
-        }
-    }
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const float oa = __shfl_xor(amax, off);
-        const float om = __shfl_xor(max, off);
-        const int oi = __shfl_xor(idx, off);
-        if (oa > amax || (oa == amax && oi < idx)) { amax = oa; max = om; idx = oi; }
-    }
+    if (a3 == amax) idx = 4 * lane + 3;
+    if (a2 == amax) idx = 4 * lane + 2;
+    if (a1 == amax) idx = 4 * lane + 1;
+    if (a0 == amax) idx = 4 * lane;
+    idx = wave_min_i(idx);
+    const int sel = idx & 3;
+    const float cand = sel == 0 ? f.x : (sel == 1 ? f.y : (sel == 2 ? f.z : f.w));
+    const float max = readlane_f(cand, __builtin_amdgcn_readfirstlane(idx >> 2));
 
     uint32_t packed = 0;
     int sum = 0;
@@ -156,8 +152,8 @@ __device__ __forceinline__ void q8k_chunk(const float4 f, int64_t row, int64_t b
         d = 1.0f / iscale;
         if (SCALED) d *= dscale;
     }
-    sum += __shfl_xor(sum, 1);
-    sum += __shfl_xor(sum, 2);  // lanes 4j..4j+3 now hold bsums[j]
+    sum += dpp_i<kQuadSwap1>(sum);
+    sum += dpp_i<kQuadSwap2>(sum);  // lanes 4j..4j+3 now hold bsums[j]
     if (AOS) {
         uint8_t *b = out.aos + blk * 292;  // 292 = 4 * 73: 4-byte aligned
         if (lane == 0) *(float *)b = d;
@@ -171,7 +167,7 @@ __device__ __forceinline__ void q8k_chunk(const float4 f, int64_t row, int64_t b
         // quants of sub-block j) as two f16 pieces p1 + p2 (22 significant bits), [p1[8] | p2[8]].
         const int64_t tb = b_in_row * out.v.m_stride + row;
         if (lane == 0) out.v.dT[tb] = d;
-        const int sum32 = sum + __shfl_xor(sum, 4);
+        const int sum32 = sum + dpp_i<kHalfMirror>(sum);  // eight lanes = one 32-element sub-block
         if ((lane & 7) == 0) {
             const float v = d * (float)sum32;
             const _Float16 p1 = (_Float16)v;
