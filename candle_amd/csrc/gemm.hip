@@ -10,7 +10,7 @@
 // The sub-block scales sit between the int8 contraction and the accumulator, so they are folded
 // into the int8 weights as two digits and the block is contracted with two MFMAs per K-slice:
 //   Q4K:  sc = 8*sh + sl (3-bit digits): operands sh*q4, sl*q4 <= 105;  I = 8*acc_hi + acc_lo
-//   Q6K:  P = sc*(q6-32) (13 bits signed): operands P >> 7, P & 127;    I = 128*acc_hi + acc_lo
+//   Q6K:  P = sc*(q6-32) (13 bits signed) = 256*ph + pl, pl in [-128, 127];  I = 256*acc_hi + acc_lo
 //   Q5K:  as Q4K with 5-bit quants (k_quants.rs:1361-1447): P = sc*q5 (11 bits), split like Q6K's
 // I is the same integer as on the CPU.  The Q4K min term is a small f32 contraction over the
 // eight sub-blocks; it runs on the f16 MFMA with both factors split in two f16 pieces (products
@@ -67,14 +67,6 @@ template <int DT, int MT> struct Tile {
 
 __device__ __forceinline__ uint32_t pk_mul_u16(uint32_t a, uint32_t b) {
     const us2 r = __builtin_bit_cast(us2, a) * __builtin_bit_cast(us2, b);
-    return __builtin_bit_cast(uint32_t, r);
-}
-__device__ __forceinline__ uint32_t pk_sub_u16(uint32_t a, uint32_t b) {
-    const us2 r = __builtin_bit_cast(us2, a) - __builtin_bit_cast(us2, b);
-    return __builtin_bit_cast(uint32_t, r);
-}
-__device__ __forceinline__ uint32_t pk_ashr7_i16(uint32_t a) {
-    const ss2 r = __builtin_bit_cast(ss2, a) >> (ss2){7, 7};
     return __builtin_bit_cast(uint32_t, r);
 }
 __device__ __forceinline__ uint32_t dup16(uint32_t v) { return (v & 0xffffu) | (v << 16); }
@@ -308,7 +300,7 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g
 }
 
 // Q5K: the Q4K nibbles plus a fifth bit per quant (words {L, H} per 32 qs bytes, bit 8c + i for byte c
-// of qs word i); scale times quant has up to 11 bits and is split at bit 7, as for Q6K.
+// of qs word i); scale times quant has up to 11 bits and is split as Q6K's products are.
 __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g, const WHead<CQ_DTYPE_Q5K> &wb,
                                              int lane, v4i (&bl)[8], v4i (&bh)[8], float &dw, v8h &wmin) {
     const int h = lane >> 5;
@@ -321,18 +313,19 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g
     for (int gi = 0; gi < 4; gi++) {
         // qs bytes 32g + 16h + [0,16) = qs words 4h .. 4h+3: low nibbles = K-slice 2g, high nibbles = slice 2g+1
         const uint4 q = *(const uint4 *)(wl + g.col[gi]);
-        const uint32_t s0 = dup16(rec[gi] & 0xff), s1 = dup16((rec[gi] >> 8) & 0xff);
+        const unsigned short s0 = (unsigned short)(rec[gi] & 0xff), s1 = (unsigned short)((rec[gi] >> 8) & 0xff);
         const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const uint32_t lo5 = (qw[i] & 0x0F0F0F0Fu) | (((fl[gi] >> (4 * h + i)) & 0x01010101u) << 4);
             const uint32_t hi5 = ((qw[i] >> 4) & 0x0F0F0F0Fu) | (((fh[gi] >> (4 * h + i)) & 0x01010101u) << 4);
-            const uint32_t a02 = pk_mul_u16(lo5 & 0x00FF00FFu, s0), a13 = pk_mul_u16((lo5 >> 8) & 0x00FF00FFu, s0);
-            const uint32_t b02 = pk_mul_u16(hi5 & 0x00FF00FFu, s1), b13 = pk_mul_u16((hi5 >> 8) & 0x00FF00FFu, s1);
-            bl[2 * gi][i] = (int)(__builtin_amdgcn_perm(a13, a02, 0x06020400u) & 0x7F7F7F7Fu);
-            bh[2 * gi][i] = (int)__builtin_amdgcn_perm(pk_ashr7_i16(a13), pk_ashr7_i16(a02), 0x06020400u);
-            bl[2 * gi + 1][i] = (int)(__builtin_amdgcn_perm(b13, b02, 0x06020400u) & 0x7F7F7F7Fu);
-            bh[2 * gi + 1][i] = (int)__builtin_amdgcn_perm(pk_ashr7_i16(b13), pk_ashr7_i16(b02), 0x06020400u);
+            int lo, hi;
+            cq_scaled_digits(lo5, s0, (unsigned short)128, lo, hi);   // digits of sc * q5, sub-block 2g
+            bl[2 * gi][i] = lo;
+            bh[2 * gi][i] = hi;
+            cq_scaled_digits(hi5, s1, (unsigned short)128, lo, hi);   // sub-block 2g+1
+            bl[2 * gi + 1][i] = lo;
+            bh[2 * gi + 1][i] = hi;
         }
     }
     wmin = __builtin_bit_cast(v8h, cq_min_term_operand(wb.dd, rec, h != 0));
@@ -359,21 +352,19 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g
         const int sb = 4 * x + nib;                  // scale byte index for h = 0; h adds 2 (same word)
         const uint32_t sw = scw[sb >> 2];
         const int sc = (int)(int8_t)((sw >> (8 * (sb & 3) + 16 * h)) & 0xff);
-        const uint32_t sc16 = dup16((uint32_t)sc);
+        const unsigned short sc16 = (unsigned short)sc, c16 = (unsigned short)(128 - 32 * sc);
         const uint32_t qw[4] = {ql[x].x, ql[x].y, ql[x].z, ql[x].w};
         const uint32_t hw[2] = {qhv[x].x, qhv[x].y};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const uint32_t H = hw[i >> 1];
-            const int sh = (i & 1) * 4 + 2 * nib;
-            const uint32_t q6 = ((qw[i] >> (4 * nib)) & 0x0F0F0F0Fu) | (((H >> sh) & 0x03030303u) << 4);
-            // the four elements as 16-bit lanes, minus 32, times the group scale (low 16 bits kept)
-            const uint32_t e02 = pk_sub_u16(q6 & 0x00FF00FFu, 0x00200020u);
-            const uint32_t e13 = pk_sub_u16((q6 >> 8) & 0x00FF00FFu, 0x00200020u);
-            const uint32_t p02 = pk_mul_u16(e02, sc16), p13 = pk_mul_u16(e13, sc16);
-            // gather bytes [p02.0, p13.0, p02.2, p13.2]
-            bl[s][i] = (int)(__builtin_amdgcn_perm(p13, p02, 0x06020400u) & 0x7F7F7F7Fu);
-            bh[s][i] = (int)__builtin_amdgcn_perm(pk_ashr7_i16(p13), pk_ashr7_i16(p02), 0x06020400u);
+            const int sh = (i & 1) * 4 + 2 * nib;   // where the two high bits sit in H's bytes; wanted at bit 4
+            const uint32_t hb = sh < 4 ? H << (4 - sh) : H >> (sh - 4);
+            const uint32_t q6 = ((qw[i] >> (4 * nib)) & 0x0F0F0F0Fu) | (hb & 0x30303030u);
+            int lo, hi;
+            cq_scaled_digits(q6, sc16, c16, lo, hi);   // digits of sc * (q6 - 32)
+            bl[s][i] = lo;
+            bh[s][i] = hi;
         }
     }
     wmin = v8h{};
@@ -395,7 +386,7 @@ __device__ __forceinline__ void block_step(const uint8_t *__restrict__ cur, uint
                                            uint8_t *__restrict__ wl, const cq_weight &w, const cq_act_view &a,
                                            const LaneGeo &g, int64_t m0, int64_t n_tile, bool n_ok, bool more, int64_t b,
                                            int wave, int lane, const WHead<DT> &hcur, v16f (&out)[MT], const DumpLane &dl) {
-    constexpr int SHIFT = DT == CQ_DTYPE_Q4K ? 3 : 7;
+    constexpr int SHIFT = DT == CQ_DTYPE_Q4K ? 3 : 8;
     constexpr int SPLIT = TRAIL ? MT / 2 : MT;   // tiles [SPLIT, MT) follow the barrier
     v4i bl[8], bh[8];
     float dw = 0.0f;

@@ -262,6 +262,23 @@ __device__ __forceinline__ int wave_min_i(int v) {
                min(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
 }
 
+// Q5K / Q6K on the int8 matrix core: the four byte-sized quants of word `q`, each times the group scale (plus an
+// offset), as two int8 digit words.  In 16-bit lanes T = q * s + c with c = 128 + offset (mod 2^16), so that
+// P = q * s + offset = T - 128 = 256 * hi + lo with hi = the high byte of T (signed) and lo = its low byte ^ 0x80 in
+// [-128, 127]; needs |P| <= 2^15 - 256.  Q6K: s = the group scale, offset = -32 * s; Q5K: s = the sub-block
+// scale, offset = 0.  Output bytes are in the order of q's.
+typedef unsigned short cq_us2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void cq_scaled_digits(uint32_t q, unsigned short s16, unsigned short c16, int &lo, int &hi) {
+    const cq_us2 s = {s16, s16}, c = {c16, c16};   // splats: the packed instruction takes one half twice
+    const cq_us2 e02 = __builtin_bit_cast(cq_us2, __builtin_amdgcn_perm(q, 0u, 0x0c060c04u));   // bytes 0, 2 as 16-bit lanes
+    const cq_us2 e13 = __builtin_bit_cast(cq_us2, __builtin_amdgcn_perm(q, 0u, 0x0c070c05u));   // bytes 1, 3
+    const uint32_t t02 = __builtin_bit_cast(uint32_t, (cq_us2)(e02 * s + c));
+    const uint32_t t13 = __builtin_bit_cast(uint32_t, (cq_us2)(e13 * s + c));
+    lo = (int)(__builtin_amdgcn_perm(t13, t02, 0x06020400u) ^ 0x80808080u);
+    hi = (int)__builtin_amdgcn_perm(t13, t02, 0x07030501u);
+}
+__device__ __forceinline__ uint32_t cq_dup16(uint32_t v) { return (v & 0xffffu) | (v << 16); }
+
 // Operand of the Q4K / Q5K min term on the f16 matrix core: the eight values -dmin * min_j of a block, each split in
 // two f16 pieces p1 = f16(v), p2 = f16(v - p1) (v has 17 significant bits; p1 + p2 == v).  Done in packed f16
 // arithmetic: the f16 product IS p1 (correctly rounded), and the f16 fma dmin * min - p1 is the product's rounding

@@ -33,14 +33,6 @@ __device__ __forceinline__ uint32_t pk_mul_u16(uint32_t a, uint32_t b) {
     const us2 r = __builtin_bit_cast(us2, a) * __builtin_bit_cast(us2, b);
     return __builtin_bit_cast(uint32_t, r);
 }
-__device__ __forceinline__ uint32_t pk_sub_u16(uint32_t a, uint32_t b) {
-    const us2 r = __builtin_bit_cast(us2, a) - __builtin_bit_cast(us2, b);
-    return __builtin_bit_cast(uint32_t, r);
-}
-__device__ __forceinline__ uint32_t pk_ashr7_i16(uint32_t a) {
-    const ss2 r = __builtin_bit_cast(ss2, a) >> (ss2){7, 7};
-    return __builtin_bit_cast(uint32_t, r);
-}
 __device__ __forceinline__ uint32_t dup16(uint32_t v) { return (v & 0xffffu) | (v << 16); }
 
 // Buffer descriptor over `base` (wave-uniform): raw bytes, no stride, no bounds.  The copies below
@@ -127,7 +119,7 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, int lane, const 
 }
 
 // Q5K: the quants are the Q4K nibbles plus a fifth bit (words {L, H} per 32 qs bytes, bit 8c + i for
-// byte c of qs word i); scale times quant has up to 11 bits and is split at bit 7 like Q6K's.
+// byte c of qs word i); scale times quant has up to 11 bits and is split as Q6K's products are.
 __device__ __forceinline__ void block_unpack(const uint8_t *wl, int lane, const WHead<CQ_DTYPE_Q5K> &wb, v4i (&bl)[4],
                                              v4i (&bh)[4], float &dw, v8h &wmin) {
     const uint32_t r = lane & 15, kq = lane >> 4;
@@ -139,14 +131,15 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, int lane, const 
 #pragma unroll
     for (int gi = 0; gi < 4; gi++) {
         const uint4 q = *(const uint4 *)(wl + swz_col(r, 2 * gi + (kq & 1)));
-        const uint32_t sc16 = dup16((rec[gi] >> (8 * hi)) & 0xff);   // scale of sub-block 2g + hi
+        const unsigned short sc16 = (unsigned short)((rec[gi] >> (8 * hi)) & 0xff);   // scale of sub-block 2g + hi
         const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const uint32_t q5 = ((qw[i] >> nsh) & 0x0F0F0F0Fu) | (((fifth[gi] >> (w0 + i)) & 0x01010101u) << 4);
-            const uint32_t p02 = pk_mul_u16(q5 & 0x00FF00FFu, sc16), p13 = pk_mul_u16((q5 >> 8) & 0x00FF00FFu, sc16);
-            bl[gi][i] = (int)(__builtin_amdgcn_perm(p13, p02, 0x06020400u) & 0x7F7F7F7Fu);
-            bh[gi][i] = (int)__builtin_amdgcn_perm(pk_ashr7_i16(p13), pk_ashr7_i16(p02), 0x06020400u);
+            int lo, hi;
+            cq_scaled_digits(q5, sc16, (unsigned short)128, lo, hi);   // digits of sc * q5
+            bl[gi][i] = lo;
+            bh[gi][i] = hi;
         }
     }
     wmin = __builtin_bit_cast(v8h, cq_min_term_operand(wb.dd, rec, (kq & 1) != 0));
@@ -170,19 +163,17 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, int lane, const 
         for (int nib = 0; nib < 2; nib++) {
             const int s = 2 * hf + nib;
             const int sc = (int)(int8_t)((sw >> (16 * (kq & 1) + 8 * nib)) & 0xff);
-            const uint32_t sc16 = dup16((uint32_t)sc);
+            const unsigned short sc16 = (unsigned short)sc, c16 = (unsigned short)(128 - 32 * sc);
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const uint32_t H = hw[i >> 1];
-                const int sh = (i & 1) * 4 + 2 * nib;
-                const uint32_t q6 = ((qw[i] >> (4 * nib)) & 0x0F0F0F0Fu) | (((H >> sh) & 0x03030303u) << 4);
-                // the four elements as 16-bit lanes, minus 32, times the group scale (low 16 bits kept)
-                const uint32_t e02 = pk_sub_u16(q6 & 0x00FF00FFu, 0x00200020u);
-                const uint32_t e13 = pk_sub_u16((q6 >> 8) & 0x00FF00FFu, 0x00200020u);
-                const uint32_t p02 = pk_mul_u16(e02, sc16), p13 = pk_mul_u16(e13, sc16);
-                // gather bytes [p02.0, p13.0, p02.2, p13.2]
-                bl[s][i] = (int)(__builtin_amdgcn_perm(p13, p02, 0x06020400u) & 0x7F7F7F7Fu);
-                bh[s][i] = (int)__builtin_amdgcn_perm(pk_ashr7_i16(p13), pk_ashr7_i16(p02), 0x06020400u);
+                const int sh = (i & 1) * 4 + 2 * nib;   // where the two high bits sit in H's bytes; wanted at bit 4
+                const uint32_t hb = sh < 4 ? H << (4 - sh) : H >> (sh - 4);
+                const uint32_t q6 = ((qw[i] >> (4 * nib)) & 0x0F0F0F0Fu) | (hb & 0x30303030u);
+                int lo, hi;
+                cq_scaled_digits(q6, sc16, c16, lo, hi);   // digits of sc * (q6 - 32)
+                bl[s][i] = lo;
+                bh[s][i] = hi;
             }
         }
     }
@@ -199,7 +190,7 @@ __global__ void __launch_bounds__(kThreads) skinny_kernel(cq_weight w, cq_act_vi
     typedef Buf<DT, RT> B;
     constexpr bool MINS = is_k4(DT);
     constexpr int NT = (RT + 1) / 2;   // 16-row tiles
-    constexpr int SHIFT = DT == CQ_DTYPE_Q4K ? 3 : 7;
+    constexpr int SHIFT = DT == CQ_DTYPE_Q4K ? 3 : 8;
     extern __shared__ __align__(16) uint8_t smem[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -359,7 +350,7 @@ __device__ __forceinline__ void res_block(const uint8_t *__restrict__ wl, const 
                                           const cq_mfma_dump &dump, int64_t at, int64_t rs, int64_t m) {
     typedef Res<DT, RT> R;
     constexpr bool MINS = is_k4(DT);
-    constexpr int SHIFT = DT == CQ_DTYPE_Q4K ? 3 : 7;
+    constexpr int SHIFT = DT == CQ_DTYPE_Q4K ? 3 : 8;
     const uint32_t r = lane & 15, kq = lane >> 4;
     v4i bl[4], bh[4];
     float dw;
