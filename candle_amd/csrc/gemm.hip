@@ -65,11 +65,11 @@ template <int DT, int MT> struct Tile {
     static constexpr int kTotal = oWgt + kWaves * kWgtWave;
 };
 
-__device__ __forceinline__ uint32_t pk_mul_u16(uint32_t a, uint32_t b) {
-    const us2 r = __builtin_bit_cast(us2, a) * __builtin_bit_cast(us2, b);
+// both 16-bit halves of `a` times `b` (a splat: the packed instruction takes one half of its operand twice)
+__device__ __forceinline__ uint32_t pk_mul_u16(uint32_t a, unsigned short b) {
+    const us2 r = __builtin_bit_cast(us2, a) * (us2){b, b};
     return __builtin_bit_cast(uint32_t, r);
 }
-__device__ __forceinline__ uint32_t dup16(uint32_t v) { return (v & 0xffffu) | (v << 16); }
 
 // Buffer descriptor over `base` (wave-uniform): raw bytes, no stride, no bounds.  The copies below
 // are buffer loads rather than global loads on purpose: with a global (FLAT-encoded) LDS copy in
@@ -284,8 +284,8 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g
     for (int gi = 0; gi < 4; gi++) {
         // qs bytes 32g + 16h + [0,16): low nibbles = K-slice 2g, high nibbles = slice 2g+1
         const uint4 q = *(const uint4 *)(wl + g.col[gi]);
-        const uint32_t s0 = rec[gi] & 0xff, s1 = (rec[gi] >> 8) & 0xff;
-        const uint32_t sl0 = dup16(s0 & 7), sh0 = dup16(s0 >> 3), sl1 = dup16(s1 & 7), sh1 = dup16(s1 >> 3);
+        const unsigned short sl0 = (unsigned short)(rec[gi] & 7), sh0 = (unsigned short)((rec[gi] >> 3) & 31);
+        const unsigned short sl1 = (unsigned short)((rec[gi] >> 8) & 7), sh1 = (unsigned short)((rec[gi] >> 11) & 31);
         const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
         for (int i = 0; i < 4; i++) {

@@ -277,7 +277,6 @@ __device__ __forceinline__ void cq_scaled_digits(uint32_t q, unsigned short s16,
     lo = (int)(__builtin_amdgcn_perm(t13, t02, 0x06020400u) ^ 0x80808080u);
     hi = (int)__builtin_amdgcn_perm(t13, t02, 0x07030501u);
 }
-__device__ __forceinline__ uint32_t cq_dup16(uint32_t v) { return (v & 0xffffu) | (v << 16); }
 
 // Operand of the Q4K / Q5K min term on the f16 matrix core: the eight values -dmin * min_j of a block, each split in
 // two f16 pieces p1 = f16(v), p2 = f16(v - p1) (v has 17 significant bits; p1 + p2 == v).  Done in packed f16

@@ -29,11 +29,11 @@ constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
 constexpr int kMaxLds = 160 * 1024;   // LDS of a CU, which a single workgroup may take
 
-__device__ __forceinline__ uint32_t pk_mul_u16(uint32_t a, uint32_t b) {
-    const us2 r = __builtin_bit_cast(us2, a) * __builtin_bit_cast(us2, b);
+// both 16-bit halves of `a` times `b` (a splat: the packed instruction takes one half of its operand twice)
+__device__ __forceinline__ uint32_t pk_mul_u16(uint32_t a, unsigned short b) {
+    const us2 r = __builtin_bit_cast(us2, a) * (us2){b, b};
     return __builtin_bit_cast(uint32_t, r);
 }
-__device__ __forceinline__ uint32_t dup16(uint32_t v) { return (v & 0xffffu) | (v << 16); }
 
 // Buffer descriptor over `base` (wave-uniform): raw bytes, no stride, no bounds.  The copies below
 // are buffer loads rather than global loads on purpose: with a global (FLAT-encoded) LDS copy in
@@ -104,7 +104,7 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, int lane, const 
     for (int gi = 0; gi < 4; gi++) {
         const uint4 q = *(const uint4 *)(wl + swz_col(r, 2 * gi + (kq & 1)));
         const uint32_t sj = (rec[gi] >> (8 * hi)) & 0xff;   // scale of sub-block 2g + hi
-        const uint32_t sl = dup16(sj & 7), sh = dup16(sj >> 3);
+        const unsigned short sl = (unsigned short)(sj & 7), sh = (unsigned short)(sj >> 3);
         const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
