@@ -354,7 +354,7 @@ static size_t act_ws_layout(int act_dtype, int64_t m, int64_t k, uint8_t *base, 
     } else {
         const size_t o_d = take((size_t)(m_pad * (k / 32)) * 4);
         const size_t o_s = take((size_t)(m * (k / 32)) * 4);
-        const size_t o_h = take((size_t)(m * (k / 32)) * 2);
+        const size_t o_h = take((size_t)(m_pad * (k / 32)) * 2);   // padded: the Q8_1 tile kernel copies whole tiles
         if (base) {
             view.qs = (int8_t *)(base + o_qs); view.d = (float *)(base + o_d);
             view.bsum32 = (int32_t *)(base + o_s); view.s16 = (uint16_t *)(base + o_h);
@@ -418,7 +418,7 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
     CQ_HIP_CHECK(hipSetDevice(w->dev));
     hipStream_t s = (hipStream_t)stream;
     if (flags & CQ_FLAG_ACT_Q8_1) {
-        // the reference's CUDA formulation (cuda.rs:298-365): activations to Q8_1, one dot-product kernel for every row count
+        // the reference's CUDA formulation (cuda.rs:298-365): activations to Q8_1; a dot-product kernel up to 32 rows, the matrix cores beyond
         if (act != CQ_DTYPE_Q8_1 || !cq_matmul_q8_1_supported(w))
             return cq_set_error(CQ_ERR_UNSUPPORTED, "Q8_1 activations are for Q4K and Q6K weights with rows that fit the LDS (dtype %d, k = %lld)",
                                 w->dtype, (long long)w->k);
@@ -428,7 +428,8 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
         act_ws_layout(act, m, w->k, (uint8_t *)ws, &v);
         if (!(flags & CQ_FLAG_REUSE_ACT))
             CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, nullptr, m, w->k, pre, v, cq_no_clear(), s));
-        CQ_HIP_CHECK(cq_launch_matmul_q8_1(w, v, m, y_dev, s));
+        if (cq_gemm_q81_supported(w, m)) CQ_HIP_CHECK(cq_launch_gemm_q81(w, v, m, y_dev, s));   // matrix cores beyond 32 rows
+        else CQ_HIP_CHECK(cq_launch_matmul_q8_1(w, v, m, y_dev, s));
         return CQ_OK;
     }
     // In the one-launch kernels every workgroup reads x (and aux) in its prologue while others already store y:

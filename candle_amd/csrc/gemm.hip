@@ -521,6 +521,211 @@ __global__ void __launch_bounds__(kThreads) gemm_grouped_kernel(GroupArgs ga, cq
     gemm_body<DT, 1>(w, a, ga.row0[tile], ga.row_end[tile], y, ksplit);
 }
 
+// ------------------------------------------------ K-quant weights x Q8_1 activations (tile kernel) ----
+// The formulation of the reference's CUDA arm (mul_mat_via_q8_1, quantized/cuda.rs:298-365; dot bodies
+// candle-kernels/src/quantized.cu:2141-2166 for Q4K, :2258-2281 for Q6K) on the matrix cores, activations quantized
+// by the CPU rule of BlockQ8_1::from_float (k_quants.rs:665-691).  Per 32-element Q8_1 block j of a weight block
+//   Q4K:  (d * sc_j) * d8_j * dot_j  -  (dmin * m_j) * s8_j          dot_j = sum_32 q4 * q8
+//   Q6K:  d * d8_j * (sc_g * dot_g + sc_g' * dot_g')                 g, g' the two 16-element groups of block j
+// A Q8_1 block is one K-slice of the 32x32x32 int8 MFMA, so dot_j is one result element (Q6K: the two-digit operands
+// of the Q8K kernel above give sc_g * dot_g + sc_g' * dot_g' as 256 * hi + lo).  Its scale is an outer product
+// (weight row factor x activation row factor): a bf16 MFMA lays it out in the accumulator layout, the weight factor
+// (17 significant bits) as three bf16 pieces, the activation factor (an f16 value) as two, all six products exact.
+// The Q4K min term is one f16 MFMA per tile and weight block: s8 is an f16, dmin * m_j goes in as two f16 pieces.
+// Work split, LDS images and copies as in the Q8K kernel; two activation stages, the waves in step.
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+
+template <int DT, int MT> struct Tile81 {
+    static constexpr int kAct = MT * 8 * 1024;
+    static constexpr int kD8 = MT * 32 * 32;                                 // [32*MT rows][8 blocks] f32
+    static constexpr int kS8 = DT == CQ_DTYPE_Q4K ? (MT < 2 ? 2 : MT) * 32 * 16 : 0;   // [32*MT rows][8 blocks] f16, whole 64-row copies
+    static constexpr int oD8 = kAct, oS8 = oD8 + kD8;
+    static constexpr int kStage = oS8 + kS8;
+    static constexpr int kWgtWave = DT == CQ_DTYPE_Q4K ? 4096 : 6144;
+    static constexpr int oWgt = 2 * kStage;
+    static constexpr int kTotal = oWgt + kWaves * kWgtWave;
+};
+
+template <int DT, int MT>
+__device__ __forceinline__ void stage_acts81(uint8_t *buf, const cq_act_view &a, const LaneGeo &g, int64_t k, int64_t m0,
+                                             int64_t b, int wave, int lane) {
+    typedef Tile81<DT, MT> T;
+#pragma unroll
+    for (int j = 0; j < MT * 8 / kWaves; j++) {
+        const int idx = wave + kWaves * j;           // = (t*2 + kh)*4 + rg
+        const int rg = idx & 3, kh = (idx >> 2) & 1, t = idx >> 3;
+        dma16(a.qs + (m0 + t * 32 + rg * 8) * k + b * 256 + kh * 128, g.act_off, buf + idx * 1024);
+    }
+    const uint32_t nb = (uint32_t)(k >> 5);
+    // block scales: 32 rows x 8 floats per copy (lane l: row l/2, half l%2)
+#pragma unroll
+    for (int t = 0; t < MT; t++) {
+        if (t + 4 == wave)
+            dma16((const uint8_t *)(a.d + (m0 + t * 32) * (int64_t)nb + b * 8), (uint32_t)(lane >> 1) * nb * 4u + (uint32_t)(lane & 1) * 16u,
+                  buf + T::oD8 + t * 1024);
+    }
+    // the blocks' `s` fields: 64 rows x 8 halves per copy (lane l: row l)
+    if (DT == CQ_DTYPE_Q4K) {
+#pragma unroll
+        for (int j = 0; j < (MT + 1) / 2; j++) {
+            if (j == wave && (MT > 1 || lane < 32))
+                dma16((const uint8_t *)(a.s16 + (m0 + j * 64) * (int64_t)nb + b * 8), (uint32_t)lane * nb * 2u, buf + T::oS8 + j * 1024);
+        }
+    }
+}
+
+// v (at most 24 significant bits) as bf16 pieces b1 + b2 + b3, each the leading eight bits of what the pieces before
+// it leave: lanes 0..31 carry [b1, b1, b2, b2] in K-slots 0..3, lanes 32..63 carry [b3, b3] in K-slots 8, 9.
+__device__ __forceinline__ v8bf weight_scale_operand(float v, int h) {
+    const uint32_t vb = __float_as_uint(v);
+    const float r1 = v - __uint_as_float(vb & 0xffff0000u);
+    const uint32_t rb = __float_as_uint(r1);
+    const float r2 = r1 - __uint_as_float(rb & 0xffff0000u);
+    const uint32_t tb = __float_as_uint(r2);
+    const uint32_t b11 = __builtin_amdgcn_perm(vb, vb, 0x07060706u), b22 = __builtin_amdgcn_perm(rb, rb, 0x07060706u);
+    const uint32_t b33 = __builtin_amdgcn_perm(tb, tb, 0x07060706u);
+    const v4u pk = {h ? b33 : b11, h ? 0u : b22, 0u, 0u};
+    return __builtin_bit_cast(v8bf, pk);
+}
+// The activation block scale (an f16 value: two bf16 pieces a1 + a2, exact) as [a1, a2, a1, a2] in K-slots 0..3 of
+// both lane halves: with the operand above the products sum to (a1 + a2) * (b1 + b2 + b3).
+__device__ __forceinline__ v8bf act_scale_operand(float v) {
+    const uint32_t vb = __float_as_uint(v);
+    const float r1 = v - __uint_as_float(vb & 0xffff0000u);
+    const uint32_t a12 = __builtin_amdgcn_perm(__float_as_uint(r1), vb, 0x07060302u);
+    const v4u pk = {a12, a12, 0u, 0u};
+    return __builtin_bit_cast(v8bf, pk);
+}
+
+template <int DT, int MT>
+__global__ void __launch_bounds__(kThreads) gemm_q81_kernel(cq_weight w, cq_act_view a, int64_t m, float *__restrict__ y) {
+    static_assert(DT == CQ_DTYPE_Q4K || DT == CQ_DTYPE_Q6K, "Q4K and Q6K only");
+    typedef Tile81<DT, MT> T;
+    constexpr bool K4 = DT == CQ_DTYPE_Q4K;
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int h = lane >> 5, col = lane & 31;
+    const int64_t k = w.k, kb = k >> 8;
+    const int64_t m0 = (int64_t)blockIdx.y * (MT * 32);
+    const int64_t n_tile = ((int64_t)blockIdx.x * kWaves + wave) * 32;
+    const bool n_ok = n_tile < w.n;   // wave-uniform; a wave past the last row only helps with the copies
+    const int64_t n = n_tile + col;
+    const int64_t nc = n_ok ? n : 0;
+    const LaneGeo g = lane_geo(lane, k);
+    uint8_t *__restrict__ wl = smem + T::oWgt + wave * T::kWgtWave;
+
+    v16f out[MT];
+#pragma unroll
+    for (int t = 0; t < MT; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) out[t][i] = 0.0f;
+
+    WHead<DT> hcur, hnxt;
+    stage_acts81<DT, MT>(smem, a, g, k, m0, 0, wave, lane);
+    if (n_ok) stage_weights<DT>(wl, w, g, n_tile, 0);
+    load_head(w, nc * kb, hcur);
+    hnxt = hcur;
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+
+    for (int64_t b = 0; b < kb; b++) {
+        const uint8_t *__restrict__ cur = smem + (b & 1) * T::kStage;
+        uint8_t *__restrict__ nxt = smem + ((b & 1) ^ 1) * T::kStage;
+        const bool more = b + 1 < kb;
+        if (more) {
+            stage_acts81<DT, MT>(nxt, a, g, k, m0, b + 1, wave, lane);
+            load_head(w, nc * kb + b + 1, hnxt);
+        }
+        if (n_ok) {
+            // weight operands of the eight Q8_1 blocks, their scale operands, the min-term operand
+            v4i bl[8], bh[8];
+            v8bf ws[K4 ? 8 : 1];
+            v8h wmin = {};
+            if constexpr (K4) {
+                const float dw = cq_h2f((uint16_t)(hcur.dd & 0xffff));
+                const uint32_t rec[4] = {hcur.rec.x, hcur.rec.y, hcur.rec.z, hcur.rec.w};   // {sc[2g], sc[2g+1], mn[2g], mn[2g+1]}
+#pragma unroll
+                for (int gi = 0; gi < 4; gi++) {
+                    // qs bytes 32g + 16h + [0,16): low nibbles = block 2g, high nibbles = block 2g+1
+                    const uint4 q = *(const uint4 *)(wl + g.col[gi]);
+                    const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        bl[2 * gi][i] = (int)(qw[i] & 0x0F0F0F0Fu);
+                        bl[2 * gi + 1][i] = (int)((qw[i] >> 4) & 0x0F0F0F0Fu);
+                    }
+                    ws[2 * gi] = weight_scale_operand(dw * (float)(rec[gi] & 0xff), h);          // d * sc_j: exact in f32
+                    ws[2 * gi + 1] = weight_scale_operand(dw * (float)((rec[gi] >> 8) & 0xff), h);
+                }
+                wmin = __builtin_bit_cast(v8h, cq_min_term_operand(hcur.dd, rec, h != 0));
+            } else {
+                float dw;
+                block_unpack(wl, g, hcur, lane, bl, bh, dw, wmin);
+                ws[0] = weight_scale_operand(dw, h);
+            }
+            if (more) stage_weights<DT>(wl, w, g, n_tile, b + 1);
+
+            // steps q = (tile t, block s): the MFMAs of step q, and in their shadow the scaling of step q-1
+            auto afrag = [&](int q) -> v4i {
+                const int t = q >> 3, s = q & 7;
+                return *(const v4i *)(cur + g.col[s & 3] + (t * 2 + (s >> 2)) * 4096);
+            };
+            auto d8raw = [&](int q) -> float {
+                const int t = q >> 3, s = q & 7;
+                return *(const float *)(cur + T::oD8 + (t * 32 + col) * 32 + s * 4);
+            };
+            v16i acc[2], acch[2];
+            v16f sc[2];
+            v4i av[3];
+            float dv[3];
+            av[0] = afrag(0); av[1] = afrag(1);
+            dv[0] = d8raw(0); dv[1] = d8raw(1);
+            const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            const v16f zerof = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int q = 0; q <= MT * 8; q++) {
+                if (q + 2 < MT * 8) { av[(q + 2) % 3] = afrag(q + 2); dv[(q + 2) % 3] = d8raw(q + 2); }
+                if (q < MT * 8) {
+                    if (K4 && (q & 7) == 0) {
+                        // min term of tile t: out -= sum_j (dmin * m_j) * s8_j
+                        const v8h s8 = *(const v8h *)(cur + T::oS8 + ((q >> 3) * 32 + col) * 16);
+                        out[q >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(s8, wmin, out[q >> 3], 0, 0, 0);
+                    }
+                    acc[q & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[q % 3], bl[q & 7], zero, 0, 0, 0);
+                    if (!K4) acch[q & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[q % 3], bh[q & 7], zero, 0, 0, 0);
+                    sc[q & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(act_scale_operand(dv[q % 3]), ws[K4 ? (q & 7) : 0], zerof, 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);   // the MFMAs stay in front of the scaling of the step before
+                if (q > 0) {
+                    const int p = (q - 1) & 1, t = (q - 1) >> 3;
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        const int I = K4 ? acc[p][i] : (acch[p][i] << 8) + acc[p][i];
+                        out[t][i] = __builtin_fmaf((float)I, sc[p][i], out[t][i]);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        hcur = hnxt;
+        __builtin_amdgcn_s_waitcnt(0);   // the next stage and the wave's next weights have landed in LDS
+        __syncthreads();
+    }
+
+    if (n_ok) {
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int64_t row = m0 + t * 32 + (i >> 2) * 8 + h * 4 + (i & 3);
+                if (row < m) y[row * w.n + n] = out[t][i];
+            }
+        }
+    }
+}
+
 int g_cus = 0;
 int num_cus() {
     if (g_cus == 0) {
@@ -645,6 +850,24 @@ hipError_t launch_grouped(const cq_weight *const *experts, int n_experts, const 
     return hipGetLastError();
 }
 
+template <int DT, int MT>
+hipError_t launch_q81_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
+    const size_t lds = Tile81<DT, MT>::kTotal;
+    if (hipError_t e = cq_ensure_lds<gemm_q81_kernel<DT, MT>>(w->dev, lds); e != hipSuccess) return e;
+    dim3 grid((unsigned)n_tiles(w), (unsigned)((m + MT * 32 - 1) / (MT * 32)), 1);
+    CQ_LAUNCH((gemm_q81_kernel<DT, MT>), grid, kThreads, lds, s, *w, a, m, y);
+    return hipGetLastError();
+}
+template <int DT>
+hipError_t launch_q81_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
+    // the tallest tile that still gives every CU a workgroup
+    int mt = 4;
+    while (mt > 1 && (m <= 16 * mt || n_tiles(w) * ((m + mt * 32 - 1) / (mt * 32)) < num_cus())) mt >>= 1;
+    if (mt == 1) return launch_q81_mt<DT, 1>(w, a, m, y, s);
+    if (mt == 2) return launch_q81_mt<DT, 2>(w, a, m, y, s);
+    return launch_q81_mt<DT, 4>(w, a, m, y, s);
+}
+
 }  // namespace
 
 bool cq_gemm_grouped_supported(const cq_weight *const *experts, int n_experts, const int32_t *offsets, int act_dtype) {
@@ -694,4 +917,18 @@ hipError_t cq_launch_gemm(const cq_weight *w, cq_act_view a, int act_dtype, int6
     if (w->dtype == CQ_DTYPE_Q4K) return launch_dt<CQ_DTYPE_Q4K>(w, a, m, y, y_cleared, s);
     if (w->dtype == CQ_DTYPE_Q5K) return launch_dt<CQ_DTYPE_Q5K>(w, a, m, y, y_cleared, s);
     return launch_dt<CQ_DTYPE_Q6K>(w, a, m, y, y_cleared, s);
+}
+
+// K-quant weights x Q8_1 activations on the matrix cores (see gemm_q81_kernel).  The workspace rows are padded to whole
+// 128-row tiles beyond 32 rows, scales and `s` fields included.
+bool cq_gemm_q81_supported(const cq_weight *w, int64_t m) {
+    return (w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q6K) && m > 32 && w->k >= 256 && w->k <= (1 << 24) && w->n % 32 == 0;
+}
+
+hipError_t cq_launch_gemm_q81(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
+    if (!cq_gemm_q81_supported(w, m)) return hipErrorNotSupported;
+    if (w->n == 0) return hipSuccess;
+    if (a.m_stride < (m + 127) / 128 * 128) return hipErrorInvalidValue;   // rows the last tile may read
+    if (w->dtype == CQ_DTYPE_Q4K) return launch_q81_dt<CQ_DTYPE_Q4K>(w, a, m, y, s);
+    return launch_q81_dt<CQ_DTYPE_Q6K>(w, a, m, y, s);
 }

@@ -124,6 +124,9 @@ bool cq_matvec_row_fits(const cq_weight *w);          // K small enough for the 
 // Q4K / Q6K weights with Q8_1 activations (the reference's CUDA formulation), any number of rows
 bool cq_matmul_q8_1_supported(const cq_weight *w);
 hipError_t cq_launch_matmul_q8_1(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s);
+// the same on the matrix cores, for more than 32 rows (gemm.hip)
+bool cq_gemm_q81_supported(const cq_weight *w, int64_t m);
+hipError_t cq_launch_gemm_q81(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s);
 bool cq_matvec_fused_supported(const cq_weight *w);   // m == 1: quantizer fused into the matvec launch
 hipError_t cq_launch_matvec_fused(const cq_weight *w, const float *x, cq_pre pre, float *y, hipStream_t s);
 // 2 <= m <= 4 rows in the one-launch kernel (short rows only)

@@ -61,7 +61,7 @@ enum {
     CQ_FLAG_ACT_Q8_1 = 4,     /* Q4K / Q6K weights x Q8_1 activations: the formulation of the reference's CUDA arm
                                  (mul_mat_via_q8_1, cuda.rs:298-365; quantized.cu:2141-2166, :2258-2281) with the
                                  activations quantized by BlockQ8_1::from_float (k_quants.rs:665-691), instead of the
-                                 CPU formulation's Q8K.  One dot-product kernel for every row count; combines with
+                                 CPU formulation's Q8K.  A dot-product kernel up to 32 rows, the matrix cores beyond; combines with
                                  CQ_FLAG_REUSE_ACT only; the grouped calls do not take it.  Its results differ from
                                  the CPU QMatMul's by the two activation quantizers' noise (about 1e-3 relative).    */
     CQ_FLAG_REUSE_ACT = 8,    /* the workspace already holds this x, quantized by an earlier cq_qmatmul call with the

@@ -83,7 +83,10 @@ def _exact(dt, x, blocks, n, k):
 
 
 @pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K])
-@pytest.mark.parametrize("m,k,n", [(1, 256, 8), (3, 512, 37), (11, 1024, 64), (9, 4096, 48)])
+@pytest.mark.parametrize("m,k,n", [(1, 256, 8), (3, 512, 37), (11, 1024, 64), (9, 4096, 48),
+                                   # more than 32 rows and n % 32 == 0: the matrix-core kernel (one, two and four
+                                   # 32-row tiles per workgroup, a last tile and a last workgroup that are not full)
+                                   (33, 512, 64), (70, 1024, 96), (130, 256, 32), (200, 768, 288), (300, 512, 8192)])
 def test_q8_1_variant_matches_oracle_and_exact_formula(qh, dt, m, k, n):
     rng = np.random.default_rng(1000 * m + n)
     w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
@@ -97,9 +100,16 @@ def test_q8_1_variant_matches_oracle_and_exact_formula(qh, dt, m, k, n):
     # a wrong integer anywhere moves a result by far more than f32 rounding does
     assert np.abs(got - exact).max() <= 2e-5 * np.abs(exact).max() + 1e-6
     # batch invariance: a row's result does not depend on the rows beside it (quantized_tests.rs:181-216)
-    if m > 1:
+    if 1 < m <= 32:
         one = qh.qmatmul(qw, dev(x[1:2]), flags=qh.FLAG_ACT_Q8_1).cpu().numpy()
         assert np.array_equal(one[0], got[1])
+    if m > 32:
+        # the same within the matrix-core kernel (another tile height, other neighbours), and to rounding against
+        # the dot-product kernel that takes up to 32 rows
+        part = qh.qmatmul(qw, dev(x[m - 33:]), flags=qh.FLAG_ACT_Q8_1).cpu().numpy()
+        assert np.array_equal(part, got[m - 33:])
+        few = qh.qmatmul(qw, dev(x[:5]), flags=qh.FLAG_ACT_Q8_1).cpu().numpy()
+        check_f32(got[:5], few)
 
 
 @pytest.mark.parametrize("dt", [orc.Q4K, orc.Q6K])
