@@ -52,14 +52,16 @@ extern "C" int cq_device_count(void) {
 // ------------------------------------------------------------ dtype tables ----
 extern "C" int64_t cq_block_size(int dt) {
     switch (dt) {
-    case CQ_DTYPE_Q4_0: case CQ_DTYPE_Q8_0: case CQ_DTYPE_Q8_1: return 32;
-    case CQ_DTYPE_Q4K: case CQ_DTYPE_Q5K: case CQ_DTYPE_Q6K: case CQ_DTYPE_Q8K: return 256;
+    case CQ_DTYPE_Q4_0: case CQ_DTYPE_Q5_0: case CQ_DTYPE_Q8_0: case CQ_DTYPE_Q8_1: return 32;
+    case CQ_DTYPE_Q3K: case CQ_DTYPE_Q4K: case CQ_DTYPE_Q5K: case CQ_DTYPE_Q6K: case CQ_DTYPE_Q8K: return 256;
     default: return 0;
     }
 }
 extern "C" int64_t cq_type_size(int dt) {
     switch (dt) {
     case CQ_DTYPE_Q4_0: return 18;
+    case CQ_DTYPE_Q5_0: return 22;
+    case CQ_DTYPE_Q3K: return 110;
     case CQ_DTYPE_Q8_0: return 34;
     case CQ_DTYPE_Q8_1: return 36;
     case CQ_DTYPE_Q4K: return 144;
@@ -71,14 +73,15 @@ extern "C" int64_t cq_type_size(int dt) {
 }
 extern "C" int cq_vec_dot_type(int dt) {
     switch (dt) {
-    case CQ_DTYPE_Q4_0: case CQ_DTYPE_Q8_0: return CQ_DTYPE_Q8_0;
-    case CQ_DTYPE_Q4K: case CQ_DTYPE_Q5K: case CQ_DTYPE_Q6K: return CQ_DTYPE_Q8K;
+    case CQ_DTYPE_Q4_0: case CQ_DTYPE_Q5_0: case CQ_DTYPE_Q8_0: return CQ_DTYPE_Q8_0;
+    case CQ_DTYPE_Q3K: case CQ_DTYPE_Q4K: case CQ_DTYPE_Q5K: case CQ_DTYPE_Q6K: return CQ_DTYPE_Q8K;
     default: return -1;
     }
 }
 
 static bool is_weight_dtype(int dt) {
-    return dt == CQ_DTYPE_Q4_0 || dt == CQ_DTYPE_Q8_0 || dt == CQ_DTYPE_Q4K || dt == CQ_DTYPE_Q5K || dt == CQ_DTYPE_Q6K;
+    return dt == CQ_DTYPE_Q4_0 || dt == CQ_DTYPE_Q5_0 || dt == CQ_DTYPE_Q8_0 || dt == CQ_DTYPE_Q3K || dt == CQ_DTYPE_Q4K ||
+           dt == CQ_DTYPE_Q5K || dt == CQ_DTYPE_Q6K;
 }
 
 // --------------------------------------------------------------- weights ----
@@ -98,11 +101,11 @@ static int weight_alloc(int dev, int dt, int64_t n, int64_t k, cq_weight **out) 
     CQ_HIP_CHECK(hipSetDevice(dev));
     cq_weight *w = new (std::nothrow) cq_weight();
     if (!w) return cq_set_error(CQ_ERR_INVALID, "out of host memory");
-    w->dev = dev; w->dtype = dt; w->n = n; w->k = k;
+    w->dev = dev; w->dtype = cq_storage_dtype(dt); w->ggml_dtype = dt; w->n = n; w->k = k;
     const int64_t nb = n * (k / bs);
     w->ggml_bytes = (size_t)nb * (size_t)cq_type_size(dt);
     size_t s0 = 0, s1 = 0, s2 = 0, s3 = 0;
-    switch (dt) {
+    switch (w->dtype) {
     case CQ_DTYPE_Q4_0: s0 = (size_t)nb * 16; s1 = (size_t)nb * 2; break;
     case CQ_DTYPE_Q8_0: s0 = (size_t)nb * 32; s1 = (size_t)nb * 2; break;
     case CQ_DTYPE_Q4K: s0 = (size_t)nb * 128; s1 = (size_t)nb * CQ_Q4K_HDR; break;
@@ -131,10 +134,46 @@ static int weight_alloc(int dev, int dt, int64_t n, int64_t k, cq_weight **out) 
     return CQ_OK;
 }
 
+// GGML blocks of the caller's type (device memory) into the planes, and back.  A type held in another type's planes
+// goes through that type's blocks in a temporary (set-up paths: they synchronize before freeing it).
+static int64_t weight_blocks(const cq_weight *w) { return w->n * (w->k / cq_block_size(w->dtype)); }
+static hipError_t blocks_to_planes(const cq_weight *w, uint8_t *ggml_aos_dev, hipStream_t s) {
+    if (w->ggml_dtype == w->dtype) return cq_launch_repack(w, ggml_aos_dev, s);
+    void *tmp = nullptr;
+    hipError_t e = hipMalloc(&tmp, (size_t)weight_blocks(w) * (size_t)cq_type_size(w->dtype) + 256);
+    if (e != hipSuccess) return e;
+    e = cq_launch_transcode(w->ggml_dtype, ggml_aos_dev, (uint8_t *)tmp, weight_blocks(w), false, s);
+    if (e == hipSuccess) e = cq_launch_repack(w, (const uint8_t *)tmp, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    (void)hipFree(tmp);
+    return e;
+}
+static hipError_t planes_to_blocks(const cq_weight *w, uint8_t *ggml_aos_dev, hipStream_t s) {
+    if (w->ggml_dtype == w->dtype) return cq_launch_unpack(w, ggml_aos_dev, s);
+    void *tmp = nullptr;
+    hipError_t e = hipMalloc(&tmp, (size_t)weight_blocks(w) * (size_t)cq_type_size(w->dtype) + 256);
+    if (e != hipSuccess) return e;
+    e = cq_launch_unpack(w, (uint8_t *)tmp, s);
+    if (e == hipSuccess) e = cq_launch_transcode(w->ggml_dtype, ggml_aos_dev, (uint8_t *)tmp, weight_blocks(w), true, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    (void)hipFree(tmp);
+    return e;
+}
+
 extern "C" int cq_weight_zeros(int dev, int dt, int64_t n, int64_t k, cq_weight **out) {
     int rc = weight_alloc(dev, dt, n, k, out);
     if (rc) return rc;
     hipError_t e = hipMemset((*out)->base, 0, (*out)->alloc_bytes);
+    if (e == hipSuccess && (*out)->ggml_dtype != (*out)->dtype && (*out)->ggml_bytes) {
+        // all-zero blocks of the caller's type are not all-zero planes of the holding type (a zero quant is stored
+        // with its offset): encode them
+        void *tmp = nullptr;
+        e = hipMalloc(&tmp, (*out)->ggml_bytes + 256);
+        if (e == hipSuccess) e = hipMemset(tmp, 0, (*out)->ggml_bytes);
+        if (e == hipSuccess) e = blocks_to_planes(*out, (uint8_t *)tmp, nullptr);
+        if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
+        if (tmp) (void)hipFree(tmp);
+    }
     if (e != hipSuccess) {
         cq_weight_destroy(*out);
         *out = nullptr;
@@ -159,7 +198,7 @@ extern "C" int cq_weight_create(int dev, int dt, const void *host_blocks, size_t
     void *tmp = nullptr;
     hipError_t e = hipMalloc(&tmp, nbytes + 256);
     if (e == hipSuccess) e = hipMemcpy(tmp, host_blocks, nbytes, hipMemcpyHostToDevice);
-    if (e == hipSuccess) e = cq_launch_repack(w, (const uint8_t *)tmp, nullptr);
+    if (e == hipSuccess) e = blocks_to_planes(w, (uint8_t *)tmp, nullptr);
     if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
     if (tmp) (void)hipFree(tmp);
     if (e != hipSuccess) {
@@ -226,8 +265,8 @@ extern "C" int cq_weight_quantize(cq_weight *w, const float *src_dev, void *stre
     void *tmp = nullptr;
     CQ_HIP_CHECK(hipMalloc(&tmp, w->ggml_bytes + 256));
     const int64_t nb = w->n * (w->k / cq_block_size(w->dtype));
-    hipError_t e = cq_launch_quantize_weight(w->dtype, src_dev, nb, (uint8_t *)tmp, s);
-    if (e == hipSuccess) e = cq_launch_repack(w, (const uint8_t *)tmp, s);
+    hipError_t e = cq_launch_quantize_weight(w->ggml_dtype, src_dev, nb, (uint8_t *)tmp, s);
+    if (e == hipSuccess) e = blocks_to_planes(w, (uint8_t *)tmp, s);
     if (e == hipSuccess) e = hipStreamSynchronize(s);  // the temporary is freed below
     (void)hipFree(tmp);
     if (e != hipSuccess) return cq_set_error(CQ_ERR_HIP, "weight quantize failed: %s", hipGetErrorString(e));
@@ -259,7 +298,7 @@ extern "C" int cq_weight_to_ggml(const cq_weight *w, void *host_dst, size_t nbyt
     void *tmp = nullptr;
     CQ_HIP_CHECK(hipMalloc(&tmp, nbytes + 256));
     hipError_t e = hipDeviceSynchronize();
-    if (e == hipSuccess) e = cq_launch_unpack(w, (uint8_t *)tmp, nullptr);
+    if (e == hipSuccess) e = planes_to_blocks(w, (uint8_t *)tmp, nullptr);
     if (e == hipSuccess) e = hipMemcpy(host_dst, tmp, nbytes, hipMemcpyDeviceToHost);
     (void)hipFree(tmp);
     if (e != hipSuccess) return cq_set_error(CQ_ERR_HIP, "weight download failed: %s", hipGetErrorString(e));
@@ -267,7 +306,7 @@ extern "C" int cq_weight_to_ggml(const cq_weight *w, void *host_dst, size_t nbyt
 }
 
 extern "C" size_t cq_weight_size_in_bytes(const cq_weight *w) { return w ? w->ggml_bytes : 0; }
-extern "C" int cq_weight_dtype(const cq_weight *w) { return w ? w->dtype : -1; }
+extern "C" int cq_weight_dtype(const cq_weight *w) { return w ? w->ggml_dtype : -1; }
 extern "C" int cq_weight_device(const cq_weight *w) { return w ? w->dev : -1; }
 extern "C" int cq_weight_shape(const cq_weight *w, int64_t *n, int64_t *k) {
     if (!w) return cq_set_error(CQ_ERR_INVALID, "null weight");
@@ -366,7 +405,7 @@ static size_t act_ws_layout(int act_dtype, int64_t m, int64_t k, uint8_t *base, 
 
 static int act_dtype_for(const cq_weight *w, int flags) {
     int a = cq_vec_dot_type(w->dtype);
-    if ((flags & CQ_FLAG_ACT_Q8_1) && (w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q6K)) a = CQ_DTYPE_Q8_1;
+    if ((flags & CQ_FLAG_ACT_Q8_1) && (w->ggml_dtype == CQ_DTYPE_Q4K || w->ggml_dtype == CQ_DTYPE_Q6K)) a = CQ_DTYPE_Q8_1;
     return a;
 }
 
@@ -421,7 +460,7 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
         // the reference's CUDA formulation (cuda.rs:298-365): activations to Q8_1; a dot-product kernel up to 32 rows, the matrix cores beyond
         if (act != CQ_DTYPE_Q8_1 || !cq_matmul_q8_1_supported(w))
             return cq_set_error(CQ_ERR_UNSUPPORTED, "Q8_1 activations are for Q4K and Q6K weights with rows that fit the LDS (dtype %d, k = %lld)",
-                                w->dtype, (long long)w->k);
+                                w->ggml_dtype, (long long)w->k);
         if (flags & ~(CQ_FLAG_ACT_Q8_1 | CQ_FLAG_REUSE_ACT))
             return cq_set_error(CQ_ERR_INVALID, "CQ_FLAG_ACT_Q8_1 combines with CQ_FLAG_REUSE_ACT only");
         cq_act_view v;

@@ -39,9 +39,10 @@
 
 struct cq_weight {
     int dev;
-    int dtype;
+    int dtype;           // the type whose planes hold the blocks: what every kernel dispatches on
+    int ggml_dtype;      // the type the caller sees; differs from dtype for Q5_0 (held as Q8_0) and Q3K (held as Q6K)
     int64_t n, k;
-    size_t ggml_bytes;   // n * k/block * type_size
+    size_t ggml_bytes;   // n * k/block * type_size of ggml_dtype
     void *base;          // the single device allocation
     size_t alloc_bytes;
     uint8_t *p0;         // qs / ql
@@ -91,6 +92,12 @@ bool cq_timing_take(hipEvent_t *start, hipEvent_t *stop);
 // repack.hip
 hipError_t cq_launch_repack(const cq_weight *w, const uint8_t *aos_dev, hipStream_t s);   // GGML AoS -> planes
 hipError_t cq_launch_unpack(const cq_weight *w, uint8_t *aos_dev, hipStream_t s);         // planes -> GGML AoS
+// Types held in another type's planes (same values, same arithmetic): Q5_0 as Q8_0, Q3K as Q6K.
+inline int cq_storage_dtype(int ggml_dtype) {
+    return ggml_dtype == CQ_DTYPE_Q5_0 ? CQ_DTYPE_Q8_0 : ggml_dtype == CQ_DTYPE_Q3K ? CQ_DTYPE_Q6K : ggml_dtype;
+}
+hipError_t cq_launch_transcode(int ggml_dtype, uint8_t *ggml_aos_dev, uint8_t *storage_aos_dev, int64_t nblocks, bool inverse,
+                               hipStream_t s);
 // A step of the caller's model computed on the way into the activation quantizer (CQ_PRE_*):
 // rms_norm: x / sqrt(mean(x^2) + eps) * aux[k]; silu_mul: silu(x) * aux[m][k] (aux indexed like x).
 struct cq_pre {

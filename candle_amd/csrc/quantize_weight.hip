@@ -7,6 +7,7 @@
 //   Q4K  :1252-1311 + utils.rs:201-258 (make_qkx1_quants) + :49-59 (get_scale_min_k4)
 //   Q5K  :1450-1525, the same with 32 levels
 //   Q6K  :1643-1713 + utils.rs:61-198  (make_qx_quants, n=16, nmax=32, rmse_type=1)
+//   Q5_0 :393-425                 Q3K  :1011-1090 + utils.rs:261-326 (make_q3_quants, nmax=4, do_rmse)
 #include "qhip_internal.h"
 
 namespace {
@@ -276,6 +277,122 @@ __global__ void quantize_q6k(const float *__restrict__ src, int64_t nblocks, uin
     store_u16(y + 208, dh);
 }
 
+__global__ void quantize_q5_0(const float *__restrict__ src, int64_t nblocks, uint8_t *__restrict__ out) {
+    const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    const float *x = src + b * 32;
+    float amax = 0.0f, max = 0.0f;
+    for (int j = 0; j < 32; j++) {
+        const float v = x[j];
+        if (amax < fabsf(v)) { amax = fabsf(v); max = v; }
+    }
+    const float d = max / -16.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    uint8_t *y = out + b * 22;
+    store_u16(y, cq_f2h(d));
+    uint32_t qh = 0;
+    for (int j = 0; j < 16; j++) {
+        const float x0 = x[j] * id, x1 = x[j + 16] * id;
+        const int8_t s0 = cq_as_i8(x0 + 16.5f), s1 = cq_as_i8(x1 + 16.5f);
+        const uint8_t xi0 = (uint8_t)(s0 < 31 ? s0 : 31), xi1 = (uint8_t)(s1 < 31 ? s1 : 31);
+        y[6 + j] = (uint8_t)((xi0 & 0x0F) | ((xi1 & 0x0F) << 4));
+        qh |= (((uint32_t)xi0 & 0x10u) >> 4) << j;
+        qh |= (((uint32_t)xi1 & 0x10u) >> 4) << (j + 16);
+    }
+    y[2] = (uint8_t)qh; y[3] = (uint8_t)(qh >> 8); y[4] = (uint8_t)(qh >> 16); y[5] = (uint8_t)(qh >> 24);
+}
+
+// utils.rs:261-326 with nmax = 4, do_rmse = true, n = 16: only the returned scale is used
+__device__ float make_q3_quants_16(const float *x) {
+    const int n = 16, nmax = 4;
+    int8_t l[16];
+    float max = 0.0f, amax = 0.0f;
+    for (int i = 0; i < n; i++) {
+        const float ax = fabsf(x[i]);
+        if (ax > amax) { amax = ax; max = x[i]; }
+    }
+    if (amax == 0.0f) return 0.0f;
+    const float iscale = -(float)nmax / max;
+    float sumlx = 0.0f, suml2 = 0.0f;
+    for (int i = 0; i < n; i++) {
+        int li = cq_nearest_int(iscale * x[i]);
+        li = li < -nmax ? -nmax : (li > nmax - 1 ? nmax - 1 : li);
+        l[i] = (int8_t)li;
+        const float w = x[i] * x[i];
+        sumlx += w * x[i] * (float)li;
+        suml2 += w * (float)(li * li);
+    }
+    for (int t = 0; t < 5; t++) {
+        int n_changed = 0;
+        for (int i = 0; i < n; i++) {
+            const float w = x[i] * x[i];
+            float slx = sumlx - w * x[i] * (float)l[i];
+            if (slx > 0.0f) {
+                float sl2 = suml2 - w * (float)((int)l[i] * (int)l[i]);
+                int new_l = cq_nearest_int(x[i] * sl2 / slx);
+                new_l = new_l < -nmax ? -nmax : (new_l > nmax - 1 ? nmax - 1 : new_l);
+                if (new_l != (int)l[i]) {
+                    slx += w * x[i] * (float)new_l;
+                    sl2 += w * (float)(new_l * new_l);
+                    if (sl2 > 0.0f && slx * slx * suml2 > sumlx * sumlx * sl2) {
+                        l[i] = (int8_t)new_l;
+                        sumlx = slx;
+                        suml2 = sl2;
+                        n_changed++;
+                    }
+                }
+            }
+        }
+        if (n_changed == 0) break;
+    }
+    return sumlx / suml2;
+}
+
+__global__ void quantize_q3k(const float *__restrict__ src, int64_t nblocks, uint8_t *__restrict__ out) {
+    const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    const float *x = src + b * 256;
+    uint8_t *y = out + b * 110;
+    uint8_t *hmask = y, *qs = y + 32, *sc = y + 96;
+    float scales[16];
+    for (int j = 0; j < 16; j++) scales[j] = make_q3_quants_16(x + 16 * j);
+    float max_scale = 0.0f;
+    for (int j = 0; j < 16; j++)
+        if (fabsf(scales[j]) > fabsf(max_scale)) max_scale = scales[j];
+    for (int i = 0; i < 108; i++) y[i] = 0;
+    uint16_t dh = cq_f2h(0.0f);
+    if (max_scale != 0.0f) {
+        const float iscale = -32.0f / max_scale;
+        for (int j = 0; j < 16; j++) {
+            int lv = cq_nearest_int(iscale * scales[j]);
+            lv = (lv < -32 ? -32 : (lv > 31 ? 31 : lv)) + 32;
+            if (j < 8) sc[j] = (uint8_t)(lv & 0xF);
+            else sc[j - 8] |= (uint8_t)((lv & 0xF) << 4);
+            lv >>= 4;
+            sc[j % 4 + 8] |= (uint8_t)(lv << (2 * (j / 4)));
+        }
+        dh = cq_f2h(1.0f / iscale);
+    }
+    store_u16(y + 108, dh);
+    const float dall = cq_h2f(dh);
+    // element e: two low bits into qs[32 * (e / 128) + e % 32] at 2 * ((e % 128) / 32), the third into hmask[e % 32] bit e / 32
+    for (int j = 0; j < 16; j++) {
+        const int low = j < 8 ? (sc[j] & 0xF) : (sc[j - 8] >> 4);
+        const int s6 = (low | (((sc[8 + j % 4] >> (2 * (j / 4))) & 3) << 4)) - 32;
+        const float d = dall * (float)s6;
+        for (int ii = 0; ii < 16; ii++) {
+            const int e = 16 * j + ii;
+            int lv = 0;
+            if (d != 0.0f) {
+                lv = cq_nearest_int(x[e] / d);
+                lv = (lv < -4 ? -4 : (lv > 3 ? 3 : lv)) + 4;
+            }
+            if (lv > 3) { hmask[e % 32] |= (uint8_t)(1u << (e / 32)); lv -= 4; }
+            qs[32 * (e / 128) + e % 32] |= (uint8_t)(lv << (2 * ((e % 128) / 32)));
+        }
+    }
+}
+
 }  // namespace
 
 hipError_t cq_launch_quantize_weight(int dtype, const float *src, int64_t nblocks, uint8_t *aos_dev, hipStream_t s) {
@@ -285,6 +402,8 @@ hipError_t cq_launch_quantize_weight(int dtype, const float *src, int64_t nblock
     switch (dtype) {
     case CQ_DTYPE_Q4_0: quantize_q4_0<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q8_0: quantize_q8_0<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
+    case CQ_DTYPE_Q5_0: quantize_q5_0<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
+    case CQ_DTYPE_Q3K: quantize_q3k<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q4K: quantize_q4k<16><<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q5K: quantize_q4k<32><<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q6K: quantize_q6k<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;

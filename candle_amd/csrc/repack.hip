@@ -208,6 +208,85 @@ __global__ void repack_q6k(const uint8_t *__restrict__ aos, uint8_t *__restrict_
     }
 }
 
+// ---- types held in another type's planes --------------------------------------------------------
+// Q5_0 {f16 d; u8 qh[4]; u8 qs[16]} (k_quants.rs:61-67) holds d and 32 five-bit quants q, value d * (q - 16): exactly a
+// Q8_0 block {f16 d; i8 qs[32]} with qs = q - 16, whose dequantization (k_quants.rs:568-584) and dot product with Q8_0
+// activations (:631-649) are the arithmetic of Q5_0's (:428-451, :371-391) operation for operation.
+__global__ void transcode_q5_0_q8_0(uint8_t *__restrict__ q5, uint8_t *__restrict__ q8, int64_t nblocks, bool inverse) {
+    const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    uint8_t *x = q5 + b * 22, *y = q8 + b * 34;
+    if (!inverse) {
+        y[0] = x[0];
+        y[1] = x[1];
+        const uint32_t qh = (uint32_t)x[2] | ((uint32_t)x[3] << 8) | ((uint32_t)x[4] << 16) | ((uint32_t)x[5] << 24);
+        for (int j = 0; j < 16; j++) {
+            const int x0 = (int)((x[6 + j] & 0x0F) | (((qh >> j) & 1u) << 4)) - 16;
+            const int x1 = (int)((x[6 + j] >> 4) | (((qh >> (j + 16)) & 1u) << 4)) - 16;
+            y[2 + j] = (uint8_t)(int8_t)x0;
+            y[2 + j + 16] = (uint8_t)(int8_t)x1;
+        }
+    } else {
+        x[0] = y[0];
+        x[1] = y[1];
+        uint32_t qh = 0;
+        for (int j = 0; j < 16; j++) {
+            const uint32_t v0 = (uint32_t)((int)(int8_t)y[2 + j] + 16) & 31u, v1 = (uint32_t)((int)(int8_t)y[2 + j + 16] + 16) & 31u;
+            x[6 + j] = (uint8_t)((v0 & 0x0F) | ((v1 & 0x0F) << 4));
+            qh |= (v0 >> 4) << j;
+            qh |= (v1 >> 4) << (j + 16);
+        }
+        x[2] = (uint8_t)qh; x[3] = (uint8_t)(qh >> 8); x[4] = (uint8_t)(qh >> 16); x[5] = (uint8_t)(qh >> 24);
+    }
+}
+
+// Q3K {u8 hmask[32]; u8 qs[64]; u8 scales[12]; f16 d} (k_quants.rs:107-114): sixteen groups of sixteen three-bit quants,
+// value (d * (sc_j - 32)) * (q - 4) with six-bit sc_j: exactly a Q6K block {ql, qh, i8 scales[16], f16 d} with
+// scales[j] = sc_j - 32 and six-bit quants q + 28 (so that q6 - 32 = q - 4), whose dequantization (k_quants.rs:1716-1746)
+// and dot product with Q8K activations (:1585-1641) are those of Q3K (:1094-1146, :890-1009): the same integers, the
+// same products in the same order.
+__device__ __forceinline__ int q3k_scale6(const uint8_t *sc, int j) {
+    const int low = j < 8 ? (sc[j] & 0xF) : (sc[j - 8] >> 4);
+    return low | (((sc[8 + j % 4] >> (2 * (j / 4))) & 3) << 4);
+}
+__global__ void transcode_q3k_q6k(uint8_t *__restrict__ q3, uint8_t *__restrict__ q6, int64_t nblocks, bool inverse) {
+    const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    uint8_t *x = q3 + b * 110, *y = q6 + b * 210;
+    uint8_t *hmask = x, *qs = x + 32, *sc3 = x + 96;
+    uint8_t *ql = y, *qh = y + 128, *sc6 = y + 192;
+    if (!inverse) {
+        for (int i = 0; i < 192; i++) y[i] = 0;
+        for (int e = 0; e < 256; e++) {
+            const int half = e / 128, r = e % 128, quad = r / 32, l = r % 32;
+            const int low = (qs[32 * half + l] >> (2 * quad)) & 3;
+            const int v = low + 4 * ((hmask[e % 32] >> (e / 32)) & 1) + 28;   // (q - 4) + 32
+            ql[64 * half + 32 * (quad & 1) + l] |= (uint8_t)((v & 0xF) << (4 * (quad >> 1)));
+            qh[32 * half + l] |= (uint8_t)((v >> 4) << (2 * quad));
+        }
+        for (int j = 0; j < 16; j++) sc6[j] = (uint8_t)(int8_t)(q3k_scale6(sc3, j) - 32);
+        y[208] = x[108];
+        y[209] = x[109];
+    } else {
+        for (int i = 0; i < 108; i++) x[i] = 0;
+        for (int e = 0; e < 256; e++) {
+            const int half = e / 128, r = e % 128, quad = r / 32, l = r % 32;
+            const int v6 = ((ql[64 * half + 32 * (quad & 1) + l] >> (4 * (quad >> 1))) & 0xF) | (((qh[32 * half + l] >> (2 * quad)) & 3) << 4);
+            const int v = v6 - 28;   // 0..7
+            qs[32 * half + l] |= (uint8_t)((v & 3) << (2 * quad));
+            hmask[e % 32] |= (uint8_t)((v >> 2) << (e / 32));
+        }
+        for (int j = 0; j < 16; j++) {
+            const int lv = (int)(int8_t)sc6[j] + 32;
+            if (j < 8) sc3[j] |= (uint8_t)(lv & 0xF);
+            else sc3[j - 8] |= (uint8_t)((lv & 0xF) << 4);
+            sc3[8 + j % 4] |= (uint8_t)((lv >> 4) << (2 * (j / 4)));
+        }
+        x[108] = y[208];
+        x[109] = y[209];
+    }
+}
+
 hipError_t launch(const cq_weight *w, uint8_t *aos, bool inverse, hipStream_t s) {
     const int64_t bs = cq_block_size(w->dtype);
     const int64_t nblocks = w->n * (w->k / bs);
@@ -251,4 +330,18 @@ hipError_t cq_launch_repack(const cq_weight *w, const uint8_t *aos_dev, hipStrea
 }
 hipError_t cq_launch_unpack(const cq_weight *w, uint8_t *aos_dev, hipStream_t s) {
     return launch(w, aos_dev, true, s);
+}
+
+// GGML blocks of type `ggml_dtype` <-> GGML blocks of the type whose planes hold them (cq_storage_dtype).
+hipError_t cq_launch_transcode(int ggml_dtype, uint8_t *ggml_aos_dev, uint8_t *storage_aos_dev, int64_t nblocks, bool inverse,
+                               hipStream_t s) {
+    if (nblocks == 0) return hipSuccess;
+    const int threads = 128;
+    const unsigned grid = (unsigned)((nblocks + threads - 1) / threads);
+    switch (ggml_dtype) {
+    case CQ_DTYPE_Q5_0: transcode_q5_0_q8_0<<<grid, threads, 0, s>>>(ggml_aos_dev, storage_aos_dev, nblocks, inverse); break;
+    case CQ_DTYPE_Q3K: transcode_q3k_q6k<<<grid, threads, 0, s>>>(ggml_aos_dev, storage_aos_dev, nblocks, inverse); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
 }

@@ -27,6 +27,11 @@
  *   silu_mul (op.rs:607-609, quantized_llama.rs:60-62) : closed form in float64 (no reference
  *        golden prints silu of known inputs on this path; PARITY UNPINNED beyond that: the last
  *        bits depend on the platform's expf)
+ *   q5_0 quantize, dequant, q5_0 x q8_0 dot (k_quants.rs:352-452) : :289-319 (128 round-trip values), :317
+ *        (RMSE bound), :795-805 (dot-product error <= 0.001353), numpy brute force from unpacked blocks
+ *   q3k quantize (make_q3_quants, utils.rs:261-326), dequant, q3k x q8k dot (k_quants.rs:874-1148)
+ *                                               : :484-529 (spot values, < 0.03, < 3.5, RMSE <= 0.004),
+ *        :795-805 (dot-product error <= 0.016148), numpy brute force from unpacked blocks
  *   q4_1 quantize, dequant, q4_1 x q8_1 dot (k_quants.rs:257-350; oracle only, the
  *        product has no Q4_1 weights)            : :256-287 (128 round-trip values), :393-434
  *        (RMSE bound), :795 + :866 (dot-product error <= 0.008 on cos vectors, x2 on ramps)
@@ -65,6 +70,10 @@ typedef struct { uint8_t ql[QK_K / 2]; uint8_t qh[QK_K / 4]; int8_t scales[QK_K 
 typedef struct { float d; int8_t qs[QK_K]; int16_t bsums[QK_K / 16]; } block_q8k; /* 292 */
 #pragma pack(pop)
 
+typedef struct { uint16_t d; uint8_t qh[4]; uint8_t qs[16]; } block_q5_0;       /* 22, k_quants.rs:61-67 */
+typedef struct { uint8_t hmask[QK_K / 8]; uint8_t qs[QK_K / 4]; uint8_t scales[12]; uint16_t d; } block_q3k; /* 110, k_quants.rs:107-114 */
+_Static_assert(sizeof(block_q5_0) == 22, "q5_0");
+_Static_assert(sizeof(block_q3k) == 110, "q3k");
 _Static_assert(sizeof(block_q4_0) == 18, "q4_0");
 _Static_assert(sizeof(block_q4_1) == 20, "q4_1");
 _Static_assert(sizeof(block_q8_0) == 34, "q8_0");
@@ -214,6 +223,80 @@ static float vec_dot_q4_0_q8_0(int64_t n, const block_q4_0 *xs, const block_q8_0
     for (int64_t i = 0; i < n / 32; i++) {
         int32_t sum_i = sumi_q4_0_q8_0(&xs[i], &ys[i]);
         sumf += (float)sum_i * orc_f16_to_f32(xs[i].d) * orc_f16_to_f32(ys[i].d);
+    }
+    return sumf;
+}
+
+/* --------------------------------------------------------------- Q5_0 ---- */
+/* k_quants.rs:393-425 (from_float) */
+int orc_quantize_q5_0(const float *xs, void *out, int64_t k) {
+    if (k % 32 != 0) return -1;
+    block_q5_0 *ys = (block_q5_0 *)out;
+    for (int64_t i = 0; i < k / 32; i++) {
+        const float *x = xs + i * 32;
+        float amax = 0.0f, max = 0.0f;
+        for (int j = 0; j < 32; j++) {
+            if (amax < fabsf(x[j])) { amax = fabsf(x[j]); max = x[j]; }
+        }
+        float d = max / -16.0f;
+        float id = d != 0.0f ? 1.0f / d : 0.0f;
+        ys[i].d = orc_f32_to_f16(d);
+        uint32_t qh = 0;
+        for (int j = 0; j < 16; j++) {
+            float x0 = x[j] * id, x1 = x[j + 16] * id;
+            int8_t s0 = as_i8(x0 + 16.5f), s1 = as_i8(x1 + 16.5f);
+            uint8_t xi0 = (uint8_t)(s0 < 31 ? s0 : 31), xi1 = (uint8_t)(s1 < 31 ? s1 : 31);
+            ys[i].qs[j] = (uint8_t)((xi0 & 0x0F) | ((xi1 & 0x0F) << 4));
+            qh |= (((uint32_t)xi0 & 0x10u) >> 4) << j;
+            qh |= (((uint32_t)xi1 & 0x10u) >> 4) << (j + 16);
+        }
+        ys[i].qh[0] = (uint8_t)qh; ys[i].qh[1] = (uint8_t)(qh >> 8);
+        ys[i].qh[2] = (uint8_t)(qh >> 16); ys[i].qh[3] = (uint8_t)(qh >> 24);
+    }
+    return 0;
+}
+
+static inline uint32_t q5_0_qh(const block_q5_0 *x) {
+    return (uint32_t)x->qh[0] | ((uint32_t)x->qh[1] << 8) | ((uint32_t)x->qh[2] << 16) | ((uint32_t)x->qh[3] << 24);
+}
+
+/* k_quants.rs:428-451 (to_float) */
+int orc_dequantize_q5_0(const void *in, float *ys, int64_t k) {
+    if (k % 32 != 0) return -1;
+    const block_q5_0 *xs = (const block_q5_0 *)in;
+    for (int64_t i = 0; i < k / 32; i++) {
+        float d = orc_f16_to_f32(xs[i].d);
+        uint32_t qh = q5_0_qh(&xs[i]);
+        for (int j = 0; j < 16; j++) {
+            uint8_t xh_0 = (uint8_t)(((qh >> j) << 4) & 0x10);
+            uint8_t xh_1 = (uint8_t)((qh >> (j + 12)) & 0x10);
+            int32_t x0 = (int32_t)((xs[i].qs[j] & 0x0F) | xh_0) - 16;
+            int32_t x1 = (int32_t)((xs[i].qs[j] >> 4) | xh_1) - 16;
+            ys[i * 32 + j] = (float)x0 * d;
+            ys[i * 32 + j + 16] = (float)x1 * d;
+        }
+    }
+    return 0;
+}
+
+/* k_quants.rs:371-391 (vec_dot_unopt of Q5_0 x Q8_0) */
+static int32_t sumi_q5_0_q8_0(const block_q5_0 *x, const block_q8_0 *y) {
+    uint32_t qh = q5_0_qh(x);
+    int32_t sumi = 0;
+    for (int j = 0; j < 16; j++) {
+        uint8_t xh_0 = (uint8_t)(((qh & (1u << j)) >> j) << 4);
+        uint8_t xh_1 = (uint8_t)((qh & (1u << (j + 16))) >> (j + 12));
+        int32_t x0 = ((int32_t)(x->qs[j] & 0x0F) | (int32_t)xh_0) - 16;
+        int32_t x1 = ((int32_t)(x->qs[j] >> 4) | (int32_t)xh_1) - 16;
+        sumi += x0 * (int32_t)y->qs[j] + x1 * (int32_t)y->qs[j + 16];
+    }
+    return sumi;
+}
+static float vec_dot_q5_0_q8_0(int64_t n, const block_q5_0 *xs, const block_q8_0 *ys) {
+    float sumf = 0.0f;
+    for (int64_t i = 0; i < n / 32; i++) {
+        int32_t sumi = sumi_q5_0_q8_0(&xs[i], &ys[i]);
+        sumf += (float)sumi * orc_f16_to_f32(xs[i].d) * orc_f16_to_f32(ys[i].d);
     }
     return sumf;
 }
@@ -944,18 +1027,171 @@ static inline int32_t int_q6k_q8k(const block_q6k *x, const block_q8k *y) {
     return total;
 }
 
+/* ---------------------------------------------------------------- Q3K ---- */
+/* utils.rs:261-326 (make_q3_quants; from_float calls it with nmax = 4, do_rmse = true and uses the returned
+ * scale only) */
+static float make_q3_quants(const float *x, int n, int32_t nmax, int do_rmse) {
+    int8_t l[32];
+    float max = 0.0f, amax = 0.0f;
+    for (int i = 0; i < n; i++) {
+        float ax = fabsf(x[i]);
+        if (ax > amax) { amax = ax; max = x[i]; }
+    }
+    if (amax == 0.0f) return 0.0f;
+    float iscale = -(float)nmax / max;
+    if (do_rmse) {
+        float sumlx = 0.0f, suml2 = 0.0f;
+        for (int i = 0; i < n; i++) {
+            int32_t li = clampi(nearest_int(iscale * x[i]), -nmax, nmax - 1);
+            l[i] = (int8_t)li;
+            float w = x[i] * x[i];
+            sumlx += w * x[i] * (float)li;
+            suml2 += w * (float)(li * li);
+        }
+        for (int t = 0; t < 5; t++) {
+            int n_changed = 0;
+            for (int i = 0; i < n; i++) {
+                float w = x[i] * x[i];
+                float slx = sumlx - w * x[i] * (float)l[i];
+                if (slx > 0.0f) {
+                    float sl2 = suml2 - w * (float)((int32_t)l[i] * (int32_t)l[i]);
+                    int32_t new_l = clampi(nearest_int(x[i] * sl2 / slx), -nmax, nmax - 1);
+                    if (new_l != (int32_t)l[i]) {
+                        slx += w * x[i] * (float)new_l;
+                        sl2 += w * (float)(new_l * new_l);
+                        if (sl2 > 0.0f && slx * slx * suml2 > sumlx * sumlx * sl2) {
+                            l[i] = (int8_t)new_l;
+                            sumlx = slx;
+                            suml2 = sl2;
+                            n_changed++;
+                        }
+                    }
+                }
+            }
+            if (n_changed == 0) break;
+        }
+        return sumlx / suml2;
+    }
+    return 1.0f / iscale;
+}
+
+/* the 6-bit scale of 16-element group j, k_quants.rs:1055-1061 */
+static inline int32_t q3k_scale(const block_q3k *b, int j) {
+    int32_t sc = j < 8 ? (b->scales[j] & 0xF) : (b->scales[j - 8] >> 4);
+    return sc | (((b->scales[8 + j % 4] >> (2 * (j / 4))) & 3) << 4);
+}
+/* the signed 3-bit quant of element e: two low bits from qs, minus 4 unless its hmask bit is set */
+static inline int32_t q3k_quant(const block_q3k *b, int e) {
+    int half = e / 128, r = e % 128;
+    int32_t low = (b->qs[32 * half + r % 32] >> (2 * (r / 32))) & 3;
+    return low - ((b->hmask[e % 32] >> (e / 32)) & 1 ? 0 : 4);
+}
+
+/* k_quants.rs:1011-1090 (from_float) */
+int orc_quantize_q3k(const float *xs, void *out, int64_t k) {
+    if (k % QK_K != 0) return -1;
+    block_q3k *ys = (block_q3k *)out;
+    for (int64_t i = 0; i < k / QK_K; i++) {
+        const float *x = xs + i * QK_K;
+        block_q3k *block = &ys[i];
+        float scales[QK_K / 16];
+        for (int j = 0; j < QK_K / 16; j++) scales[j] = make_q3_quants(x + 16 * j, 16, 4, 1);
+        float max_scale = 0.0f;
+        for (int j = 0; j < QK_K / 16; j++)
+            if (fabsf(scales[j]) > fabsf(max_scale)) max_scale = scales[j];
+        memset(block->scales, 0, 12);
+        if (max_scale != 0.0f) {
+            float iscale = -32.0f / max_scale;
+            for (int j = 0; j < QK_K / 16; j++) {
+                int32_t l_val = clampi(nearest_int(iscale * scales[j]), -32, 31) + 32;
+                if (j < 8) block->scales[j] = (uint8_t)(l_val & 0xF);
+                else block->scales[j - 8] |= (uint8_t)((l_val & 0xF) << 4);
+                l_val >>= 4;
+                block->scales[j % 4 + 8] |= (uint8_t)(l_val << (2 * (j / 4)));
+            }
+            block->d = orc_f32_to_f16(1.0f / iscale);
+        } else {
+            block->d = orc_f32_to_f16(0.0f);
+        }
+        int8_t l[QK_K];
+        memset(l, 0, sizeof l);
+        for (int j = 0; j < QK_K / 16; j++) {
+            int32_t sc = q3k_scale(block, j) - 32;
+            float d = orc_f16_to_f32(block->d) * (float)sc;
+            if (d != 0.0f) {
+                for (int ii = 0; ii < 16; ii++) {
+                    int32_t l_val = nearest_int(x[16 * j + ii] / d);
+                    l[16 * j + ii] = (int8_t)(clampi(l_val, -4, 3) + 4);
+                }
+            }
+        }
+        memset(block->hmask, 0, QK_K / 8);
+        int m = 0;
+        uint8_t hm = 1;
+        for (int e = 0; e < QK_K; e++) {
+            if (l[e] > 3) { block->hmask[m] |= hm; l[e] -= 4; }
+            if (++m == QK_K / 8) { m = 0; hm = (uint8_t)(hm << 1); }
+        }
+        for (int j = 0; j < QK_K; j += 128)
+            for (int lv = 0; lv < 32; lv++)
+                block->qs[j / 4 + lv] = (uint8_t)(l[j + lv] | (l[j + lv + 32] << 2) | (l[j + lv + 64] << 4) | (l[j + lv + 96] << 6));
+    }
+    return 0;
+}
+
+/* k_quants.rs:1094-1146 (to_float): y = (d_all * (scale - 32)) * q */
+int orc_dequantize_q3k(const void *in, float *ys, int64_t k) {
+    if (k % QK_K != 0) return -1;
+    const block_q3k *xs = (const block_q3k *)in;
+    for (int64_t i = 0; i < k / QK_K; i++) {
+        float d_all = orc_f16_to_f32(xs[i].d);
+        for (int e = 0; e < QK_K; e++) {
+            float dl = d_all * ((float)(int8_t)q3k_scale(&xs[i], e / 16) - 32.0f);
+            ys[i * QK_K + e] = dl * (float)(int8_t)q3k_quant(&xs[i], e);
+        }
+    }
+    return 0;
+}
+
+/* k_quants.rs:890-1009 (vec_dot_unopt of Q3K x Q8K): eight integer lanes (element index mod 8) per block,
+ * sums[l] += (d * d8) * aux32[l], the eight sums added at the end. */
+static void ints_q3k_q8k(const block_q3k *x, const block_q8k *y, int32_t aux32[8]) {
+    for (int l = 0; l < 8; l++) aux32[l] = 0;
+    for (int j = 0; j < QK_K / 16; j++) {
+        int32_t scale = q3k_scale(x, j) - 32;
+        for (int h = 0; h < 2; h++)
+            for (int l = 0; l < 8; l++) {
+                int e = 16 * j + 8 * h + l;
+                int16_t p = (int16_t)((int16_t)y->qs[e] * (int16_t)q3k_quant(x, e));
+                aux32[l] += scale * (int32_t)p;
+            }
+    }
+}
+static float vec_dot_q3k_q8k(int64_t n, const block_q3k *xs, const block_q8k *ys) {
+    float sums[8] = {0};
+    for (int64_t i = 0; i < n / QK_K; i++) {
+        int32_t aux32[8];
+        ints_q3k_q8k(&xs[i], &ys[i], aux32);
+        float d = orc_f16_to_f32(xs[i].d) * ys[i].d;
+        for (int l = 0; l < 8; l++) sums[l] += d * (float)aux32[l];
+    }
+    float total = 0.0f;
+    for (int l = 0; l < 8; l++) total += sums[l];
+    return total;
+}
+
 /* -------------------------------------------------------- type dispatch ---- */
 int64_t orc_block_size(int dtype) {
     switch (dtype) {
-    case ORC_Q4_0: case ORC_Q4_1: case ORC_Q8_0: case ORC_Q8_1: return 32;
-    case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return QK_K;
+    case ORC_Q4_0: case ORC_Q4_1: case ORC_Q5_0: case ORC_Q8_0: case ORC_Q8_1: return 32;
+    case ORC_Q3K: case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return QK_K;
     default: return 0;
     }
 }
 int64_t orc_type_size(int dtype) {
     switch (dtype) {
-    case ORC_Q4_0: return 18; case ORC_Q4_1: return 20; case ORC_Q8_0: return 34; case ORC_Q8_1: return 36;
-    case ORC_Q4K: return 144; case ORC_Q5K: return 176; case ORC_Q6K: return 210; case ORC_Q8K: return 292;
+    case ORC_Q4_0: return 18; case ORC_Q4_1: return 20; case ORC_Q5_0: return 22; case ORC_Q8_0: return 34; case ORC_Q8_1: return 36;
+    case ORC_Q3K: return 110; case ORC_Q4K: return 144; case ORC_Q5K: return 176; case ORC_Q6K: return 210; case ORC_Q8K: return 292;
     default: return 0;
     }
 }
@@ -963,9 +1199,9 @@ int64_t orc_type_size(int dtype) {
  * k_quants.rs:160, :565, :1155, :1569, :1752). */
 int orc_vec_dot_type(int dtype) {
     switch (dtype) {
-    case ORC_Q4_0: case ORC_Q8_0: return ORC_Q8_0;
+    case ORC_Q4_0: case ORC_Q5_0: case ORC_Q8_0: return ORC_Q8_0;   /* Q5_0: k_quants.rs:356 */
     case ORC_Q4_1: return ORC_Q8_1;   /* k_quants.rs:260 */
-    case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return ORC_Q8K;
+    case ORC_Q3K: case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return ORC_Q8K;   /* Q3K: k_quants.rs:877 */
     default: return -1;
     }
 }
@@ -974,6 +1210,8 @@ int orc_quantize(int dtype, const float *xs, void *out, int64_t k) {
     switch (dtype) {
     case ORC_Q4_0: return orc_quantize_q4_0(xs, out, k);
     case ORC_Q4_1: return orc_quantize_q4_1(xs, out, k);
+    case ORC_Q5_0: return orc_quantize_q5_0(xs, out, k);
+    case ORC_Q3K: return orc_quantize_q3k(xs, out, k);
     case ORC_Q8_0: return orc_quantize_q8_0(xs, out, k);
     case ORC_Q8_1: return orc_quantize_q8_1(xs, out, k);
     case ORC_Q4K: return orc_quantize_q4k(xs, out, k);
@@ -988,6 +1226,8 @@ int orc_dequantize(int dtype, const void *in, float *ys, int64_t k) {
     switch (dtype) {
     case ORC_Q4_0: return orc_dequantize_q4_0(in, ys, k);
     case ORC_Q4_1: return orc_dequantize_q4_1(in, ys, k);
+    case ORC_Q5_0: return orc_dequantize_q5_0(in, ys, k);
+    case ORC_Q3K: return orc_dequantize_q3k(in, ys, k);
     case ORC_Q8_0: return orc_dequantize_q8_0(in, ys, k);
     case ORC_Q4K: return orc_dequantize_q4k(in, ys, k);
     case ORC_Q5K: return orc_dequantize_q5k(in, ys, k);
@@ -1004,6 +1244,8 @@ int orc_vec_dot(int dtype, int64_t n, const void *xs, const void *ys, float *out
     switch (dtype) {
     case ORC_Q4_0: *out = vec_dot_q4_0_q8_0(n, xs, ys); return 0;
     case ORC_Q4_1: return vec_dot_q4_1_q8_1(n, xs, ys, out);
+    case ORC_Q5_0: *out = vec_dot_q5_0_q8_0(n, xs, ys); return 0;
+    case ORC_Q3K: *out = vec_dot_q3k_q8k(n, xs, ys); return 0;
     case ORC_Q8_0: *out = vec_dot_q8_0_q8_0(n, xs, ys); return 0;
     case ORC_Q4K: *out = vec_dot_q4k_q8k(n, xs, ys); return 0;
     case ORC_Q5K: *out = vec_dot_q5k_q8k(n, xs, ys); return 0;
@@ -1064,6 +1306,16 @@ int orc_block_int_dots(int dtype, int64_t m, int64_t k, int64_t n, const void *a
                 case ORC_Q8_0:
                     out_i[o] = sumi_q8_0_q8_0((const block_q8_0 *)w + b, (const block_q8_0 *)a + b);
                     break;
+                case ORC_Q5_0:
+                    out_i[o] = sumi_q5_0_q8_0((const block_q5_0 *)w + b, (const block_q8_0 *)a + b);
+                    break;
+                case ORC_Q3K: {
+                    int32_t aux32[8], t = 0;
+                    ints_q3k_q8k((const block_q3k *)w + b, (const block_q8k *)a + b, aux32);
+                    for (int l = 0; l < 8; l++) t += aux32[l];
+                    out_i[o] = t;
+                    break;
+                }
                 case ORC_Q8K:
                     out_i[o] = sumi_q8k_q8k((const block_q8k *)w + b, (const block_q8k *)a + b);
                     break;

@@ -107,6 +107,10 @@ def test_metadata_calls_need_no_gpu(lib):
     lib.cq_type_size.restype = ctypes.c_int
     lib.cq_vec_dot_type.restype = ctypes.c_int
     Q4_0, Q8_0, Q4K, Q6K, Q8K = 2, 8, 12, 14, 15
+    Q5_0, Q3K = 6, 11
+    assert (lib.cq_block_size(Q5_0), lib.cq_type_size(Q5_0), lib.cq_vec_dot_type(Q5_0)) == (32, 22, Q8_0)    # k_quants.rs:61-67, :356
+    assert (lib.cq_block_size(Q3K), lib.cq_type_size(Q3K), lib.cq_vec_dot_type(Q3K)) == (256, 110, Q8K)     # k_quants.rs:107-114, :877
+    assert (lib.cq_block_size(10), lib.cq_type_size(10), lib.cq_vec_dot_type(10)) == (0, 0, -1)             # Q2K: not handled
     assert (lib.cq_block_size(Q4_0), lib.cq_type_size(Q4_0)) == (32, 18)
     assert (lib.cq_block_size(Q8_0), lib.cq_type_size(Q8_0)) == (32, 34)
     assert (lib.cq_block_size(Q4K), lib.cq_type_size(Q4K)) == (256, 144)

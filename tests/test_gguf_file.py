@@ -200,7 +200,7 @@ def test_type_table_matches_library():
     """The parser's own size table against the device library's `cq_block_size` / `cq_type_size`."""
     from candle_amd import qhip
     L = qhip.load()
-    for t in (2, 8, 9, 12, 14, 15):
+    for t in (2, 6, 8, 9, 11, 12, 13, 14, 15):
         assert G.ggml_block_size(t) == L.cq_block_size(t), t
         assert G.ggml_type_size(t) == L.cq_type_size(t), t
 
@@ -211,7 +211,8 @@ def _model_file(tmp_path, rng):
     k, n = 512, 96
     host = {}
     for name, dt in (("blk.0.attn_q.weight", 12), ("blk.0.ffn_down.weight", 14),
-                     ("blk.0.attn_k.weight", 2), ("token_embd.weight", 8)):
+                     ("blk.0.attn_k.weight", 2), ("token_embd.weight", 8),
+                     ("blk.0.attn_v.weight", 6), ("blk.0.ffn_up.weight", 11), ("blk.0.ffn_gate.weight", 13)):
         w = (rng.standard_normal((n, k)) * 0.1).astype(np.float32)
         host[name] = HostQTensor(dt, O.quantize(dt, w), (n, k))
     host["blk.0.attn_norm.weight"] = HostQTensor(0, rng.standard_normal(k).astype(np.float32), (k,))
@@ -263,7 +264,7 @@ def test_load_gguf_to_device_and_matmul(tmp_path):
 
 @pytest.mark.gpu
 def test_load_gguf_rejects_types_without_device_kernels(tmp_path):
-    path = str(tmp_path / "q5.gguf")
-    G.save_gguf(path, {"w": HostQTensor(11, bytes(110), (1, 256))}, {})
-    with pytest.raises(GgufError, match="Q3K tensors are not supported on the device"):
+    path = str(tmp_path / "q2.gguf")
+    G.save_gguf(path, {"w": HostQTensor(10, bytes(84), (1, 256))}, {})
+    with pytest.raises(GgufError, match="Q2K tensors are not supported on the device"):
         G.load_gguf(path)

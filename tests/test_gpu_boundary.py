@@ -55,7 +55,7 @@ def test_flat_storage_runs_the_reference_goldens(qh, goldens, seeded_inputs):
         assert np.array_equal(out, out2)
 
 
-@pytest.mark.parametrize("dt", [orc.Q4_0, orc.Q8_0, orc.Q4K, orc.Q5K, orc.Q6K])
+@pytest.mark.parametrize("dt", [orc.Q4_0, orc.Q5_0, orc.Q8_0, orc.Q3K, orc.Q4K, orc.Q5K, orc.Q6K])
 @pytest.mark.parametrize("m", [1, 3, 16, 80])
 def test_shape_at_call_equals_shape_at_creation(qh, dt, m):
     """Every kernel family (one-launch decode, split-K, tile) reads flat storage like shaped storage, and one
@@ -78,6 +78,32 @@ def test_shape_at_call_equals_shape_at_creation(qh, dt, m):
     ref2 = orc.matmul(dt, x2.cpu().numpy(), blocks, 2 * n)
     assert np.linalg.norm(a2 - ref2) <= 1e-4 * np.linalg.norm(ref2)
     assert np.array_equal(flat.dequantize().cpu().numpy().ravel(), orc.dequantize(dt, blocks))
+
+
+@pytest.mark.parametrize("dt", [orc.Q5_0, orc.Q3K])
+def test_types_held_in_another_types_planes(qh, dt):
+    """Q5_0 lives in Q8_0 planes and Q3K in Q6K planes: the caller sees the type it created (dtype, GGML byte size,
+    all-zero blocks from `zeros`, its own bytes back), whatever the device holds; the prefill tile kernel and the
+    Q8K-formulation integers follow the oracle's Q5_0 / Q3K code."""
+    rng = np.random.default_rng(int(dt))
+    n, k = 64, 1024
+    nbytes = n * k // orc.BLOCK_SIZE[dt] * orc.TYPE_SIZE[dt]
+    z = qh.QWeight.zeros(dt, n, k)
+    assert z.dtype == dt and z.size_in_bytes == nbytes
+    assert not z.to_ggml().any()
+    assert not z.dequantize().cpu().numpy().any()
+    flat = qh.QWeight.zeros_flat(dt, n * k)
+    assert flat.dtype == dt and not flat.to_ggml().any()
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    q = z.quantize_(dev(w))                                   # QTensor::quantize into existing storage
+    blocks = orc.quantize(dt, w)
+    assert np.array_equal(q.to_ggml(), blocks)
+    x = rng.standard_normal((70, k)).astype(np.float32)      # more than 32 rows: the tile kernels
+    got = qh.qmatmul(q, dev(x)).cpu().numpy()
+    ref = orc.matmul(dt, x, blocks, n)
+    assert np.linalg.norm(got - ref) <= 1e-4 * np.linalg.norm(ref)
+    with pytest.raises(qh.QHipError, match="Q8_1 activations are for Q4K and Q6K"):
+        qh.qmatmul(q, dev(x), flags=qh.FLAG_ACT_Q8_1)
 
 
 def test_shape_errors(qh):

@@ -48,7 +48,9 @@ def make_inputs(seed, m, k, n, wscale=0.02, outliers=False):
     return w, x
 
 
-WEIGHT_DTYPES = [orc.Q4_0, orc.Q8_0, orc.Q4K, orc.Q5K, orc.Q6K]
+# Q5_0 and Q3K are held on the device in the planes of Q8_0 and Q6K (same values, same arithmetic): every test below
+# takes them through the boundary like the others and compares with the oracle's own Q5_0 / Q3K code
+WEIGHT_DTYPES = [orc.Q4_0, orc.Q5_0, orc.Q8_0, orc.Q3K, orc.Q4K, orc.Q5K, orc.Q6K]
 
 
 # ------------------------------------------------------------ activation quantizers ----
@@ -694,7 +696,7 @@ def test_few_rows_one_launch_equals_single_rows(qh, dt, m, k, n):
     qw = qh.QWeight.from_ggml(dt, blocks, n, k)
     xd = dev(x)
     got = qh.qmatmul(qw, xd)
-    elems = {orc.Q4_0: 32, orc.Q8_0: 16, orc.Q4K: 64, orc.Q5K: 64, orc.Q6K: 32}[dt]   # weights per 16-byte lane unit
+    elems = {orc.Q4_0: 32, orc.Q5_0: 16, orc.Q8_0: 16, orc.Q3K: 32, orc.Q4K: 64, orc.Q5K: 64, orc.Q6K: 32}[dt]   # weights per 16-byte lane unit
     units = k // elems
     per_lane = -(-units // 64) * elems
     if units <= (384 if m == 2 else 256) and (per_lane <= 64 or (per_lane <= 128 and m <= 3) or m <= 2):   # the library's rule

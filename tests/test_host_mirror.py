@@ -34,6 +34,9 @@ def test_python_mirror_dtype_table():
     assert (GgmlDType.Q4_0.block_size(), GgmlDType.Q4_0.type_size()) == (32, 18)
     assert GgmlDType.Q4K.vec_dot_type() == GgmlDType.Q8K
     assert GgmlDType.Q8_0.vec_dot_type() == GgmlDType.Q8_0
+    assert GgmlDType.from_str("q5_0") == GgmlDType.Q5_0 == 6 and GgmlDType.from_str("q3k") == GgmlDType.Q3K == 11
+    assert (GgmlDType.Q5_0.block_size(), GgmlDType.Q5_0.type_size(), GgmlDType.Q5_0.vec_dot_type()) == (32, 22, GgmlDType.Q8_0)
+    assert (GgmlDType.Q3K.block_size(), GgmlDType.Q3K.type_size(), GgmlDType.Q3K.vec_dot_type()) == (256, 110, GgmlDType.Q8K)
     with pytest.raises(ValueError):
         GgmlDType.from_str("q9_9")
 
@@ -82,7 +85,7 @@ def test_python_qtensor_roundtrip_and_f16():
     import torch
     from candle_amd.quantized import QTensor
     src = torch.linspace(-0.5, 0.5, 4 * 1024, device="cuda").reshape(4, 1024)
-    for name, bound in (("q4k", 0.017), ("q6k", 0.008), ("q8_0", 0.005), ("q4_0", 0.05)):
+    for name, bound in (("q4k", 0.017), ("q6k", 0.008), ("q8_0", 0.005), ("q4_0", 0.05), ("q5_0", 0.02), ("q3k", 0.03)):
         q = QTensor.quantize(src, name)
         back = q.dequantize()
         assert back.shape == src.shape and float((back - src).abs().max()) < bound, name
