@@ -52,7 +52,7 @@ extern "C" int cq_device_count(void) {
 // ------------------------------------------------------------ dtype tables ----
 extern "C" int64_t cq_block_size(int dt) {
     switch (dt) {
-    case CQ_DTYPE_Q4_0: case CQ_DTYPE_Q5_0: case CQ_DTYPE_Q8_0: case CQ_DTYPE_Q8_1: return 32;
+    case CQ_DTYPE_Q4_0: case CQ_DTYPE_Q4_1: case CQ_DTYPE_Q5_0: case CQ_DTYPE_Q5_1: case CQ_DTYPE_Q8_0: case CQ_DTYPE_Q8_1: return 32;
     case CQ_DTYPE_Q3K: case CQ_DTYPE_Q4K: case CQ_DTYPE_Q5K: case CQ_DTYPE_Q6K: case CQ_DTYPE_Q8K: return 256;
     default: return 0;
     }
@@ -60,7 +60,9 @@ extern "C" int64_t cq_block_size(int dt) {
 extern "C" int64_t cq_type_size(int dt) {
     switch (dt) {
     case CQ_DTYPE_Q4_0: return 18;
+    case CQ_DTYPE_Q4_1: return 20;
     case CQ_DTYPE_Q5_0: return 22;
+    case CQ_DTYPE_Q5_1: return 24;
     case CQ_DTYPE_Q3K: return 110;
     case CQ_DTYPE_Q8_0: return 34;
     case CQ_DTYPE_Q8_1: return 36;
@@ -74,13 +76,15 @@ extern "C" int64_t cq_type_size(int dt) {
 extern "C" int cq_vec_dot_type(int dt) {
     switch (dt) {
     case CQ_DTYPE_Q4_0: case CQ_DTYPE_Q5_0: case CQ_DTYPE_Q8_0: return CQ_DTYPE_Q8_0;
+    case CQ_DTYPE_Q4_1: case CQ_DTYPE_Q5_1: return CQ_DTYPE_Q8_1;   /* k_quants.rs:260, :457 */
     case CQ_DTYPE_Q3K: case CQ_DTYPE_Q4K: case CQ_DTYPE_Q5K: case CQ_DTYPE_Q6K: return CQ_DTYPE_Q8K;
     default: return -1;
     }
 }
 
 static bool is_weight_dtype(int dt) {
-    return dt == CQ_DTYPE_Q4_0 || dt == CQ_DTYPE_Q5_0 || dt == CQ_DTYPE_Q8_0 || dt == CQ_DTYPE_Q3K || dt == CQ_DTYPE_Q4K ||
+    return dt == CQ_DTYPE_Q4_0 || dt == CQ_DTYPE_Q4_1 || dt == CQ_DTYPE_Q5_0 || dt == CQ_DTYPE_Q5_1 || dt == CQ_DTYPE_Q8_0 ||
+           dt == CQ_DTYPE_Q3K || dt == CQ_DTYPE_Q4K ||
            dt == CQ_DTYPE_Q5K || dt == CQ_DTYPE_Q6K;
 }
 
@@ -112,6 +116,7 @@ static int weight_alloc(int dev, int dt, int64_t n, int64_t k, cq_weight **out) 
     case CQ_DTYPE_Q5K: s0 = (size_t)nb * 128; s1 = (size_t)nb * CQ_Q4K_HDR; s2 = (size_t)nb * 32; break;
     case CQ_DTYPE_Q6K: s0 = (size_t)nb * 128; s1 = (size_t)nb * 64; s2 = (size_t)nb * 16; s3 = (size_t)nb * 2; break;
     }
+    if (cq_has_min32(dt)) s2 = (size_t)nb * 2;   // the blocks' minima beside the Q8_0 planes
     const size_t o1 = cq_align_up(s0 + CQ_TAIL_PAD, 256);
     const size_t o2 = cq_align_up(o1 + s1 + CQ_TAIL_PAD, 256);
     const size_t o3 = cq_align_up(o2 + s2 + CQ_TAIL_PAD, 256);
@@ -142,7 +147,7 @@ static hipError_t blocks_to_planes(const cq_weight *w, uint8_t *ggml_aos_dev, hi
     void *tmp = nullptr;
     hipError_t e = hipMalloc(&tmp, (size_t)weight_blocks(w) * (size_t)cq_type_size(w->dtype) + 256);
     if (e != hipSuccess) return e;
-    e = cq_launch_transcode(w->ggml_dtype, ggml_aos_dev, (uint8_t *)tmp, weight_blocks(w), false, s);
+    e = cq_launch_transcode(w->ggml_dtype, ggml_aos_dev, (uint8_t *)tmp, (uint16_t *)w->p2, weight_blocks(w), false, s);
     if (e == hipSuccess) e = cq_launch_repack(w, (const uint8_t *)tmp, s);
     if (e == hipSuccess) e = hipStreamSynchronize(s);
     (void)hipFree(tmp);
@@ -154,7 +159,7 @@ static hipError_t planes_to_blocks(const cq_weight *w, uint8_t *ggml_aos_dev, hi
     hipError_t e = hipMalloc(&tmp, (size_t)weight_blocks(w) * (size_t)cq_type_size(w->dtype) + 256);
     if (e != hipSuccess) return e;
     e = cq_launch_unpack(w, (uint8_t *)tmp, s);
-    if (e == hipSuccess) e = cq_launch_transcode(w->ggml_dtype, ggml_aos_dev, (uint8_t *)tmp, weight_blocks(w), true, s);
+    if (e == hipSuccess) e = cq_launch_transcode(w->ggml_dtype, ggml_aos_dev, (uint8_t *)tmp, (uint16_t *)w->p2, weight_blocks(w), true, s);
     if (e == hipSuccess) e = hipStreamSynchronize(s);
     (void)hipFree(tmp);
     return e;
@@ -478,7 +483,9 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
                           (pre.kind != CQ_PRE_NONE &&
                            ranges_overlap(y_dev, m * w->n, pre.aux, pre.kind == CQ_PRE_RMS_NORM ? w->k : m * w->k));
     // decode (one activation row): a single launch that quantizes x in its prologue
-    if (m == 1 && !in_place && !(flags & (CQ_FLAG_REUSE_ACT | CQ_FLAG_FORCE_GEMM | CQ_FLAG_STAGED_ACT | CQ_FLAG_ACT_Q8_1)) &&
+    // (Q4_1 / Q5_1: the second launch that adds their m * s term reads the quantized row from the workspace)
+    const bool min32 = cq_has_min32(w->ggml_dtype);
+    if (m == 1 && !in_place && !min32 && !(flags & (CQ_FLAG_REUSE_ACT | CQ_FLAG_FORCE_GEMM | CQ_FLAG_STAGED_ACT | CQ_FLAG_ACT_Q8_1)) &&
         cq_matvec_fused_supported(w)) {
         CQ_HIP_CHECK(cq_launch_matvec_fused(w, x_dev, pre, y_dev, s));
         return CQ_OK;
@@ -526,7 +533,7 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
                             (long long)w->k);
     // two to four rows of short enough weight rows: the one-launch kernel again, every unpacked weight unit
     // contracted with each activation row
-    if (flags == 0 && pre.kind == CQ_PRE_NONE && !in_place && cq_matvec_fused_rows_supported(w, m)) {
+    if (flags == 0 && pre.kind == CQ_PRE_NONE && !in_place && !min32 && cq_matvec_fused_rows_supported(w, m)) {
         CQ_HIP_CHECK(cq_launch_matvec_fused_rows(w, x_dev, m, y_dev, s));
         return CQ_OK;
     }
@@ -548,6 +555,7 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
         case kGemm: CQ_HIP_CHECK(cq_launch_gemm(w, v, act, m, y_dev, y_cleared, s)); break;
         case kMatvec: CQ_HIP_CHECK(cq_launch_matvec(w, v, act, m, y_dev, s)); break;
     }
+    if (min32) CQ_HIP_CHECK(cq_launch_min32_term(w, v, m, y_dev, s));
     return CQ_OK;
 }
 
@@ -581,7 +589,7 @@ extern "C" int cq_qmatmul_multi(const cq_weight *const *ws, int count, int pre, 
     if (!ws || !ys_dev || count < 1) return cq_set_error(CQ_ERR_INVALID, "null argument");
     for (int i = 0; i < count; i++) {
         if (!ws[i]) return cq_set_error(CQ_ERR_INVALID, "null weight %d", i);
-        if (ws[i]->dtype != ws[0]->dtype || ws[i]->k != ws[0]->k || ws[i]->dev != ws[0]->dev)
+        if (ws[i]->ggml_dtype != ws[0]->ggml_dtype || ws[i]->k != ws[0]->k || ws[i]->dev != ws[0]->dev)
             return cq_set_error(CQ_ERR_INVALID, "weight %d differs in dtype, row length or device from weight 0", i);
     }
     const cq_pre p{pre, aux_dev, eps};
@@ -592,7 +600,7 @@ extern "C" int cq_qmatmul_multi(const cq_weight *const *ws, int count, int pre, 
             return cq_set_error(CQ_ERR_INVALID, "output %d overlaps the activations: cq_qmatmul_multi does not work in place", i);
     }
     // one activation row (or up to four of short weight rows), two or three weights: one launch over all their rows
-    if (m >= 1 && m <= 4 && flags == 0 && cq_matvec_fused_multi_supported(ws, count, pre, m)) {
+    if (m >= 1 && m <= 4 && flags == 0 && !cq_has_min32(ws[0]->ggml_dtype) && cq_matvec_fused_multi_supported(ws, count, pre, m)) {
         if (!x_dev) return cq_set_error(CQ_ERR_INVALID, "null argument");
         if ((uintptr_t)x_dev & 15) return cq_set_error(CQ_ERR_INVALID, "x must be 16-byte aligned");
         for (int i = 0; i < count; i++)
@@ -671,7 +679,7 @@ static int grouped_impl(const cq_weight *const *experts, int n_experts, const fl
     if (!w0) return cq_set_error(CQ_ERR_INVALID, "null expert");
     for (int e = 0; e < n_experts; e++) {
         if (!experts[e]) return cq_set_error(CQ_ERR_INVALID, "null expert %d", e);
-        if (experts[e]->dtype != w0->dtype || experts[e]->n != w0->n || experts[e]->k != w0->k || experts[e]->dev != w0->dev)
+        if (experts[e]->ggml_dtype != w0->ggml_dtype || experts[e]->n != w0->n || experts[e]->k != w0->k || experts[e]->dev != w0->dev)
             return cq_set_error(CQ_ERR_INVALID, "expert %d differs in dtype, shape or device from expert 0", e);
         if (offsets[e + 1] < offsets[e]) return cq_set_error(CQ_ERR_INVALID, "offsets must be non-decreasing");
     }
@@ -682,6 +690,8 @@ static int grouped_impl(const cq_weight *const *experts, int n_experts, const fl
     if (rc || total == 0 || w0->n == 0 || w0->k == 0) return rc;
     const int act = act_dtype_for(w0, flags);
     if (act == CQ_DTYPE_Q8_1) return cq_set_error(CQ_ERR_UNSUPPORTED, "grouped matmul takes the CPU formulation only");
+    if (cq_has_min32(w0->ggml_dtype))
+        return cq_set_error(CQ_ERR_UNSUPPORTED, "grouped matmul does not take Q4_1 / Q5_1 experts (their m * s term has no grouped launch)");
     if ((rc = check_pre(pre))) return rc;
     CQ_HIP_CHECK(hipSetDevice(w0->dev));
     hipStream_t s = (hipStream_t)stream;

@@ -1,6 +1,6 @@
 // Device planes -> f32 / f16 (QTensor::dequantize, dequantize_f16;
 // candle-core/src/quantized/mod.rs:361-382, CUDA precedent cuda.rs:69-181).
-// The f32 values are those of T::to_float (k_quants.rs:163-183, :568-584, :1313-1341, :1527-1564,
+// The f32 values are those of T::to_float (k_quants.rs:163-183, :329-349, :533-558, :568-584, :1313-1341, :1527-1564,
 // :1716-1746): same products in the same order, no contraction.  The f16 output is the
 // f32 output rounded to nearest-even, as the reference's tests require
 // (candle-core/tests/quantized_tests.rs:229-234).
@@ -47,19 +47,22 @@ __global__ void dequant_q4_0(const uint8_t *__restrict__ qs, const uint16_t *__r
     put16<F16>(d32, d16, b * 32 + 16, hi);
 }
 
-template <bool F16>
-__global__ void dequant_q8_0(const uint8_t *__restrict__ qs, const uint16_t *__restrict__ dpl, int64_t nunits,
-                             float *d32, uint16_t *d16) {
+// MIN: Q4_1 / Q5_1 held as Q8_0 planes plus the plane of block minima: q * d + m (k_quants.rs:329-349, :533-558)
+template <bool F16, bool MIN>
+__global__ void dequant_q8_0(const uint8_t *__restrict__ qs, const uint16_t *__restrict__ dpl,
+                             const uint16_t *__restrict__ mpl, int64_t nunits, float *d32, uint16_t *d16) {
     const int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // 16 elements each
     if (u >= nunits) return;
     const uint4 q = *(const uint4 *)(qs + u * 16);
     const float d = cq_h2f(dpl[u >> 1]);
+    const float mn = MIN ? cq_h2f(mpl[u >> 1]) : 0.0f;
     const uint32_t w[4] = {q.x, q.y, q.z, q.w};
     float out[16];
 #pragma unroll
     for (int j = 0; j < 16; j++) {
         const int8_t v = (int8_t)((w[j >> 2] >> (8 * (j & 3))) & 0xff);
         out[j] = (float)v * d;
+        if (MIN) out[j] = out[j] + mn;
     }
     put16<F16>(d32, d16, u * 16, out);
 }
@@ -140,7 +143,11 @@ hipError_t launch(const cq_weight *w, float *d32, uint16_t *d16, hipStream_t s) 
         dequant_q4_0<F16><<<grid(total / 32), threads, 0, s>>>(w->p0, (const uint16_t *)w->p1, total / 32, d32, d16);
         break;
     case CQ_DTYPE_Q8_0:
-        dequant_q8_0<F16><<<grid(total / 16), threads, 0, s>>>(w->p0, (const uint16_t *)w->p1, total / 16, d32, d16);
+        if (cq_has_min32(w->ggml_dtype))
+            dequant_q8_0<F16, true><<<grid(total / 16), threads, 0, s>>>(w->p0, (const uint16_t *)w->p1, (const uint16_t *)w->p2,
+                                                                         total / 16, d32, d16);
+        else
+            dequant_q8_0<F16, false><<<grid(total / 16), threads, 0, s>>>(w->p0, (const uint16_t *)w->p1, nullptr, total / 16, d32, d16);
         break;
     case CQ_DTYPE_Q4K:
         dequant_q4k<F16, false><<<grid(total / 32), threads, 0, s>>>(w->p0, w->p1, nullptr, total / 32, d32, d16);

@@ -40,14 +40,14 @@
 struct cq_weight {
     int dev;
     int dtype;           // the type whose planes hold the blocks: what every kernel dispatches on
-    int ggml_dtype;      // the type the caller sees; differs from dtype for Q5_0 (held as Q8_0) and Q3K (held as Q6K)
+    int ggml_dtype;      // the type the caller sees; differs from dtype for Q5_0, Q4_1, Q5_1 (held as Q8_0) and Q3K (as Q6K)
     int64_t n, k;
     size_t ggml_bytes;   // n * k/block * type_size of ggml_dtype
     void *base;          // the single device allocation
     size_t alloc_bytes;
     uint8_t *p0;         // qs / ql
     uint8_t *p1;         // d (Q4_0,Q8_0) / hd (Q4K) / qh (Q6K)
-    uint8_t *p2;         // sc (Q6K) / qh (Q5K)
+    uint8_t *p2;         // sc (Q6K) / qh (Q5K) / m (Q4_1, Q5_1: f16 block minima beside the Q8_0 planes)
     uint8_t *p3;         // d  (Q6K)
 };
 
@@ -93,11 +93,19 @@ bool cq_timing_take(hipEvent_t *start, hipEvent_t *stop);
 hipError_t cq_launch_repack(const cq_weight *w, const uint8_t *aos_dev, hipStream_t s);   // GGML AoS -> planes
 hipError_t cq_launch_unpack(const cq_weight *w, uint8_t *aos_dev, hipStream_t s);         // planes -> GGML AoS
 // Types held in another type's planes (same values, same arithmetic): Q5_0 as Q8_0, Q3K as Q6K.
+// Q4_1 and Q5_1 (value d * q + m) are Q8_0 planes with qs = q plus the plane p2 of the blocks' minima m (f16): the
+// holding type's kernels give the sum_i * d * d8 part of their dot product, cq_launch_min32_term adds sum_b m_b * s8_b.
+inline bool cq_has_min32(int ggml_dtype) { return ggml_dtype == CQ_DTYPE_Q4_1 || ggml_dtype == CQ_DTYPE_Q5_1; }
 inline int cq_storage_dtype(int ggml_dtype) {
-    return ggml_dtype == CQ_DTYPE_Q5_0 ? CQ_DTYPE_Q8_0 : ggml_dtype == CQ_DTYPE_Q3K ? CQ_DTYPE_Q6K : ggml_dtype;
+    if (ggml_dtype == CQ_DTYPE_Q5_0 || cq_has_min32(ggml_dtype)) return CQ_DTYPE_Q8_0;
+    return ggml_dtype == CQ_DTYPE_Q3K ? CQ_DTYPE_Q6K : ggml_dtype;
 }
-hipError_t cq_launch_transcode(int ggml_dtype, uint8_t *ggml_aos_dev, uint8_t *storage_aos_dev, int64_t nblocks, bool inverse,
-                               hipStream_t s);
+// `min_plane`: the f16 minima of Q4_1 / Q5_1 blocks (cq_weight::p2), else unused
+hipError_t cq_launch_transcode(int ggml_dtype, uint8_t *ggml_aos_dev, uint8_t *storage_aos_dev, uint16_t *min_plane,
+                               int64_t nblocks, bool inverse, hipStream_t s);
+// y[r, c] += sum_b m[c, b] * s8[r, b] for Q4_1 / Q5_1 weights, s8 the `s` field of the activation's Q8_1 block
+// (k_quants.rs:665-691) recomputed from the workspace's block sums and scales.
+hipError_t cq_launch_min32_term(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s);
 // A step of the caller's model computed on the way into the activation quantizer (CQ_PRE_*):
 // rms_norm: x / sqrt(mean(x^2) + eps) * aux[k]; silu_mul: silu(x) * aux[m][k] (aux indexed like x).
 struct cq_pre {

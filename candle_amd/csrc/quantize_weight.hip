@@ -7,7 +7,7 @@
 //   Q4K  :1252-1311 + utils.rs:201-258 (make_qkx1_quants) + :49-59 (get_scale_min_k4)
 //   Q5K  :1450-1525, the same with 32 levels
 //   Q6K  :1643-1713 + utils.rs:61-198  (make_qx_quants, n=16, nmax=32, rmse_type=1)
-//   Q5_0 :393-425                 Q3K  :1011-1090 + utils.rs:261-326 (make_q3_quants, nmax=4, do_rmse)
+//   Q4_1 :296-326   Q5_1 :496-530   Q5_0 :393-425   Q3K  :1011-1090 + utils.rs:261-326 (make_q3_quants, nmax=4, do_rmse)
 #include "qhip_internal.h"
 
 namespace {
@@ -302,6 +302,38 @@ __global__ void quantize_q5_0(const float *__restrict__ src, int64_t nblocks, ui
     y[2] = (uint8_t)qh; y[3] = (uint8_t)(qh >> 8); y[4] = (uint8_t)(qh >> 16); y[5] = (uint8_t)(qh >> 24);
 }
 
+// Q4_1 (k_quants.rs:296-326) and, FIVE, Q5_1 (:496-530): d = (max - min) / levels, quants round((x - min) / d)
+template <bool FIVE>
+__global__ void quantize_q4_1(const float *__restrict__ src, int64_t nblocks, uint8_t *__restrict__ out) {
+    const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    const float *x = src + b * 32;
+    float min = INFINITY, max = -INFINITY;
+    for (int j = 0; j < 32; j++) {
+        min = fminf(x[j], min);   // f32::min / f32::max: a NaN operand loses
+        max = fmaxf(x[j], max);
+    }
+    const float d = (max - min) / (FIVE ? 31.0f : 15.0f);
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    uint8_t *y = out + b * (FIVE ? 24 : 20);
+    store_u16(y, cq_f2h(d));
+    store_u16(y + 2, cq_f2h(min));
+    uint32_t qh = 0;
+    for (int j = 0; j < 16; j++) {
+        const float x0 = (x[j] - min) * id;
+        const float x1 = (x[16 + j] - min) * id;
+        uint8_t xi0 = cq_as_u8(x0 + 0.5f), xi1 = cq_as_u8(x1 + 0.5f);
+        if (!FIVE) {
+            if (xi0 > 15) xi0 = 15;
+            if (xi1 > 15) xi1 = 15;
+        }
+        y[(FIVE ? 8 : 4) + j] = (uint8_t)((xi0 & 0x0F) | ((xi1 & 0x0F) << 4));
+        qh |= (((uint32_t)xi0 & 0x10u) >> 4) << j;
+        qh |= (((uint32_t)xi1 & 0x10u) >> 4) << (j + 16);
+    }
+    if (FIVE) { y[4] = (uint8_t)qh; y[5] = (uint8_t)(qh >> 8); y[6] = (uint8_t)(qh >> 16); y[7] = (uint8_t)(qh >> 24); }
+}
+
 // utils.rs:261-326 with nmax = 4, do_rmse = true, n = 16: only the returned scale is used
 __device__ float make_q3_quants_16(const float *x) {
     const int n = 16, nmax = 4;
@@ -403,6 +435,8 @@ hipError_t cq_launch_quantize_weight(int dtype, const float *src, int64_t nblock
     case CQ_DTYPE_Q4_0: quantize_q4_0<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q8_0: quantize_q8_0<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q5_0: quantize_q5_0<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
+    case CQ_DTYPE_Q4_1: quantize_q4_1<false><<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
+    case CQ_DTYPE_Q5_1: quantize_q4_1<true><<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q3K: quantize_q3k<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q4K: quantize_q4k<16><<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q5K: quantize_q4k<32><<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;

@@ -240,6 +240,40 @@ __global__ void transcode_q5_0_q8_0(uint8_t *__restrict__ q5, uint8_t *__restric
     }
 }
 
+// Q4_1 {f16 d; f16 m; u8 qs[16]} and Q5_1 {f16 d; f16 m; u8 qh[4]; u8 qs[16]} (k_quants.rs:51-57, :69-76): value d * q + m.
+// The quants (0..15, 0..31) and d go into a Q8_0 block, m into its own plane.
+template <bool FIVE>
+__global__ void transcode_q4_1_q8_0(uint8_t *__restrict__ src, uint8_t *__restrict__ q8, uint16_t *__restrict__ mins,
+                                    int64_t nblocks, bool inverse) {
+    const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    constexpr int TS = FIVE ? 24 : 20, QS = FIVE ? 8 : 4;
+    uint8_t *x = src + b * TS, *y = q8 + b * 34;
+    if (!inverse) {
+        y[0] = x[0];
+        y[1] = x[1];
+        mins[b] = (uint16_t)(x[2] | (x[3] << 8));
+        const uint32_t qh = FIVE ? ((uint32_t)x[4] | ((uint32_t)x[5] << 8) | ((uint32_t)x[6] << 16) | ((uint32_t)x[7] << 24)) : 0u;
+        for (int j = 0; j < 16; j++) {
+            y[2 + j] = (uint8_t)((x[QS + j] & 0x0F) | (((qh >> j) & 1u) << 4));
+            y[2 + j + 16] = (uint8_t)((x[QS + j] >> 4) | (((qh >> (j + 16)) & 1u) << 4));
+        }
+    } else {
+        x[0] = y[0];
+        x[1] = y[1];
+        x[2] = (uint8_t)(mins[b] & 0xff);
+        x[3] = (uint8_t)(mins[b] >> 8);
+        uint32_t qh = 0;
+        for (int j = 0; j < 16; j++) {
+            const uint32_t v0 = y[2 + j], v1 = y[2 + j + 16];
+            x[QS + j] = (uint8_t)((v0 & 0x0F) | ((v1 & 0x0F) << 4));
+            qh |= ((v0 >> 4) & 1u) << j;
+            qh |= ((v1 >> 4) & 1u) << (j + 16);
+        }
+        if (FIVE) { x[4] = (uint8_t)qh; x[5] = (uint8_t)(qh >> 8); x[6] = (uint8_t)(qh >> 16); x[7] = (uint8_t)(qh >> 24); }
+    }
+}
+
 // Q3K {u8 hmask[32]; u8 qs[64]; u8 scales[12]; f16 d} (k_quants.rs:107-114): sixteen groups of sixteen three-bit quants,
 // value (d * (sc_j - 32)) * (q - 4) with six-bit sc_j: exactly a Q6K block {ql, qh, i8 scales[16], f16 d} with
 // scales[j] = sc_j - 32 and six-bit quants q + 28 (so that q6 - 32 = q - 4), whose dequantization (k_quants.rs:1716-1746)
@@ -333,13 +367,15 @@ hipError_t cq_launch_unpack(const cq_weight *w, uint8_t *aos_dev, hipStream_t s)
 }
 
 // GGML blocks of type `ggml_dtype` <-> GGML blocks of the type whose planes hold them (cq_storage_dtype).
-hipError_t cq_launch_transcode(int ggml_dtype, uint8_t *ggml_aos_dev, uint8_t *storage_aos_dev, int64_t nblocks, bool inverse,
-                               hipStream_t s) {
+hipError_t cq_launch_transcode(int ggml_dtype, uint8_t *ggml_aos_dev, uint8_t *storage_aos_dev, uint16_t *min_plane,
+                               int64_t nblocks, bool inverse, hipStream_t s) {
     if (nblocks == 0) return hipSuccess;
     const int threads = 128;
     const unsigned grid = (unsigned)((nblocks + threads - 1) / threads);
     switch (ggml_dtype) {
     case CQ_DTYPE_Q5_0: transcode_q5_0_q8_0<<<grid, threads, 0, s>>>(ggml_aos_dev, storage_aos_dev, nblocks, inverse); break;
+    case CQ_DTYPE_Q4_1: transcode_q4_1_q8_0<false><<<grid, threads, 0, s>>>(ggml_aos_dev, storage_aos_dev, min_plane, nblocks, inverse); break;
+    case CQ_DTYPE_Q5_1: transcode_q4_1_q8_0<true><<<grid, threads, 0, s>>>(ggml_aos_dev, storage_aos_dev, min_plane, nblocks, inverse); break;
     case CQ_DTYPE_Q3K: transcode_q3k_q6k<<<grid, threads, 0, s>>>(ggml_aos_dev, storage_aos_dev, nblocks, inverse); break;
     default: return hipErrorInvalidValue;
     }

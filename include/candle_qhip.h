@@ -36,7 +36,10 @@ extern "C" {
 /* GgmlDType ids handled by this library (mod.rs:133-190). */
 enum {
     CQ_DTYPE_Q4_0 = 2,
+    CQ_DTYPE_Q4_1 = 3,  /* held as Q8_0 planes (qs = q) plus a plane of block minima; the m * s term of the dot
+                           product with Q8_1 activations (k_quants.rs:267-294) is added by a second small launch      */
     CQ_DTYPE_Q5_0 = 6,  /* held on the device as Q8_0 planes (qs = q - 16): the same values, the same arithmetic     */
+    CQ_DTYPE_Q5_1 = 7,  /* like Q4_1, with five-bit quants                                                            */
     CQ_DTYPE_Q8_0 = 8,
     CQ_DTYPE_Q8_1 = 9,  /* activation format only */
     CQ_DTYPE_Q3K = 11,  /* held on the device as Q6K planes (scale - 32, quant + 28): the same values and arithmetic */

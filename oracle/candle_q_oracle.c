@@ -32,8 +32,9 @@
  *   q3k quantize (make_q3_quants, utils.rs:261-326), dequant, q3k x q8k dot (k_quants.rs:874-1148)
  *                                               : :484-529 (spot values, < 0.03, < 3.5, RMSE <= 0.004),
  *        :795-805 (dot-product error <= 0.016148), numpy brute force from unpacked blocks
- *   q4_1 quantize, dequant, q4_1 x q8_1 dot (k_quants.rs:257-350; oracle only, the
- *        product has no Q4_1 weights)            : :256-287 (128 round-trip values), :393-434
+ *   q5_1 quantize, dequant, q5_1 x q8_1 dot (k_quants.rs:454-560) : :321-351 (128 round-trip values), :349
+ *        (RMSE bound), :795-805 (dot-product error <= 0.00149), numpy brute force from unpacked blocks
+ *   q4_1 quantize, dequant, q4_1 x q8_1 dot (k_quants.rs:257-350)            : :256-287 (128 round-trip values), :393-434
  *        (RMSE bound), :795 + :866 (dot-product error <= 0.008 on cos vectors, x2 on ramps)
  *   q8_1 quantize (k_quants.rs:665-691)         : d and qs by the q8_0 goldens (same
  *        arithmetic); the `s` field by the reference's q4_1 x q8_1 dot-product bounds above
@@ -71,6 +72,8 @@ typedef struct { float d; int8_t qs[QK_K]; int16_t bsums[QK_K / 16]; } block_q8k
 #pragma pack(pop)
 
 typedef struct { uint16_t d; uint8_t qh[4]; uint8_t qs[16]; } block_q5_0;       /* 22, k_quants.rs:61-67 */
+typedef struct { uint16_t d; uint16_t m; uint8_t qh[4]; uint8_t qs[16]; } block_q5_1; /* 24, k_quants.rs:69-76 */
+_Static_assert(sizeof(block_q5_1) == 24, "q5_1");
 typedef struct { uint8_t hmask[QK_K / 8]; uint8_t qs[QK_K / 4]; uint8_t scales[12]; uint16_t d; } block_q3k; /* 110, k_quants.rs:107-114 */
 _Static_assert(sizeof(block_q5_0) == 22, "q5_0");
 _Static_assert(sizeof(block_q3k) == 110, "q3k");
@@ -425,6 +428,85 @@ static int vec_dot_q4_1_q8_1(int64_t n, const block_q4_1 *xs, const block_q8_1 *
             int32_t v1 = xs[i].qs[j] >> 4;
             sumi += v0 * (int32_t)ys[i].qs[j] + v1 * (int32_t)ys[i].qs[j + 16];
         }
+        sumf += (float)sumi * orc_f16_to_f32(xs[i].d) * orc_f16_to_f32(ys[i].d) +
+                orc_f16_to_f32(xs[i].m) * orc_f16_to_f32(ys[i].s);
+    }
+    *out = sumf;
+    return 0;
+}
+
+/* --------------------------------------------------------------- Q5_1 ---- */
+/* k_quants.rs:496-530 (from_float) */
+int orc_quantize_q5_1(const float *xs, void *out, int64_t k) {
+    if (k % 32 != 0) return -1;
+    block_q5_1 *ys = (block_q5_1 *)out;
+    for (int64_t i = 0; i < k / 32; i++) {
+        const float *x = xs + i * 32;
+        float min = INFINITY, max = -INFINITY;
+        for (int j = 0; j < 32; j++) {
+            min = fminf(x[j], min);
+            max = fmaxf(x[j], max);
+        }
+        float d = (max - min) / 31.0f;
+        float id = d != 0.0f ? 1.0f / d : 0.0f;
+        ys[i].d = orc_f32_to_f16(d);
+        ys[i].m = orc_f32_to_f16(min);
+        uint32_t qh = 0;
+        for (int j = 0; j < 16; j++) {
+            float x0 = (x[j] - min) * id;
+            float x1 = (x[16 + j] - min) * id;
+            uint8_t xi0 = as_u8(x0 + 0.5f), xi1 = as_u8(x1 + 0.5f);
+            ys[i].qs[j] = (uint8_t)((xi0 & 0x0F) | ((xi1 & 0x0F) << 4));
+            qh |= (((uint32_t)xi0 & 0x10u) >> 4) << j;
+            qh |= (((uint32_t)xi1 & 0x10u) >> 4) << (j + 16);
+        }
+        ys[i].qh[0] = (uint8_t)qh; ys[i].qh[1] = (uint8_t)(qh >> 8);
+        ys[i].qh[2] = (uint8_t)(qh >> 16); ys[i].qh[3] = (uint8_t)(qh >> 24);
+    }
+    return 0;
+}
+
+static inline uint32_t q5_1_qh(const block_q5_1 *x) {
+    return (uint32_t)x->qh[0] | ((uint32_t)x->qh[1] << 8) | ((uint32_t)x->qh[2] << 16) | ((uint32_t)x->qh[3] << 24);
+}
+/* the five-bit quant of element e (0..31) */
+static inline int32_t q5_1_quant(const block_q5_1 *x, int e) {
+    uint32_t qh = q5_1_qh(x);
+    int j = e & 15;
+    int32_t lo = e < 16 ? (x->qs[j] & 0x0F) : (x->qs[j] >> 4);
+    return lo | (int32_t)(((qh >> e) & 1u) << 4);
+}
+
+/* k_quants.rs:533-558 (to_float) */
+int orc_dequantize_q5_1(const void *in, float *ys, int64_t k) {
+    if (k % 32 != 0) return -1;
+    const block_q5_1 *xs = (const block_q5_1 *)in;
+    for (int64_t i = 0; i < k / 32; i++) {
+        float d = orc_f16_to_f32(xs[i].d), m = orc_f16_to_f32(xs[i].m);
+        for (int e = 0; e < 32; e++) ys[i * 32 + e] = (float)q5_1_quant(&xs[i], e) * d + m;
+    }
+    return 0;
+}
+
+/* k_quants.rs:463-494 (vec_dot_unopt of Q5_1 x Q8_1; the block count must be even) */
+static int32_t sumi_q5_1_q8_1(const block_q5_1 *x, const block_q8_1 *y) {
+    int32_t sumi = 0;
+    for (int j = 0; j < 16; j++)
+        sumi += q5_1_quant(x, j) * (int32_t)y->qs[j] + q5_1_quant(x, j + 16) * (int32_t)y->qs[j + 16];
+    return sumi;
+}
+static int32_t sumi_q4_1_q8_1(const block_q4_1 *x, const block_q8_1 *y) {
+    int32_t sumi = 0;
+    for (int j = 0; j < 16; j++)
+        sumi += (int32_t)(x->qs[j] & 0x0F) * (int32_t)y->qs[j] + (int32_t)(x->qs[j] >> 4) * (int32_t)y->qs[j + 16];
+    return sumi;
+}
+static int vec_dot_q5_1_q8_1(int64_t n, const block_q5_1 *xs, const block_q8_1 *ys, float *out) {
+    int64_t nb = n / 32;
+    if (nb % 2 != 0) return -1;
+    float sumf = 0.0f;
+    for (int64_t i = 0; i < nb; i++) {
+        int32_t sumi = sumi_q5_1_q8_1(&xs[i], &ys[i]);
         sumf += (float)sumi * orc_f16_to_f32(xs[i].d) * orc_f16_to_f32(ys[i].d) +
                 orc_f16_to_f32(xs[i].m) * orc_f16_to_f32(ys[i].s);
     }
@@ -1183,14 +1265,14 @@ static float vec_dot_q3k_q8k(int64_t n, const block_q3k *xs, const block_q8k *ys
 /* -------------------------------------------------------- type dispatch ---- */
 int64_t orc_block_size(int dtype) {
     switch (dtype) {
-    case ORC_Q4_0: case ORC_Q4_1: case ORC_Q5_0: case ORC_Q8_0: case ORC_Q8_1: return 32;
+    case ORC_Q4_0: case ORC_Q4_1: case ORC_Q5_0: case ORC_Q5_1: case ORC_Q8_0: case ORC_Q8_1: return 32;
     case ORC_Q3K: case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return QK_K;
     default: return 0;
     }
 }
 int64_t orc_type_size(int dtype) {
     switch (dtype) {
-    case ORC_Q4_0: return 18; case ORC_Q4_1: return 20; case ORC_Q5_0: return 22; case ORC_Q8_0: return 34; case ORC_Q8_1: return 36;
+    case ORC_Q4_0: return 18; case ORC_Q4_1: return 20; case ORC_Q5_0: return 22; case ORC_Q5_1: return 24; case ORC_Q8_0: return 34; case ORC_Q8_1: return 36;
     case ORC_Q3K: return 110; case ORC_Q4K: return 144; case ORC_Q5K: return 176; case ORC_Q6K: return 210; case ORC_Q8K: return 292;
     default: return 0;
     }
@@ -1200,7 +1282,7 @@ int64_t orc_type_size(int dtype) {
 int orc_vec_dot_type(int dtype) {
     switch (dtype) {
     case ORC_Q4_0: case ORC_Q5_0: case ORC_Q8_0: return ORC_Q8_0;   /* Q5_0: k_quants.rs:356 */
-    case ORC_Q4_1: return ORC_Q8_1;   /* k_quants.rs:260 */
+    case ORC_Q4_1: case ORC_Q5_1: return ORC_Q8_1;   /* k_quants.rs:260, :457 */
     case ORC_Q3K: case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return ORC_Q8K;   /* Q3K: k_quants.rs:877 */
     default: return -1;
     }
@@ -1211,6 +1293,7 @@ int orc_quantize(int dtype, const float *xs, void *out, int64_t k) {
     case ORC_Q4_0: return orc_quantize_q4_0(xs, out, k);
     case ORC_Q4_1: return orc_quantize_q4_1(xs, out, k);
     case ORC_Q5_0: return orc_quantize_q5_0(xs, out, k);
+    case ORC_Q5_1: return orc_quantize_q5_1(xs, out, k);
     case ORC_Q3K: return orc_quantize_q3k(xs, out, k);
     case ORC_Q8_0: return orc_quantize_q8_0(xs, out, k);
     case ORC_Q8_1: return orc_quantize_q8_1(xs, out, k);
@@ -1227,6 +1310,7 @@ int orc_dequantize(int dtype, const void *in, float *ys, int64_t k) {
     case ORC_Q4_0: return orc_dequantize_q4_0(in, ys, k);
     case ORC_Q4_1: return orc_dequantize_q4_1(in, ys, k);
     case ORC_Q5_0: return orc_dequantize_q5_0(in, ys, k);
+    case ORC_Q5_1: return orc_dequantize_q5_1(in, ys, k);
     case ORC_Q3K: return orc_dequantize_q3k(in, ys, k);
     case ORC_Q8_0: return orc_dequantize_q8_0(in, ys, k);
     case ORC_Q4K: return orc_dequantize_q4k(in, ys, k);
@@ -1245,6 +1329,7 @@ int orc_vec_dot(int dtype, int64_t n, const void *xs, const void *ys, float *out
     case ORC_Q4_0: *out = vec_dot_q4_0_q8_0(n, xs, ys); return 0;
     case ORC_Q4_1: return vec_dot_q4_1_q8_1(n, xs, ys, out);
     case ORC_Q5_0: *out = vec_dot_q5_0_q8_0(n, xs, ys); return 0;
+    case ORC_Q5_1: return vec_dot_q5_1_q8_1(n, xs, ys, out);
     case ORC_Q3K: *out = vec_dot_q3k_q8k(n, xs, ys); return 0;
     case ORC_Q8_0: *out = vec_dot_q8_0_q8_0(n, xs, ys); return 0;
     case ORC_Q4K: *out = vec_dot_q4k_q8k(n, xs, ys); return 0;
@@ -1308,6 +1393,12 @@ int orc_block_int_dots(int dtype, int64_t m, int64_t k, int64_t n, const void *a
                     break;
                 case ORC_Q5_0:
                     out_i[o] = sumi_q5_0_q8_0((const block_q5_0 *)w + b, (const block_q8_0 *)a + b);
+                    break;
+                case ORC_Q4_1:
+                    out_i[o] = sumi_q4_1_q8_1((const block_q4_1 *)w + b, (const block_q8_1 *)a + b);
+                    break;
+                case ORC_Q5_1:
+                    out_i[o] = sumi_q5_1_q8_1((const block_q5_1 *)w + b, (const block_q8_1 *)a + b);
                     break;
                 case ORC_Q3K: {
                     int32_t aux32[8], t = 0;

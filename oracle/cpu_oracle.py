@@ -17,12 +17,12 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libcandle_q_oracle.so")
 
 # GgmlDType ids (candle-core/src/quantized/mod.rs:173-190)
-Q4_0, Q4_1, Q5_0, Q8_0, Q8_1, Q3K, Q4K, Q5K, Q6K, Q8K = 2, 3, 6, 8, 9, 11, 12, 13, 14, 15
-BLOCK_SIZE = {Q4_0: 32, Q4_1: 32, Q5_0: 32, Q8_0: 32, Q8_1: 32, Q3K: 256, Q4K: 256, Q5K: 256, Q6K: 256, Q8K: 256}
-TYPE_SIZE = {Q4_0: 18, Q4_1: 20, Q5_0: 22, Q8_0: 34, Q8_1: 36, Q3K: 110, Q4K: 144, Q5K: 176, Q6K: 210, Q8K: 292}
-# Q4_1 exists in the oracle only: the reference's Q4_1 vectors pin the `s` field of Q8_1 blocks
-VEC_DOT_TYPE = {Q4_0: Q8_0, Q4_1: Q8_1, Q5_0: Q8_0, Q8_0: Q8_0, Q3K: Q8K, Q4K: Q8K, Q5K: Q8K, Q6K: Q8K, Q8K: Q8K}
-NAMES = {Q4_0: "q4_0", Q4_1: "q4_1", Q5_0: "q5_0", Q8_0: "q8_0", Q8_1: "q8_1", Q3K: "q3k", Q4K: "q4k", Q5K: "q5k", Q6K: "q6k", Q8K: "q8k"}
+Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1, Q3K, Q4K, Q5K, Q6K, Q8K = 2, 3, 6, 7, 8, 9, 11, 12, 13, 14, 15
+BLOCK_SIZE = {Q4_0: 32, Q4_1: 32, Q5_0: 32, Q5_1: 32, Q8_0: 32, Q8_1: 32, Q3K: 256, Q4K: 256, Q5K: 256, Q6K: 256, Q8K: 256}
+TYPE_SIZE = {Q4_0: 18, Q4_1: 20, Q5_0: 22, Q5_1: 24, Q8_0: 34, Q8_1: 36, Q3K: 110, Q4K: 144, Q5K: 176, Q6K: 210, Q8K: 292}
+# the reference's Q4_1 vectors also pin the `s` field of Q8_1 blocks
+VEC_DOT_TYPE = {Q4_0: Q8_0, Q4_1: Q8_1, Q5_0: Q8_0, Q5_1: Q8_1, Q8_0: Q8_0, Q3K: Q8K, Q4K: Q8K, Q5K: Q8K, Q6K: Q8K, Q8K: Q8K}
+NAMES = {Q4_0: "q4_0", Q4_1: "q4_1", Q5_0: "q5_0", Q5_1: "q5_1", Q8_0: "q8_0", Q8_1: "q8_1", Q3K: "q3k", Q4K: "q4k", Q5K: "q5k", Q6K: "q6k", Q8K: "q8k"}
 
 
 def build(force: bool = False) -> str:

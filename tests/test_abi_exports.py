@@ -108,6 +108,8 @@ def test_metadata_calls_need_no_gpu(lib):
     lib.cq_vec_dot_type.restype = ctypes.c_int
     Q4_0, Q8_0, Q4K, Q6K, Q8K = 2, 8, 12, 14, 15
     Q5_0, Q3K = 6, 11
+    assert (lib.cq_block_size(3), lib.cq_type_size(3), lib.cq_vec_dot_type(3)) == (32, 20, 9)      # Q4_1 x Q8_1, k_quants.rs:51-57, :260
+    assert (lib.cq_block_size(7), lib.cq_type_size(7), lib.cq_vec_dot_type(7)) == (32, 24, 9)      # Q5_1 x Q8_1, k_quants.rs:69-76, :457
     assert (lib.cq_block_size(Q5_0), lib.cq_type_size(Q5_0), lib.cq_vec_dot_type(Q5_0)) == (32, 22, Q8_0)    # k_quants.rs:61-67, :356
     assert (lib.cq_block_size(Q3K), lib.cq_type_size(Q3K), lib.cq_vec_dot_type(Q3K)) == (256, 110, Q8K)     # k_quants.rs:107-114, :877
     assert (lib.cq_block_size(10), lib.cq_type_size(10), lib.cq_vec_dot_type(10)) == (0, 0, -1)             # Q2K: not handled

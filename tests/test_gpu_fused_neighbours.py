@@ -152,7 +152,7 @@ def test_matmul_with_rms_norm(qh, dt, m, k, n):
     qw = qh.QWeight.from_ggml(dt, wq, n, k)
     got = qh.qmatmul(qw, dev(x), pre=qh.PRE_RMS_NORM, aux=dev(alpha), eps=eps)
     # the same kernels on host-prepared input, in the kernels' order of operations: same bits
-    if dt in (orc.Q4_0, orc.Q5_0, orc.Q8_0):   # the types with Q8_0 activations
+    if dt in (orc.Q4_0, orc.Q4_1, orc.Q5_0, orc.Q5_1, orc.Q8_0):   # the types with 32-element activation blocks
         assert torch.equal(got, qh.qmatmul(qw, dev(canonical_rms_norm(x, alpha, eps)), staged(qh, m)))
     elif m == 1:   # one row: x * alpha through the matmul, the result times the row's scale
         plain = qh.qmatmul(qw, dev((x * alpha[None, :]).astype(np.float32))).cpu().numpy()

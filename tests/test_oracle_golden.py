@@ -6,7 +6,7 @@ import pytest
 
 from oracle import cpu_oracle as orc
 
-DT = {"q4_0": orc.Q4_0, "q4_1": orc.Q4_1, "q5_0": orc.Q5_0, "q8_0": orc.Q8_0, "q3k": orc.Q3K, "q4k": orc.Q4K, "q5k": orc.Q5K, "q6k": orc.Q6K, "q8k": orc.Q8K}
+DT = {"q4_0": orc.Q4_0, "q4_1": orc.Q4_1, "q5_0": orc.Q5_0, "q5_1": orc.Q5_1, "q8_0": orc.Q8_0, "q3k": orc.Q3K, "q4k": orc.Q4K, "q5k": orc.Q5K, "q6k": orc.Q6K, "q8k": orc.Q8K}
 
 
 # ---------------------------------------------------------------- f16 ----
@@ -83,6 +83,18 @@ def test_q5_0_roundtrip_golden(goldens):
     assert np.array_equal(rounded.view(np.uint32), want.view(np.uint32)), (rounded, want)   # includes the sign of -0.0
 
 
+def test_q5_1_roundtrip_golden(goldens):
+    """quantize_q5_1 (quantized_tests.rs:321-351): the ramp 0..127 comes back exactly."""
+    g = goldens["q5_1_roundtrip_ramp128"]
+    src = np.arange(128, dtype=np.float32)
+    blocks = orc.quantize(orc.Q5_1, src)
+    assert blocks.size == 4 * 24
+    dst = orc.dequantize(orc.Q5_1, blocks)
+    t = np.float32(1000.0) * dst
+    rounded = (np.copysign(np.floor(np.abs(t) + np.float32(0.5)), t)).astype(np.float32) / np.float32(1000.0)
+    assert rounded.tolist() == g["dst"]
+
+
 # ------------------------------------------- G4: K-quant round trips ----
 def _test_vector2(bound, size=1024):
     v = np.arange(size, dtype=np.float32)
@@ -112,7 +124,7 @@ def _ggml_like(offset):
     return (np.float32(0.1) + np.float32(2.0) * np.cos(i + np.float32(offset), dtype=np.float32)).astype(np.float32)
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q3k", "q4k", "q5k", "q6k", "q8k", "q8_0"])
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q3k", "q4k", "q5k", "q6k", "q8k", "q8_0"])
 def test_quantization_total_error(goldens, name):
     src = _ggml_like(0.0)
     dst = orc.dequantize(DT[name], orc.quantize(DT[name], src))
@@ -122,7 +134,7 @@ def test_quantization_total_error(goldens, name):
 
 
 # ------------------------------------------------- G6: dot product error ----
-@pytest.mark.parametrize("name", ["q4_0", "q5_0", "q8_0", "q3k", "q4k", "q5k", "q6k", "q8k"])
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q3k", "q4k", "q5k", "q6k", "q8k"])
 def test_dot_product_error(goldens, name):
     g = goldens["dot_product_error"]
     ramp = (np.arange(4096, dtype=np.float32) / np.float32(4096))
@@ -288,7 +300,7 @@ def test_q8_1_is_q8_0_plus_s():
     assert (np.abs(s.astype(np.float64) - exact) <= ulp).all()
 
 
-# ---- Q4_1 (oracle only): the reference vectors that depend on the `s` field of Q8_1 blocks ----
+# ---- Q4_1: the reference vectors that depend on the `s` field of Q8_1 blocks ----
 def test_q4_1_roundtrip_golden(goldens):
     """quantize_q4_1 (quantized_tests.rs:256-287): ramp 0..127 through Q4_1 and back, 3 decimals."""
     g = goldens["q4_1_roundtrip_ramp128"]
@@ -407,7 +419,7 @@ def _unpack_q3k(w):
     return d, sc, q
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q5_0", "q8_0", "q3k", "q4k", "q5k", "q6k", "q8k"])
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q3k", "q4k", "q5k", "q6k", "q8k"])
 def test_int_dots_and_matmul_bruteforce(name):
     """Integer block dots recomputed by int64 numpy from independently unpacked blocks,
     and the f32 result against a float64 evaluation of the same formula."""
@@ -447,6 +459,22 @@ def test_int_dots_and_matmul_bruteforce(name):
             I = np.einsum("nbl,mbl->mnb", qw.reshape(n, kb, 256).astype(np.int64), q8.astype(np.int64))
             assert np.array_equal(oi, I)
             ref = (dw.reshape(n, kb)[None].astype(np.float64) * d8[:, None] * I).sum(-1)
+    elif name in ("q4_1", "q5_1"):
+        ab = a.reshape(m, -1, 36)
+        da = ab[:, :, :2].copy().view(np.float16)[..., 0].astype(np.float64)
+        sa = ab[:, :, 2:4].copy().view(np.float16)[..., 0].astype(np.float64)
+        qa = ab[:, :, 4:].copy().view(np.int8).astype(np.int64)
+        wb = w.reshape(n, -1, 20 if name == "q4_1" else 24)
+        dw = wb[:, :, :2].copy().view(np.float16)[..., 0].astype(np.float64)
+        mw = wb[:, :, 2:4].copy().view(np.float16)[..., 0].astype(np.float64)
+        nib = wb[:, :, -16:].astype(np.int64)
+        qw = np.concatenate([nib & 0xF, nib >> 4], axis=-1)
+        if name == "q5_1":
+            qh = wb[:, :, 4:8].copy().view(np.uint32)[..., 0].astype(np.int64)
+            qw = qw | (((qh[..., None] >> np.arange(32)) & 1) << 4)
+        I = np.einsum("nbl,mbl->mnb", qw, qa)
+        assert np.array_equal(oi, I)
+        ref = (I * dw[None] * da[:, None] + mw[None] * sa[:, None]).sum(-1)
     else:
         ab = a.reshape(m, -1, 34)
         da = ab[:, :, :2].copy().view(np.float16)[..., 0].astype(np.float64)
