@@ -53,7 +53,7 @@ extern "C" int cq_device_count(void) {
 extern "C" int64_t cq_block_size(int dt) {
     switch (dt) {
     case CQ_DTYPE_Q4_0: case CQ_DTYPE_Q4_1: case CQ_DTYPE_Q5_0: case CQ_DTYPE_Q5_1: case CQ_DTYPE_Q8_0: case CQ_DTYPE_Q8_1: return 32;
-    case CQ_DTYPE_Q3K: case CQ_DTYPE_Q4K: case CQ_DTYPE_Q5K: case CQ_DTYPE_Q6K: case CQ_DTYPE_Q8K: return 256;
+    case CQ_DTYPE_Q2K: case CQ_DTYPE_Q3K: case CQ_DTYPE_Q4K: case CQ_DTYPE_Q5K: case CQ_DTYPE_Q6K: case CQ_DTYPE_Q8K: return 256;
     default: return 0;
     }
 }
@@ -63,6 +63,7 @@ extern "C" int64_t cq_type_size(int dt) {
     case CQ_DTYPE_Q4_1: return 20;
     case CQ_DTYPE_Q5_0: return 22;
     case CQ_DTYPE_Q5_1: return 24;
+    case CQ_DTYPE_Q2K: return 84;
     case CQ_DTYPE_Q3K: return 110;
     case CQ_DTYPE_Q8_0: return 34;
     case CQ_DTYPE_Q8_1: return 36;
@@ -77,14 +78,14 @@ extern "C" int cq_vec_dot_type(int dt) {
     switch (dt) {
     case CQ_DTYPE_Q4_0: case CQ_DTYPE_Q5_0: case CQ_DTYPE_Q8_0: return CQ_DTYPE_Q8_0;
     case CQ_DTYPE_Q4_1: case CQ_DTYPE_Q5_1: return CQ_DTYPE_Q8_1;   /* k_quants.rs:260, :457 */
-    case CQ_DTYPE_Q3K: case CQ_DTYPE_Q4K: case CQ_DTYPE_Q5K: case CQ_DTYPE_Q6K: return CQ_DTYPE_Q8K;
+    case CQ_DTYPE_Q2K: case CQ_DTYPE_Q3K: case CQ_DTYPE_Q4K: case CQ_DTYPE_Q5K: case CQ_DTYPE_Q6K: return CQ_DTYPE_Q8K;
     default: return -1;
     }
 }
 
 static bool is_weight_dtype(int dt) {
     return dt == CQ_DTYPE_Q4_0 || dt == CQ_DTYPE_Q4_1 || dt == CQ_DTYPE_Q5_0 || dt == CQ_DTYPE_Q5_1 || dt == CQ_DTYPE_Q8_0 ||
-           dt == CQ_DTYPE_Q3K || dt == CQ_DTYPE_Q4K ||
+           dt == CQ_DTYPE_Q2K || dt == CQ_DTYPE_Q3K || dt == CQ_DTYPE_Q4K ||
            dt == CQ_DTYPE_Q5K || dt == CQ_DTYPE_Q6K;
 }
 
@@ -117,10 +118,14 @@ static int weight_alloc(int dev, int dt, int64_t n, int64_t k, cq_weight **out) 
     case CQ_DTYPE_Q6K: s0 = (size_t)nb * 128; s1 = (size_t)nb * 64; s2 = (size_t)nb * 16; s3 = (size_t)nb * 2; break;
     }
     if (cq_has_min32(dt)) s2 = (size_t)nb * 2;   // the blocks' minima beside the Q8_0 planes
+    size_t s4 = 0, s5 = 0;
+    if (cq_has_min16(dt)) { s4 = (size_t)nb * 16; s5 = (size_t)nb * 2; }   // the groups' minima and dmin beside the Q6K planes
     const size_t o1 = cq_align_up(s0 + CQ_TAIL_PAD, 256);
     const size_t o2 = cq_align_up(o1 + s1 + CQ_TAIL_PAD, 256);
     const size_t o3 = cq_align_up(o2 + s2 + CQ_TAIL_PAD, 256);
-    w->alloc_bytes = cq_align_up(o3 + s3 + CQ_TAIL_PAD, 256);
+    const size_t o4 = cq_align_up(o3 + s3 + CQ_TAIL_PAD, 256);
+    const size_t o5 = cq_align_up(o4 + s4 + CQ_TAIL_PAD, 256);
+    w->alloc_bytes = cq_align_up(o5 + s5 + CQ_TAIL_PAD, 256);
     hipError_t e = hipMalloc(&w->base, w->alloc_bytes);
     if (e != hipSuccess) {
         const size_t bytes = w->alloc_bytes;
@@ -131,6 +136,8 @@ static int weight_alloc(int dev, int dt, int64_t n, int64_t k, cq_weight **out) 
     w->p1 = (uint8_t *)w->base + o1;
     w->p2 = (uint8_t *)w->base + o2;
     w->p3 = (uint8_t *)w->base + o3;
+    w->p4 = (uint8_t *)w->base + o4;
+    w->p5 = (uint8_t *)w->base + o5;
     // creating a weight is the set-up call every user of a device goes through: the scratch array of
     // cq_qmatmul_static is looked up here, so that the first matmul on the device has nothing left to set up
     // (a failure is reported by cq_qmatmul_static itself, which looks again)
@@ -147,7 +154,7 @@ static hipError_t blocks_to_planes(const cq_weight *w, uint8_t *ggml_aos_dev, hi
     void *tmp = nullptr;
     hipError_t e = hipMalloc(&tmp, (size_t)weight_blocks(w) * (size_t)cq_type_size(w->dtype) + 256);
     if (e != hipSuccess) return e;
-    e = cq_launch_transcode(w->ggml_dtype, ggml_aos_dev, (uint8_t *)tmp, (uint16_t *)w->p2, weight_blocks(w), false, s);
+    e = cq_launch_transcode(w, ggml_aos_dev, (uint8_t *)tmp, weight_blocks(w), false, s);
     if (e == hipSuccess) e = cq_launch_repack(w, (const uint8_t *)tmp, s);
     if (e == hipSuccess) e = hipStreamSynchronize(s);
     (void)hipFree(tmp);
@@ -159,7 +166,7 @@ static hipError_t planes_to_blocks(const cq_weight *w, uint8_t *ggml_aos_dev, hi
     hipError_t e = hipMalloc(&tmp, (size_t)weight_blocks(w) * (size_t)cq_type_size(w->dtype) + 256);
     if (e != hipSuccess) return e;
     e = cq_launch_unpack(w, (uint8_t *)tmp, s);
-    if (e == hipSuccess) e = cq_launch_transcode(w->ggml_dtype, ggml_aos_dev, (uint8_t *)tmp, (uint16_t *)w->p2, weight_blocks(w), true, s);
+    if (e == hipSuccess) e = cq_launch_transcode(w, ggml_aos_dev, (uint8_t *)tmp, weight_blocks(w), true, s);
     if (e == hipSuccess) e = hipStreamSynchronize(s);
     (void)hipFree(tmp);
     return e;
@@ -484,7 +491,7 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
                            ranges_overlap(y_dev, m * w->n, pre.aux, pre.kind == CQ_PRE_RMS_NORM ? w->k : m * w->k));
     // decode (one activation row): a single launch that quantizes x in its prologue
     // (Q4_1 / Q5_1: the second launch that adds their m * s term reads the quantized row from the workspace)
-    const bool min32 = cq_has_min32(w->ggml_dtype);
+    const bool min32 = cq_has_min32(w->ggml_dtype) || cq_has_min16(w->ggml_dtype);   // (Q2K: likewise, its dmin term)
     if (m == 1 && !in_place && !min32 && !(flags & (CQ_FLAG_REUSE_ACT | CQ_FLAG_FORCE_GEMM | CQ_FLAG_STAGED_ACT | CQ_FLAG_ACT_Q8_1)) &&
         cq_matvec_fused_supported(w)) {
         CQ_HIP_CHECK(cq_launch_matvec_fused(w, x_dev, pre, y_dev, s));
@@ -555,7 +562,8 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
         case kGemm: CQ_HIP_CHECK(cq_launch_gemm(w, v, act, m, y_dev, y_cleared, s)); break;
         case kMatvec: CQ_HIP_CHECK(cq_launch_matvec(w, v, act, m, y_dev, s)); break;
     }
-    if (min32) CQ_HIP_CHECK(cq_launch_min32_term(w, v, m, y_dev, s));
+    if (cq_has_min32(w->ggml_dtype)) CQ_HIP_CHECK(cq_launch_min32_term(w, v, m, y_dev, s));
+    if (cq_has_min16(w->ggml_dtype)) CQ_HIP_CHECK(cq_launch_min16_term(w, v, m, y_dev, s));
     return CQ_OK;
 }
 
@@ -600,7 +608,8 @@ extern "C" int cq_qmatmul_multi(const cq_weight *const *ws, int count, int pre, 
             return cq_set_error(CQ_ERR_INVALID, "output %d overlaps the activations: cq_qmatmul_multi does not work in place", i);
     }
     // one activation row (or up to four of short weight rows), two or three weights: one launch over all their rows
-    if (m >= 1 && m <= 4 && flags == 0 && !cq_has_min32(ws[0]->ggml_dtype) && cq_matvec_fused_multi_supported(ws, count, pre, m)) {
+    if (m >= 1 && m <= 4 && flags == 0 && !cq_has_min32(ws[0]->ggml_dtype) && !cq_has_min16(ws[0]->ggml_dtype) &&
+        cq_matvec_fused_multi_supported(ws, count, pre, m)) {
         if (!x_dev) return cq_set_error(CQ_ERR_INVALID, "null argument");
         if ((uintptr_t)x_dev & 15) return cq_set_error(CQ_ERR_INVALID, "x must be 16-byte aligned");
         for (int i = 0; i < count; i++)
@@ -690,8 +699,8 @@ static int grouped_impl(const cq_weight *const *experts, int n_experts, const fl
     if (rc || total == 0 || w0->n == 0 || w0->k == 0) return rc;
     const int act = act_dtype_for(w0, flags);
     if (act == CQ_DTYPE_Q8_1) return cq_set_error(CQ_ERR_UNSUPPORTED, "grouped matmul takes the CPU formulation only");
-    if (cq_has_min32(w0->ggml_dtype))
-        return cq_set_error(CQ_ERR_UNSUPPORTED, "grouped matmul does not take Q4_1 / Q5_1 experts (their m * s term has no grouped launch)");
+    if (cq_has_min32(w0->ggml_dtype) || cq_has_min16(w0->ggml_dtype))
+        return cq_set_error(CQ_ERR_UNSUPPORTED, "grouped matmul does not take Q4_1 / Q5_1 / Q2K experts (their offset term has no grouped launch)");
     if ((rc = check_pre(pre))) return rc;
     CQ_HIP_CHECK(hipSetDevice(w0->dev));
     hipStream_t s = (hipStream_t)stream;

@@ -1,7 +1,7 @@
 // Device planes -> f32 / f16 (QTensor::dequantize, dequantize_f16;
 // candle-core/src/quantized/mod.rs:361-382, CUDA precedent cuda.rs:69-181).
-// The f32 values are those of T::to_float (k_quants.rs:163-183, :329-349, :533-558, :568-584, :1313-1341, :1527-1564,
-// :1716-1746): same products in the same order, no contraction.  The f16 output is the
+// The f32 values are those of T::to_float (k_quants.rs:163-183, :329-349, :533-558, :568-584, :841-872, :1094-1146, :1313-1341,
+// :1527-1564, :1716-1746): same products in the same order, no contraction.  The f16 output is the
 // f32 output rounded to nearest-even, as the reference's tests require
 // (candle-core/tests/quantized_tests.rs:229-234).
 // One thread per 16-byte lane of the main plane; a wave covers 1 KiB of it.
@@ -100,9 +100,11 @@ __global__ void dequant_q4k(const uint8_t *__restrict__ qs, const uint8_t *__res
     put16<F16>(d32, d16, base + 32, hi);
 }
 
-template <bool F16>
+// MIN: Q2K held as Q6K planes plus the groups' minima and dmin: (d * sc) * q - dmin * m (k_quants.rs:841-872)
+template <bool F16, bool MIN>
 __global__ void dequant_q6k(const uint8_t *__restrict__ ql, const uint8_t *__restrict__ qh,
-                            const int8_t *__restrict__ sc, const uint16_t *__restrict__ dpl, int64_t nunits,
+                            const int8_t *__restrict__ sc, const uint16_t *__restrict__ dpl,
+                            const uint8_t *__restrict__ mins, const uint16_t *__restrict__ dmins, int64_t nunits,
                             float *d32, uint16_t *d16) {
     const int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // 16 bytes of ql = 32 elements
     if (u >= nunits) return;
@@ -127,6 +129,17 @@ __global__ void dequant_q6k(const uint8_t *__restrict__ ql, const uint8_t *__res
         const int q_hi = (int)((byte >> 4) | (((hb >> (sh + 2)) & 3) << 4)) - 32;
         lo[e] = d * s_lo * (float)q_lo;
         hi[e] = d * s_hi * (float)q_hi;
+    }
+    if (MIN) {
+        // the lane's low-nibble elements are group 8h + 2t + p%2 of the block, the high-nibble ones four groups on
+        const int j = 8 * h + 2 * t + (p & 1);
+        const float dmin = cq_h2f(dmins[b]);
+        const float ml_lo = dmin * (float)mins[b * 16 + j], ml_hi = dmin * (float)mins[b * 16 + j + 4];
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            lo[e] = lo[e] - ml_lo;
+            hi[e] = hi[e] - ml_hi;
+        }
     }
     put16<F16>(d32, d16, base, lo);
     put16<F16>(d32, d16, base + 64, hi);
@@ -156,8 +169,12 @@ hipError_t launch(const cq_weight *w, float *d32, uint16_t *d16, hipStream_t s) 
         dequant_q4k<F16, true><<<grid(total / 32), threads, 0, s>>>(w->p0, w->p1, w->p2, total / 32, d32, d16);
         break;
     case CQ_DTYPE_Q6K:
-        dequant_q6k<F16><<<grid(total / 32), threads, 0, s>>>(w->p0, w->p1, (const int8_t *)w->p2,
-                                                              (const uint16_t *)w->p3, total / 32, d32, d16);
+        if (cq_has_min16(w->ggml_dtype))
+            dequant_q6k<F16, true><<<grid(total / 32), threads, 0, s>>>(w->p0, w->p1, (const int8_t *)w->p2, (const uint16_t *)w->p3,
+                                                                        w->p4, (const uint16_t *)w->p5, total / 32, d32, d16);
+        else
+            dequant_q6k<F16, false><<<grid(total / 32), threads, 0, s>>>(w->p0, w->p1, (const int8_t *)w->p2, (const uint16_t *)w->p3,
+                                                                         nullptr, nullptr, total / 32, d32, d16);
         break;
     default: return hipErrorInvalidValue;
     }

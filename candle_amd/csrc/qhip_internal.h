@@ -40,7 +40,7 @@
 struct cq_weight {
     int dev;
     int dtype;           // the type whose planes hold the blocks: what every kernel dispatches on
-    int ggml_dtype;      // the type the caller sees; differs from dtype for Q5_0, Q4_1, Q5_1 (held as Q8_0) and Q3K (as Q6K)
+    int ggml_dtype;      // the type the caller sees; differs from dtype for Q5_0, Q4_1, Q5_1 (held as Q8_0), Q3K and Q2K (as Q6K)
     int64_t n, k;
     size_t ggml_bytes;   // n * k/block * type_size of ggml_dtype
     void *base;          // the single device allocation
@@ -49,6 +49,8 @@ struct cq_weight {
     uint8_t *p1;         // d (Q4_0,Q8_0) / hd (Q4K) / qh (Q6K)
     uint8_t *p2;         // sc (Q6K) / qh (Q5K) / m (Q4_1, Q5_1: f16 block minima beside the Q8_0 planes)
     uint8_t *p3;         // d  (Q6K)
+    uint8_t *p4;         // Q2K (held as Q6K): the sixteen group minima of a block, one byte each
+    uint8_t *p5;         // Q2K: dmin (f16)
 };
 
 // ---------------------------------------------------------------------------
@@ -96,13 +98,19 @@ hipError_t cq_launch_unpack(const cq_weight *w, uint8_t *aos_dev, hipStream_t s)
 // Q4_1 and Q5_1 (value d * q + m) are Q8_0 planes with qs = q plus the plane p2 of the blocks' minima m (f16): the
 // holding type's kernels give the sum_i * d * d8 part of their dot product, cq_launch_min32_term adds sum_b m_b * s8_b.
 inline bool cq_has_min32(int ggml_dtype) { return ggml_dtype == CQ_DTYPE_Q4_1 || ggml_dtype == CQ_DTYPE_Q5_1; }
+// Q2K (value d * sc_j * q - dmin * m_j, sixteen groups of sixteen) is a Q6K block with scales sc_j and six-bit quants
+// q + 32, plus the planes p4 / p5 of the groups' minima and dmin: the Q6K kernels give sum_b d * d8 * I_b of its dot
+// product with Q8K activations, cq_launch_min16_term subtracts sum_b dmin * d8 * sum_j bsums_j * m_j.
+inline bool cq_has_min16(int ggml_dtype) { return ggml_dtype == CQ_DTYPE_Q2K; }
 inline int cq_storage_dtype(int ggml_dtype) {
     if (ggml_dtype == CQ_DTYPE_Q5_0 || cq_has_min32(ggml_dtype)) return CQ_DTYPE_Q8_0;
-    return ggml_dtype == CQ_DTYPE_Q3K ? CQ_DTYPE_Q6K : ggml_dtype;
+    return ggml_dtype == CQ_DTYPE_Q3K || ggml_dtype == CQ_DTYPE_Q2K ? CQ_DTYPE_Q6K : ggml_dtype;
 }
-// `min_plane`: the f16 minima of Q4_1 / Q5_1 blocks (cq_weight::p2), else unused
-hipError_t cq_launch_transcode(int ggml_dtype, uint8_t *ggml_aos_dev, uint8_t *storage_aos_dev, uint16_t *min_plane,
-                               int64_t nblocks, bool inverse, hipStream_t s);
+// `w` supplies the planes beside the holding type's blocks: the minima of Q4_1 / Q5_1 (p2), of Q2K (p4, p5)
+hipError_t cq_launch_transcode(const cq_weight *w, uint8_t *ggml_aos_dev, uint8_t *storage_aos_dev, int64_t nblocks, bool inverse,
+                               hipStream_t s);
+// y[r, c] -= sum_b (d8[r, b] * dmin[c, b]) * sum_j bsums[r, b, j] * m[c, b, j] for Q2K weights (k_quants.rs:727-733, :762)
+hipError_t cq_launch_min16_term(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s);
 // y[r, c] += sum_b m[c, b] * s8[r, b] for Q4_1 / Q5_1 weights, s8 the `s` field of the activation's Q8_1 block
 // (k_quants.rs:665-691) recomputed from the workspace's block sums and scales.
 hipError_t cq_launch_min32_term(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s);

@@ -7,6 +7,7 @@
 //   Q4K  :1252-1311 + utils.rs:201-258 (make_qkx1_quants) + :49-59 (get_scale_min_k4)
 //   Q5K  :1450-1525, the same with 32 levels
 //   Q6K  :1643-1713 + utils.rs:61-198  (make_qx_quants, n=16, nmax=32, rmse_type=1)
+//   Q2K  :770-839 (make_qkx1_quants over 16 elements, 3 levels)
 //   Q4_1 :296-326   Q5_1 :496-530   Q5_0 :393-425   Q3K  :1011-1090 + utils.rs:261-326 (make_q3_quants, nmax=4, do_rmse)
 #include "qhip_internal.h"
 
@@ -52,9 +53,10 @@ __global__ void quantize_q8_0(const float *__restrict__ src, int64_t nblocks, ui
 }
 
 // utils.rs:201-258
+template <int N = 32>
 __device__ void make_qkx1_quants(const float *x, int nmax, float &out_scale, float &out_min) {
-    const int n = 32, ntry = 5;
-    uint8_t l[32];
+    const int n = N, ntry = 5;
+    uint8_t l[N];
     for (int i = 0; i < n; i++) l[i] = 0;
     float min = x[0], max = x[0];
     for (int i = 1; i < n; i++) {
@@ -302,6 +304,50 @@ __global__ void quantize_q5_0(const float *__restrict__ src, int64_t nblocks, ui
     y[2] = (uint8_t)qh; y[3] = (uint8_t)(qh >> 8); y[4] = (uint8_t)(qh >> 16); y[5] = (uint8_t)(qh >> 24);
 }
 
+// Q2K (k_quants.rs:770-839): sixteen groups of sixteen, make_qkx1_quants with three levels, 4-bit scales and minima
+__global__ void quantize_q2k(const float *__restrict__ src, int64_t nblocks, uint8_t *__restrict__ out) {
+    const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    const float *x = src + b * 256;
+    uint8_t *y = out + b * 84;
+    uint8_t *sc = y, *qs = y + 16;
+    const float Q4SCALE = 15.0f;
+    float mins[16], scales[16];
+    for (int j = 0; j < 16; j++) make_qkx1_quants<16>(x + 16 * j, 3, scales[j], mins[j]);
+    float max_scale = 0.0f, max_min = 0.0f;
+    for (int j = 0; j < 16; j++) {
+        max_scale = fmaxf(scales[j], max_scale);
+        max_min = fmaxf(mins[j], max_min);
+    }
+    uint16_t dh = cq_f2h(0.0f), dmh = cq_f2h(0.0f);
+    if (max_scale > 0.0f) {
+        const float iscale = Q4SCALE / max_scale;
+        for (int j = 0; j < 16; j++) sc[j] = (uint8_t)cq_nearest_int(iscale * scales[j]);
+        dh = cq_f2h(max_scale / Q4SCALE);
+    } else {
+        for (int j = 0; j < 16; j++) sc[j] = 0;
+    }
+    if (max_min > 0.0f) {
+        const float iscale = Q4SCALE / max_min;
+        for (int j = 0; j < 16; j++) sc[j] |= (uint8_t)((uint8_t)cq_nearest_int(iscale * mins[j]) << 4);
+        dmh = cq_f2h(max_min / Q4SCALE);
+    }
+    store_u16(y + 80, dh);
+    store_u16(y + 82, dmh);
+    for (int i = 0; i < 64; i++) qs[i] = 0;
+    const float dall = cq_h2f(dh), dmin = cq_h2f(dmh);
+    for (int j = 0; j < 16; j++) {
+        const float d = dall * (float)(sc[j] & 0xF);
+        if (d == 0.0f) continue;
+        const float dm = dmin * (float)(sc[j] >> 4);
+        for (int ii = 0; ii < 16; ii++) {
+            const int e = 16 * j + ii;
+            const int ll = cq_clampi(cq_nearest_int((x[e] + dm) / d), 0, 3);
+            qs[32 * (e / 128) + e % 32] |= (uint8_t)(ll << (2 * ((e % 128) / 32)));
+        }
+    }
+}
+
 // Q4_1 (k_quants.rs:296-326) and, FIVE, Q5_1 (:496-530): d = (max - min) / levels, quants round((x - min) / d)
 template <bool FIVE>
 __global__ void quantize_q4_1(const float *__restrict__ src, int64_t nblocks, uint8_t *__restrict__ out) {
@@ -438,6 +484,7 @@ hipError_t cq_launch_quantize_weight(int dtype, const float *src, int64_t nblock
     case CQ_DTYPE_Q4_1: quantize_q4_1<false><<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q5_1: quantize_q4_1<true><<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q3K: quantize_q3k<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
+    case CQ_DTYPE_Q2K: quantize_q2k<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q4K: quantize_q4k<16><<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q5K: quantize_q4k<32><<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q6K: quantize_q6k<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;

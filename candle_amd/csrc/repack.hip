@@ -321,6 +321,46 @@ __global__ void transcode_q3k_q6k(uint8_t *__restrict__ q3, uint8_t *__restrict_
     }
 }
 
+// Q2K {u8 scales[16]; u8 qs[64]; f16 d; f16 dmin} (k_quants.rs:96-103): value (d * sc_j) * q - dmin * m_j, sc_j and m_j
+// the nibbles of scales[j].  The first term is a Q6K block with scales sc_j and quants q + 32; m_j and dmin go to
+// planes of their own.
+__global__ void transcode_q2k_q6k(uint8_t *__restrict__ q2, uint8_t *__restrict__ q6, uint8_t *__restrict__ mins,
+                                  uint16_t *__restrict__ dmins, int64_t nblocks, bool inverse) {
+    const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    uint8_t *x = q2 + b * 84, *y = q6 + b * 210;
+    uint8_t *sc2 = x, *qs = x + 16;
+    uint8_t *ql = y, *qh = y + 128, *sc6 = y + 192, *mb = mins + b * 16;
+    if (!inverse) {
+        for (int i = 0; i < 192; i++) y[i] = 0;
+        for (int e = 0; e < 256; e++) {
+            const int half = e / 128, r = e % 128, quad = r / 32, l = r % 32;
+            const int v = ((qs[32 * half + l] >> (2 * quad)) & 3) + 32;
+            ql[64 * half + 32 * (quad & 1) + l] |= (uint8_t)((v & 0xF) << (4 * (quad >> 1)));
+            qh[32 * half + l] |= (uint8_t)((v >> 4) << (2 * quad));
+        }
+        for (int j = 0; j < 16; j++) {
+            sc6[j] = (uint8_t)(sc2[j] & 0xF);
+            mb[j] = (uint8_t)(sc2[j] >> 4);
+        }
+        y[208] = x[80];
+        y[209] = x[81];
+        dmins[b] = (uint16_t)(x[82] | (x[83] << 8));
+    } else {
+        for (int i = 16; i < 80; i++) x[i] = 0;
+        for (int e = 0; e < 256; e++) {
+            const int half = e / 128, r = e % 128, quad = r / 32, l = r % 32;
+            const int v6 = ((ql[64 * half + 32 * (quad & 1) + l] >> (4 * (quad >> 1))) & 0xF) | (((qh[32 * half + l] >> (2 * quad)) & 3) << 4);
+            qs[32 * half + l] |= (uint8_t)(((v6 - 32) & 3) << (2 * quad));
+        }
+        for (int j = 0; j < 16; j++) sc2[j] = (uint8_t)((sc6[j] & 0xF) | (mb[j] << 4));
+        x[80] = y[208];
+        x[81] = y[209];
+        x[82] = (uint8_t)(dmins[b] & 0xff);
+        x[83] = (uint8_t)(dmins[b] >> 8);
+    }
+}
+
 hipError_t launch(const cq_weight *w, uint8_t *aos, bool inverse, hipStream_t s) {
     const int64_t bs = cq_block_size(w->dtype);
     const int64_t nblocks = w->n * (w->k / bs);
@@ -367,8 +407,10 @@ hipError_t cq_launch_unpack(const cq_weight *w, uint8_t *aos_dev, hipStream_t s)
 }
 
 // GGML blocks of type `ggml_dtype` <-> GGML blocks of the type whose planes hold them (cq_storage_dtype).
-hipError_t cq_launch_transcode(int ggml_dtype, uint8_t *ggml_aos_dev, uint8_t *storage_aos_dev, uint16_t *min_plane,
-                               int64_t nblocks, bool inverse, hipStream_t s) {
+hipError_t cq_launch_transcode(const cq_weight *w, uint8_t *ggml_aos_dev, uint8_t *storage_aos_dev, int64_t nblocks, bool inverse,
+                               hipStream_t s) {
+    const int ggml_dtype = w->ggml_dtype;
+    uint16_t *min_plane = (uint16_t *)w->p2;
     if (nblocks == 0) return hipSuccess;
     const int threads = 128;
     const unsigned grid = (unsigned)((nblocks + threads - 1) / threads);
@@ -377,6 +419,7 @@ hipError_t cq_launch_transcode(int ggml_dtype, uint8_t *ggml_aos_dev, uint8_t *s
     case CQ_DTYPE_Q4_1: transcode_q4_1_q8_0<false><<<grid, threads, 0, s>>>(ggml_aos_dev, storage_aos_dev, min_plane, nblocks, inverse); break;
     case CQ_DTYPE_Q5_1: transcode_q4_1_q8_0<true><<<grid, threads, 0, s>>>(ggml_aos_dev, storage_aos_dev, min_plane, nblocks, inverse); break;
     case CQ_DTYPE_Q3K: transcode_q3k_q6k<<<grid, threads, 0, s>>>(ggml_aos_dev, storage_aos_dev, nblocks, inverse); break;
+    case CQ_DTYPE_Q2K: transcode_q2k_q6k<<<grid, threads, 0, s>>>(ggml_aos_dev, storage_aos_dev, w->p4, (uint16_t *)w->p5, nblocks, inverse); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

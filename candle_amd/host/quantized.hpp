@@ -38,11 +38,11 @@ inline void check_hip(hipError_t e, const char *what) {
 }
 
 // ---- GgmlDType (mod.rs:133-247) --------------------------------------------------------------
-enum class GgmlDType : uint32_t { Q4_0 = 2, Q4_1 = 3, Q5_0 = 6, Q5_1 = 7, Q8_0 = 8, Q8_1 = 9, Q3K = 11, Q4K = 12, Q5K = 13, Q6K = 14, Q8K = 15 };
+enum class GgmlDType : uint32_t { Q4_0 = 2, Q4_1 = 3, Q5_0 = 6, Q5_1 = 7, Q8_0 = 8, Q8_1 = 9, Q2K = 10, Q3K = 11, Q4K = 12, Q5K = 13, Q6K = 14, Q8K = 15 };
 
 inline GgmlDType ggml_dtype_from_u32(uint32_t u) {   // mod.rs:152-171
     switch (u) {
-        case 2: case 3: case 6: case 7: case 8: case 9: case 11: case 12: case 13: case 14: case 15: return static_cast<GgmlDType>(u);
+        case 2: case 3: case 6: case 7: case 8: case 9: case 10: case 11: case 12: case 13: case 14: case 15: return static_cast<GgmlDType>(u);
         default: throw Error("unknown or unsupported dtype for ggml: " + std::to_string(u));
     }
 }

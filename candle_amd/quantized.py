@@ -30,6 +30,7 @@ class GgmlDType(enum.IntEnum):
     Q5_1 = 7
     Q8_0 = 8
     Q8_1 = 9
+    Q2K = 10
     Q3K = 11
     Q4K = 12
     Q5K = 13
@@ -39,7 +40,7 @@ class GgmlDType(enum.IntEnum):
     @classmethod
     def from_str(cls, name: str) -> "GgmlDType":
         """Names accepted by the reference's Python `Tensor.quantize` (lib.rs:1082-1098)."""
-        table = {"q4_0": cls.Q4_0, "q4_1": cls.Q4_1, "q5_0": cls.Q5_0, "q5_1": cls.Q5_1, "q8_0": cls.Q8_0, "q8_1": cls.Q8_1, "q3k": cls.Q3K, "q4k": cls.Q4K,
+        table = {"q4_0": cls.Q4_0, "q4_1": cls.Q4_1, "q5_0": cls.Q5_0, "q5_1": cls.Q5_1, "q8_0": cls.Q8_0, "q8_1": cls.Q8_1, "q2k": cls.Q2K, "q3k": cls.Q3K, "q4k": cls.Q4K,
                  "q5k": cls.Q5K, "q6k": cls.Q6K,
                  "q8k": cls.Q8K, "f32": cls.F32, "f16": cls.F16}
         key = name.lower()
@@ -66,7 +67,7 @@ class GgmlDType(enum.IntEnum):
         return GgmlDType(qhip.load().cq_vec_dot_type(int(self)))
 
 
-_WEIGHT_TYPES = (GgmlDType.Q4_0, GgmlDType.Q4_1, GgmlDType.Q5_0, GgmlDType.Q5_1, GgmlDType.Q8_0, GgmlDType.Q3K, GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K)
+_WEIGHT_TYPES = (GgmlDType.Q4_0, GgmlDType.Q4_1, GgmlDType.Q5_0, GgmlDType.Q5_1, GgmlDType.Q8_0, GgmlDType.Q2K, GgmlDType.Q3K, GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K)
 
 
 class QTensor:

@@ -42,6 +42,8 @@ enum {
     CQ_DTYPE_Q5_1 = 7,  /* like Q4_1, with five-bit quants                                                            */
     CQ_DTYPE_Q8_0 = 8,
     CQ_DTYPE_Q8_1 = 9,  /* activation format only */
+    CQ_DTYPE_Q2K = 10,  /* held as Q6K planes (scale, quant + 32) plus the groups' minima and dmin; the dmin term of the
+                           dot product (k_quants.rs:717-767) is subtracted by a second small launch                   */
     CQ_DTYPE_Q3K = 11,  /* held on the device as Q6K planes (scale - 32, quant + 28): the same values and arithmetic */
     CQ_DTYPE_Q4K = 12,
     CQ_DTYPE_Q5K = 13,

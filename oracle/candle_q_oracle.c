@@ -29,6 +29,9 @@
  *        bits depend on the platform's expf)
  *   q5_0 quantize, dequant, q5_0 x q8_0 dot (k_quants.rs:352-452) : :289-319 (128 round-trip values), :317
  *        (RMSE bound), :795-805 (dot-product error <= 0.001353), numpy brute force from unpacked blocks
+ *   q2k quantize (make_qkx1_quants with 3 levels over 16 elements), dequant, q2k x q8k dot (k_quants.rs:698-872)
+ *                                               : :437-482 (spot values, < 0.1, < 6.0, RMSE <= 0.0075),
+ *        :795-805 (dot-product error <= 0.004086), numpy brute force from unpacked blocks
  *   q3k quantize (make_q3_quants, utils.rs:261-326), dequant, q3k x q8k dot (k_quants.rs:874-1148)
  *                                               : :484-529 (spot values, < 0.03, < 3.5, RMSE <= 0.004),
  *        :795-805 (dot-product error <= 0.016148), numpy brute force from unpacked blocks
@@ -75,6 +78,8 @@ typedef struct { uint16_t d; uint8_t qh[4]; uint8_t qs[16]; } block_q5_0;       
 typedef struct { uint16_t d; uint16_t m; uint8_t qh[4]; uint8_t qs[16]; } block_q5_1; /* 24, k_quants.rs:69-76 */
 _Static_assert(sizeof(block_q5_1) == 24, "q5_1");
 typedef struct { uint8_t hmask[QK_K / 8]; uint8_t qs[QK_K / 4]; uint8_t scales[12]; uint16_t d; } block_q3k; /* 110, k_quants.rs:107-114 */
+typedef struct { uint8_t scales[QK_K / 16]; uint8_t qs[QK_K / 4]; uint16_t d; uint16_t dmin; } block_q2k;    /* 84, k_quants.rs:96-103 */
+_Static_assert(sizeof(block_q2k) == 84, "q2k");
 _Static_assert(sizeof(block_q5_0) == 22, "q5_0");
 _Static_assert(sizeof(block_q3k) == 110, "q3k");
 _Static_assert(sizeof(block_q4_0) == 18, "q4_0");
@@ -1109,6 +1114,100 @@ static inline int32_t int_q6k_q8k(const block_q6k *x, const block_q8k *y) {
     return total;
 }
 
+/* ---------------------------------------------------------------- Q2K ---- */
+/* the two-bit quant of element e */
+static inline int32_t q2k_quant(const block_q2k *b, int e) {
+    return (b->qs[32 * (e / 128) + e % 32] >> (2 * ((e % 128) / 32))) & 3;
+}
+
+/* k_quants.rs:770-839 (from_float; make_qkx1_quants(3, 5, 16 elements), utils.rs:201-258) */
+int orc_quantize_q2k(const float *xs, void *out, int64_t k) {
+    if (k % QK_K != 0) return -1;
+    block_q2k *ys = (block_q2k *)out;
+    const float Q4SCALE = 15.0f;
+    for (int64_t i = 0; i < k / QK_K; i++) {
+        const float *x = xs + i * QK_K;
+        block_q2k *block = &ys[i];
+        float mins[QK_K / 16], scales[QK_K / 16];
+        for (int j = 0; j < QK_K / 16; j++) make_qkx1_quants(3, 5, x + 16 * j, 16, &scales[j], &mins[j]);
+        float max_scale = 0.0f, max_min = 0.0f;
+        for (int j = 0; j < QK_K / 16; j++) {
+            max_scale = fmaxf(scales[j], max_scale);
+            max_min = fmaxf(mins[j], max_min);
+        }
+        if (max_scale > 0.0f) {
+            float iscale = Q4SCALE / max_scale;
+            for (int j = 0; j < QK_K / 16; j++) block->scales[j] = (uint8_t)nearest_int(iscale * scales[j]);
+            block->d = orc_f32_to_f16(max_scale / Q4SCALE);
+        } else {
+            for (int j = 0; j < QK_K / 16; j++) block->scales[j] = 0;
+            block->d = orc_f32_to_f16(0.0f);
+        }
+        if (max_min > 0.0f) {
+            float iscale = Q4SCALE / max_min;
+            for (int j = 0; j < QK_K / 16; j++) {
+                uint8_t l = (uint8_t)nearest_int(iscale * mins[j]);
+                block->scales[j] |= (uint8_t)(l << 4);
+            }
+            block->dmin = orc_f32_to_f16(max_min / Q4SCALE);
+        } else {
+            block->dmin = orc_f32_to_f16(0.0f);
+        }
+        uint8_t big_l[QK_K];
+        memset(big_l, 0, sizeof big_l);
+        for (int j = 0; j < QK_K / 16; j++) {
+            float d = orc_f16_to_f32(block->d) * (float)(block->scales[j] & 0xF);
+            if (d == 0.0f) continue;
+            float dm = orc_f16_to_f32(block->dmin) * (float)(block->scales[j] >> 4);
+            for (int ii = 0; ii < 16; ii++)
+                big_l[16 * j + ii] = (uint8_t)clampi(nearest_int((x[16 * j + ii] + dm) / d), 0, 3);
+        }
+        for (int j = 0; j < QK_K; j += 128)
+            for (int ll = 0; ll < 32; ll++)
+                block->qs[j / 4 + ll] = (uint8_t)(big_l[j + ll] | (big_l[j + ll + 32] << 2) | (big_l[j + ll + 64] << 4) | (big_l[j + ll + 96] << 6));
+    }
+    return 0;
+}
+
+/* k_quants.rs:841-872 (to_float): y = (d * sc) * q - (dmin * m) */
+int orc_dequantize_q2k(const void *in, float *ys, int64_t k) {
+    if (k % QK_K != 0) return -1;
+    const block_q2k *xs = (const block_q2k *)in;
+    for (int64_t i = 0; i < k / QK_K; i++) {
+        float d = orc_f16_to_f32(xs[i].d), min = orc_f16_to_f32(xs[i].dmin);
+        for (int e = 0; e < QK_K; e++) {
+            uint8_t sc = xs[i].scales[e / 16];
+            float dl = d * (float)(sc & 0xF), ml = min * (float)(sc >> 4);
+            ys[i * QK_K + e] = dl * (float)q2k_quant(&xs[i], e) - ml;
+        }
+    }
+    return 0;
+}
+
+/* k_quants.rs:717-767 (vec_dot_unopt of Q2K x Q8K): per block dall * isum - dmin * summs */
+static void ints_q2k_q8k(const block_q2k *x, const block_q8k *y, int32_t *isum, int32_t *summs) {
+    int32_t s = 0, t = 0;
+    for (int j = 0; j < QK_K / 16; j++) {
+        s += (int32_t)y->bsums[j] * (int32_t)(x->scales[j] >> 4);
+        int32_t isuml = 0;
+        for (int l = 0; l < 16; l++) isuml += (int32_t)y->qs[16 * j + l] * q2k_quant(x, 16 * j + l);
+        t += (int32_t)(x->scales[j] & 0xF) * isuml;
+    }
+    *isum = t;
+    *summs = s;
+}
+static float vec_dot_q2k_q8k(int64_t n, const block_q2k *xs, const block_q8k *ys) {
+    float sumf = 0.0f;
+    for (int64_t i = 0; i < n / QK_K; i++) {
+        int32_t isum, summs;
+        ints_q2k_q8k(&xs[i], &ys[i], &isum, &summs);
+        float dall = ys[i].d * orc_f16_to_f32(xs[i].d);
+        float dmin = ys[i].d * orc_f16_to_f32(xs[i].dmin);
+        sumf += dall * (float)isum - dmin * (float)summs;
+    }
+    return sumf;
+}
+
 /* ---------------------------------------------------------------- Q3K ---- */
 /* utils.rs:261-326 (make_q3_quants; from_float calls it with nmax = 4, do_rmse = true and uses the returned
  * scale only) */
@@ -1266,14 +1365,14 @@ static float vec_dot_q3k_q8k(int64_t n, const block_q3k *xs, const block_q8k *ys
 int64_t orc_block_size(int dtype) {
     switch (dtype) {
     case ORC_Q4_0: case ORC_Q4_1: case ORC_Q5_0: case ORC_Q5_1: case ORC_Q8_0: case ORC_Q8_1: return 32;
-    case ORC_Q3K: case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return QK_K;
+    case ORC_Q2K: case ORC_Q3K: case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return QK_K;
     default: return 0;
     }
 }
 int64_t orc_type_size(int dtype) {
     switch (dtype) {
     case ORC_Q4_0: return 18; case ORC_Q4_1: return 20; case ORC_Q5_0: return 22; case ORC_Q5_1: return 24; case ORC_Q8_0: return 34; case ORC_Q8_1: return 36;
-    case ORC_Q3K: return 110; case ORC_Q4K: return 144; case ORC_Q5K: return 176; case ORC_Q6K: return 210; case ORC_Q8K: return 292;
+    case ORC_Q2K: return 84; case ORC_Q3K: return 110; case ORC_Q4K: return 144; case ORC_Q5K: return 176; case ORC_Q6K: return 210; case ORC_Q8K: return 292;
     default: return 0;
     }
 }
@@ -1283,7 +1382,7 @@ int orc_vec_dot_type(int dtype) {
     switch (dtype) {
     case ORC_Q4_0: case ORC_Q5_0: case ORC_Q8_0: return ORC_Q8_0;   /* Q5_0: k_quants.rs:356 */
     case ORC_Q4_1: case ORC_Q5_1: return ORC_Q8_1;   /* k_quants.rs:260, :457 */
-    case ORC_Q3K: case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return ORC_Q8K;   /* Q3K: k_quants.rs:877 */
+    case ORC_Q2K: case ORC_Q3K: case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return ORC_Q8K;   /* Q2K: k_quants.rs:701, Q3K: :877 */
     default: return -1;
     }
 }
@@ -1294,6 +1393,7 @@ int orc_quantize(int dtype, const float *xs, void *out, int64_t k) {
     case ORC_Q4_1: return orc_quantize_q4_1(xs, out, k);
     case ORC_Q5_0: return orc_quantize_q5_0(xs, out, k);
     case ORC_Q5_1: return orc_quantize_q5_1(xs, out, k);
+    case ORC_Q2K: return orc_quantize_q2k(xs, out, k);
     case ORC_Q3K: return orc_quantize_q3k(xs, out, k);
     case ORC_Q8_0: return orc_quantize_q8_0(xs, out, k);
     case ORC_Q8_1: return orc_quantize_q8_1(xs, out, k);
@@ -1311,6 +1411,7 @@ int orc_dequantize(int dtype, const void *in, float *ys, int64_t k) {
     case ORC_Q4_1: return orc_dequantize_q4_1(in, ys, k);
     case ORC_Q5_0: return orc_dequantize_q5_0(in, ys, k);
     case ORC_Q5_1: return orc_dequantize_q5_1(in, ys, k);
+    case ORC_Q2K: return orc_dequantize_q2k(in, ys, k);
     case ORC_Q3K: return orc_dequantize_q3k(in, ys, k);
     case ORC_Q8_0: return orc_dequantize_q8_0(in, ys, k);
     case ORC_Q4K: return orc_dequantize_q4k(in, ys, k);
@@ -1330,6 +1431,7 @@ int orc_vec_dot(int dtype, int64_t n, const void *xs, const void *ys, float *out
     case ORC_Q4_1: return vec_dot_q4_1_q8_1(n, xs, ys, out);
     case ORC_Q5_0: *out = vec_dot_q5_0_q8_0(n, xs, ys); return 0;
     case ORC_Q5_1: return vec_dot_q5_1_q8_1(n, xs, ys, out);
+    case ORC_Q2K: *out = vec_dot_q2k_q8k(n, xs, ys); return 0;
     case ORC_Q3K: *out = vec_dot_q3k_q8k(n, xs, ys); return 0;
     case ORC_Q8_0: *out = vec_dot_q8_0_q8_0(n, xs, ys); return 0;
     case ORC_Q4K: *out = vec_dot_q4k_q8k(n, xs, ys); return 0;
@@ -1400,6 +1502,13 @@ int orc_block_int_dots(int dtype, int64_t m, int64_t k, int64_t n, const void *a
                 case ORC_Q5_1:
                     out_i[o] = sumi_q5_1_q8_1((const block_q5_1 *)w + b, (const block_q8_1 *)a + b);
                     break;
+                case ORC_Q2K: {
+                    int32_t isum, summs;
+                    ints_q2k_q8k((const block_q2k *)w + b, (const block_q8k *)a + b, &isum, &summs);
+                    out_i[o] = isum;
+                    if (out_mn) out_mn[o] = summs;
+                    break;
+                }
                 case ORC_Q3K: {
                     int32_t aux32[8], t = 0;
                     ints_q3k_q8k((const block_q3k *)w + b, (const block_q8k *)a + b, aux32);

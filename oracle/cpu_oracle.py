@@ -17,12 +17,12 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libcandle_q_oracle.so")
 
 # GgmlDType ids (candle-core/src/quantized/mod.rs:173-190)
-Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1, Q3K, Q4K, Q5K, Q6K, Q8K = 2, 3, 6, 7, 8, 9, 11, 12, 13, 14, 15
-BLOCK_SIZE = {Q4_0: 32, Q4_1: 32, Q5_0: 32, Q5_1: 32, Q8_0: 32, Q8_1: 32, Q3K: 256, Q4K: 256, Q5K: 256, Q6K: 256, Q8K: 256}
-TYPE_SIZE = {Q4_0: 18, Q4_1: 20, Q5_0: 22, Q5_1: 24, Q8_0: 34, Q8_1: 36, Q3K: 110, Q4K: 144, Q5K: 176, Q6K: 210, Q8K: 292}
+Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1, Q2K, Q3K, Q4K, Q5K, Q6K, Q8K = 2, 3, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15
+BLOCK_SIZE = {Q4_0: 32, Q4_1: 32, Q5_0: 32, Q5_1: 32, Q8_0: 32, Q8_1: 32, Q2K: 256, Q3K: 256, Q4K: 256, Q5K: 256, Q6K: 256, Q8K: 256}
+TYPE_SIZE = {Q4_0: 18, Q4_1: 20, Q5_0: 22, Q5_1: 24, Q8_0: 34, Q8_1: 36, Q2K: 84, Q3K: 110, Q4K: 144, Q5K: 176, Q6K: 210, Q8K: 292}
 # the reference's Q4_1 vectors also pin the `s` field of Q8_1 blocks
-VEC_DOT_TYPE = {Q4_0: Q8_0, Q4_1: Q8_1, Q5_0: Q8_0, Q5_1: Q8_1, Q8_0: Q8_0, Q3K: Q8K, Q4K: Q8K, Q5K: Q8K, Q6K: Q8K, Q8K: Q8K}
-NAMES = {Q4_0: "q4_0", Q4_1: "q4_1", Q5_0: "q5_0", Q5_1: "q5_1", Q8_0: "q8_0", Q8_1: "q8_1", Q3K: "q3k", Q4K: "q4k", Q5K: "q5k", Q6K: "q6k", Q8K: "q8k"}
+VEC_DOT_TYPE = {Q4_0: Q8_0, Q4_1: Q8_1, Q5_0: Q8_0, Q5_1: Q8_1, Q8_0: Q8_0, Q2K: Q8K, Q3K: Q8K, Q4K: Q8K, Q5K: Q8K, Q6K: Q8K, Q8K: Q8K}
+NAMES = {Q4_0: "q4_0", Q4_1: "q4_1", Q5_0: "q5_0", Q5_1: "q5_1", Q8_0: "q8_0", Q8_1: "q8_1", Q2K: "q2k", Q3K: "q3k", Q4K: "q4k", Q5K: "q5k", Q6K: "q6k", Q8K: "q8k"}
 
 
 def build(force: bool = False) -> str:
@@ -140,7 +140,7 @@ def block_int_dots(dtype: int, act_blocks: np.ndarray, m: int, rhs_blocks: np.nd
     act_blocks = np.ascontiguousarray(act_blocks, dtype=np.uint8)
     rhs_blocks = np.ascontiguousarray(rhs_blocks, dtype=np.uint8)
     oi = np.zeros((m, n, kb), dtype=np.int32)
-    om = np.zeros((m, n, kb), dtype=np.int32) if dtype in (Q4K, Q5K) else None
+    om = np.zeros((m, n, kb), dtype=np.int32) if dtype in (Q2K, Q4K, Q5K) else None
     i32p = C.POINTER(C.c_int32)
     _check(lib().orc_block_int_dots(dtype, m, k, n, act_blocks.ctypes.data, rhs_blocks.ctypes.data,
                                     oi.ctypes.data_as(i32p),

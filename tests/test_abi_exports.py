@@ -112,7 +112,8 @@ def test_metadata_calls_need_no_gpu(lib):
     assert (lib.cq_block_size(7), lib.cq_type_size(7), lib.cq_vec_dot_type(7)) == (32, 24, 9)      # Q5_1 x Q8_1, k_quants.rs:69-76, :457
     assert (lib.cq_block_size(Q5_0), lib.cq_type_size(Q5_0), lib.cq_vec_dot_type(Q5_0)) == (32, 22, Q8_0)    # k_quants.rs:61-67, :356
     assert (lib.cq_block_size(Q3K), lib.cq_type_size(Q3K), lib.cq_vec_dot_type(Q3K)) == (256, 110, Q8K)     # k_quants.rs:107-114, :877
-    assert (lib.cq_block_size(10), lib.cq_type_size(10), lib.cq_vec_dot_type(10)) == (0, 0, -1)             # Q2K: not handled
+    assert (lib.cq_block_size(10), lib.cq_type_size(10), lib.cq_vec_dot_type(10)) == (256, 84, Q8K)         # Q2K, k_quants.rs:96-103, :701
+    assert (lib.cq_block_size(1), lib.cq_type_size(1), lib.cq_vec_dot_type(1)) == (0, 0, -1)                # F16: not handled
     assert (lib.cq_block_size(Q4_0), lib.cq_type_size(Q4_0)) == (32, 18)
     assert (lib.cq_block_size(Q8_0), lib.cq_type_size(Q8_0)) == (32, 34)
     assert (lib.cq_block_size(Q4K), lib.cq_type_size(Q4K)) == (256, 144)

@@ -200,7 +200,7 @@ def test_type_table_matches_library():
     """The parser's own size table against the device library's `cq_block_size` / `cq_type_size`."""
     from candle_amd import qhip
     L = qhip.load()
-    for t in (2, 3, 6, 7, 8, 9, 11, 12, 13, 14, 15):
+    for t in (2, 3, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15):
         assert G.ggml_block_size(t) == L.cq_block_size(t), t
         assert G.ggml_type_size(t) == L.cq_type_size(t), t
 
@@ -213,7 +213,7 @@ def _model_file(tmp_path, rng):
     for name, dt in (("blk.0.attn_q.weight", 12), ("blk.0.ffn_down.weight", 14),
                      ("blk.0.attn_k.weight", 2), ("token_embd.weight", 8),
                      ("blk.0.attn_v.weight", 6), ("blk.0.ffn_up.weight", 11), ("blk.0.ffn_gate.weight", 13),
-                     ("blk.0.attn_output.weight", 3), ("output.weight", 7)):
+                     ("blk.0.attn_output.weight", 3), ("output.weight", 7), ("blk.1.ffn_up.weight", 10)):
         w = (rng.standard_normal((n, k)) * 0.1).astype(np.float32)
         host[name] = HostQTensor(dt, O.quantize(dt, w), (n, k))
     host["blk.0.attn_norm.weight"] = HostQTensor(0, rng.standard_normal(k).astype(np.float32), (k,))
@@ -265,7 +265,7 @@ def test_load_gguf_to_device_and_matmul(tmp_path):
 
 @pytest.mark.gpu
 def test_load_gguf_rejects_types_without_device_kernels(tmp_path):
-    path = str(tmp_path / "q2.gguf")
-    G.save_gguf(path, {"w": HostQTensor(10, bytes(84), (1, 256))}, {})
-    with pytest.raises(GgufError, match="Q2K tensors are not supported on the device"):
+    path = str(tmp_path / "q8k.gguf")
+    G.save_gguf(path, {"w": HostQTensor(15, bytes(292), (1, 256))}, {})   # an activation format, not a weight type
+    with pytest.raises(GgufError, match="Q8K tensors are not supported on the device"):
         G.load_gguf(path)

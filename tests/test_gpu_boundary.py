@@ -55,7 +55,7 @@ def test_flat_storage_runs_the_reference_goldens(qh, goldens, seeded_inputs):
         assert np.array_equal(out, out2)
 
 
-@pytest.mark.parametrize("dt", [orc.Q4_0, orc.Q4_1, orc.Q5_0, orc.Q5_1, orc.Q8_0, orc.Q3K, orc.Q4K, orc.Q5K, orc.Q6K])
+@pytest.mark.parametrize("dt", [orc.Q4_0, orc.Q4_1, orc.Q5_0, orc.Q5_1, orc.Q8_0, orc.Q2K, orc.Q3K, orc.Q4K, orc.Q5K, orc.Q6K])
 @pytest.mark.parametrize("m", [1, 3, 16, 80])
 def test_shape_at_call_equals_shape_at_creation(qh, dt, m):
     """Every kernel family (one-launch decode, split-K, tile) reads flat storage like shaped storage, and one
@@ -80,7 +80,7 @@ def test_shape_at_call_equals_shape_at_creation(qh, dt, m):
     assert np.array_equal(flat.dequantize().cpu().numpy().ravel(), orc.dequantize(dt, blocks))
 
 
-@pytest.mark.parametrize("dt", [orc.Q4_1, orc.Q5_0, orc.Q5_1, orc.Q3K])
+@pytest.mark.parametrize("dt", [orc.Q4_1, orc.Q5_0, orc.Q5_1, orc.Q2K, orc.Q3K])
 def test_types_held_in_another_types_planes(qh, dt):
     """Q5_0 lives in Q8_0 planes, Q3K in Q6K planes, Q4_1 and Q5_1 in Q8_0 planes plus a plane of minima: the caller sees the type it created (dtype, GGML byte size,
     all-zero blocks from `zeros`, its own bytes back), whatever the device holds; the prefill tile kernel and the
@@ -104,9 +104,13 @@ def test_types_held_in_another_types_planes(qh, dt):
     assert np.linalg.norm(got - ref) <= 1e-4 * np.linalg.norm(ref)
     with pytest.raises(qh.QHipError, match="Q8_1 activations are for Q4K and Q6K"):
         qh.qmatmul(q, dev(x), flags=qh.FLAG_ACT_Q8_1)
-    if dt in (orc.Q4_1, orc.Q5_1):
-        # the offset term alone: an all-zero-quant weight (d = 0, m = c) gives c * sum_b s8_b for every output
+    if dt in (orc.Q4_1, orc.Q5_1, orc.Q2K):
+        # the offset term (almost) alone: Q4_1 / Q5_1 store a constant block as d = 0, m = c; Q2K a block of -0.375
+        # with a few -0.25 as minima of 0.375 and small scales
         const = np.full((n, k), 0.375, np.float32)
+        if dt == orc.Q2K:
+            const = -const
+            const[:, ::16] = -0.25
         qc = qh.QWeight.from_ggml(dt, orc.quantize(dt, const), n, k)
         got_c = qh.qmatmul(qc, dev(x[:3])).cpu().numpy()
         ref_c = orc.matmul(dt, x[:3], orc.quantize(dt, const), n)
@@ -120,7 +124,7 @@ def test_shape_errors(qh):
     assert L.cq_weight_zeros_flat(0, orc.Q4K, 300, C.byref(h)) == -1          # not whole blocks
     assert b"block size" in L.cq_last_error()
     assert L.cq_weight_create_flat(0, orc.Q4K, None, 145, C.byref(h)) == -1  # not whole blocks of bytes
-    assert L.cq_weight_zeros_flat(0, 10, 256, C.byref(h)) == -2              # Q2K: no device kernels
+    assert L.cq_weight_zeros_flat(0, 1, 256, C.byref(h)) == -2               # F16: not a quantized storage of this library
     qw = qh.QWeight.zeros_flat(orc.Q4K, 4 * 512)
     with pytest.raises(qh.QHipError, match="does not cover"):
         qw.set_shape(3, 512)

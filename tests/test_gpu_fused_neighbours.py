@@ -154,7 +154,8 @@ def test_matmul_with_rms_norm(qh, dt, m, k, n):
     # the same kernels on host-prepared input, in the kernels' order of operations: same bits
     if dt in (orc.Q4_0, orc.Q4_1, orc.Q5_0, orc.Q5_1, orc.Q8_0):   # the types with 32-element activation blocks
         assert torch.equal(got, qh.qmatmul(qw, dev(canonical_rms_norm(x, alpha, eps)), staged(qh, m)))
-    elif m == 1:   # one row: x * alpha through the matmul, the result times the row's scale
+    elif m == 1 and dt != orc.Q2K:   # one row: x * alpha through the matmul, the result times the row's scale
+        # (Q2K: two sums, the scale inside each: equal to rounding only, covered by the oracle comparison below)
         plain = qh.qmatmul(qw, dev((x * alpha[None, :]).astype(np.float32))).cpu().numpy()
         assert np.array_equal(got.cpu().numpy(), plain * canonical_scale(x, eps)[:, None])
     # the reference sequence rms_norm -> QMatMul::forward

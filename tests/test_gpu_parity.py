@@ -49,9 +49,9 @@ def make_inputs(seed, m, k, n, wscale=0.02, outliers=False):
 
 
 # Q5_0 and Q3K are held on the device in the planes of Q8_0 and Q6K (same values, same arithmetic), Q4_1 and Q5_1 in
-# Q8_0 planes plus a plane of minima whose term a second launch adds: every test below takes them through the boundary
+# Q8_0 planes plus a plane of minima whose term a second launch adds (Q2K likewise in Q6K planes): every test below takes them through the boundary
 # like the others and compares with the oracle's own code for the type
-WEIGHT_DTYPES = [orc.Q4_0, orc.Q4_1, orc.Q5_0, orc.Q5_1, orc.Q8_0, orc.Q3K, orc.Q4K, orc.Q5K, orc.Q6K]
+WEIGHT_DTYPES = [orc.Q4_0, orc.Q4_1, orc.Q5_0, orc.Q5_1, orc.Q8_0, orc.Q2K, orc.Q3K, orc.Q4K, orc.Q5K, orc.Q6K]
 
 
 # ------------------------------------------------------------ activation quantizers ----
@@ -697,10 +697,10 @@ def test_few_rows_one_launch_equals_single_rows(qh, dt, m, k, n):
     qw = qh.QWeight.from_ggml(dt, blocks, n, k)
     xd = dev(x)
     got = qh.qmatmul(qw, xd)
-    elems = {orc.Q4_0: 32, orc.Q4_1: 16, orc.Q5_0: 16, orc.Q5_1: 16, orc.Q8_0: 16, orc.Q3K: 32, orc.Q4K: 64, orc.Q5K: 64, orc.Q6K: 32}[dt]   # weights per 16-byte lane unit
+    elems = {orc.Q4_0: 32, orc.Q4_1: 16, orc.Q5_0: 16, orc.Q5_1: 16, orc.Q8_0: 16, orc.Q2K: 32, orc.Q3K: 32, orc.Q4K: 64, orc.Q5K: 64, orc.Q6K: 32}[dt]   # weights per 16-byte lane unit
     units = k // elems
     per_lane = -(-units // 64) * elems
-    one_launch = dt not in (orc.Q4_1, orc.Q5_1)   # their m * s term is a second launch over the workspace
+    one_launch = dt not in (orc.Q4_1, orc.Q5_1, orc.Q2K)   # their offset term is a second launch over the workspace
     if one_launch and units <= (384 if m == 2 else 256) and (per_lane <= 64 or (per_lane <= 128 and m <= 3) or m <= 2):   # the library's rule
         for r in range(m):
             assert torch.equal(got[r:r + 1], qh.qmatmul(qw, xd[r:r + 1].contiguous())), r
