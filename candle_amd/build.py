@@ -11,7 +11,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libcandle_qhip.so")
 SOURCES = ["api.hip", "repack.hip", "quantize_act.hip", "quantize_weight.hip", "dequantize.hip", "matvec.hip",
-           "gemm.hip", "gemm_blk32.hip", "skinny.hip", "moe.hip", "min_term.hip", "no_alloc.hip"]
+           "gemm.hip", "gemm_blk32.hip", "skinny.hip", "moe.hip", "min_term.hip", "q8k_weight.hip", "no_alloc.hip"]
 # -ffp-contract=off: quantizers must perform single IEEE operations in the reference's order.
 # -packed-fp32-ops off: packed FP32 instructions are not to be generated on this hardware pool.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fno-fast-math",

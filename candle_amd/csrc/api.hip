@@ -78,7 +78,7 @@ extern "C" int cq_vec_dot_type(int dt) {
     switch (dt) {
     case CQ_DTYPE_Q4_0: case CQ_DTYPE_Q5_0: case CQ_DTYPE_Q8_0: return CQ_DTYPE_Q8_0;
     case CQ_DTYPE_Q4_1: case CQ_DTYPE_Q5_1: return CQ_DTYPE_Q8_1;   /* k_quants.rs:260, :457 */
-    case CQ_DTYPE_Q2K: case CQ_DTYPE_Q3K: case CQ_DTYPE_Q4K: case CQ_DTYPE_Q5K: case CQ_DTYPE_Q6K: return CQ_DTYPE_Q8K;
+    case CQ_DTYPE_Q2K: case CQ_DTYPE_Q3K: case CQ_DTYPE_Q4K: case CQ_DTYPE_Q5K: case CQ_DTYPE_Q6K: case CQ_DTYPE_Q8K: return CQ_DTYPE_Q8K;
     default: return -1;
     }
 }
@@ -86,7 +86,7 @@ extern "C" int cq_vec_dot_type(int dt) {
 static bool is_weight_dtype(int dt) {
     return dt == CQ_DTYPE_Q4_0 || dt == CQ_DTYPE_Q4_1 || dt == CQ_DTYPE_Q5_0 || dt == CQ_DTYPE_Q5_1 || dt == CQ_DTYPE_Q8_0 ||
            dt == CQ_DTYPE_Q2K || dt == CQ_DTYPE_Q3K || dt == CQ_DTYPE_Q4K ||
-           dt == CQ_DTYPE_Q5K || dt == CQ_DTYPE_Q6K;
+           dt == CQ_DTYPE_Q5K || dt == CQ_DTYPE_Q6K || dt == CQ_DTYPE_Q8K;
 }
 
 // --------------------------------------------------------------- weights ----
@@ -116,6 +116,7 @@ static int weight_alloc(int dev, int dt, int64_t n, int64_t k, cq_weight **out) 
     case CQ_DTYPE_Q4K: s0 = (size_t)nb * 128; s1 = (size_t)nb * CQ_Q4K_HDR; break;
     case CQ_DTYPE_Q5K: s0 = (size_t)nb * 128; s1 = (size_t)nb * CQ_Q4K_HDR; s2 = (size_t)nb * 32; break;
     case CQ_DTYPE_Q6K: s0 = (size_t)nb * 128; s1 = (size_t)nb * 64; s2 = (size_t)nb * 16; s3 = (size_t)nb * 2; break;
+    case CQ_DTYPE_Q8K: s0 = (size_t)nb * 256; s1 = (size_t)nb * 4; s2 = (size_t)nb * 32; break;
     }
     if (cq_has_min32(dt)) s2 = (size_t)nb * 2;   // the blocks' minima beside the Q8_0 planes
     size_t s4 = 0, s5 = 0;
@@ -468,6 +469,17 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
     const int act = act_dtype_for(w, flags);
     CQ_HIP_CHECK(hipSetDevice(w->dev));
     hipStream_t s = (hipStream_t)stream;
+    if (w->dtype == CQ_DTYPE_Q8K) {
+        // Q8K weights (a type of the reference's tests, not of checkpoints): the quantizer launch and one dot-product kernel
+        if (flags & ~(CQ_FLAG_REUSE_ACT | CQ_FLAG_FORCE_MATVEC | CQ_FLAG_STAGED_ACT))
+            return cq_set_error(CQ_ERR_UNSUPPORTED, "Q8K weights have a dot-product kernel only (flags %d)", flags);
+        cq_act_view v;
+        act_ws_layout(act, m, w->k, (uint8_t *)ws, &v);
+        if (!(flags & CQ_FLAG_REUSE_ACT))
+            CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, nullptr, m, w->k, pre, v, cq_no_clear(), s));
+        CQ_HIP_CHECK(cq_launch_q8k_weight_matmul(w, v, m, y_dev, s));
+        return CQ_OK;
+    }
     if (flags & CQ_FLAG_ACT_Q8_1) {
         // the reference's CUDA formulation (cuda.rs:298-365): activations to Q8_1; a dot-product kernel up to 32 rows, the matrix cores beyond
         if (act != CQ_DTYPE_Q8_1 || !cq_matmul_q8_1_supported(w))
@@ -638,6 +650,7 @@ extern "C" int cq_qmatmul_int_dots(const cq_weight *w, const float *x_dev, int64
     int rc = check_matmul_args(w, x_dev, m, out_i, ws, ws_bytes, need);
     if (rc || m == 0 || w->n == 0 || w->k == 0) return rc;
     const int act = cq_vec_dot_type(w->dtype);
+    if (w->dtype == CQ_DTYPE_Q8K) return cq_set_error(CQ_ERR_UNSUPPORTED, "no integer dump for Q8K weights");
     if (!cq_matvec_row_fits(w)) return cq_set_error(CQ_ERR_UNSUPPORTED, "rows of %lld elements do not fit the LDS", (long long)w->k);
     CQ_HIP_CHECK(hipSetDevice(w->dev));
     hipStream_t s = (hipStream_t)stream;
@@ -699,8 +712,8 @@ static int grouped_impl(const cq_weight *const *experts, int n_experts, const fl
     if (rc || total == 0 || w0->n == 0 || w0->k == 0) return rc;
     const int act = act_dtype_for(w0, flags);
     if (act == CQ_DTYPE_Q8_1) return cq_set_error(CQ_ERR_UNSUPPORTED, "grouped matmul takes the CPU formulation only");
-    if (cq_has_min32(w0->ggml_dtype) || cq_has_min16(w0->ggml_dtype))
-        return cq_set_error(CQ_ERR_UNSUPPORTED, "grouped matmul does not take Q4_1 / Q5_1 / Q2K experts (their offset term has no grouped launch)");
+    if (cq_has_min32(w0->ggml_dtype) || cq_has_min16(w0->ggml_dtype) || w0->dtype == CQ_DTYPE_Q8K)
+        return cq_set_error(CQ_ERR_UNSUPPORTED, "grouped matmul does not take Q4_1 / Q5_1 / Q2K / Q8K experts (no grouped launch for them)");
     if ((rc = check_pre(pre))) return rc;
     CQ_HIP_CHECK(hipSetDevice(w0->dev));
     hipStream_t s = (hipStream_t)stream;

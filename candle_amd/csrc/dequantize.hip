@@ -176,6 +176,7 @@ hipError_t launch(const cq_weight *w, float *d32, uint16_t *d16, hipStream_t s) 
             dequant_q6k<F16, false><<<grid(total / 32), threads, 0, s>>>(w->p0, w->p1, (const int8_t *)w->p2, (const uint16_t *)w->p3,
                                                                          nullptr, nullptr, total / 32, d32, d16);
         break;
+    case CQ_DTYPE_Q8K: return cq_launch_dequantize_q8k(w, d32, d16, s);
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

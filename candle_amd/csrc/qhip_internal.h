@@ -111,6 +111,10 @@ hipError_t cq_launch_transcode(const cq_weight *w, uint8_t *ggml_aos_dev, uint8_
                                hipStream_t s);
 // y[r, c] -= sum_b (d8[r, b] * dmin[c, b]) * sum_j bsums[r, b, j] * m[c, b, j] for Q2K weights (k_quants.rs:727-733, :762)
 hipError_t cq_launch_min16_term(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s);
+// Q8K as a weight type (q8k_weight.hip): planes p0 qs, p1 d (f32), p2 bsums
+hipError_t cq_launch_repack_q8k(const cq_weight *w, uint8_t *aos, bool inverse, hipStream_t s);
+hipError_t cq_launch_dequantize_q8k(const cq_weight *w, float *d32, uint16_t *d16, hipStream_t s);
+hipError_t cq_launch_q8k_weight_matmul(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s);
 // y[r, c] += sum_b m[c, b] * s8[r, b] for Q4_1 / Q5_1 weights, s8 the `s` field of the activation's Q8_1 block
 // (k_quants.rs:665-691) recomputed from the workspace's block sums and scales.
 hipError_t cq_launch_min32_term(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s);

@@ -485,6 +485,8 @@ hipError_t cq_launch_quantize_weight(int dtype, const float *src, int64_t nblock
     case CQ_DTYPE_Q5_1: quantize_q4_1<true><<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q3K: quantize_q3k<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q2K: quantize_q2k<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
+    // Q8K (k_quants.rs:1788-1825): the activation quantizer writing GGML blocks, one 256-element row per block
+    case CQ_DTYPE_Q8K: return cq_launch_quantize_act_aos(CQ_DTYPE_Q8K, src, nblocks, 256, cq_no_pre(), aos_dev, s);
     case CQ_DTYPE_Q4K: quantize_q4k<16><<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q5K: quantize_q4k<32><<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;
     case CQ_DTYPE_Q6K: quantize_q6k<<<grid, threads, 0, s>>>(src, nblocks, aos_dev); break;

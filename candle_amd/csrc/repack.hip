@@ -392,6 +392,7 @@ hipError_t launch(const cq_weight *w, uint8_t *aos, bool inverse, hipStream_t s)
         repack_q6k<<<grid, threads, 0, s>>>(aos, w->p0, w->p1, w->p2, (uint16_t *)w->p3, nblocks, inverse);
         break;
     }
+    case CQ_DTYPE_Q8K: return cq_launch_repack_q8k(w, aos, inverse, s);
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

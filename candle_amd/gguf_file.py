@@ -40,7 +40,7 @@ _GGML_TYPES = {
     15: ("Q8K", 256, 292),
 }
 # Types the device library holds as weights (everything else parses but cannot be uploaded).
-DEVICE_WEIGHT_TYPES = (2, 3, 6, 7, 8, 10, 11, 12, 13, 14)
+DEVICE_WEIGHT_TYPES = (2, 3, 6, 7, 8, 10, 11, 12, 13, 14, 15)
 
 
 def ggml_type_name(dtype: int) -> str:

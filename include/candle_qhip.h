@@ -48,7 +48,8 @@ enum {
     CQ_DTYPE_Q4K = 12,
     CQ_DTYPE_Q5K = 13,
     CQ_DTYPE_Q6K = 14,
-    CQ_DTYPE_Q8K = 15   /* activation format only */
+    CQ_DTYPE_Q8K = 15   /* the activation format of the K-quants; as a weight type (k_quants.rs:1749-1839, a type of the
+                           reference's tests rather than of checkpoints) it has one plain dot-product kernel        */
 };
 
 /* error codes */

@@ -213,7 +213,8 @@ def _model_file(tmp_path, rng):
     for name, dt in (("blk.0.attn_q.weight", 12), ("blk.0.ffn_down.weight", 14),
                      ("blk.0.attn_k.weight", 2), ("token_embd.weight", 8),
                      ("blk.0.attn_v.weight", 6), ("blk.0.ffn_up.weight", 11), ("blk.0.ffn_gate.weight", 13),
-                     ("blk.0.attn_output.weight", 3), ("output.weight", 7), ("blk.1.ffn_up.weight", 10)):
+                     ("blk.0.attn_output.weight", 3), ("output.weight", 7), ("blk.1.ffn_up.weight", 10),
+                     ("blk.1.ffn_down.weight", 15)):
         w = (rng.standard_normal((n, k)) * 0.1).astype(np.float32)
         host[name] = HostQTensor(dt, O.quantize(dt, w), (n, k))
     host["blk.0.attn_norm.weight"] = HostQTensor(0, rng.standard_normal(k).astype(np.float32), (k,))
@@ -265,7 +266,7 @@ def test_load_gguf_to_device_and_matmul(tmp_path):
 
 @pytest.mark.gpu
 def test_load_gguf_rejects_types_without_device_kernels(tmp_path):
-    path = str(tmp_path / "q8k.gguf")
-    G.save_gguf(path, {"w": HostQTensor(15, bytes(292), (1, 256))}, {})   # an activation format, not a weight type
-    with pytest.raises(GgufError, match="Q8K tensors are not supported on the device"):
+    path = str(tmp_path / "q8_1.gguf")
+    G.save_gguf(path, {"w": HostQTensor(9, bytes(36), (1, 32))}, {})   # an activation format, not a weight type
+    with pytest.raises(GgufError, match="Q8_1 tensors are not supported on the device"):
         G.load_gguf(path)

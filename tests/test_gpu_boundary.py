@@ -45,7 +45,7 @@ def test_flat_storage_runs_the_reference_goldens(qh, goldens, seeded_inputs):
     assert np.array_equal(qw.to_ggml(), orc.quantize(orc.Q4_0, rhs))
     g = goldens["seeded_matmul_m11_k512_n21"]
     lhs, rhs = seeded_inputs
-    for name, dt in (("q4k", orc.Q4K), ("q5k", orc.Q5K), ("q6k", orc.Q6K)):
+    for name, dt in (("q4k", orc.Q4K), ("q5k", orc.Q5K), ("q6k", orc.Q6K), ("q8k", orc.Q8K)):
         qw = qh.QWeight.zeros_flat(dt, 21 * 512).quantize_(dev(rhs))
         out = qh.qmatmul_shaped(qw, (21, 512), dev(lhs)).cpu().numpy().ravel()
         spot = [float(np.round(np.float32(1000.0) * out[i]) / np.float32(1000.0)) for i in g["flat_indices"]]
@@ -116,6 +116,35 @@ def test_types_held_in_another_types_planes(qh, dt):
         ref_c = orc.matmul(dt, x[:3], orc.quantize(dt, const), n)
         assert np.abs(got_c - ref_c).max() <= 1e-4 * np.abs(ref_c).max()
         assert np.abs(ref_c).max() > 1.0     # the term is not negligible here
+
+
+@pytest.mark.parametrize("m,k,n", [(1, 256, 7), (3, 4096, 64), (40, 1024, 33), (2, 11008, 5)])
+def test_q8k_as_a_weight_type(qh, m, k, n):
+    """BlockQ8K as GgmlType (k_quants.rs:1749-1839; the reference's tests quantize to it and multiply by it,
+    quantized_tests.rs:672-717, :1124-1150): bytes back (any pattern, all-zero blocks from `zeros`), dequantize and the
+    device quantizer bit-exact, the product against the oracle, rows independent of their neighbours."""
+    rng = np.random.default_rng(m * k + n)
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    w[0] = 0.0
+    blocks = orc.quantize(orc.Q8K, w)
+    qw = qh.QWeight.from_ggml(orc.Q8K, blocks, n, k)
+    assert qw.dtype == orc.Q8K and qw.size_in_bytes == blocks.size and np.array_equal(qw.to_ggml(), blocks)
+    rnd = rng.integers(0, 256, size=blocks.size, dtype=np.uint8)
+    assert np.array_equal(qh.QWeight.from_ggml(orc.Q8K, rnd, n, k).to_ggml(), rnd)
+    assert not qh.QWeight.zeros(orc.Q8K, n, k).to_ggml().any()
+    want = orc.dequantize(orc.Q8K, blocks).reshape(n, k)
+    assert np.array_equal(qw.dequantize().cpu().numpy().view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(qw.dequantize_f16().cpu().numpy().view(np.uint16), want.astype(np.float16).view(np.uint16))
+    assert np.array_equal(qh.QWeight.zeros(orc.Q8K, n, k).quantize_(dev(w)).to_ggml(), blocks)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    got = qh.qmatmul(qw, dev(x)).cpu().numpy()
+    ref = orc.matmul(orc.Q8K, x, blocks, n)
+    for r in range(m):
+        assert np.linalg.norm(got[r] - ref[r]) <= 1e-4 * max(np.linalg.norm(ref[r]), 1e-30)
+    if m > 1:
+        assert np.array_equal(qh.qmatmul(qw, dev(x[1:2])).cpu().numpy()[0], got[1])
+    with pytest.raises(qh.QHipError, match="dot-product kernel only"):
+        qh.qmatmul(qw, dev(x), flags=qh.FLAG_FORCE_GEMM)
 
 
 def test_shape_errors(qh):

@@ -85,7 +85,7 @@ def test_python_qtensor_roundtrip_and_f16():
     import torch
     from candle_amd.quantized import QTensor
     src = torch.linspace(-0.5, 0.5, 4 * 1024, device="cuda").reshape(4, 1024)
-    for name, bound in (("q4k", 0.017), ("q6k", 0.008), ("q8_0", 0.005), ("q4_0", 0.05), ("q5_0", 0.02), ("q3k", 0.03), ("q4_1", 0.04), ("q5_1", 0.02), ("q2k", 0.1)):
+    for name, bound in (("q4k", 0.017), ("q6k", 0.008), ("q8_0", 0.005), ("q4_0", 0.05), ("q5_0", 0.02), ("q3k", 0.03), ("q4_1", 0.04), ("q5_1", 0.02), ("q2k", 0.1), ("q8k", 0.005)):
         q = QTensor.quantize(src, name)
         back = q.dequantize()
         assert back.shape == src.shape and float((back - src).abs().max()) < bound, name
