@@ -366,6 +366,36 @@ def test_gemm_needs_32_row_multiple(qh, dt):
     check_f32(qh.qmatmul(qw, dev(x)).cpu().numpy(), orc.matmul(dt, x, blocks, n))
 
 
+@pytest.mark.parametrize("dt,m,k,n", [(orc.Q3K, 1, 4096, 32000), (orc.Q3K, 512, 4096, 14336), (orc.Q2K, 1, 11008, 4096),
+                                      (orc.Q2K, 512, 14336, 4096), (orc.Q5_0, 16, 4096, 11008), (orc.Q5_0, 512, 4096, 14336),
+                                      (orc.Q4_1, 1, 4096, 11008), (orc.Q5_1, 512, 4096, 4096), (orc.Q8K, 3, 4096, 4096)])
+def test_other_weight_types_at_model_shapes(qh, dt, m, k, n):
+    """The types that are held in another type's planes (and Q8K weights) at the shapes of the BASELINE configurations:
+    weights quantized on the device, sampled weight rows (first, last, tile edges, random) over all activation rows
+    against the oracle's own code for the type, and the bytes of the sampled rows against the oracle's quantizer."""
+    rng = np.random.default_rng(k + n + int(dt))
+    gen = torch.Generator(device="cuda").manual_seed(k + int(dt))
+    wt = torch.randn((n, k), generator=gen, device="cuda") * 0.02
+    qw = qh.QWeight.zeros(dt, n, k).quantize_(wt)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    idx = rng.choice(x.size, size=max(1, x.size // 100), replace=False)
+    x.ravel()[idx] = np.where(rng.random(idx.size) < 0.5, -8.0, 8.0).astype(np.float32)
+    got = qh.qmatmul(qw, dev(x)).cpu().numpy()
+    rows = np.unique(np.concatenate([[0, 31, 32, 255, 256, n // 2, n - 257, n - 256, n - 33, n - 32, n - 1],
+                                     rng.choice(n, size=21, replace=False)]))
+    row_bytes = k // orc.BLOCK_SIZE[dt] * orc.TYPE_SIZE[dt]
+    blocks = qw.to_ggml().reshape(n, row_bytes)[rows]
+    assert np.array_equal(blocks.ravel(), orc.quantize(dt, wt[torch.from_numpy(rows).cuda()].cpu().numpy()))
+    del wt
+    ms = np.arange(m) if m <= 16 else np.unique(np.concatenate([[0, 31, 32, 127, 128, m - 1], rng.choice(m, size=10, replace=False)]))
+    want = orc.matmul(dt, x[ms], blocks.ravel(), len(rows))
+    g = got[np.ix_(ms, rows)].astype(np.float64)
+    assert np.linalg.norm(g - want) <= REL_L2_TOL * np.linalg.norm(want)
+    for i in range(len(ms)):
+        nrm = np.linalg.norm(want[i])
+        assert np.linalg.norm(g[i] - want[i]) <= REL_L2_TOL * nrm, (int(ms[i]), np.linalg.norm(g[i] - want[i]) / nrm)
+
+
 @pytest.mark.parametrize("dt", [orc.Q4K, orc.Q5K, orc.Q6K])
 @pytest.mark.parametrize("m,k,n", [(512, 4096, 14336), (512, 14336, 4096)])
 def test_prefill_gemm_config3(qh, dt, m, k, n):
