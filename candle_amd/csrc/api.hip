@@ -427,11 +427,19 @@ extern "C" size_t cq_workspace_bytes(const cq_weight *w, int64_t m, int flags) {
     return act_ws_layout(act_dtype_for(w, flags), m, w->k, nullptr, nullptr);
 }
 
+// candle's vec_dot of these three types refuses rows with an odd number of blocks (k_quants.rs:273, 363, 469)
+static int check_vec_dot_rows(const cq_weight *w) {
+    if ((w->ggml_dtype == CQ_DTYPE_Q4_1 || w->ggml_dtype == CQ_DTYPE_Q5_0 || w->ggml_dtype == CQ_DTYPE_Q5_1) && (w->k / 32) % 2)
+        return cq_set_error(CQ_ERR_INVALID, "vec_dot: %lld, nb is not divisible by 2", (long long)w->k);
+    return CQ_OK;
+}
+
 static int check_matmul_args(const cq_weight *w, const float *x, int64_t m, const void *y, void *ws, size_t ws_bytes,
                              size_t need) {
     if (!w) return cq_set_error(CQ_ERR_INVALID, "null weight");
     if (m < 0) return cq_set_error(CQ_ERR_INVALID, "negative row count");
     if (m == 0 || w->n == 0) return CQ_OK;
+    if (int rc = check_vec_dot_rows(w)) return rc;
     if (!x || !y) return cq_set_error(CQ_ERR_INVALID, "null argument");
     if ((uintptr_t)x & 15) return cq_set_error(CQ_ERR_INVALID, "x must be 16-byte aligned");
     if (!ws || ws_bytes < need)
@@ -502,9 +510,11 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
                           (pre.kind != CQ_PRE_NONE &&
                            ranges_overlap(y_dev, m * w->n, pre.aux, pre.kind == CQ_PRE_RMS_NORM ? w->k : m * w->k));
     // decode (one activation row): a single launch that quantizes x in its prologue
-    // (Q4_1 / Q5_1: the second launch that adds their m * s term reads the quantized row from the workspace)
+    // (Q4_1 / Q5_1 / Q2K: the one-launch kernels add the offset term themselves when no model step is fused in front;
+    // otherwise a second launch adds it from the quantized rows in the workspace)
     const bool min32 = cq_has_min32(w->ggml_dtype) || cq_has_min16(w->ggml_dtype);   // (Q2K: likewise, its dmin term)
-    if (m == 1 && !in_place && !min32 && !(flags & (CQ_FLAG_REUSE_ACT | CQ_FLAG_FORCE_GEMM | CQ_FLAG_STAGED_ACT | CQ_FLAG_ACT_Q8_1)) &&
+    if (m == 1 && !in_place && !(min32 && pre.kind != CQ_PRE_NONE) &&
+        !(flags & (CQ_FLAG_REUSE_ACT | CQ_FLAG_FORCE_GEMM | CQ_FLAG_STAGED_ACT | CQ_FLAG_ACT_Q8_1)) &&
         cq_matvec_fused_supported(w)) {
         CQ_HIP_CHECK(cq_launch_matvec_fused(w, x_dev, pre, y_dev, s));
         return CQ_OK;
@@ -552,7 +562,7 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
                             (long long)w->k);
     // two to four rows of short enough weight rows: the one-launch kernel again, every unpacked weight unit
     // contracted with each activation row
-    if (flags == 0 && pre.kind == CQ_PRE_NONE && !in_place && !min32 && cq_matvec_fused_rows_supported(w, m)) {
+    if (flags == 0 && pre.kind == CQ_PRE_NONE && !in_place && cq_matvec_fused_rows_supported(w, m)) {
         CQ_HIP_CHECK(cq_launch_matvec_fused_rows(w, x_dev, m, y_dev, s));
         return CQ_OK;
     }
@@ -622,6 +632,9 @@ extern "C" int cq_qmatmul_multi(const cq_weight *const *ws, int count, int pre, 
     // one activation row (or up to four of short weight rows), two or three weights: one launch over all their rows
     if (m >= 1 && m <= 4 && flags == 0 && !cq_has_min32(ws[0]->ggml_dtype) && !cq_has_min16(ws[0]->ggml_dtype) &&
         cq_matvec_fused_multi_supported(ws, count, pre, m)) {
+        for (int i = 0; i < count; i++)
+            if (ws[i]->n > 0)
+                if (int rc = check_vec_dot_rows(ws[i])) return rc;
         if (!x_dev) return cq_set_error(CQ_ERR_INVALID, "null argument");
         if ((uintptr_t)x_dev & 15) return cq_set_error(CQ_ERR_INVALID, "x must be 16-byte aligned");
         for (int i = 0; i < count; i++)

@@ -534,6 +534,99 @@ __device__ __forceinline__ float unit_value(const uint8_t *smem, const UnitW<DT>
     return ((float)I * w.dw) * ad;
 }
 
+// ---- offset terms of the types held in another type's planes ------------------------------------
+// Q4_1 / Q5_1 (Q8_0 planes plus the plane p2 of block minima) add sum_b m_b * s8_b, Q2K (Q6K planes plus p4, p5)
+// subtracts sum_b (d8_b * dmin_b) * sum_j bsums_j * m_j: the sums of the kernels in min_term.hip, formed from the
+// quantized row in LDS with the same operations in the same order (chunk and block sums per lane, added lane after
+// lane), so that the one-launch decode gives the bits of the launches that go through the workspace.  Called by whole
+// waves; `lr` = the weight row.  Returns the value to add to the row's result.
+// The weight side of the first pass (512 blocks of 32 / 64 blocks of 256) of a row's offset term, requested ahead.
+template <int DT> struct OffsetRow {
+    uint4 mw;        // Q4_1 / Q5_1: the lane's eight block minima (f16); Q2K: the sixteen group minima of the lane's block
+    uint16_t dmin;   // Q2K: the block's dmin
+};
+template <int DT> __device__ __forceinline__ void offset_load(const cq_weight &ws, int64_t lr, int64_t sb, OffsetRow<DT> &o) {
+    const int lane = threadIdx.x & 63;
+    if constexpr (DT == CQ_DTYPE_Q8_0) {
+        const int64_t nb = ws.k / 32;
+        const uint16_t *mins = (const uint16_t *)ws.p2 + lr * nb;
+        const int64_t b = sb + lane * 8;
+        if ((nb & 7) == 0) {   // whole groups of eight: one 16-byte load (lanes past the row re-read its last group)
+            o.mw = *(const uint4 *)(mins + (b < nb ? b : nb - 8));
+        } else {
+            uint32_t h[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) h[i] = mins[b + i < nb ? b + i : nb - 1];
+            o.mw = make_uint4(h[0] | h[1] << 16, h[2] | h[3] << 16, h[4] | h[5] << 16, h[6] | h[7] << 16);
+        }
+    } else {
+        const int64_t kb = ws.k / 256;
+        const int64_t b = sb + lane < kb ? sb + lane : kb - 1;
+        o.mw = *(const uint4 *)(ws.p4 + (lr * kb + b) * 16);
+        o.dmin = ((const uint16_t *)ws.p5)[lr * kb + b];
+    }
+}
+// `first` = the first pass of a Q4_1 / Q5_1 row as loaded by offset_load; later passes (longer rows) and Q2K rows load as they go.
+template <int DT>
+__device__ __forceinline__ float offset_term(const uint8_t *smem, const LdsRow r, const cq_weight &ws, int64_t lr,
+                                             const OffsetRow<DT> &first) {
+    const int lane = threadIdx.x & 63;
+    float acc = 0.0f;
+    if constexpr (DT == CQ_DTYPE_Q8_0) {
+        const int64_t nb = ws.k / 32;
+        for (int64_t sb = 0; sb < nb; sb += 64 * 8) {
+            OffsetRow<DT> o = first;
+            if (sb > 0) offset_load<DT>(ws, lr, sb, o);
+            const int64_t b = sb + lane * 8;
+            const uint32_t mh[4] = {o.mw.x, o.mw.y, o.mw.z, o.mw.w};
+            int32_t bs[8];
+            float d[8];
+            if ((nb & 7) == 0) {
+                const int64_t bc = b < nb ? b : nb - 8;
+                const int4 s0 = lds_get<int4>(smem, r.bs + 4 * (uint32_t)bc), s1 = lds_get<int4>(smem, r.bs + 4 * (uint32_t)bc + 16);
+                const float4 d0 = lds_get<float4>(smem, r.d + 4 * (uint32_t)bc), d1 = lds_get<float4>(smem, r.d + 4 * (uint32_t)bc + 16);
+                bs[0] = s0.x; bs[1] = s0.y; bs[2] = s0.z; bs[3] = s0.w; bs[4] = s1.x; bs[5] = s1.y; bs[6] = s1.z; bs[7] = s1.w;
+                d[0] = d0.x; d[1] = d0.y; d[2] = d0.z; d[3] = d0.w; d[4] = d1.x; d[5] = d1.y; d[6] = d1.z; d[7] = d1.w;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const int64_t bc = b + i < nb ? b + i : nb - 1;
+                    bs[i] = lds_get<int32_t>(smem, r.bs + 4 * (uint32_t)bc);
+                    d[i] = lds_get<float>(smem, r.d + 4 * (uint32_t)bc);
+                }
+            }
+            float t = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float hs = cq_h2f(cq_f2h((float)bs[i]));
+                const float sv = cq_h2f(cq_f2h(hs * d[i]));
+                const float p = cq_h2f((uint16_t)(mh[i >> 1] >> (16 * (i & 1)))) * sv;
+                t += b + i < nb ? p : 0.0f;
+            }
+            for (int jj = 0; jj < 64 && sb + jj * 8 < nb; jj++) acc += readlane_f(t, jj);
+        }
+        return acc;
+    } else {
+        const int64_t kb = ws.k / 256;
+        for (int64_t sb = 0; sb < kb; sb += 64) {
+            OffsetRow<DT> o;
+            offset_load<DT>(ws, lr, sb, o);
+            const int64_t b = sb + lane;
+            float term = 0.0f;
+            if (b < kb) {
+                const uint32_t w4[4] = {o.mw.x, o.mw.y, o.mw.z, o.mw.w};
+                int summs = 0;
+#pragma unroll
+                for (int g = 0; g < 16; g++)
+                    summs += (int)lds_get<int16_t>(smem, r.bs + 32 * (uint32_t)b + 2 * g) * (int)((w4[g >> 2] >> (8 * (g & 3))) & 0xff);
+                term = (lds_get<float>(smem, r.d + 4 * (uint32_t)b) * cq_h2f(o.dmin)) * (float)summs;
+            }
+            for (int jj = 0; jj < 64 && sb + jj < kb; jj++) acc += readlane_f(term, jj);
+        }
+        return -acc;
+    }
+}
+
 // --------------------------------------------------------------------- fused kernel (m = 1) ----
 // Loads of one weight row for this lane: units lane, lane + 64, ...  Lanes past the end of the row
 // re-read its last unit (same cache line as a neighbour, no extra traffic) and are masked when
@@ -652,11 +745,21 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
         }
         return row - first;
     };
-    auto load_launch_row = [&](int64_t row, UnitRaw<DT> (&buf)[UPL]) {
+    // Q4_1 / Q5_1 / Q2K weights (a wave-uniform property of the launch): the minima of a row travel with the row's
+    // units, requested when they are and summed when the row's result is stored.
+    constexpr bool kOffsets = PRE == CQ_PRE_NONE && NWT == 1 && (DT == CQ_DTYPE_Q8_0 || DT == CQ_DTYPE_Q6K);
+    bool offsets = false;
+    if constexpr (kOffsets) offsets = w.ggml_dtype != w.dtype && (cq_has_min32(w.ggml_dtype) || cq_has_min16(w.ggml_dtype));
+    auto load_launch_row = [&](int64_t row, UnitRaw<DT> (&buf)[UPL], OffsetRow<DT> &o) {
         cq_weight ws;
         float *ys;
         const int64_t lr = pick(row, ws, ys);
         load_row<DT, UPL>(ws, lr, units, buf);
+        // (Q2K's minima are loaded where they are summed: carrying them costs the Q6K kernel more registers than
+        // the wait costs time)
+        if constexpr (kOffsets && DT == CQ_DTYPE_Q8_0) {
+            if (offsets) offset_load<DT>(ws, lr, 0, o);
+        }
     };
     // rows of this wave (>= DEPTH): n / T, plus one for the first n % T waves (both from the host)
     const int64_t cnt = rows_per_wave + (row0 < rows_extra ? 1 : 0);
@@ -686,8 +789,9 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     UnitRaw<DT> a[UPL], b[DEPTH == 2 ? UPL : 1];
-    load_launch_row(row0, a);
-    if constexpr (DEPTH == 2) load_launch_row(row0 + T, b);
+    OffsetRow<DT> oa = {}, ob = {};
+    load_launch_row(row0, a, oa);
+    if constexpr (DEPTH == 2) load_launch_row(row0 + T, b, ob);
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     const LdsRow r = lds_row<DT>(w.k, 0);
@@ -767,7 +871,7 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
     __syncthreads();
     float yscale = 1.0f;
     if constexpr (kRms && kPairs) yscale = row_scale();
-    auto put = [&](int64_t row, Sums<MB> v) {
+    auto put = [&](int64_t row, Sums<MB> v, const OffsetRow<DT> &o) {
         cq_weight ws;
         float *ys;
         const int64_t lr = pick(row, ws, ys);
@@ -775,6 +879,9 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
         for (int m = 0; m < MB; m++) {
             float t = v.v[m];
             if constexpr (kRms && kPairs) t *= yscale;
+            if constexpr (kOffsets) {
+                if (offsets) t += offset_term<DT>(smem, rm[m], ws, lr, o);   // the f32 addition the workspace path's second launch makes
+            }
             if (lane == 0) ys[m * ws.n + lr] = t;
         }
     };
@@ -782,8 +889,9 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
     if constexpr (DEPTH == 1) {
         for (int64_t i = 0; i < cnt; i++) {
             const Sums<MB> s = row_dot_rows<DT, UPL, MB>(smem, rm, units, a);
-            if (i + 1 < cnt) load_launch_row(row0 + (i + 1) * T, a);
-            put(row0 + i * T, s);
+            const OffsetRow<DT> o = oa;
+            if (i + 1 < cnt) load_launch_row(row0 + (i + 1) * T, a, oa);
+            put(row0 + i * T, s, o);
         }
     } else {
         int64_t i = 0;
@@ -792,26 +900,27 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
             // the refill of a buffer is issued before the arithmetic on its old contents (which move
             // to other registers), so a wave keeps up to three rows in flight
             Sums<MB> s0, s1;
+            const OffsetRow<DT> o0 = oa, o1 = ob;
             if constexpr (UPL <= 2) {
                 UnitRaw<DT> ta[UPL], tb[UPL];
 #pragma unroll
                 for (int c = 0; c < UPL; c++) ta[c] = a[c];
-                load_launch_row(row0 + (i + 2) * T, a);
+                load_launch_row(row0 + (i + 2) * T, a, oa);
                 __builtin_amdgcn_sched_barrier(0);
                 s0 = row_dot_rows<DT, UPL, MB>(smem, rm, units, ta);
 #pragma unroll
                 for (int c = 0; c < UPL; c++) tb[c] = b[c];
-                load_launch_row(row0 + (i + 3) * T, b);
+                load_launch_row(row0 + (i + 3) * T, b, ob);
                 __builtin_amdgcn_sched_barrier(0);
                 s1 = row_dot_rows<DT, UPL, MB>(smem, rm, units, tb);
             } else {
                 s0 = row_dot_rows<DT, UPL, MB>(smem, rm, units, a);
-                load_launch_row(row0 + (i + 2) * T, a);
+                load_launch_row(row0 + (i + 2) * T, a, oa);
                 s1 = row_dot_rows<DT, UPL, MB>(smem, rm, units, b);
-                load_launch_row(row0 + (i + 3) * T, b);
+                load_launch_row(row0 + (i + 3) * T, b, ob);
             }
-            put(row0 + i * T, s0);
-            put(row0 + (i + 1) * T, s1);
+            put(row0 + i * T, s0, o0);
+            put(row0 + (i + 1) * T, s1, o1);
         }
         // tail: two or three rows left (a = row i, b = row i+1, maybe row i+2 still to load)
         const bool third = i + 2 < cnt;
@@ -820,16 +929,17 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
             // wave reductions) interleave
             const Sums<MB> s0 = row_dot_rows<DT, UPL, MB>(smem, rm, units, a);
             const Sums<MB> s1 = row_dot_rows<DT, UPL, MB>(smem, rm, units, b);
-            put(row0 + i * T, s0);
-            put(row0 + (i + 1) * T, s1);
+            put(row0 + i * T, s0, oa);
+            put(row0 + (i + 1) * T, s1, ob);
         } else {
             const Sums<MB> s0 = row_dot_rows<DT, UPL, MB>(smem, rm, units, a);
-            load_launch_row(row0 + (i + 2) * T, a);
+            const OffsetRow<DT> o0 = oa;
+            load_launch_row(row0 + (i + 2) * T, a, oa);
             const Sums<MB> s1 = row_dot_rows<DT, UPL, MB>(smem, rm, units, b);
-            put(row0 + i * T, s0);
-            put(row0 + (i + 1) * T, s1);
+            put(row0 + i * T, s0, o0);
+            put(row0 + (i + 1) * T, s1, ob);
             const Sums<MB> s2 = row_dot_rows<DT, UPL, MB>(smem, rm, units, a);
-            put(row0 + (i + 2) * T, s2);
+            put(row0 + (i + 2) * T, s2, oa);
         }
     }
 }

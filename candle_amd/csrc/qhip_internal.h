@@ -97,11 +97,11 @@ hipError_t cq_launch_unpack(const cq_weight *w, uint8_t *aos_dev, hipStream_t s)
 // Types held in another type's planes (same values, same arithmetic): Q5_0 as Q8_0, Q3K as Q6K.
 // Q4_1 and Q5_1 (value d * q + m) are Q8_0 planes with qs = q plus the plane p2 of the blocks' minima m (f16): the
 // holding type's kernels give the sum_i * d * d8 part of their dot product, cq_launch_min32_term adds sum_b m_b * s8_b.
-inline bool cq_has_min32(int ggml_dtype) { return ggml_dtype == CQ_DTYPE_Q4_1 || ggml_dtype == CQ_DTYPE_Q5_1; }
+__host__ __device__ inline bool cq_has_min32(int ggml_dtype) { return ggml_dtype == CQ_DTYPE_Q4_1 || ggml_dtype == CQ_DTYPE_Q5_1; }
 // Q2K (value d * sc_j * q - dmin * m_j, sixteen groups of sixteen) is a Q6K block with scales sc_j and six-bit quants
 // q + 32, plus the planes p4 / p5 of the groups' minima and dmin: the Q6K kernels give sum_b d * d8 * I_b of its dot
 // product with Q8K activations, cq_launch_min16_term subtracts sum_b dmin * d8 * sum_j bsums_j * m_j.
-inline bool cq_has_min16(int ggml_dtype) { return ggml_dtype == CQ_DTYPE_Q2K; }
+__host__ __device__ inline bool cq_has_min16(int ggml_dtype) { return ggml_dtype == CQ_DTYPE_Q2K; }
 inline int cq_storage_dtype(int ggml_dtype) {
     if (ggml_dtype == CQ_DTYPE_Q5_0 || cq_has_min32(ggml_dtype)) return CQ_DTYPE_Q8_0;
     return ggml_dtype == CQ_DTYPE_Q3K || ggml_dtype == CQ_DTYPE_Q2K ? CQ_DTYPE_Q6K : ggml_dtype;

@@ -37,13 +37,14 @@ extern "C" {
 enum {
     CQ_DTYPE_Q4_0 = 2,
     CQ_DTYPE_Q4_1 = 3,  /* held as Q8_0 planes (qs = q) plus a plane of block minima; the m * s term of the dot
-                           product with Q8_1 activations (k_quants.rs:267-294) is added by a second small launch      */
+                           product with Q8_1 activations (k_quants.rs:267-294) is added by the one-launch decode kernels
+                           themselves, by a second small launch otherwise                                           */
     CQ_DTYPE_Q5_0 = 6,  /* held on the device as Q8_0 planes (qs = q - 16): the same values, the same arithmetic     */
     CQ_DTYPE_Q5_1 = 7,  /* like Q4_1, with five-bit quants                                                            */
     CQ_DTYPE_Q8_0 = 8,
     CQ_DTYPE_Q8_1 = 9,  /* activation format only */
     CQ_DTYPE_Q2K = 10,  /* held as Q6K planes (scale, quant + 32) plus the groups' minima and dmin; the dmin term of the
-                           dot product (k_quants.rs:717-767) is subtracted by a second small launch                   */
+                           dot product (k_quants.rs:717-767) is subtracted the same way                                */
     CQ_DTYPE_Q3K = 11,  /* held on the device as Q6K planes (scale - 32, quant + 28): the same values and arithmetic */
     CQ_DTYPE_Q4K = 12,
     CQ_DTYPE_Q5K = 13,
@@ -157,7 +158,10 @@ int cq_quantize_act(int dev, int act_dtype, const float *x_dev, int64_t m, int64
 size_t cq_workspace_bytes(const cq_weight *w, int64_t m, int flags);
 /* QCudaStorage::fwd (cuda.rs:478-499) = <QTensor as CustomOp1>::cuda_fwd (mod.rs:514-524):
  * y[m, n] = x[m, k] . W[n, k]^T with x quantized to W's VecDotType first (k_quants.rs:1842-1883).
- * x contiguous f32; m = product of the leading dims of the input tensor. */
+ * x contiguous f32; m = product of the leading dims of the input tensor.
+ * Q4_1, Q5_0 and Q5_1 weights with an odd number of 32-element blocks per row are refused with
+ * CQ_ERR_INVALID, as their vec_dot refuses them (k_quants.rs:273, 363, 469); so do the other matmul
+ * entry points. */
 int cq_qmatmul(const cq_weight *w, const float *x_dev, int64_t m, float *y_dev, int flags,
                void *workspace_dev, size_t workspace_bytes, void *stream);
 /* The same with the weight's shape given at the call, exactly as QCudaStorage::fwd(&self, self_shape, ..)

@@ -1429,7 +1429,10 @@ int orc_vec_dot(int dtype, int64_t n, const void *xs, const void *ys, float *out
     switch (dtype) {
     case ORC_Q4_0: *out = vec_dot_q4_0_q8_0(n, xs, ys); return 0;
     case ORC_Q4_1: return vec_dot_q4_1_q8_1(n, xs, ys, out);
-    case ORC_Q5_0: *out = vec_dot_q5_0_q8_0(n, xs, ys); return 0;
+    case ORC_Q5_0:
+        if ((n / 32) % 2 != 0) return -1;   /* k_quants.rs:363: nb is not divisible by 2 */
+        *out = vec_dot_q5_0_q8_0(n, xs, ys);
+        return 0;
     case ORC_Q5_1: return vec_dot_q5_1_q8_1(n, xs, ys, out);
     case ORC_Q2K: *out = vec_dot_q2k_q8k(n, xs, ys); return 0;
     case ORC_Q3K: *out = vec_dot_q3k_q8k(n, xs, ys); return 0;
@@ -1461,7 +1464,8 @@ int orc_matmul(int dtype, int64_t m, int64_t k, int64_t n, const float *lhs, con
     for (int64_t r = 0; r < m; r++) {
         for (int64_t c = 0; c < n; c++) {
             float v;
-            orc_vec_dot(dtype, k, (const uint8_t *)rhs_t + c * w_row_bytes, lhs_b + r * a_row_bytes, &v);
+            int rc = orc_vec_dot(dtype, k, (const uint8_t *)rhs_t + c * w_row_bytes, lhs_b + r * a_row_bytes, &v);
+            if (rc) { free(lhs_b); return rc; }   /* vec_dot's Err ends the matmul (k_quants.rs:1876-1880) */
             dst[r * n + c] = v;
         }
     }

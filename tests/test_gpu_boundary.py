@@ -80,6 +80,35 @@ def test_shape_at_call_equals_shape_at_creation(qh, dt, m):
     assert np.array_equal(flat.dequantize().cpu().numpy().ravel(), orc.dequantize(dt, blocks))
 
 
+@pytest.mark.parametrize("dt", [orc.Q4_1, orc.Q5_0, orc.Q5_1])
+@pytest.mark.parametrize("m", [1, 3, 40])
+def test_odd_block_counts_are_refused_like_the_reference(qh, dt, m):
+    """vec_dot of Q4_1, Q5_0 and Q5_1 bails out on rows with an odd number of blocks (k_quants.rs:273, 363, 469), and
+    with it the matmul; weights of such shapes can still be created, read back and dequantized.  Q4_0 and Q8_0 have
+    no such rule."""
+    rng = np.random.default_rng(7 * int(dt) + m)
+    n, k = 16, 96
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    blocks = orc.quantize(dt, w)
+    q = qh.QWeight.from_ggml(dt, blocks, n, k)
+    assert np.array_equal(q.to_ggml(), blocks)
+    assert np.array_equal(q.dequantize().cpu().numpy(), orc.dequantize(dt, blocks).reshape(n, k))
+    with pytest.raises(ValueError):
+        orc.matmul(dt, x, blocks, n)
+    for flags in (0, qh.FLAG_STAGED_ACT, qh.FLAG_FORCE_MATVEC):
+        with pytest.raises(qh.QHipError, match="nb is not divisible by 2"):
+            qh.qmatmul(q, dev(x), flags)
+    with pytest.raises(qh.QHipError, match="nb is not divisible by 2"):
+        qh.qmatmul_multi([q, q], dev(x))
+    assert qh.qmatmul(q, dev(x[:0])).shape == (0, n)          # no rows: no vec_dot, no error
+    for ok in (orc.Q4_0, orc.Q8_0):
+        b = orc.quantize(ok, w)
+        got = qh.qmatmul(qh.QWeight.from_ggml(ok, b, n, k), dev(x)).cpu().numpy()
+        ref = orc.matmul(ok, x, b, n)
+        assert np.linalg.norm(got - ref) <= 1e-4 * np.linalg.norm(ref)
+
+
 @pytest.mark.parametrize("dt", [orc.Q4_1, orc.Q5_0, orc.Q5_1, orc.Q2K, orc.Q3K])
 def test_types_held_in_another_types_planes(qh, dt):
     """Q5_0 lives in Q8_0 planes, Q3K in Q6K planes, Q4_1 and Q5_1 in Q8_0 planes plus a plane of minima: the caller sees the type it created (dtype, GGML byte size,

@@ -49,7 +49,7 @@ def make_inputs(seed, m, k, n, wscale=0.02, outliers=False):
 
 
 # Q5_0 and Q3K are held on the device in the planes of Q8_0 and Q6K (same values, same arithmetic), Q4_1 and Q5_1 in
-# Q8_0 planes plus a plane of minima whose term a second launch adds (Q2K likewise in Q6K planes): every test below takes them through the boundary
+# Q8_0 planes plus a plane of minima whose term the one-launch kernels add themselves and a second launch adds elsewhere (Q2K likewise in Q6K planes): every test below takes them through the boundary
 # like the others and compares with the oracle's own code for the type
 WEIGHT_DTYPES = [orc.Q4_0, orc.Q4_1, orc.Q5_0, orc.Q5_1, orc.Q8_0, orc.Q2K, orc.Q3K, orc.Q4K, orc.Q5K, orc.Q6K]
 
@@ -730,12 +730,35 @@ def test_few_rows_one_launch_equals_single_rows(qh, dt, m, k, n):
     elems = {orc.Q4_0: 32, orc.Q4_1: 16, orc.Q5_0: 16, orc.Q5_1: 16, orc.Q8_0: 16, orc.Q2K: 32, orc.Q3K: 32, orc.Q4K: 64, orc.Q5K: 64, orc.Q6K: 32}[dt]   # weights per 16-byte lane unit
     units = k // elems
     per_lane = -(-units // 64) * elems
-    one_launch = dt not in (orc.Q4_1, orc.Q5_1, orc.Q2K)   # their offset term is a second launch over the workspace
-    if one_launch and units <= (384 if m == 2 else 256) and (per_lane <= 64 or (per_lane <= 128 and m <= 3) or m <= 2):   # the library's rule
+    if units <= (384 if m == 2 else 256) and (per_lane <= 64 or (per_lane <= 128 and m <= 3) or m <= 2):   # the library's rule
         for r in range(m):
             assert torch.equal(got[r:r + 1], qh.qmatmul(qw, xd[r:r + 1].contiguous())), r
     two = qh.qmatmul(qw, xd, qh.FLAG_STAGED_ACT)
     assert (torch.linalg.norm(got - two) / torch.linalg.norm(two)).item() <= 2e-6
+    check_f32(got.cpu().numpy(), orc.matmul(dt, x, blocks, n))
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4])
+@pytest.mark.parametrize("dt,k,n", [(dt, k, n) for dt in (orc.Q4_1, orc.Q5_1, orc.Q2K)
+                                    for k, n in [(256, 8), (512, 40), (2048, 64), (4096, 300), (11008, 24), (14336, 16),
+                                                 (64, 16), (192, 33), (1088, 64), (4160, 48)]
+                                    if dt != orc.Q2K or k % 256 == 0])
+def test_offset_types_one_launch_equals_workspace_path(qh, dt, m, k, n):
+    """Q4_1 / Q5_1 / Q2K: the one-launch kernels add the offset term (block minima times the activation blocks' scaled
+    sums) themselves; the other paths add it in a second launch over the quantized rows in the workspace.  Same
+    operations in the same order: equal bits at one row.  Row lengths with whole and partial groups of eight 32-element blocks,
+    one and several passes of 64 lanes over the blocks (an even number of blocks: the reference takes no other)."""
+    w, x = make_inputs(23 * dt + m + k + n, m, k, n, outliers=True)
+    w = w + 0.5 * np.abs(w).mean()          # offsets that matter
+    blocks = orc.quantize(dt, w)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    xd = dev(x)
+    got = qh.qmatmul(qw, xd)
+    two = qh.qmatmul(qw, xd, qh.FLAG_STAGED_ACT)
+    if m == 1:
+        assert torch.equal(got, two)
+    else:   # several rows: the kernels behind the workspace add up the main term in another order
+        assert (torch.linalg.norm(got - two) / torch.linalg.norm(two)).item() <= 2e-6
     check_f32(got.cpu().numpy(), orc.matmul(dt, x, blocks, n))
 
 
@@ -745,7 +768,7 @@ def _random_cases(count, seed):
     cases = []
     for _ in range(count):
         dt = int(rng.choice(WEIGHT_DTYPES))
-        blk = 32 if dt in (orc.Q4_0, orc.Q8_0) else 256
+        blk = 32 if dt in (orc.Q4_0, orc.Q4_1, orc.Q5_0, orc.Q5_1, orc.Q8_0) else 256
         k = blk * int(rng.integers(1, (2048 // blk) + 1))
         m = int(rng.choice([1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 31, 32, 33, 40, 64, 65, 70]))
         n = int(rng.choice([1, 2, 7, 8, 15, 16, 17, 31, 32, 33, 48, 63, 64, 96, 100, 128, 255, 256, 257, 300]))
@@ -760,4 +783,11 @@ def test_random_shapes_match_oracle(qh, dt, m, k, n):
     w, x = make_inputs(dt * 1000003 + m * 10007 + k * 101 + n, m, k, n, outliers=True)
     blocks = orc.quantize(dt, w)
     qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    if dt in (orc.Q4_1, orc.Q5_0, orc.Q5_1) and (k // 32) % 2:
+        # the reference's vec_dot of these types refuses an odd number of blocks (k_quants.rs:273, 363, 469)
+        with pytest.raises(ValueError):
+            orc.matmul(dt, x, blocks, n)
+        with pytest.raises(qh.QHipError, match="not divisible by 2"):
+            qh.qmatmul(qw, dev(x))
+        return
     check_f32(qh.qmatmul(qw, dev(x)).cpu().numpy(), orc.matmul(dt, x, blocks, n))
