@@ -717,7 +717,7 @@ template <> struct FusedMore<1> {};
 // `more` names the planes, outputs and row ranges of the weights behind the first.
 // MB > 1 (with PRE none and one weight): MB activation rows x[MB][k], outputs y[MB][n]; every weight row is
 // unpacked once and contracted with each of them.
-template <int DT, int UPL, int NW, int DEPTH, int PRE, int NWT = 1, int MB = 1>
+template <int DT, int UPL, int NW, int DEPTH, int PRE, int NWT = 1, int MB = 1, bool OFFSETS = false>
 __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float *x, cq_pre pre,
                                                         float *__restrict__ y, int64_t total_waves,
                                                         int64_t rows_per_wave, int64_t rows_extra, FusedMore<NWT> more) {
@@ -745,11 +745,12 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
         }
         return row - first;
     };
-    // Q4_1 / Q5_1 / Q2K weights (a wave-uniform property of the launch): the minima of a row travel with the row's
-    // units, requested when they are and summed when the row's result is stored.
-    constexpr bool kOffsets = PRE == CQ_PRE_NONE && NWT == 1 && (DT == CQ_DTYPE_Q8_0 || DT == CQ_DTYPE_Q6K);
-    bool offsets = false;
-    if constexpr (kOffsets) offsets = w.ggml_dtype != w.dtype && (cq_has_min32(w.ggml_dtype) || cq_has_min16(w.ggml_dtype));
+    // OFFSETS: Q4_1 / Q5_1 / Q2K weights (instances of their own, so that the kernels of the plain Q8_0 and Q6K
+    // weights carry nothing for them): the minima of a row travel with the row's units, requested when they are and
+    // summed when the row's result is stored.
+    static_assert(!OFFSETS || (PRE == CQ_PRE_NONE && NWT == 1 && (DT == CQ_DTYPE_Q8_0 || DT == CQ_DTYPE_Q6K)), "offset terms: Q8_0 / Q6K planes, one weight, no fused step");
+    constexpr bool kOffsets = OFFSETS;
+    constexpr bool offsets = OFFSETS;
     auto load_launch_row = [&](int64_t row, UnitRaw<DT> (&buf)[UPL], OffsetRow<DT> &o) {
         cq_weight ws;
         float *ys;
@@ -1230,9 +1231,25 @@ hipError_t launch_fused_upl(const cq_weight *w, int64_t n, FusedMore<NWT> more, 
     int64_t wgs = n / (NW * depth);
     if (wgs > max_wgs) wgs = max_wgs;
     const int64_t tw = wgs * NW, rpw = n / tw, extra = n % tw;
+    // weights with an offset term (Q4_1 / Q5_1 in Q8_0 planes, Q2K in Q6K planes) take the instances that add it
+    constexpr bool kCanOffset = PRE == CQ_PRE_NONE && NWT == 1 && (DT == CQ_DTYPE_Q8_0 || DT == CQ_DTYPE_Q6K);
+    const bool offsets = w->ggml_dtype != w->dtype && (cq_has_min32(w->ggml_dtype) || cq_has_min16(w->ggml_dtype));
+    if (offsets && !kCanOffset) return hipErrorInvalidValue;
     if constexpr (UPL <= 2) {   // (longer rows never run two deep: no instance of that)
         if (depth == 2) {
+            if constexpr (kCanOffset) {
+                if (offsets) {
+                    CQ_LAUNCH((fused_kernel<DT, UPL, NW, 2, PRE, NWT, MB, true>), (unsigned)wgs, NW * 64, lds, s, *w, x, pre, y, tw, rpw, extra, more);
+                    return hipGetLastError();
+                }
+            }
             CQ_LAUNCH((fused_kernel<DT, UPL, NW, 2, PRE, NWT, MB>), (unsigned)wgs, NW * 64, lds, s, *w, x, pre, y, tw, rpw, extra, more);
+            return hipGetLastError();
+        }
+    }
+    if constexpr (kCanOffset) {
+        if (offsets) {
+            CQ_LAUNCH((fused_kernel<DT, UPL, NW, 1, PRE, NWT, MB, true>), (unsigned)wgs, NW * 64, lds, s, *w, x, pre, y, tw, rpw, extra, more);
             return hipGetLastError();
         }
     }
