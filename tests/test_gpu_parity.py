@@ -791,3 +791,56 @@ def test_random_shapes_match_oracle(qh, dt, m, k, n):
             qh.qmatmul(qw, dev(x))
         return
     check_f32(qh.qmatmul(qw, dev(x)).cpu().numpy(), orc.matmul(dt, x, blocks, n))
+
+
+def _pattern_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(count):
+        dt = int(rng.choice(WEIGHT_DTYPES + [orc.Q8K]))
+        blk = 32 if dt in (orc.Q4_0, orc.Q4_1, orc.Q5_0, orc.Q5_1, orc.Q8_0) else 256
+        k = blk * (2 * int(rng.integers(1, 33)) if blk == 32 else int(rng.choice([1, 2, 3, 5, 8, 16, 43])))
+        m = int(rng.choice([1, 2, 3, 4, 5, 8, 9, 16, 17, 33, 64, 65, 129]))
+        n = int(rng.choice([1, 7, 8, 16, 31, 32, 33, 64, 100, 128, 257]))
+        cases.append((dt, m, k, n, i % 4))
+    return cases
+
+
+@pytest.mark.parametrize("dt,m,k,n,kind", _pattern_cases(64, 20250117))
+def test_input_patterns_match_oracle(qh, dt, m, k, n, kind):
+    """Inputs that exercise the quantizers' special cases rather than their typical ones, through whatever kernel the
+    automatic choice and the forced dot-product path land on: all-zero rows, blocks and weight rows and a row with a
+    single non-zero (scale 0 / one live quant); equal magnitudes with both signs (the first-index rules of the
+    maximum searches) and constant blocks; positive weights with large minima against a ramp; scales 0.01 - 100."""
+    rng = np.random.default_rng(dt * 7919 + m * 131 + k + n + kind)
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    if kind == 0:
+        x[rng.integers(0, m)] = 0
+        x[:, :min(k, 256)] = 0
+        r = rng.integers(0, m)
+        x[r] = 0
+        x[r, rng.integers(0, k)] = -3.0
+        w[rng.integers(0, n)] = 0
+    elif kind == 1:
+        x = np.where(rng.random((m, k)) < 0.5, -1.5, 1.5).astype(np.float32)
+        w = np.where(rng.random((n, k)) < 0.5, -0.25, 0.25).astype(np.float32) + np.float32(0.125 * (n % 2))
+    elif kind == 2:
+        w = np.abs(w) + np.float32(0.05)
+        x = ((np.arange(m * k, dtype=np.float32).reshape(m, k) % 97) - 48) / 16
+    else:
+        x *= np.float32(10.0 ** int(rng.integers(-2, 3)))
+        w *= np.float32(10.0 ** int(rng.integers(-2, 2)))
+    blocks = orc.quantize(dt, w)
+    ref = orc.matmul(dt, x, blocks, n)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    assert np.array_equal(qh.QWeight.zeros(dt, n, k).quantize_(dev(w)).to_ggml(), blocks)   # device quantizer: same bytes
+    ref64 = ref.astype(np.float64)
+    for flags in (0, qh.FLAG_FORCE_MATVEC):
+        got = qh.qmatmul(qw, dev(x), flags).cpu().numpy()
+        if n >= 32:
+            check_f32(got, ref)
+        else:   # a handful of outputs per row, some of them sums that nearly cancel: the bar over the whole result
+            assert np.isfinite(got).all()
+            assert np.linalg.norm(got - ref64) <= REL_L2_TOL * np.linalg.norm(ref64)
+        assert not got[~x.any(axis=1)].any()          # a row of zeros gives zeros, offsets or not
