@@ -540,89 +540,50 @@ __device__ __forceinline__ float unit_value(const uint8_t *smem, const UnitW<DT>
 // quantized row in LDS with the same operations in the same order (chunk and block sums per lane, added lane after
 // lane), so that the one-launch decode gives the bits of the launches that go through the workspace.  Called by whole
 // waves; `lr` = the weight row.  Returns the value to add to the row's result.
-// The weight side of the first pass (512 blocks of 32 / 64 blocks of 256) of a row's offset term, requested ahead.
+// The rows of the one-launch kernels have at most 16 384 elements: one lane per group of eight 32-element blocks
+// (Q4_1 / Q5_1, whole groups only) or per 256-element block (Q2K) covers a row, so the weight side of a row's term
+// is one unconditional request per lane, made together with the row's units (a request behind a branch or in a loop
+// would make the compiler wait for everything in flight, the next row's units included).
 template <int DT> struct OffsetRow {
     uint4 mw;        // Q4_1 / Q5_1: the lane's eight block minima (f16); Q2K: the sixteen group minima of the lane's block
     uint16_t dmin;   // Q2K: the block's dmin
 };
-template <int DT> __device__ __forceinline__ void offset_load(const cq_weight &ws, int64_t lr, int64_t sb, OffsetRow<DT> &o) {
-    const int lane = threadIdx.x & 63;
+template <int DT> __device__ __forceinline__ void offset_load(const cq_weight &ws, int64_t lr, OffsetRow<DT> &o) {
+    const uint32_t lane = threadIdx.x & 63;
     if constexpr (DT == CQ_DTYPE_Q8_0) {
-        const int64_t nb = ws.k / 32;
-        const uint16_t *mins = (const uint16_t *)ws.p2 + lr * nb;
-        const int64_t b = sb + lane * 8;
-        if ((nb & 7) == 0) {   // whole groups of eight: one 16-byte load (lanes past the row re-read its last group)
-            o.mw = *(const uint4 *)(mins + (b < nb ? b : nb - 8));
-        } else {
-            uint32_t h[8];
-#pragma unroll
-            for (int i = 0; i < 8; i++) h[i] = mins[b + i < nb ? b + i : nb - 1];
-            o.mw = make_uint4(h[0] | h[1] << 16, h[2] | h[3] << 16, h[4] | h[5] << 16, h[6] | h[7] << 16);
-        }
+        const uint32_t nb = (uint32_t)(ws.k / 32), b = lane * 8;   // lanes past the row re-read its last group
+        o.mw = *(const uint4 *)((const uint16_t *)ws.p2 + lr * nb + (b < nb ? b : nb - 8));
     } else {
-        const int64_t kb = ws.k / 256;
-        const int64_t b = sb + lane < kb ? sb + lane : kb - 1;
+        const uint32_t kb = (uint32_t)(ws.k / 256), b = lane < kb ? lane : kb - 1;
         o.mw = *(const uint4 *)(ws.p4 + (lr * kb + b) * 16);
         o.dmin = ((const uint16_t *)ws.p5)[lr * kb + b];
     }
 }
-// `first` = the first pass of a Q4_1 / Q5_1 row as loaded by offset_load; later passes (longer rows) and Q2K rows load as they go.
 template <int DT>
-__device__ __forceinline__ float offset_term(const uint8_t *smem, const LdsRow r, const cq_weight &ws, int64_t lr,
-                                             const OffsetRow<DT> &first) {
-    const int lane = threadIdx.x & 63;
+__device__ __forceinline__ float offset_term(const uint8_t *smem, const LdsRow r, const cq_weight &ws, const OffsetRow<DT> &o) {
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t mw[4] = {o.mw.x, o.mw.y, o.mw.z, o.mw.w};
     float acc = 0.0f;
     if constexpr (DT == CQ_DTYPE_Q8_0) {
-        const int64_t nb = ws.k / 32;
-        for (int64_t sb = 0; sb < nb; sb += 64 * 8) {
-            OffsetRow<DT> o = first;
-            if (sb > 0) offset_load<DT>(ws, lr, sb, o);
-            const int64_t b = sb + lane * 8;
-            const uint32_t mh[4] = {o.mw.x, o.mw.y, o.mw.z, o.mw.w};
-            int32_t bs[8];
-            float d[8];
-            if ((nb & 7) == 0) {
-                const int64_t bc = b < nb ? b : nb - 8;
-                const int4 s0 = lds_get<int4>(smem, r.bs + 4 * (uint32_t)bc), s1 = lds_get<int4>(smem, r.bs + 4 * (uint32_t)bc + 16);
-                const float4 d0 = lds_get<float4>(smem, r.d + 4 * (uint32_t)bc), d1 = lds_get<float4>(smem, r.d + 4 * (uint32_t)bc + 16);
-                bs[0] = s0.x; bs[1] = s0.y; bs[2] = s0.z; bs[3] = s0.w; bs[4] = s1.x; bs[5] = s1.y; bs[6] = s1.z; bs[7] = s1.w;
-                d[0] = d0.x; d[1] = d0.y; d[2] = d0.z; d[3] = d0.w; d[4] = d1.x; d[5] = d1.y; d[6] = d1.z; d[7] = d1.w;
-            } else {
+        const uint32_t nb = (uint32_t)(ws.k / 32), b = lane * 8, bc = b < nb ? b : nb - 8;
+        // the blocks' scaled sums, left in place of the integer sums by the kernel's prologue
+        const float4 s0 = lds_get<float4>(smem, r.bs + 4 * bc), s1 = lds_get<float4>(smem, r.bs + 4 * bc + 16);
+        const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+        float t = 0.0f;
 #pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    const int64_t bc = b + i < nb ? b + i : nb - 1;
-                    bs[i] = lds_get<int32_t>(smem, r.bs + 4 * (uint32_t)bc);
-                    d[i] = lds_get<float>(smem, r.d + 4 * (uint32_t)bc);
-                }
-            }
-            float t = 0.0f;
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const float hs = cq_h2f(cq_f2h((float)bs[i]));
-                const float sv = cq_h2f(cq_f2h(hs * d[i]));
-                const float p = cq_h2f((uint16_t)(mh[i >> 1] >> (16 * (i & 1)))) * sv;
-                t += b + i < nb ? p : 0.0f;
-            }
-            for (int jj = 0; jj < 64 && sb + jj * 8 < nb; jj++) acc += readlane_f(t, jj);
-        }
+        for (int i = 0; i < 8; i++) t += cq_h2f((uint16_t)(mw[i >> 1] >> (16 * (i & 1)))) * sv[i];
+        t = b < nb ? t : 0.0f;
+        for (uint32_t jj = 0; jj * 8 < nb; jj++) acc += readlane_f(t, jj);
         return acc;
     } else {
-        const int64_t kb = ws.k / 256;
-        for (int64_t sb = 0; sb < kb; sb += 64) {
-            OffsetRow<DT> o;
-            offset_load<DT>(ws, lr, sb, o);
-            const int64_t b = sb + lane;
-            float term = 0.0f;
-            if (b < kb) {
-                const uint32_t w4[4] = {o.mw.x, o.mw.y, o.mw.z, o.mw.w};
-                int summs = 0;
+        const uint32_t kb = (uint32_t)(ws.k / 256), b = lane < kb ? lane : kb - 1;
+        int summs = 0;
 #pragma unroll
-                for (int g = 0; g < 16; g++)
-                    summs += (int)lds_get<int16_t>(smem, r.bs + 32 * (uint32_t)b + 2 * g) * (int)((w4[g >> 2] >> (8 * (g & 3))) & 0xff);
-                term = (lds_get<float>(smem, r.d + 4 * (uint32_t)b) * cq_h2f(o.dmin)) * (float)summs;
-            }
-            for (int jj = 0; jj < 64 && sb + jj < kb; jj++) acc += readlane_f(term, jj);
-        }
+        for (int g = 0; g < 16; g++)
+            summs += (int)lds_get<int16_t>(smem, r.bs + 32 * b + 2 * g) * (int)((mw[g >> 2] >> (8 * (g & 3))) & 0xff);
+        float term = (lds_get<float>(smem, r.d + 4 * b) * cq_h2f(o.dmin)) * (float)summs;
+        term = lane < kb ? term : 0.0f;
+        for (uint32_t jj = 0; jj < kb; jj++) acc += readlane_f(term, jj);
         return -acc;
     }
 }
@@ -750,17 +711,12 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
     // summed when the row's result is stored.
     static_assert(!OFFSETS || (PRE == CQ_PRE_NONE && NWT == 1 && (DT == CQ_DTYPE_Q8_0 || DT == CQ_DTYPE_Q6K)), "offset terms: Q8_0 / Q6K planes, one weight, no fused step");
     constexpr bool kOffsets = OFFSETS;
-    constexpr bool offsets = OFFSETS;
     auto load_launch_row = [&](int64_t row, UnitRaw<DT> (&buf)[UPL], OffsetRow<DT> &o) {
         cq_weight ws;
         float *ys;
         const int64_t lr = pick(row, ws, ys);
         load_row<DT, UPL>(ws, lr, units, buf);
-        // (Q2K's minima are loaded where they are summed: carrying them costs the Q6K kernel more registers than
-        // the wait costs time)
-        if constexpr (kOffsets && DT == CQ_DTYPE_Q8_0) {
-            if (offsets) offset_load<DT>(ws, lr, 0, o);
-        }
+        if constexpr (kOffsets) offset_load<DT>(ws, lr, o);
     };
     // rows of this wave (>= DEPTH): n / T, plus one for the first n % T waves (both from the host)
     const int64_t cnt = rows_per_wave + (row0 < rows_extra ? 1 : 0);
@@ -870,6 +826,19 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
         else quantize_row_to_lds<DT, XCH, NW>(smem, w.k, wave, rm[m], fxa[m]);
     }
     __syncthreads();
+    if constexpr (OFFSETS && DT == CQ_DTYPE_Q8_0) {
+        // Q4_1 / Q5_1: the activation blocks' scaled sums s = f16(f16(sum) * d) of the Q8_1 format are the same for
+        // every weight row: computed once per workgroup, in place of the integer sums (which Q8_0 planes do not use)
+        const uint32_t nb = (uint32_t)(w.k / 32);
+#pragma unroll
+        for (int m = 0; m < MB; m++) {
+            for (uint32_t b = threadIdx.x; b < nb; b += NW * 64) {
+                const float hs = cq_h2f(cq_f2h((float)lds_get<int32_t>(smem, rm[m].bs + 4 * b)));
+                lds_put<float>(smem, rm[m].bs + 4 * b, cq_h2f(cq_f2h(hs * lds_get<float>(smem, rm[m].d + 4 * b))));
+            }
+        }
+        __syncthreads();
+    }
     float yscale = 1.0f;
     if constexpr (kRms && kPairs) yscale = row_scale();
     auto put = [&](int64_t row, Sums<MB> v, const OffsetRow<DT> &o) {
@@ -881,7 +850,7 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
             float t = v.v[m];
             if constexpr (kRms && kPairs) t *= yscale;
             if constexpr (kOffsets) {
-                if (offsets) t += offset_term<DT>(smem, rm[m], ws, lr, o);   // the f32 addition the workspace path's second launch makes
+                t += offset_term<DT>(smem, rm[m], ws, o);   // the f32 addition the workspace path's second launch makes
             }
             if (lane == 0) ys[m * ws.n + lr] = t;
         }
@@ -1522,6 +1491,8 @@ bool cq_matvec_row_fits(const cq_weight *w) {
 }
 
 bool cq_matvec_fused_supported(const cq_weight *w) {
+    // Q4_1 / Q5_1: the kernels that add the offset term take a row's minima in whole groups of eight blocks
+    if (cq_has_min32(w->ggml_dtype) && w->k % 256 != 0) return false;
     switch (w->dtype) {
     case CQ_DTYPE_Q4_0: return fused_ok<CQ_DTYPE_Q4_0>(w);
     case CQ_DTYPE_Q8_0: return fused_ok<CQ_DTYPE_Q8_0>(w);
