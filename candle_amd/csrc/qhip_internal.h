@@ -67,7 +67,8 @@ struct cq_act_view {
     int16_t *bsums;  // Q8K
     // Q8K, for the GEMM only (block-major so that a tile of rows is contiguous per block):
     float *dT;         // [k/256][m_stride] f32, the same values as d
-    uint16_t *minp;    // [k/256][m_stride][16] f16, d * sub-block sums as two f16 pieces p1[8] | p2[8]
+    uint16_t *minp;    // [k/256][m_stride][16] f16, d * sub-block sums as two f16 pieces p1[8] | p2[8] (the tile kernel's min term)
+    uint16_t *bsh;     // [k/256][m_stride][16] f16: the block's sixteen bsums as f16 (exact), the small-batch kernels' min term
     int64_t m_stride;  // rows allocated: at least 256 more than the rows quantized, so that the GEMM
                        // may read (and ignore) whole 128-row tiles past the last row
     int32_t *bsum32; // Q8_0 / Q8_1
@@ -328,6 +329,30 @@ __device__ __forceinline__ cq_u32x4 cq_min_term_operand(uint32_t dd, const uint3
         const cq_half2 p1 = ndmin * mn;
         const cq_half2 p2 = __builtin_elementwise_fma(ndmin, mn, -p1);
         out[g] = second ? __builtin_bit_cast(uint32_t, p2) : __builtin_bit_cast(uint32_t, p1);
+    }
+    return out;
+}
+
+// The same term with its range taken out of the operands (the Q8K matrix-core kernels): the activation side of the
+// contraction is the block's sixteen 16-element sums bsums_j as f16 (|bsums_j| <= 2048: exact, whatever the activations'
+// magnitude), the block scale d8 multiplies the result afterwards.  Weight side per group j: -dmin * min_{j/2} in two
+// f16 pieces as above.  `half` picks the groups 8*half .. 8*half+7 (sub-blocks 4*half .. 4*half+3, each value twice in a
+// row), `second` the piece.
+__device__ __forceinline__ cq_u32x4 cq_min_term_groups(uint32_t dd, const uint32_t (&rec)[4], bool half, bool second) {
+    const uint32_t nd = (dd >> 16) ^ 0x8000u;   // -dmin
+    const cq_half2 ndmin = __builtin_bit_cast(cq_half2, nd | (nd << 16));
+    const cq_half2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+    cq_u32x4 out;
+#pragma unroll
+    for (int g = 0; g < 2; g++) {
+        const uint32_t rg = half ? rec[2 + g] : rec[g];
+        const uint32_t n2 = __builtin_amdgcn_perm(rg, 0u, 0x0c070c06u) | 0x64006400u;   // the two min bytes as 1024 + n
+        const cq_half2 mn = __builtin_bit_cast(cq_half2, n2) - k1024;
+        const cq_half2 p1 = ndmin * mn;
+        const cq_half2 p2 = __builtin_elementwise_fma(ndmin, mn, -p1);
+        const uint32_t u = second ? __builtin_bit_cast(uint32_t, p2) : __builtin_bit_cast(uint32_t, p1);
+        out[2 * g] = __builtin_amdgcn_perm(u, u, 0x01000100u);       // sub-block 2g' twice
+        out[2 * g + 1] = __builtin_amdgcn_perm(u, u, 0x03020302u);   // sub-block 2g'+1 twice
     }
     return out;
 }

@@ -56,7 +56,7 @@ __device__ __forceinline__ void dma4(const void *base, uint32_t off, uint8_t *ld
 //         Q6K also [16 rows][4 chunks] of the 64-byte qh plane (chunk c at c ^ ((r/2)%4)),
 //         Q5K also [16 rows][32 B] of the fifth-bit plane
 //   act : [RT row groups][2 K-halves][8 rows][8 chunks], same swizzle
-//   d8  : [8*RT] f32         minp : [8*RT][2 pieces][8] f16 (Q4K)
+//   d8  : [8*RT] f32         minp : [8*RT][16] f16: the rows' bsums (Q4K / Q5K)
 constexpr bool is_k4(int dt) { return dt == CQ_DTYPE_Q4K || dt == CQ_DTYPE_Q5K; }   // types with a min term
 
 template <int DT, int RT> struct Buf {
@@ -115,7 +115,7 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, int lane, const 
     }
     // min term operand: 32 K-slots = activation pieces [1,1,2,2] x weight pieces [1,2,1,2] of the
     // eight sub-block values -dmin*min_j
-    wmin = __builtin_bit_cast(v8h, cq_min_term_operand(wb.dd, rec, (kq & 1) != 0));
+    wmin = __builtin_bit_cast(v8h, cq_min_term_groups(wb.dd, rec, (kq & 1) != 0, (kq >> 1) != 0));   // K-slots 8kq..: groups 8(kq%2).., piece kq/2
 }
 
 // Q5K: the quants are the Q4K nibbles plus a fifth bit (words {L, H} per 32 qs bytes, bit 8c + i for
@@ -142,7 +142,7 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, int lane, const 
             bh[gi][i] = hi;
         }
     }
-    wmin = __builtin_bit_cast(v8h, cq_min_term_operand(wb.dd, rec, (kq & 1) != 0));
+    wmin = __builtin_bit_cast(v8h, cq_min_term_groups(wb.dd, rec, (kq & 1) != 0, (kq >> 1) != 0));   // K-slots 8kq..: groups 8(kq%2).., piece kq/2
 }
 
 __device__ __forceinline__ void block_unpack(const uint8_t *wl, int lane, const WHead<CQ_DTYPE_Q6K> &wb, v4i (&bl)[4],
@@ -232,7 +232,7 @@ __global__ void __launch_bounds__(kThreads) skinny_kernel(cq_weight w, cq_act_vi
             dma16(a.qs + (m0 + rg * 8) * k + b * 256 + kh * 128, act_off, buf + B::oAct + i * 1024);
         }
         if (lane < 8 * RT) dma4(a.dT + b * a.m_stride + m0, lane * 4u, buf + B::oD8);
-        if (MINS && lane < 16 * RT) dma16(a.minp + (b * a.m_stride + m0) * 16, lane * 16u, buf + B::oMin);
+        if (MINS && lane < 16 * RT) dma16(a.bsh + (b * a.m_stride + m0) * 16, lane * 16u, buf + B::oMin);
         WHead<DT> head;
         load_head(w, (n_tile + r) * kb + b, head);
         __builtin_amdgcn_s_waitcnt(0);   // everything above has landed
@@ -245,12 +245,14 @@ __global__ void __launch_bounds__(kThreads) skinny_kernel(cq_weight w, cq_act_vi
 #pragma unroll
         for (int t = 0; t < NT; t++) {
             const v4f d8 = *(const v4f *)(buf + B::oD8 + (t * 16 + 4 * kq < 8u * RT ? t * 16 + 4 * kq : 0) * 4);
+            // min term: sum_j bsums_j * (-dmin * min_{j/2}), the sums exact in f16 whatever the activations' magnitude
+            // (their scale d8 multiplies afterwards, with the main term)
+            v4f mn = {0.0f, 0.0f, 0.0f, 0.0f};
             if (MINS) {
                 const uint32_t row = t * 16 + r < 8u * RT ? t * 16 + r : 8u * RT - 1;
-                const v8h ma = *(const v8h *)(buf + B::oMin + row * 32 + (kq >> 1) * 16);
-                if (!DUMP) out[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ma, wmin, out[t], 0, 0, 0);
+                const v8h ma = *(const v8h *)(buf + B::oMin + row * 32 + (kq & 1) * 16);
+                mn = __builtin_amdgcn_mfma_f32_16x16x32_f16(ma, wmin, mn, 0, 0, 0);
                 if (DUMP && dump.mn) {
-                    const v4f mn = __builtin_amdgcn_mfma_f32_16x16x32_f16(ma, wmin, (v4f){0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
                         const int64_t orow = m0 + t * 16 + kq * 4 + i;
@@ -272,7 +274,8 @@ __global__ void __launch_bounds__(kThreads) skinny_kernel(cq_weight w, cq_act_vi
                     const int64_t orow = m0 + t * 16 + kq * 4 + i;
                     if (orow < m) dump.i[(orow * w.n + n_tile + r) * kb + b] = I;
                 } else {
-                    out[t][i] = __builtin_fmaf((float)I * dw, d8[i], out[t][i]);
+                    const float v = MINS ? __builtin_fmaf((float)I, dw, mn[i]) : (float)I * dw;
+                    out[t][i] = __builtin_fmaf(v, d8[i], out[t][i]);
                 }
             }
         }
@@ -308,7 +311,7 @@ __global__ void __launch_bounds__(kThreads) skinny_kernel(cq_weight w, cq_act_vi
 // weight tiles (tile t of workgroup g: g + t * G) streaming weights only.  The launcher takes it where every
 // workgroup has one tile (n <= 16 x the number of CUs); with more tiles per workgroup it measured no faster than
 // the kernel above, also with the next tile's weights copied ahead into a second buffer (NBUF == 2).
-//   per K block b  : act [RT][2 K-halves][8 rows][8 chunks] | d8 [8*RT] f32 | minp [8*RT][2][8] f16 (k4 types)
+//   per K block b  : act [RT][2 K-halves][8 rows][8 chunks] | d8 [8*RT] f32 | minp [8*RT][16] f16 (k4 types)
 //   per wave, block: weights of one tile (kWgt bytes), twice when NBUF == 2; a wave's first buffer of a tile also
 //                    carries its partial results of that tile (1 KiB per 16 activation rows)
 template <int DT, int RT> struct Res {
@@ -359,12 +362,12 @@ __device__ __forceinline__ void res_block(const uint8_t *__restrict__ wl, const 
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         const v4f d8 = *(const v4f *)(act + R::oD8 + (t * 16 + 4 * kq < 8u * RT ? t * 16 + 4 * kq : 0) * 4);
+        v4f mn = {0.0f, 0.0f, 0.0f, 0.0f};   // min term without the activation scale (see skinny_kernel)
         if (MINS) {
             const uint32_t row = t * 16 + r < 8u * RT ? t * 16 + r : 8u * RT - 1;
-            const v8h ma = *(const v8h *)(act + R::oMin + row * 32 + (kq >> 1) * 16);
-            if (!DUMP) out[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ma, wmin, out[t], 0, 0, 0);
+            const v8h ma = *(const v8h *)(act + R::oMin + row * 32 + (kq & 1) * 16);
+            mn = __builtin_amdgcn_mfma_f32_16x16x32_f16(ma, wmin, mn, 0, 0, 0);
             if (DUMP && dump.mn) {
-                const v4f mn = __builtin_amdgcn_mfma_f32_16x16x32_f16(ma, wmin, (v4f){0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const int64_t orow = t * 16 + kq * 4 + i;
@@ -386,7 +389,8 @@ __device__ __forceinline__ void res_block(const uint8_t *__restrict__ wl, const 
                 const int64_t orow = t * 16 + kq * 4 + i;
                 if (orow < m) dump.i[at + orow * rs] = I;
             } else {
-                out[t][i] = __builtin_fmaf((float)I * dw, d8[i], out[t][i]);
+                const float v = MINS ? __builtin_fmaf((float)I, dw, mn[i]) : (float)I * dw;
+                out[t][i] = __builtin_fmaf(v, d8[i], out[t][i]);
             }
         }
     }
@@ -429,7 +433,7 @@ __global__ void __launch_bounds__(kWaves * 64) skinny_resident_kernel(cq_weight 
     pl.w5 = wave_rsrc(w.p2);
     pl.aq = wave_rsrc(a.qs);
     pl.ad = wave_rsrc(a.dT);
-    pl.am = wave_rsrc(a.minp);
+    pl.am = wave_rsrc(a.bsh);
     const uint32_t kb32 = (uint32_t)kb, k32 = (uint32_t)k, mstr = (uint32_t)a.m_stride;
     // ---- the wave's K blocks: the small fields of the first tile's weights (registers; requested first, they are
     // what the unpacking starts with), activation slices once, weights of the first tile

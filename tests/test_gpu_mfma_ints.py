@@ -50,8 +50,9 @@ def k4_scales_mins(hdr12):
     return sc, mn
 
 
-def min_term_reference(dt, acts, m, blocks, n, k):
-    """(-(dmin*d8) * sum_j min_j*bsum32_j, (dmin*|d8|) * sum_j min_j*|bsum32_j|) in float64, [m, n, k/256]."""
+def min_term_reference(dt, acts, m, blocks, n, k, with_d8):
+    """(-s * sum_j min_j*bsum32_j, |s| * sum_j min_j*|bsum32_j|) in float64, [m, n, k/256], s = dmin * d8 (tile kernel)
+    or s = dmin (small-batch kernels: the activation block's scale multiplies afterwards, with the main term)."""
     kb = k // 256
     w = blocks.reshape(n, kb, orc.TYPE_SIZE[dt])
     dmin = w[..., 2:4].copy().view(np.float16)[..., 0].astype(np.float64)          # [n, kb]
@@ -62,7 +63,7 @@ def min_term_reference(dt, acts, m, blocks, n, k):
     bs32 = bs16[..., 0::2] + bs16[..., 1::2]                                        # [m, kb, 8]
     s = np.einsum("nbj,mbj->mnb", mn, bs32)
     sabs = np.einsum("nbj,mbj->mnb", mn, np.abs(bs32))
-    scale = dmin[None] * d8[:, None]
+    scale = dmin[None] * (d8 if with_d8 else np.ones_like(d8))[:, None]
     return -scale * s, np.abs(scale) * sabs
 
 
@@ -79,10 +80,13 @@ def check_dump(qh, dt, kernel, m, k, n, seed, x_scale=1.0):
     wi, wm = orc.block_int_dots(dt, acts, m, blocks, n, k)
     assert np.array_equal(oi.cpu().numpy(), wi)                  # every (row, weight row, block), bit for bit
     if dt in (orc.Q4K, orc.Q5K):
-        ref, mag = min_term_reference(dt, acts, m, blocks, n, k)
+        tile = kernel == qh.MFMA_TILE
+        ref, mag = min_term_reference(dt, acts, m, blocks, n, k, with_d8=tile)
         got = om.cpu().numpy().astype(np.float64)
-        # two f16 pieces per factor: 2^-22 per product and f32 rounding of the eight-term sum, against sum |terms|
-        assert np.all(np.abs(got - ref) <= 2.0 ** -19 * mag + 1e-30), float((np.abs(got - ref) / (mag + 1e-30)).max())
+        # tile kernel: two f16 pieces per factor, 2^-22 per product and the f32 rounding of the eight-term sum; small
+        # batch: the sums exact in f16, -dmin*min_j in two f16 pieces, every product exact, only the f32 sum rounds
+        bound = 2.0 ** -19 if tile else 2.0 ** -21
+        assert np.all(np.abs(got - ref) <= bound * mag + 1e-30), float((np.abs(got - ref) / (mag + 1e-30)).max())
     return x, blocks, qw
 
 
@@ -109,12 +113,14 @@ def test_tile_kernel_integers(qh, dt, m, k, n):
     check_dump(qh, dt, qh.MFMA_TILE, m, k, n, 13 * dt + m + k + n)
 
 
-@pytest.mark.parametrize("x_scale", [1e-2, 1.0, 30.0, 500.0])
-@pytest.mark.parametrize("kernel", ["skinny", "tile"])
+@pytest.mark.parametrize("kernel,x_scale", [("skinny", v) for v in (1e-30, 1e-8, 1e-2, 1.0, 500.0, 1e6, 1e30)] +
+                         [("tile", v) for v in (1e-2, 1.0, 30.0, 500.0)])
 def test_min_term_error_bound_across_magnitudes(qh, kernel, x_scale):
-    """The split-f16 min term keeps its bound for activations from a hundred times smaller to five hundred times
-    larger than unit variance (|d8 * bsum32| leaves the f16 range for activations beyond about 2000 throughout a
-    sub-block, and the pieces lose bits below about 1e-3: the documented range of the matrix-core kernels)."""
+    """Small-batch kernels: the min term's matrix-core operands are the integer sums of the block and -dmin*min_j, the
+    activation block's scale multiplies afterwards in f32, so the bound holds for activations of any magnitude.  Tile
+    kernel: the operand d8 * bsum32 in two f16 pieces keeps its bound from a hundred times smaller to five hundred times
+    larger than unit variance (it leaves the f16 range for activations beyond about 2000 throughout a sub-block, and
+    the pieces lose bits below about 1e-3: the documented range of that kernel)."""
     kid = qh.MFMA_SKINNY if kernel == "skinny" else qh.MFMA_TILE
     m = 16 if kernel == "skinny" else 70
     check_dump(qh, orc.Q4K, kid, m, 1024, 64, 5, x_scale)
@@ -123,20 +129,22 @@ def test_min_term_error_bound_across_magnitudes(qh, kernel, x_scale):
 @pytest.mark.parametrize("dt", [orc.Q4K, orc.Q5K, orc.Q6K])
 @pytest.mark.parametrize("m,k,n", [(16, 2048, 64), (70, 1024, 96), (512, 512, 64)])
 def test_rows_of_different_magnitudes(qh, dt, m, k, n):
-    """One batch whose rows span five orders of magnitude (0.01 .. 1000), one row with a block a thousand times the
-    others and one all-zero row: every row against the oracle at the usual bars, on both matrix-core kernels."""
+    """One batch whose rows span five orders of magnitude (0.01 .. 1000; forty, 1e-20 .. 1e20, for the small-batch
+    kernels), one row with a block a thousand times the others and one all-zero row: every row against the oracle at
+    the usual bars, on both matrix-core kernels."""
     rng = np.random.default_rng(m + k + n + int(dt))
     w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
     x = rng.standard_normal((m, k)).astype(np.float32)
-    scales = np.float32(10.0) ** rng.integers(-2, 4, size=m).astype(np.float32)
-    scales[2] = 1.0
-    x *= scales[:, None]
-    x[1] = 0.0
-    x[2, 256:512] *= np.float32(1e3)          # one block dwarfs the others of its row
     blocks = orc.quantize(dt, w)
     qw = qh.QWeight.from_ggml(dt, blocks, n, k)
-    want = orc.matmul(dt, x, blocks, n).astype(np.float64)
-    for flags in (qh.FLAG_FORCE_SKINNY, qh.FLAG_FORCE_GEMM):
+    x0 = x
+    for flags, lo, hi in ((qh.FLAG_FORCE_SKINNY, -20, 21), (qh.FLAG_FORCE_GEMM, -2, 4)):
+        scales = np.float32(10.0) ** rng.integers(lo, hi, size=m).astype(np.float32)
+        scales[2] = 1.0
+        x = x0 * scales[:, None]
+        x[1] = 0.0
+        x[2, 256:512] *= np.float32(1e3)          # one block dwarfs the others of its row
+        want = orc.matmul(dt, x, blocks, n).astype(np.float64)
         got = qh.qmatmul(qw, dev(x), flags).cpu().numpy().astype(np.float64)
         assert np.all(np.isfinite(got))
         for r in range(m):
@@ -173,7 +181,7 @@ def test_tile_kernel_integers_config3(qh, dt, k, n):
     sub = oi[torch.from_numpy(ms).cuda()][:, torch.from_numpy(cols).cuda()].cpu().numpy()
     assert np.array_equal(sub, wi)
     if dt == orc.Q4K:
-        ref, mag = min_term_reference(dt, acts, len(ms), blocks, len(cols), k)
+        ref, mag = min_term_reference(dt, acts, len(ms), blocks, len(cols), k, with_d8=True)
         got = om[torch.from_numpy(ms).cuda()][:, torch.from_numpy(cols).cuda()].cpu().numpy().astype(np.float64)
         assert np.all(np.abs(got - ref) <= 2.0 ** -19 * mag + 1e-30)
         # whole launch: the float min term against the dot-product kernels' integer through the scales is covered by
