@@ -90,6 +90,9 @@ __device__ __forceinline__ void dma4(const void *base, uint32_t off, uint8_t *ld
 }
 
 // Per-lane constants of the copies and of the operand reads.
+// Tile heights whose Q4K / Q5K min term is contracted from unscaled operands (see MinW).
+template <int MT> __device__ __host__ constexpr bool min_term_unscaled() { return MT <= 2; }
+
 struct LaneGeo {
     uint32_t act_off;   // copy of 8 rows x 128 B of activations: (l/8)*k + ((l%8) ^ (l/8))*16
     uint32_t wq_off;    // the same over the weights' 128-byte plane: (l/8)*kb*128 + ...
@@ -139,7 +142,7 @@ __device__ __forceinline__ void stage_issue(uint8_t *buf, const cq_weight &w, co
 #pragma unroll
         for (int j = 0; j < MT; j++) {
             if (j + 4 == wave)
-                dma16(a.minp + (b * a.m_stride + m0 + j * 32) * 16, lane * 16u, buf + T::oMin + j * 1024);
+                dma16((min_term_unscaled<MT>() ? a.bsh : a.minp) + (b * a.m_stride + m0 + j * 32) * 16, lane * 16u, buf + T::oMin + j * 1024);
         }
     }
 }
@@ -184,6 +187,15 @@ struct DumpLane {
     int64_t rows;   // rows m0 .. m0 + rows - 1 exist
 };
 
+// The weight operand(s) of the Q4K / Q5K min term.  Tiles of up to 64 rows take the form whose operands do not depend
+// on the activations' magnitude (the block's sixteen integer sums as f16 against -dmin * min in two pieces, the result
+// in an accumulator of its own until the activation scale multiplies it with the main term): `p1`, `p2` from
+// cq_min_term_groups.  The 128-row tiles have no registers for that accumulator (measured: 100 bytes of scratch per lane
+// and 81 -> 95 us at M = 512) and keep the operand scaled by d8 in the quantizer, which accumulates straight into the
+// result: `p1` from cq_min_term_operand.
+struct MinW {
+    v8h p1, p2;
+};
 // One block for this wave's 32 weight rows against the MT activation tiles in `cur`, as a
 // hand-laid software pipeline of 8*(MT+1) steps.  Step (t, s) issues the two int8 MFMAs of tile t,
 // K-slice s, and, in their shadow, the scaling of two of the sixteen integers of tile t-1 (VALU);
@@ -194,25 +206,27 @@ struct DumpLane {
 // it, from a zero accumulator) are stored through `dl`.
 template <int DT, int MT, int T0, int T1, int SHIFT, bool HALF, bool DUMP>
 __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, const v4i (&bl)[8], const v4i (&bh)[8],
-                                          float dw, v8h wmin, int lane, v16f (&out)[MT], const DumpLane &dl) {
+                                          float dw, const MinW &wmin, int lane, v16f (&out)[MT], const DumpLane &dl) {
     typedef Tile<DT, MT> T;
     if constexpr (T0 >= T1) return;
     constexpr bool MINS = is_k4(DT);
+    constexpr bool UNSCALED = MINS && min_term_unscaled<MT>();
     const int h = lane >> 5, col = lane & 31;
     const uint8_t *d8p = cur + T::oD8 + h * 16;        // rows 8j + 4h + [0,4) of a tile
-    const uint8_t *mnp = cur + T::oMin + col * 32;     // this lane's row of min pieces
+    const uint8_t *mnp = cur + T::oMin + col * 32;     // this lane's row of the min term's activation operand
     // operand of tile t, K-slice s: chunk 2*(s%4) + h of K-half s/4
     auto afrag = [&](int q) -> v4i {
         const int t = q >> 3, s = q & 7;
         return *(const v4i *)(cur + g.col[s & 3] + (t * 2 + (s >> 2)) * 4096);
     };
     v16i acc_lo[2], acc_hi[2];
+    v16f mn = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};   // UNSCALED: -dmin * Mn_b of the tile being scaled
     v4i a[3];
     v4f dreg[2];   // d8 of four rows each, read two steps before the scaling that needs them
-    v8h ma1, ma2;
+    v8h ma1 = {}, ma2 = {};
     a[(T0 * 8) % 3] = afrag(T0 * 8);
     a[(T0 * 8 + 1) % 3] = afrag(T0 * 8 + 1);
-    if (MINS) {
+    if (MINS && !UNSCALED) {
         ma1 = *(const v8h *)(mnp + T0 * 1024);
         ma2 = *(const v8h *)(mnp + T0 * 1024 + 16);
     }
@@ -222,21 +236,21 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, 
         if (q + 2 < T1 * 8) a[(q + 2) % 3] = afrag(q + 2);
         if (t < T1) {
             if (s == 0) {
-                if (MINS && !DUMP) {
+                if (MINS && !UNSCALED && !DUMP) {
                     // min term: out -= sum_j (dmin*min_j) * (d8*bsum32_j).  K-slots 0..7 carry piece 1
                     // of the weight factor, slots 8..15 piece 2; the activation operand carries one of
                     // its pieces in both halves.
-                    out[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma1, wmin, out[t], 0, 0, 0);
-                    out[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma2, wmin, out[t], 0, 0, 0);
+                    out[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma1, wmin.p1, out[t], 0, 0, 0);
+                    out[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma2, wmin.p1, out[t], 0, 0, 0);
                 }
-                if (MINS && DUMP && dl.mn) {
-                    v16f mn = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                    mn = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma1, wmin, mn, 0, 0, 0);
-                    mn = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma2, wmin, mn, 0, 0, 0);
+                if (MINS && !UNSCALED && DUMP && dl.mn) {
+                    v16f m0 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                    m0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma1, wmin.p1, m0, 0, 0, 0);
+                    m0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma2, wmin.p1, m0, 0, 0, 0);
 #pragma unroll
                     for (int i = 0; i < 16; i++) {
                         const int64_t row = t * 32 + (i >> 2) * 8 + h * 4 + (i & 3);
-                        if (row < dl.rows) dl.mn[row * dl.rs] = mn[i];
+                        if (row < dl.rows) dl.mn[row * dl.rs] = m0[i];
                     }
                 }
                 const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
@@ -247,12 +261,21 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, 
                 acc_hi[t & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[q % 3], bh[s], acc_hi[t & 1], 0, 0, 0);
             }
             if (s == 6) dreg[0] = *(const v4f *)(d8p + (t * 32) * 4);
-            if (s == 6 && MINS && t + 1 < T1) {
+            if (s == 6 && MINS && !UNSCALED && t + 1 < T1) {
                 ma1 = *(const v8h *)(mnp + (t + 1) * 1024);
                 ma2 = *(const v8h *)(mnp + (t + 1) * 1024 + 16);
             }
+            // UNSCALED: this tile's own min term, -dmin * sum_j bsums_j * min_{j/2} from a zero accumulator (lanes h:
+            // sums 8h .. 8h+7), behind its last MFMAs; it is added where the integers are scaled, one tile later
+            if (s == 6 && UNSCALED) ma1 = *(const v8h *)(mnp + t * 1024 + h * 16);
+            if (s == 7 && UNSCALED && (!DUMP || dl.mn)) {
+                const v16f zf = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                mn = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma1, wmin.p1, zf, 0, 0, 0);
+                mn = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma1, wmin.p2, mn, 0, 0, 0);
+            }
         }
-        if (t > T0) {
+        if (t > T0 && !UNSCALED) {
+            // scaling of two of the sixteen integers of tile t-1 per step (element i: rows 8*(i/4) + 4h + i%4)
             const int p = (t - 1) & 1;
             if ((s & 1) == 0 && s < 6) dreg[((s >> 1) + 1) & 1] = *(const v4f *)(d8p + ((t - 1) * 32 + 8 * ((s >> 1) + 1)) * 4);
 #pragma unroll
@@ -269,6 +292,42 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, 
                 out[t - 1][i] = o;
             }
         }
+        if (t > T0 && UNSCALED) {
+            // the same in steps 1..6 (the min term's MFMAs were the last of tile t-1, and this tile's follow in step 7
+            // into the same registers): three elements a step, then two; out += d8 * (I * dw + min term)
+            const int p = (t - 1) & 1;
+            if (s == 0) {
+                dreg[1] = *(const v4f *)(d8p + ((t - 1) * 32 + 8) * 4);
+                if (DUMP && dl.mn) {
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        const int64_t row = (t - 1) * 32 + (i >> 2) * 8 + h * 4 + (i & 3);
+                        // (stored with the activation scale, like the 128-row tiles' term)
+                        if (row < dl.rows) dl.mn[row * dl.rs] = mn[i] * *(const float *)(d8p + ((t - 1) * 32 + 8 * (i >> 2) + (i & 3)) * 4);
+                    }
+                }
+            }
+            if (s >= 1 && s <= 6) {
+                const int i0 = s < 5 ? 3 * (s - 1) : 12 + 2 * (s - 5), i1 = s < 5 ? i0 + 3 : i0 + 2;
+#pragma unroll
+                for (int i = i0; i < i1; i++) {
+                    if (!(HALF && i >= 8)) {   // (HALF: rows 16..31 of the tile are not wanted)
+                        const int I = (acc_hi[p][i] << SHIFT) + acc_lo[p][i];
+                        if (DUMP) {
+                            const int64_t row = (t - 1) * 32 + (i >> 2) * 8 + h * 4 + (i & 3);
+                            if (row < dl.rows) dl.i[row * dl.rs] = I;
+                        } else {
+                            float o = __builtin_fmaf(__builtin_fmaf((float)I, dw, mn[i]), dreg[(i >> 2) & 1][i & 3], out[t - 1][i]);
+                            asm volatile("" : "+v"(o));   // pins the scaling to this step (pure ops float otherwise)
+                            out[t - 1][i] = o;
+                        }
+                    }
+                    // the d8 of rows 16.. and 24.. follow their buffers' last use (elements 3 and 7)
+                    if (i == 3) dreg[0] = *(const v4f *)(d8p + ((t - 1) * 32 + 16) * 4);
+                    if (i == 7) dreg[1] = *(const v4f *)(d8p + ((t - 1) * 32 + 24) * 4);
+                }
+            }
+        }
         __builtin_amdgcn_sched_barrier(0);
     }
 }
@@ -276,7 +335,7 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, 
 // Weight operands of one block: unpacks the wave's 32 rows from `wl` into the two digit operands
 // of the eight K-slices, and returns the block scale (and the Q4K min-term operand).
 __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g, const WHead<CQ_DTYPE_Q4K> &wb,
-                                             int lane, v4i (&bl)[8], v4i (&bh)[8], float &dw, v8h &wmin) {
+                                             int lane, v4i (&bl)[8], v4i (&bh)[8], float &dw, MinW &wmin, bool unscaled) {
     const int h = lane >> 5;
     dw = cq_h2f((uint16_t)(wb.dd & 0xffff));
     const uint32_t rec[4] = {wb.rec.x, wb.rec.y, wb.rec.z, wb.rec.w};   // {sc[2g], sc[2g+1], mn[2g], mn[2g+1]}
@@ -296,13 +355,19 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g
             bh[2 * gi + 1][i] = (int)pk_mul_u16(hi4, sh1);
         }
     }
-    wmin = __builtin_bit_cast(v8h, cq_min_term_operand(wb.dd, rec, h != 0));
+    if (unscaled) {   // (a compile-time constant at every call)
+        wmin.p1 = __builtin_bit_cast(v8h, cq_min_term_groups(wb.dd, rec, h != 0, false));
+        wmin.p2 = __builtin_bit_cast(v8h, cq_min_term_groups(wb.dd, rec, h != 0, true));
+    } else {
+        wmin.p1 = __builtin_bit_cast(v8h, cq_min_term_operand(wb.dd, rec, h != 0));
+        wmin.p2 = wmin.p1;
+    }
 }
 
 // Q5K: the Q4K nibbles plus a fifth bit per quant (words {L, H} per 32 qs bytes, bit 8c + i for byte c
 // of qs word i); scale times quant has up to 11 bits and is split as Q6K's products are.
 __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g, const WHead<CQ_DTYPE_Q5K> &wb,
-                                             int lane, v4i (&bl)[8], v4i (&bh)[8], float &dw, v8h &wmin) {
+                                             int lane, v4i (&bl)[8], v4i (&bh)[8], float &dw, MinW &wmin, bool unscaled) {
     const int h = lane >> 5;
     const uint32_t row = lane & 31;
     dw = cq_h2f((uint16_t)(wb.dd & 0xffff));
@@ -328,11 +393,17 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g
             bh[2 * gi + 1][i] = hi;
         }
     }
-    wmin = __builtin_bit_cast(v8h, cq_min_term_operand(wb.dd, rec, h != 0));
+    if (unscaled) {   // (a compile-time constant at every call)
+        wmin.p1 = __builtin_bit_cast(v8h, cq_min_term_groups(wb.dd, rec, h != 0, false));
+        wmin.p2 = __builtin_bit_cast(v8h, cq_min_term_groups(wb.dd, rec, h != 0, true));
+    } else {
+        wmin.p1 = __builtin_bit_cast(v8h, cq_min_term_operand(wb.dd, rec, h != 0));
+        wmin.p2 = wmin.p1;
+    }
 }
 
 __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g, const WHead<CQ_DTYPE_Q6K> &wb,
-                                             int lane, v4i (&bl)[8], v4i (&bh)[8], float &dw, v8h &wmin) {
+                                             int lane, v4i (&bl)[8], v4i (&bh)[8], float &dw, MinW &wmin, bool unscaled) {
     const int h = lane >> 5;
     dw = cq_h2f((uint16_t)wb.d);
     const uint32_t scw[4] = {wb.sc.x, wb.sc.y, wb.sc.z, wb.sc.w};
@@ -367,7 +438,7 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g
             bh[s][i] = hi;
         }
     }
-    wmin = v8h{};
+    wmin = MinW{};
 }
 
 // One K block of one wave.  The two waves of a SIMD (waves w and w + 4 of the workgroup) run half a
@@ -390,10 +461,10 @@ __device__ __forceinline__ void block_step(const uint8_t *__restrict__ cur, uint
     constexpr int SPLIT = TRAIL ? MT / 2 : MT;   // tiles [SPLIT, MT) follow the barrier
     v4i bl[8], bh[8];
     float dw = 0.0f;
-    v8h wmin = {};
+    MinW wmin = {};
     if (more) stage_issue<DT, MT>(nxt, w, a, g, m0, b + 1, wave, lane);
     if (n_ok) {
-        block_unpack(wl, g, hcur, lane, bl, bh, dw, wmin);
+        block_unpack(wl, g, hcur, lane, bl, bh, dw, wmin, min_term_unscaled<MT>());
         if (more) stage_weights<DT>(wl, w, g, n_tile, b + 1);
         tiles_mac<DT, MT, 0, SPLIT, SHIFT, HALF, DUMP>(cur, g, bl, bh, dw, wmin, lane, out, dl);
     }
@@ -662,7 +733,8 @@ __global__ void __launch_bounds__(kThreads) gemm_q81_kernel(cq_weight w, cq_act_
                 wmin = __builtin_bit_cast(v8h, cq_min_term_operand(hcur.dd, rec, h != 0));
             } else {
                 float dw;
-                block_unpack(wl, g, hcur, lane, bl, bh, dw, wmin);
+                MinW none;
+                block_unpack(wl, g, hcur, lane, bl, bh, dw, none, false);
                 ws[0] = weight_scale_operand(dw, h);
             }
             if (more) stage_weights<DT>(wl, w, g, n_tile, b + 1);

@@ -113,32 +113,34 @@ def test_tile_kernel_integers(qh, dt, m, k, n):
     check_dump(qh, dt, qh.MFMA_TILE, m, k, n, 13 * dt + m + k + n)
 
 
-@pytest.mark.parametrize("kernel,x_scale", [("skinny", v) for v in (1e-30, 1e-8, 1e-2, 1.0, 500.0, 1e6, 1e30)] +
+@pytest.mark.parametrize("kernel,x_scale", [(kn, v) for kn in ("skinny", "tile64") for v in (1e-30, 1e-8, 1e-2, 1.0, 500.0, 1e6, 1e30)] +
                          [("tile", v) for v in (1e-2, 1.0, 30.0, 500.0)])
 def test_min_term_error_bound_across_magnitudes(qh, kernel, x_scale):
-    """Small-batch kernels: the min term's matrix-core operands are the integer sums of the block and -dmin*min_j, the
-    activation block's scale multiplies afterwards in f32, so the bound holds for activations of any magnitude.  Tile
-    kernel: the operand d8 * bsum32 in two f16 pieces keeps its bound from a hundred times smaller to five hundred times
-    larger than unit variance (it leaves the f16 range for activations beyond about 2000 throughout a sub-block, and
-    the pieces lose bits below about 1e-3: the documented range of that kernel)."""
+    """Small-batch kernels and tiles of up to 64 rows (a call of at most 64 rows has no others): the min term's
+    matrix-core operands are the integer sums of the block and -dmin*min_j, the activation block's scale multiplies
+    afterwards in f32, so the bound holds for activations of any magnitude.  128-row tiles: the operand d8 * bsum32 in
+    two f16 pieces keeps its bound from a hundred times smaller to five hundred times larger than unit variance (it
+    leaves the f16 range for activations beyond about 2000 throughout a sub-block, and the pieces lose bits below about
+    1e-3: the documented range of those tiles)."""
     kid = qh.MFMA_SKINNY if kernel == "skinny" else qh.MFMA_TILE
-    m = 16 if kernel == "skinny" else 70
+    m = {"skinny": 16, "tile64": 56, "tile": 70}[kernel]
     check_dump(qh, orc.Q4K, kid, m, 1024, 64, 5, x_scale)
 
 
 @pytest.mark.parametrize("dt", [orc.Q4K, orc.Q5K, orc.Q6K])
-@pytest.mark.parametrize("m,k,n", [(16, 2048, 64), (70, 1024, 96), (512, 512, 64)])
+@pytest.mark.parametrize("m,k,n", [(16, 2048, 64), (60, 1024, 96), (70, 1024, 96), (512, 512, 64)])
 def test_rows_of_different_magnitudes(qh, dt, m, k, n):
     """One batch whose rows span five orders of magnitude (0.01 .. 1000; forty, 1e-20 .. 1e20, for the small-batch
-    kernels), one row with a block a thousand times the others and one all-zero row: every row against the oracle at
-    the usual bars, on both matrix-core kernels."""
+    kernels and the tile kernel on at most 64 rows), one row with a block a thousand times the others and one all-zero
+    row: every row against the oracle at the usual bars, on both matrix-core kernels."""
     rng = np.random.default_rng(m + k + n + int(dt))
     w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
     x = rng.standard_normal((m, k)).astype(np.float32)
     blocks = orc.quantize(dt, w)
     qw = qh.QWeight.from_ggml(dt, blocks, n, k)
     x0 = x
-    for flags, lo, hi in ((qh.FLAG_FORCE_SKINNY, -20, 21), (qh.FLAG_FORCE_GEMM, -2, 4)):
+    wide = (-20, 21)      # the small-batch kernels and tiles of up to 64 rows (all a call of at most 64 rows has)
+    for flags, lo, hi in ((qh.FLAG_FORCE_SKINNY,) + wide, (qh.FLAG_FORCE_GEMM,) + (wide if m <= 64 else (-2, 4))):
         scales = np.float32(10.0) ** rng.integers(lo, hi, size=m).astype(np.float32)
         scales[2] = 1.0
         x = x0 * scales[:, None]
@@ -151,6 +153,29 @@ def test_rows_of_different_magnitudes(qh, dt, m, k, n):
             nrm = np.linalg.norm(want[r])
             assert np.linalg.norm(got[r] - want[r]) <= 1e-4 * nrm + 1e-38, (flags, r, float(scales[r]))
             assert np.abs(got[r] - want[r]).max() <= 1e-3 * nrm + 1e-38, (flags, r)
+
+
+@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q5K])
+def test_grouped_rows_of_different_magnitudes(qh, dt):
+    """The grouped launch of the expert FFN (32-row tiles) with token rows forty orders of magnitude apart: every row
+    against the oracle's matmul with its expert."""
+    rng = np.random.default_rng(int(dt))
+    k, n, tokens = 1024, 96, 24
+    ws = [(rng.standard_normal((n, k)) * 0.02).astype(np.float32) for _ in range(3)]
+    blocks = [orc.quantize(dt, w) for w in ws]
+    experts = [qh.QWeight.from_ggml(dt, b, n, k) for b in blocks]
+    x = rng.standard_normal((tokens, k)).astype(np.float32)
+    x *= (np.float32(10.0) ** rng.integers(-20, 21, size=tokens).astype(np.float32))[:, None]
+    offsets = np.array([0, 17, 17 + 40, 17 + 40 + 5], np.int32)
+    rid = rng.integers(0, tokens, size=int(offsets[-1])).astype(np.int32)
+    y = qh.qmatmul_grouped(experts, dev(x), torch.from_numpy(rid).cuda(), offsets).cpu().numpy().astype(np.float64)
+    assert np.all(np.isfinite(y))
+    for e in range(3):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        want = orc.matmul(dt, x[rid[lo:hi]], blocks[e], n).astype(np.float64)
+        for r in range(hi - lo):
+            nrm = np.linalg.norm(want[r])
+            assert np.linalg.norm(y[lo + r] - want[r]) <= 1e-4 * nrm + 1e-38, (e, r)
 
 
 @pytest.mark.parametrize("dt,k,n", [(orc.Q4K, 4096, 14336), (orc.Q6K, 14336, 4096)])
