@@ -251,6 +251,17 @@ __device__ __forceinline__ float min3f(float a, float b, float c) {
     asm("v_min3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
     return r;
 }
+// the same against 0.0 as the third operand: never NaN, never below / above zero
+__device__ __forceinline__ float max3f_zero(float a, float b) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, 0" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ float min3f_zero(float a, float b) {
+    float r;
+    asm("v_min3_f32 %0, %1, %2, 0" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
 __device__ __forceinline__ int half_min_i(int v) {
     v = min(v, dpp_i<kQuadSwap1>(v));
     v = min(v, dpp_i<kQuadSwap2>(v));
@@ -276,8 +287,10 @@ __device__ __forceinline__ void quantize_pair_to_lds(uint8_t *smem, const X8 &fi
     // magnitude of the lane's largest positive and largest negative value (zero if it has none), then
     // of the chunk (an out-of-range chunk goes through the arithmetic on the bytes of chunk 0; nothing
     // of it is stored)
-    const float vmax = max3f(max3f(v[0], v[1], v[2]), max3f(v[3], v[4], v[5]), max3f(v[6], v[7], v[7]));
-    const float vmin = min3f(min3f(v[0], v[1], v[2]), min3f(v[3], v[4], v[5]), min3f(v[6], v[7], v[7]));
+    // (0.0 as one operand: a lane whose eight values are all NaN ends with zero, as the reference's search, whose
+    // comparisons with a NaN are false, passes over them)
+    const float vmax = max3f(max3f(v[0], v[1], v[2]), max3f(v[3], v[4], v[5]), max3f_zero(v[6], v[7]));
+    const float vmin = min3f(min3f(v[0], v[1], v[2]), min3f(v[3], v[4], v[5]), min3f_zero(v[6], v[7]));
     const uint32_t pbits = (uint32_t)max(__builtin_bit_cast(int, vmax), 0);
     const uint32_t nbits = (uint32_t)max(__builtin_bit_cast(int, vmin) ^ (int)0x80000000, 0);
     uint32_t a_lo, a_hi;

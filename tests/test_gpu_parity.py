@@ -844,3 +844,32 @@ def test_input_patterns_match_oracle(qh, dt, m, k, n, kind):
             assert np.isfinite(got).all()
             assert np.linalg.norm(got - ref64) <= REL_L2_TOL * np.linalg.norm(ref64)
         assert not got[~x.any(axis=1)].any()          # a row of zeros gives zeros, offsets or not
+
+
+@pytest.mark.parametrize("dt", WEIGHT_DTYPES)
+@pytest.mark.parametrize("m", [1, 3, 9])
+def test_nan_activations_follow_the_reference(qh, dt, m):
+    """The reference's maximum searches skip NaN (comparisons with it are false) and its casts turn NaN into 0, so
+    activations with NaN give numbers, not NaN - unless a scale becomes infinite.  Isolated NaN, a run of NaN that fills
+    whole lanes of the quantizers (eight, sixteen, thirty-two in a row), a block of NaN and a row of NaN, through the
+    one-launch kernels (one and three rows) and the workspace path: finite where the oracle is finite, the same
+    values."""
+    rng = np.random.default_rng(100 * int(dt) + m)
+    k, n = 1024, 40
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    x[0, [3, 77, 500]] = np.nan
+    x[0, 256:264] = np.nan
+    x[0, 320:336] = np.nan
+    x[0, 512:544] = np.nan
+    x[0, 768:1024] = np.nan
+    if m > 1:
+        x[1, :] = np.nan
+    blocks = orc.quantize(dt, w)
+    ref = orc.matmul(dt, x, blocks, n)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    for flags in (0, qh.FLAG_STAGED_ACT, qh.FLAG_FORCE_MATVEC):
+        got = qh.qmatmul(qw, dev(x), flags).cpu().numpy()
+        fin = np.isfinite(ref)
+        assert np.array_equal(np.isfinite(got), fin), flags
+        assert np.linalg.norm((got - ref)[fin]) <= REL_L2_TOL * np.linalg.norm(ref[fin]), flags
