@@ -873,3 +873,50 @@ def test_nan_activations_follow_the_reference(qh, dt, m):
         fin = np.isfinite(ref)
         assert np.array_equal(np.isfinite(got), fin), flags
         assert np.linalg.norm((got - ref)[fin]) <= REL_L2_TOL * np.linalg.norm(ref[fin]), flags
+
+
+# byte offsets of the f16 fields of a block (k_quants.rs:42-155)
+_F16_FIELDS = {orc.Q4_0: [0], orc.Q4_1: [0, 2], orc.Q5_0: [0], orc.Q5_1: [0, 2], orc.Q8_0: [0], orc.Q2K: [80, 82],
+               orc.Q3K: [108], orc.Q4K: [0, 2], orc.Q5K: [0, 2], orc.Q6K: [208]}
+
+
+def _byte_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(count):
+        dt = WEIGHT_DTYPES[i % len(WEIGHT_DTYPES)]
+        kb = int(rng.choice([16, 32, 64])) if orc.BLOCK_SIZE[dt] == 32 else int(rng.choice([1, 2, 3, 8]))
+        cases.append((dt, int(rng.choice([1, 3, 8, 17, 40, 130])), kb * orc.BLOCK_SIZE[dt], int(rng.choice([16, 48, 100])), i % 3))
+    return cases
+
+
+@pytest.mark.parametrize("dt,m,k,n,mode", _byte_cases(60, 77))
+def test_weights_from_arbitrary_bytes(qh, dt, m, k, n, mode):
+    """Blocks no quantizer would write: every integer field random, all ones, or at the corners 0x00 / 0x7f / 0x80 / 0xff
+    (six-bit scales of 63, Q6K scales of -128, Q8_0 quants of -128 ...), the f16 fields finite; activations that quantize
+    to +-127 / -128.  Bytes back, dequantize and every kernel choice against the oracle: the integer ranges the
+    matrix-core kernels' digit splits assume hold for any block."""
+    rng = np.random.default_rng(dt * 131 + m + k + n + mode)
+    ts, kb = orc.TYPE_SIZE[dt], k // orc.BLOCK_SIZE[dt]
+    raw = rng.integers(0, 256, size=(n * kb, ts), dtype=np.uint8)
+    if mode == 1:
+        raw[:] = 0xff
+    if mode == 2:
+        raw[:] = rng.choice([0x00, 0x80, 0x7f, 0xff], size=raw.shape).astype(np.uint8)
+    for off in _F16_FIELDS[dt]:
+        vals = (rng.uniform(1e-3, 1.0, size=n * kb) * rng.choice([-1.0, 1.0], size=n * kb)).astype(np.float16)
+        raw[:, off:off + 2] = vals.view(np.uint8).reshape(-1, 2)
+    blocks = raw.ravel()
+    x = np.where(rng.random((m, k)) < 0.5, -3.0, 3.0).astype(np.float32) if mode else rng.standard_normal((m, k)).astype(np.float32)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    assert np.array_equal(qw.to_ggml(), blocks)
+    assert np.array_equal(qw.dequantize().cpu().numpy().ravel(), orc.dequantize(dt, blocks).ravel()[:n * k])
+    ref = orc.matmul(dt, x, blocks, n).astype(np.float64)
+    for flags in (0, qh.FLAG_STAGED_ACT, qh.FLAG_FORCE_MATVEC, qh.FLAG_FORCE_SKINNY, qh.FLAG_FORCE_GEMM):
+        try:
+            got = qh.qmatmul(qw, dev(x), flags).cpu().numpy().astype(np.float64)
+        except qh.QHipError:
+            assert flags in (qh.FLAG_FORCE_SKINNY, qh.FLAG_FORCE_GEMM)   # a forced kernel that does not take the shape
+            continue
+        assert np.isfinite(got).all()
+        assert np.linalg.norm(got - ref) <= REL_L2_TOL * np.linalg.norm(ref), flags
