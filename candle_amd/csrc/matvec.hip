@@ -860,7 +860,11 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
         __syncthreads();
     }
     float yscale = 1.0f;
-    if constexpr (kRms && kPairs) yscale = row_scale();
+    bool yscale_ok = true;   // (a NaN, infinite or zero scale: the reference's normalised row quantizes to zero blocks)
+    if constexpr (kRms && kPairs) {
+        yscale = row_scale();
+        yscale_ok = yscale > 0.0f && yscale < __builtin_inff();
+    }
     auto put = [&](int64_t row, Sums<MB> v, const OffsetRow<DT> &o) {
         cq_weight ws;
         float *ys;
@@ -868,7 +872,7 @@ __global__ void __launch_bounds__(NW * 64) fused_kernel(cq_weight w, const float
 #pragma unroll
         for (int m = 0; m < MB; m++) {
             float t = v.v[m];
-            if constexpr (kRms && kPairs) t *= yscale;
+            if constexpr (kRms && kPairs) t = yscale_ok ? t * yscale : 0.0f;
             if constexpr (kOffsets) {
                 t += offset_term<DT>(smem, rm[m], ws, o);   // the f32 addition the workspace path's second launch makes
             }

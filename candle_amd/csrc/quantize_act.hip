@@ -240,12 +240,15 @@ __global__ void __launch_bounds__(256) quantize_rms_rows_kernel(const float *__r
     float sum2 = chunk_sums[0];
     for (int64_t c = 1; c < chunks; c++) sum2 += chunk_sums[c];
     const float scale = 1.0f / sqrtf(sum2 / (float)k + eps);
+    // Q8K: a row whose scale is NaN, infinite or zero (NaN or infinities among its elements, squares that overflow) is
+    // all NaN or all zero after the reference's normalisation and quantizes to zero blocks; z alone would not
+    const float keep = scale > 0.0f && scale < __builtin_inff() ? 1.0f : __builtin_nanf("");
     for (int64_t c = wave; c < chunks; c += 4) {
         const int64_t e0 = c * 256 + 4 * lane;
         const bool active = e0 < k;
         float4 f = make_float4(0.f, 0.f, 0.f, 0.f), a = f;
         if (active) { f = *(const float4 *)(xr + e0); a = *(const float4 *)(alpha + e0); }
-        if (ACT == 0) q8k_chunk<AOS, true>(make_float4(f.x * a.x, f.y * a.y, f.z * a.z, f.w * a.w), row, c, k, out, scale);
+        if (ACT == 0) q8k_chunk<AOS, true>(make_float4(f.x * a.x * keep, f.y * a.y * keep, f.z * a.z * keep, f.w * a.w * keep), row, c, k, out, keep == keep ? scale : 0.0f);
         else q8_0_chunk<AOS, ACT == 2>(rms_scale4(f, scale, a), active, row, e0, k, out);
     }
 }

@@ -242,3 +242,37 @@ def test_fused_argument_errors(qh):
     assert call(qh.PRE_NONE, None) == 0
     torch.cuda.synchronize()
     assert torch.equal(y, qh.qmatmul(qw, xd))
+
+
+@pytest.mark.parametrize("dt", WEIGHT_DTYPES)
+@pytest.mark.parametrize("m", [1, 3, 9])
+def test_rms_norm_rows_without_a_finite_scale(qh, dt, m):
+    """A row with a NaN, with an infinity, or whose squares overflow has no finite non-zero scale: the reference's
+    normalised row is then all NaN or all zero, quantizes to zero blocks and gives zeros.  The fused calls (Q8K
+    activations keep the scale out of the quantized elements) give the same, and the other rows their usual values."""
+    rng = np.random.default_rng(31 * int(dt) + m)
+    k, n, eps = 1024, 40, 1e-5
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    alpha = rng.standard_normal(k).astype(np.float32)
+    x[0, 5] = np.nan
+    if m > 2:
+        x[1, 700] = np.inf
+        x[2, :] *= np.float32(1e25)          # squares overflow: scale 0
+    blocks = orc.quantize(dt, w)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    with np.errstate(all="ignore"):
+        normed = orc.rms_norm(x, alpha, eps)
+        ref = orc.matmul(dt, normed, blocks, n)
+    bad_rows = [0] + ([1, 2] if m > 2 else [])
+    assert not ref[bad_rows].any()                      # the reference's own answer for such rows: zeros
+    for flags in (0, qh.FLAG_STAGED_ACT):
+        got = qh.qmatmul(qw, dev(x), flags, pre=qh.PRE_RMS_NORM, aux=dev(alpha), eps=eps).cpu().numpy()
+        assert not got[bad_rows].any(), flags
+        good = [r for r in range(m) if r not in bad_rows]
+        if good:
+            check_f32(got[good], ref[good])
+    acts = qh.quantize_act(orc.VEC_DOT_TYPE[dt], dev(x), pre=qh.PRE_RMS_NORM, aux=dev(alpha), eps=eps).cpu().numpy()
+    rowb = acts.size // m
+    for r in bad_rows:
+        assert not acts.reshape(m, rowb)[r].any()       # zero blocks, as the reference's quantizer writes for them
