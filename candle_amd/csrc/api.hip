@@ -397,12 +397,11 @@ static size_t act_ws_layout(int act_dtype, int64_t m, int64_t k, uint8_t *base, 
         const size_t o_d = take((size_t)(m * (k / 256)) * 4);
         const size_t o_bs = take((size_t)(m * (k / 256)) * 32);
         const size_t o_dt = take((size_t)(m_pad * (k / 256)) * 4);
-        const size_t o_mp = take((size_t)(m_pad * (k / 256)) * 32);
         const size_t o_bh = take((size_t)(m_pad * (k / 256)) * 32);
         if (base) {
             view.qs = (int8_t *)(base + o_qs); view.d = (float *)(base + o_d);
             view.bsums = (int16_t *)(base + o_bs); view.dT = (float *)(base + o_dt);
-            view.minp = (uint16_t *)(base + o_mp); view.bsh = (uint16_t *)(base + o_bh);
+            view.bsh = (uint16_t *)(base + o_bh);
         }
     } else {
         const size_t o_d = take((size_t)(m_pad * (k / 32)) * 4);
@@ -759,7 +758,6 @@ static int grouped_impl(const cq_weight *const *experts, int n_experts, const fl
             ve.d += r0 * (w0->k / 256);
             ve.bsums += r0 * (w0->k / 256) * 16;
             ve.dT += r0;
-            ve.minp += r0 * 16;
             ve.bsh += r0 * 16;
         } else {
             ve.d += r0 * (w0->k / 32);

@@ -48,7 +48,7 @@ constexpr int kThreads = kWaves * 64;
 // LDS image of one pipeline stage:
 //   act  : [MT tiles][2 K-halves][4 row groups][8 rows][8 chunks of 16 B]   chunk c of row r sits at c ^ (r%8)
 //   d8   : [BM] f32
-//   minp : [BM][2 pieces][8] f16            d8 * bsum32_j split in two f16 pieces (Q4K)
+//   bsh  : [BM][16] f16                      the block's sixteen bsums as f16 (Q4K / Q5K min term)
 //   wgt  : per wave: [4 row groups][8 rows][8 chunks] of the 128-byte qs / ql plane (same swizzle),
 //          Q6K also [2 row groups][16 rows][4 chunks] of the 64-byte qh plane (chunk c at c ^ ((r/2)%4)),
 //          Q5K also [32 rows][32 B] of the fifth-bit plane
@@ -90,8 +90,9 @@ __device__ __forceinline__ void dma4(const void *base, uint32_t off, uint8_t *ld
 }
 
 // Per-lane constants of the copies and of the operand reads.
-// Tile heights whose Q4K / Q5K min term is contracted from unscaled operands (see MinW).
-template <int MT> __device__ __host__ constexpr bool min_term_unscaled() { return MT <= 2; }
+// Q4K / Q5K min term: tiles of up to 64 rows keep it in an accumulator of its own until the integers are scaled; the
+// 128-row tiles have no registers for that and let its MFMAs add to the scaled integers themselves (see tiles_mac).
+template <int MT> __device__ __host__ constexpr bool min_term_folded() { return MT > 2; }
 
 struct LaneGeo {
     uint32_t act_off;   // copy of 8 rows x 128 B of activations: (l/8)*k + ((l%8) ^ (l/8))*16
@@ -142,7 +143,7 @@ __device__ __forceinline__ void stage_issue(uint8_t *buf, const cq_weight &w, co
 #pragma unroll
         for (int j = 0; j < MT; j++) {
             if (j + 4 == wave)
-                dma16((min_term_unscaled<MT>() ? a.bsh : a.minp) + (b * a.m_stride + m0 + j * 32) * 16, lane * 16u, buf + T::oMin + j * 1024);
+                dma16(a.bsh + (b * a.m_stride + m0 + j * 32) * 16, lane * 16u, buf + T::oMin + j * 1024);
         }
     }
 }
@@ -187,72 +188,56 @@ struct DumpLane {
     int64_t rows;   // rows m0 .. m0 + rows - 1 exist
 };
 
-// The weight operand(s) of the Q4K / Q5K min term.  Tiles of up to 64 rows take the form whose operands do not depend
-// on the activations' magnitude (the block's sixteen integer sums as f16 against -dmin * min in two pieces, the result
-// in an accumulator of its own until the activation scale multiplies it with the main term): `p1`, `p2` from
-// cq_min_term_groups.  The 128-row tiles have no registers for that accumulator (measured: 100 bytes of scratch per lane
-// and 81 -> 95 us at M = 512) and keep the operand scaled by d8 in the quantizer, which accumulates straight into the
-// result: `p1` from cq_min_term_operand.
+// The weight operand of the Q4K / Q5K min term in its two f16 pieces (cq_min_term_groups): -dmin * min_{j/2} per
+// 16-element group j, contracted with the block's sixteen integer sums as f16.  No operand depends on the activations'
+// magnitude; the activation block's scale multiplies the sum of main and min term afterwards.
 struct MinW {
     v8h p1, p2;
 };
 // One block for this wave's 32 weight rows against the MT activation tiles in `cur`, as a
 // hand-laid software pipeline of 8*(MT+1) steps.  Step (t, s) issues the two int8 MFMAs of tile t,
-// K-slice s, and, in their shadow, the scaling of two of the sixteen integers of tile t-1 (VALU);
-// LDS reads run two steps ahead.  The accumulator pair alternates between two register sets.  A
-// scheduling barrier after every step keeps the compiler from hoisting all MFMAs to the front,
-// which would need MT accumulator sets at once.
-// DUMP: instead of scaling them into `out`, the block integers I (and the min term as the f16 MFMA delivers
-// it, from a zero accumulator) are stored through `dl`.
+// K-slice s, and, in their shadow, the scaling of integers of tile t-1 (VALU); LDS reads run ahead.
+// The accumulator pair alternates between two register sets.  A scheduling barrier after every step
+// keeps the compiler from hoisting all MFMAs to the front, which would need MT accumulator sets at
+// once.  Q6K: out += d8 * (I * dw), two elements a step.  Q4K / Q5K: out += d8 * (I * dw - dmin * Mn_b) with the min
+// term from two f16 MFMAs (the block's sums against -dmin * min in two pieces, all products exact) -
+//   tiles of up to 64 rows: behind the tile's last int8 MFMAs into an accumulator of its own, added where the
+//   integers are scaled (steps 1..6 of the next tile);
+//   128-row tiles (no registers for that accumulator): step 1 of the next tile turns the integers into I * dw in
+//   place - the registers of the high digits are free from then on - and the two MFMAs add to them; steps 2..7
+//   multiply by d8.
+// DUMP: instead of scaling them into `out`, the block integers I (and the min term as the f16 MFMAs deliver
+// it, times d8) are stored through `dl`.
 template <int DT, int MT, int T0, int T1, int SHIFT, bool HALF, bool DUMP>
 __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, const v4i (&bl)[8], const v4i (&bh)[8],
                                           float dw, const MinW &wmin, int lane, v16f (&out)[MT], const DumpLane &dl) {
     typedef Tile<DT, MT> T;
     if constexpr (T0 >= T1) return;
     constexpr bool MINS = is_k4(DT);
-    constexpr bool UNSCALED = MINS && min_term_unscaled<MT>();
+    constexpr bool FOLD = MINS && min_term_folded<MT>();
+    constexpr bool UNSCALED = MINS && !FOLD;
     const int h = lane >> 5, col = lane & 31;
     const uint8_t *d8p = cur + T::oD8 + h * 16;        // rows 8j + 4h + [0,4) of a tile
-    const uint8_t *mnp = cur + T::oMin + col * 32;     // this lane's row of the min term's activation operand
+    const uint8_t *mnp = cur + T::oMin + col * 32;     // this lane's row of sums (the min term's activation operand)
     // operand of tile t, K-slice s: chunk 2*(s%4) + h of K-half s/4
     auto afrag = [&](int q) -> v4i {
         const int t = q >> 3, s = q & 7;
         return *(const v4i *)(cur + g.col[s & 3] + (t * 2 + (s >> 2)) * 4096);
     };
     v16i acc_lo[2], acc_hi[2];
-    v16f mn = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};   // UNSCALED: -dmin * Mn_b of the tile being scaled
+    // up to 64 rows: -dmin * Mn_b of the tile being scaled; 128 rows: its I * dw - dmin * Mn_b
+    v16f mn = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     v4i a[3];
     v4f dreg[2];   // d8 of four rows each, read two steps before the scaling that needs them
-    v8h ma1 = {}, ma2 = {};
+    v8h ma1 = {};   // the block's sums of the tile whose min term comes next (lanes h: sums 8h .. 8h+7)
     a[(T0 * 8) % 3] = afrag(T0 * 8);
     a[(T0 * 8 + 1) % 3] = afrag(T0 * 8 + 1);
-    if (MINS && !UNSCALED) {
-        ma1 = *(const v8h *)(mnp + T0 * 1024);
-        ma2 = *(const v8h *)(mnp + T0 * 1024 + 16);
-    }
 #pragma unroll
     for (int q = T0 * 8; q < (T1 + 1) * 8; q++) {
         const int t = q >> 3, s = q & 7;
         if (q + 2 < T1 * 8) a[(q + 2) % 3] = afrag(q + 2);
         if (t < T1) {
             if (s == 0) {
-                if (MINS && !UNSCALED && !DUMP) {
-                    // min term: out -= sum_j (dmin*min_j) * (d8*bsum32_j).  K-slots 0..7 carry piece 1
-                    // of the weight factor, slots 8..15 piece 2; the activation operand carries one of
-                    // its pieces in both halves.
-                    out[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma1, wmin.p1, out[t], 0, 0, 0);
-                    out[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma2, wmin.p1, out[t], 0, 0, 0);
-                }
-                if (MINS && !UNSCALED && DUMP && dl.mn) {
-                    v16f m0 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                    m0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma1, wmin.p1, m0, 0, 0, 0);
-                    m0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma2, wmin.p1, m0, 0, 0, 0);
-#pragma unroll
-                    for (int i = 0; i < 16; i++) {
-                        const int64_t row = t * 32 + (i >> 2) * 8 + h * 4 + (i & 3);
-                        if (row < dl.rows) dl.mn[row * dl.rs] = m0[i];
-                    }
-                }
                 const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                 acc_lo[t & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[q % 3], bl[0], zero, 0, 0, 0);
                 acc_hi[t & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[q % 3], bh[0], zero, 0, 0, 0);
@@ -261,10 +246,6 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, 
                 acc_hi[t & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[q % 3], bh[s], acc_hi[t & 1], 0, 0, 0);
             }
             if (s == 6) dreg[0] = *(const v4f *)(d8p + (t * 32) * 4);
-            if (s == 6 && MINS && !UNSCALED && t + 1 < T1) {
-                ma1 = *(const v8h *)(mnp + (t + 1) * 1024);
-                ma2 = *(const v8h *)(mnp + (t + 1) * 1024 + 16);
-            }
             // UNSCALED: this tile's own min term, -dmin * sum_j bsums_j * min_{j/2} from a zero accumulator (lanes h:
             // sums 8h .. 8h+7), behind its last MFMAs; it is added where the integers are scaled, one tile later
             if (s == 6 && UNSCALED) ma1 = *(const v8h *)(mnp + t * 1024 + h * 16);
@@ -274,7 +255,7 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, 
                 mn = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma1, wmin.p2, mn, 0, 0, 0);
             }
         }
-        if (t > T0 && !UNSCALED) {
+        if (t > T0 && !MINS) {
             // scaling of two of the sixteen integers of tile t-1 per step (element i: rows 8*(i/4) + 4h + i%4)
             const int p = (t - 1) & 1;
             if ((s & 1) == 0 && s < 6) dreg[((s >> 1) + 1) & 1] = *(const v4f *)(d8p + ((t - 1) * 32 + 8 * ((s >> 1) + 1)) * 4);
@@ -290,6 +271,51 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, 
                 float o = __builtin_fmaf((float)I * dw, dreg[(i >> 2) & 1][i & 3], out[t - 1][i]);
                 asm volatile("" : "+v"(o));   // pins the scaling to this step (pure ops float otherwise)
                 out[t - 1][i] = o;
+            }
+        }
+        if (t < T1 && s == 7 && FOLD) ma1 = *(const v8h *)(mnp + t * 1024 + h * 16);   // this tile's sums, for step 1 of the next
+        if (t > T0 && FOLD) {
+            // 128-row tiles: step 1 turns the sixteen integers of tile t-1 into I * dw in place (the registers of the high
+            // digits are free from then on) and lets the min term's two MFMAs add to them; steps 2..7 multiply by d8
+            const int p = (t - 1) & 1;
+            if (s == 1) {
+                if (DUMP) {
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        const int64_t row = (t - 1) * 32 + (i >> 2) * 8 + h * 4 + (i & 3);
+                        if (row < dl.rows && !(HALF && i >= 8)) dl.i[row * dl.rs] = (acc_hi[p][i] << SHIFT) + acc_lo[p][i];
+                    }
+                    if (dl.mn) {
+                        v16f m0 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                        m0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma1, wmin.p1, m0, 0, 0, 0);
+                        m0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma1, wmin.p2, m0, 0, 0, 0);
+#pragma unroll
+                        for (int i = 0; i < 16; i++) {
+                            const int64_t row = (t - 1) * 32 + (i >> 2) * 8 + h * 4 + (i & 3);
+                            if (row < dl.rows) dl.mn[row * dl.rs] = m0[i] * *(const float *)(d8p + ((t - 1) * 32 + 8 * (i >> 2) + (i & 3)) * 4);
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 16; i++) mn[i] = (float)((acc_hi[p][i] << SHIFT) + acc_lo[p][i]) * dw;
+                    __builtin_amdgcn_sched_barrier(0);
+                    mn = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma1, wmin.p1, mn, 0, 0, 0);
+                    mn = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma1, wmin.p2, mn, 0, 0, 0);
+                }
+                dreg[1] = *(const v4f *)(d8p + ((t - 1) * 32 + 8) * 4);
+            }
+            if (s >= 2 && !DUMP) {
+                const int i0 = s < 6 ? 3 * (s - 2) : 12 + 2 * (s - 6), i1 = s < 6 ? i0 + 3 : i0 + 2;
+#pragma unroll
+                for (int i = i0; i < i1; i++) {
+                    if (!(HALF && i >= 8)) {
+                        float o = __builtin_fmaf(mn[i], dreg[(i >> 2) & 1][i & 3], out[t - 1][i]);
+                        asm volatile("" : "+v"(o));   // pins the scaling to this step (pure ops float otherwise)
+                        out[t - 1][i] = o;
+                    }
+                    if (i == 3) dreg[0] = *(const v4f *)(d8p + ((t - 1) * 32 + 16) * 4);
+                    if (i == 7) dreg[1] = *(const v4f *)(d8p + ((t - 1) * 32 + 24) * 4);
+                }
             }
         }
         if (t > T0 && UNSCALED) {
@@ -335,7 +361,7 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, 
 // Weight operands of one block: unpacks the wave's 32 rows from `wl` into the two digit operands
 // of the eight K-slices, and returns the block scale (and the Q4K min-term operand).
 __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g, const WHead<CQ_DTYPE_Q4K> &wb,
-                                             int lane, v4i (&bl)[8], v4i (&bh)[8], float &dw, MinW &wmin, bool unscaled) {
+                                             int lane, v4i (&bl)[8], v4i (&bh)[8], float &dw, MinW &wmin) {
     const int h = lane >> 5;
     dw = cq_h2f((uint16_t)(wb.dd & 0xffff));
     const uint32_t rec[4] = {wb.rec.x, wb.rec.y, wb.rec.z, wb.rec.w};   // {sc[2g], sc[2g+1], mn[2g], mn[2g+1]}
@@ -355,19 +381,14 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g
             bh[2 * gi + 1][i] = (int)pk_mul_u16(hi4, sh1);
         }
     }
-    if (unscaled) {   // (a compile-time constant at every call)
-        wmin.p1 = __builtin_bit_cast(v8h, cq_min_term_groups(wb.dd, rec, h != 0, false));
-        wmin.p2 = __builtin_bit_cast(v8h, cq_min_term_groups(wb.dd, rec, h != 0, true));
-    } else {
-        wmin.p1 = __builtin_bit_cast(v8h, cq_min_term_operand(wb.dd, rec, h != 0));
-        wmin.p2 = wmin.p1;
-    }
+    wmin.p1 = __builtin_bit_cast(v8h, cq_min_term_groups(wb.dd, rec, h != 0, false));
+    wmin.p2 = __builtin_bit_cast(v8h, cq_min_term_groups(wb.dd, rec, h != 0, true));
 }
 
 // Q5K: the Q4K nibbles plus a fifth bit per quant (words {L, H} per 32 qs bytes, bit 8c + i for byte c
 // of qs word i); scale times quant has up to 11 bits and is split as Q6K's products are.
 __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g, const WHead<CQ_DTYPE_Q5K> &wb,
-                                             int lane, v4i (&bl)[8], v4i (&bh)[8], float &dw, MinW &wmin, bool unscaled) {
+                                             int lane, v4i (&bl)[8], v4i (&bh)[8], float &dw, MinW &wmin) {
     const int h = lane >> 5;
     const uint32_t row = lane & 31;
     dw = cq_h2f((uint16_t)(wb.dd & 0xffff));
@@ -393,17 +414,12 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g
             bh[2 * gi + 1][i] = hi;
         }
     }
-    if (unscaled) {   // (a compile-time constant at every call)
-        wmin.p1 = __builtin_bit_cast(v8h, cq_min_term_groups(wb.dd, rec, h != 0, false));
-        wmin.p2 = __builtin_bit_cast(v8h, cq_min_term_groups(wb.dd, rec, h != 0, true));
-    } else {
-        wmin.p1 = __builtin_bit_cast(v8h, cq_min_term_operand(wb.dd, rec, h != 0));
-        wmin.p2 = wmin.p1;
-    }
+    wmin.p1 = __builtin_bit_cast(v8h, cq_min_term_groups(wb.dd, rec, h != 0, false));
+    wmin.p2 = __builtin_bit_cast(v8h, cq_min_term_groups(wb.dd, rec, h != 0, true));
 }
 
 __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g, const WHead<CQ_DTYPE_Q6K> &wb,
-                                             int lane, v4i (&bl)[8], v4i (&bh)[8], float &dw, MinW &wmin, bool unscaled) {
+                                             int lane, v4i (&bl)[8], v4i (&bh)[8], float &dw, MinW &wmin) {
     const int h = lane >> 5;
     dw = cq_h2f((uint16_t)wb.d);
     const uint32_t scw[4] = {wb.sc.x, wb.sc.y, wb.sc.z, wb.sc.w};
@@ -464,7 +480,7 @@ __device__ __forceinline__ void block_step(const uint8_t *__restrict__ cur, uint
     MinW wmin = {};
     if (more) stage_issue<DT, MT>(nxt, w, a, g, m0, b + 1, wave, lane);
     if (n_ok) {
-        block_unpack(wl, g, hcur, lane, bl, bh, dw, wmin, min_term_unscaled<MT>());
+        block_unpack(wl, g, hcur, lane, bl, bh, dw, wmin);
         if (more) stage_weights<DT>(wl, w, g, n_tile, b + 1);
         tiles_mac<DT, MT, 0, SPLIT, SHIFT, HALF, DUMP>(cur, g, bl, bh, dw, wmin, lane, out, dl);
     }
@@ -734,7 +750,7 @@ __global__ void __launch_bounds__(kThreads) gemm_q81_kernel(cq_weight w, cq_act_
             } else {
                 float dw;
                 MinW none;
-                block_unpack(wl, g, hcur, lane, bl, bh, dw, none, false);
+                block_unpack(wl, g, hcur, lane, bl, bh, dw, none);
                 ws[0] = weight_scale_operand(dw, h);
             }
             if (more) stage_weights<DT>(wl, w, g, n_tile, b + 1);

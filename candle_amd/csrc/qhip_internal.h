@@ -65,10 +65,9 @@ struct cq_act_view {
     int8_t *qs;
     float *d;
     int16_t *bsums;  // Q8K
-    // Q8K, for the GEMM only (block-major so that a tile of rows is contiguous per block):
+    // Q8K, for the matrix-core kernels (block-major so that a tile of rows is contiguous per block):
     float *dT;         // [k/256][m_stride] f32, the same values as d
-    uint16_t *minp;    // [k/256][m_stride][16] f16, d * sub-block sums as two f16 pieces p1[8] | p2[8] (the tile kernel's min term)
-    uint16_t *bsh;     // [k/256][m_stride][16] f16: the block's sixteen bsums as f16 (exact), the small-batch kernels' min term
+    uint16_t *bsh;     // [k/256][m_stride][16] f16: the block's sixteen bsums as f16 (exact), the min term's operand
     int64_t m_stride;  // rows allocated: at least 256 more than the rows quantized, so that the GEMM
                        // may read (and ignore) whole 128-row tiles past the last row
     int32_t *bsum32; // Q8_0 / Q8_1

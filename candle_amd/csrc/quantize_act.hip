@@ -163,21 +163,11 @@ __device__ __forceinline__ void q8k_chunk(const float4 f, int64_t row, int64_t b
         *(uint32_t *)(out.v.qs + row * k + b_in_row * 256 + 4 * lane) = packed;
         if (lane == 0) out.v.d[blk] = d;
         if ((lane & 3) == 0) out.v.bsums[blk * 16 + (lane >> 2)] = (int16_t)sum;
-        // For the matrix-core kernels (block-major copies): d again; for the small-batch kernels' min term the sixteen
-        // sums once more as f16 (at most 16 * 128 in magnitude: exact); for the tile kernel's d * (sum of the 32
-        // quants of sub-block j) as two f16 pieces p1 + p2 (22 significant bits), [p1[8] | p2[8]].
+        // For the matrix-core kernels (block-major copies): d again, and for their min term the sixteen sums once more
+        // as f16 (at most 16 * 128 in magnitude: exact), the operand of its contraction.
         const int64_t tb = b_in_row * out.v.m_stride + row;
         if (lane == 0) out.v.dT[tb] = d;
         if ((lane & 3) == 0) ((_Float16 *)out.v.bsh)[tb * 16 + (lane >> 2)] = (_Float16)(float)sum;
-        const int sum32 = sum + dpp_i<kHalfMirror>(sum);  // eight lanes = one 32-element sub-block
-        if ((lane & 7) == 0) {
-            const float v = d * (float)sum32;
-            const _Float16 p1 = (_Float16)v;
-            const _Float16 p2 = (_Float16)(v - (float)p1);
-            _Float16 *mp = (_Float16 *)out.v.minp + tb * 16;
-            mp[lane >> 3] = p1;
-            mp[8 + (lane >> 3)] = p2;
-        }
     }
 }
 

@@ -56,7 +56,7 @@ __device__ __forceinline__ void dma4(const void *base, uint32_t off, uint8_t *ld
 //         Q6K also [16 rows][4 chunks] of the 64-byte qh plane (chunk c at c ^ ((r/2)%4)),
 //         Q5K also [16 rows][32 B] of the fifth-bit plane
 //   act : [RT row groups][2 K-halves][8 rows][8 chunks], same swizzle
-//   d8  : [8*RT] f32         minp : [8*RT][16] f16: the rows' bsums (Q4K / Q5K)
+//   d8  : [8*RT] f32         bsh : [8*RT][16] f16: the rows' bsums (Q4K / Q5K)
 constexpr bool is_k4(int dt) { return dt == CQ_DTYPE_Q4K || dt == CQ_DTYPE_Q5K; }   // types with a min term
 
 template <int DT, int RT> struct Buf {
@@ -311,7 +311,7 @@ __global__ void __launch_bounds__(kThreads) skinny_kernel(cq_weight w, cq_act_vi
 // weight tiles (tile t of workgroup g: g + t * G) streaming weights only.  The launcher takes it where every
 // workgroup has one tile (n <= 16 x the number of CUs); with more tiles per workgroup it measured no faster than
 // the kernel above, also with the next tile's weights copied ahead into a second buffer (NBUF == 2).
-//   per K block b  : act [RT][2 K-halves][8 rows][8 chunks] | d8 [8*RT] f32 | minp [8*RT][16] f16 (k4 types)
+//   per K block b  : act [RT][2 K-halves][8 rows][8 chunks] | d8 [8*RT] f32 | bsh [8*RT][16] f16 (k4 types)
 //   per wave, block: weights of one tile (kWgt bytes), twice when NBUF == 2; a wave's first buffer of a tile also
 //                    carries its partial results of that tile (1 KiB per 16 activation rows)
 template <int DT, int RT> struct Res {

@@ -192,10 +192,9 @@ int cq_qmatmul_int_dots(const cq_weight *w, const float *x_dev, int64_t m, int32
  * the tile kernel of the prefill path (CQ_MFMA_TILE, with the tile height and K split cq_qmatmul picks for m;
  * Q8_0 and Q4_0 weights: more than 32 rows, as in cq_qmatmul).
  * out_i as above.  out_mn (Q4K, Q5K; else NULL) is a float: those kernels contract the min term on the f16 matrix
- * core and never hold the integer sum; it is stored as that contraction delivers it for one block.  Tile kernel:
- * -(dmin*d8) * sum_j min_j*bsum32_j from operands split in two f16 pieces each.  Small-batch kernels:
- * -dmin * sum_j min_{j/2}*bsums_j over the sixteen sums of a block (exact in f16) with -dmin*min in two f16 pieces,
- * before the activation block's scale multiplies it.  No counterpart in the reference. */
+ * core and never hold the integer sum: -dmin * sum_j min_{j/2}*bsums_j over the sixteen sums of a block (exact in
+ * f16) with -dmin*min in two f16 pieces, stored as that contraction delivers it for one block (small-batch kernels) or
+ * times the activation block's scale (tile kernel).  No counterpart in the reference. */
 #define CQ_MFMA_SKINNY 1
 #define CQ_MFMA_TILE 2
 int cq_qmatmul_int_dots_mfma(const cq_weight *w, const float *x_dev, int64_t m, int kernel, int32_t *out_i_dev,

@@ -83,9 +83,10 @@ def check_dump(qh, dt, kernel, m, k, n, seed, x_scale=1.0):
         tile = kernel == qh.MFMA_TILE
         ref, mag = min_term_reference(dt, acts, m, blocks, n, k, with_d8=tile)
         got = om.cpu().numpy().astype(np.float64)
-        # tile kernel: two f16 pieces per factor, 2^-22 per product and the f32 rounding of the eight-term sum; small
-        # batch: the sums exact in f16, -dmin*min_j in two f16 pieces, every product exact, only the f32 sum rounds
-        bound = 2.0 ** -19 if tile else 2.0 ** -21
+        # the sums exact in f16, -dmin*min_j in two f16 pieces: every product exact, the f32 sum of the 32 terms rounds
+        # (tile kernel: stored times d8, one more rounding; its 128-row tiles add the terms to I * dw, which the dump
+        # leaves out)
+        bound = 2.0 ** -20 if tile else 2.0 ** -21
         assert np.all(np.abs(got - ref) <= bound * mag + 1e-30), float((np.abs(got - ref) / (mag + 1e-30)).max())
     return x, blocks, qw
 
@@ -113,34 +114,30 @@ def test_tile_kernel_integers(qh, dt, m, k, n):
     check_dump(qh, dt, qh.MFMA_TILE, m, k, n, 13 * dt + m + k + n)
 
 
-@pytest.mark.parametrize("kernel,x_scale", [(kn, v) for kn in ("skinny", "tile64") for v in (1e-30, 1e-8, 1e-2, 1.0, 500.0, 1e6, 1e30)] +
-                         [("tile", v) for v in (1e-2, 1.0, 30.0, 500.0)])
+@pytest.mark.parametrize("x_scale", [1e-30, 1e-8, 1e-2, 1.0, 500.0, 1e6, 1e30])
+@pytest.mark.parametrize("kernel", ["skinny", "tile64", "tile"])
 def test_min_term_error_bound_across_magnitudes(qh, kernel, x_scale):
-    """Small-batch kernels and tiles of up to 64 rows (a call of at most 64 rows has no others): the min term's
-    matrix-core operands are the integer sums of the block and -dmin*min_j, the activation block's scale multiplies
-    afterwards in f32, so the bound holds for activations of any magnitude.  128-row tiles: the operand d8 * bsum32 in
-    two f16 pieces keeps its bound from a hundred times smaller to five hundred times larger than unit variance (it
-    leaves the f16 range for activations beyond about 2000 throughout a sub-block, and the pieces lose bits below about
-    1e-3: the documented range of those tiles)."""
+    """The min term's matrix-core operands are the integer sums of the block and -dmin*min_j; the activation block's
+    scale multiplies afterwards in f32: the bound holds for activations of any magnitude, in the small-batch kernels,
+    in tiles of up to 64 rows (an accumulator of their own) and in the 128-row tiles (the scaled integers as the
+    accumulator)."""
     kid = qh.MFMA_SKINNY if kernel == "skinny" else qh.MFMA_TILE
-    m = {"skinny": 16, "tile64": 56, "tile": 70}[kernel]
-    check_dump(qh, orc.Q4K, kid, m, 1024, 64, 5, x_scale)
+    m, n = {"skinny": (16, 64), "tile64": (56, 64), "tile": (300, 2048)}[kernel]
+    check_dump(qh, orc.Q4K, kid, m, 1024, n, 5, x_scale)
 
 
 @pytest.mark.parametrize("dt", [orc.Q4K, orc.Q5K, orc.Q6K])
-@pytest.mark.parametrize("m,k,n", [(16, 2048, 64), (60, 1024, 96), (70, 1024, 96), (512, 512, 64)])
+@pytest.mark.parametrize("m,k,n", [(16, 2048, 64), (60, 1024, 96), (70, 1024, 96), (512, 512, 64), (300, 1024, 2048)])
 def test_rows_of_different_magnitudes(qh, dt, m, k, n):
-    """One batch whose rows span five orders of magnitude (0.01 .. 1000; forty, 1e-20 .. 1e20, for the small-batch
-    kernels and the tile kernel on at most 64 rows), one row with a block a thousand times the others and one all-zero
-    row: every row against the oracle at the usual bars, on both matrix-core kernels."""
+    """One batch whose rows span forty orders of magnitude (1e-20 .. 1e20), one row with a block a thousand times the
+    others and one all-zero row: every row against the oracle at the usual bars, on both matrix-core kernels."""
     rng = np.random.default_rng(m + k + n + int(dt))
     w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
     x = rng.standard_normal((m, k)).astype(np.float32)
     blocks = orc.quantize(dt, w)
     qw = qh.QWeight.from_ggml(dt, blocks, n, k)
     x0 = x
-    wide = (-20, 21)      # the small-batch kernels and tiles of up to 64 rows (all a call of at most 64 rows has)
-    for flags, lo, hi in ((qh.FLAG_FORCE_SKINNY,) + wide, (qh.FLAG_FORCE_GEMM,) + (wide if m <= 64 else (-2, 4))):
+    for flags, lo, hi in ((qh.FLAG_FORCE_SKINNY, -20, 21), (qh.FLAG_FORCE_GEMM, -20, 21)):
         scales = np.float32(10.0) ** rng.integers(lo, hi, size=m).astype(np.float32)
         scales[2] = 1.0
         x = x0 * scales[:, None]
@@ -153,6 +150,33 @@ def test_rows_of_different_magnitudes(qh, dt, m, k, n):
             nrm = np.linalg.norm(want[r])
             assert np.linalg.norm(got[r] - want[r]) <= 1e-4 * nrm + 1e-38, (flags, r, float(scales[r]))
             assert np.abs(got[r] - want[r]).max() <= 1e-3 * nrm + 1e-38, (flags, r)
+
+
+@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q5K])
+def test_tall_tiles_rows_of_different_magnitudes(qh, dt):
+    """A launch of 128-row tiles (512 rows on 16 384 weight rows: more 32-row tiles than four rounds of compute units) with
+    rows forty orders of magnitude apart: every row against the dot-product kernels, which hold the min term as an
+    integer, and sampled weight rows against the oracle."""
+    rng = np.random.default_rng(9 + int(dt))
+    m, k, n = 512, 512, 16384
+    gen = torch.Generator(device="cuda").manual_seed(int(dt))
+    qw = qh.QWeight.zeros(dt, n, k).quantize_(torch.randn((n, k), generator=gen, device="cuda") * 0.02)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    x *= (np.float32(10.0) ** rng.integers(-20, 21, size=m).astype(np.float32))[:, None]
+    x[7] = 0.0
+    xd = dev(x)
+    got = qh.qmatmul(qw, xd, qh.FLAG_FORCE_GEMM)
+    ref = qh.qmatmul(qw, xd, qh.FLAG_FORCE_MATVEC)
+    assert bool(torch.isfinite(got).all())
+    err = (got.double() - ref.double()).norm(dim=1)
+    nrm = ref.double().norm(dim=1)
+    assert bool((err <= 1e-5 * nrm + 1e-38).all()), float((err / (nrm + 1e-38)).max())
+    cols = np.unique(np.concatenate([[0, 255, 256, n - 1], rng.choice(n, size=20, replace=False)]))
+    blocks = qw.to_ggml().reshape(n, -1)[cols].ravel()
+    want = orc.matmul(dt, x, blocks, len(cols)).astype(np.float64)
+    sub = got[:, torch.from_numpy(cols).cuda()].cpu().numpy().astype(np.float64)
+    for r in range(m):
+        assert np.linalg.norm(sub[r] - want[r]) <= 1e-4 * np.linalg.norm(want[r]) + 1e-38, r
 
 
 @pytest.mark.parametrize("dt", [orc.Q4K, orc.Q5K])
