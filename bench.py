@@ -66,6 +66,9 @@ def envelope() -> int:
     vp = C.c_void_p
     P.cqp_empty.argtypes = [C.c_int, C.c_int, C.c_int, vp, vp]
     P.cqp_stream_read.argtypes = [vp, C.c_size_t, C.c_int, C.c_int, C.c_int, vp, vp]
+    P.cqp_stream_read_pol.argtypes = [vp, C.c_size_t, C.c_int, C.c_int, C.c_int, vp, vp]
+    P.cqp_lds_read.argtypes = [vp, C.c_size_t, C.c_int, C.c_int, C.c_int, vp, vp]
+    P.cqp_lds_read_rows.argtypes = [vp, C.c_size_t, C.c_int, C.c_int, vp, vp]
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     sink = torch.zeros(4, dtype=torch.int32, device=dev)
@@ -120,6 +123,27 @@ def envelope() -> int:
                 us = timed(launch, graph)
                 row[f"grid{grid}_block{block}_u{unroll}_{mode}_us"] = round(us, 3)
                 row[f"grid{grid}_block{block}_u{unroll}_{mode}_GBs"] = round(nbytes / us / 1e3, 1)
+        # cache-policy bits on the loads (1 = sc0, 2 = nt, 16 = sc1), graph replay only
+        for aux in (0, 1, 2, 3, 16, 17, 18, 19):
+            def launch(i, s, aux=aux):
+                rc = P.cqp_stream_read_pol(vp(pool.data_ptr() + (i % slots) * span), nbytes, 2048, 256, aux,
+                                           vp(sink.data_ptr()), s)
+                assert rc == 0, rc
+            row[f"bufload_aux{aux}_graph_us"] = round(timed(launch, True), 3)
+        # requests that land in LDS, a ring of 1-KiB slots per wave (8 waves per workgroup)
+        for grid, ring, aux in ((256, 4, 0), (256, 8, 0), (256, 16, 0), (512, 8, 0), (512, 4, 0), (256, 16, 2), (256, 8, 2),
+                                (256, 16, 16)):
+            def launch(i, s, grid=grid, ring=ring, aux=aux):
+                rc = P.cqp_lds_read(vp(pool.data_ptr() + (i % slots) * span), nbytes, grid, ring, aux,
+                                    vp(sink.data_ptr()), s)
+                assert rc == 0, rc
+            row[f"lds_grid{grid}_ring{ring}_aux{aux}_graph_us"] = round(timed(launch, True), 3)
+        # the same requests with a wave owning whole rows of P consecutive KiB (the decode kernels' ownership)
+        for ppr in (1, 2, 3, 6, 9):
+            def launch(i, s, ppr=ppr):
+                rc = P.cqp_lds_read_rows(vp(pool.data_ptr() + (i % slots) * span), nbytes, 256, ppr, vp(sink.data_ptr()), s)
+                assert rc == 0, rc
+            row[f"lds_rows_of_{ppr}KiB_ring8_aux2_graph_us"] = round(timed(launch, True), 3)
         out["stream_read"][name] = row
     print(json.dumps(out), flush=True)
     return 0

@@ -681,10 +681,12 @@ extern "C" int cq_qmatmul_int_dots_mfma(const cq_weight *w, const float *x_dev, 
     if (rc || m == 0 || w->n == 0 || w->k == 0) return rc;
     const int act = cq_vec_dot_type(w->dtype);
     const bool kquant = w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q5K || w->dtype == CQ_DTYPE_Q6K;
+    const int int_min = kernel & CQ_MFMA_INT_MIN;
+    kernel &= ~CQ_MFMA_INT_MIN;
     bool ok = false;
     if (kernel == CQ_MFMA_SKINNY) ok = cq_skinny_supported(w, act);
     else if (kernel == CQ_MFMA_TILE) ok = kquant ? cq_gemm_supported(w, m, act) : m > 32 && cq_gemm32_supported(w, act);   // as cq_qmatmul
-    else return cq_set_error(CQ_ERR_INVALID, "kernel must be CQ_MFMA_SKINNY or CQ_MFMA_TILE");
+    else return cq_set_error(CQ_ERR_INVALID, "kernel must be CQ_MFMA_SKINNY or CQ_MFMA_TILE (plus CQ_MFMA_INT_MIN)");
     if (!ok) return cq_set_error(CQ_ERR_UNSUPPORTED, "that kernel does not take this weight (dtype %d, %lld x %lld) with %lld rows", w->dtype,
                                  (long long)w->n, (long long)w->k, (long long)m);
     CQ_HIP_CHECK(hipSetDevice(w->dev));
@@ -692,7 +694,7 @@ extern "C" int cq_qmatmul_int_dots_mfma(const cq_weight *w, const float *x_dev, 
     cq_act_view v;
     act_ws_layout(act, m, w->k, (uint8_t *)ws, &v);
     CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, nullptr, m, w->k, cq_no_pre(), v, cq_no_clear(), s));
-    const cq_mfma_dump d{out_i, (w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q5K) ? out_mn : nullptr};
+    const cq_mfma_dump d{out_i, (w->dtype == CQ_DTYPE_Q4K || w->dtype == CQ_DTYPE_Q5K) ? out_mn : nullptr, int_min};
     if (kernel == CQ_MFMA_SKINNY) CQ_HIP_CHECK(cq_launch_skinny_dump(w, v, act, m, d, s));
     else if (kquant) CQ_HIP_CHECK(cq_launch_gemm_dump(w, v, act, m, d, s));
     else CQ_HIP_CHECK(cq_launch_gemm32_dump(w, v, act, m, d, s));

@@ -186,6 +186,7 @@ struct DumpLane {
     float *mn;      // the same of cq_mfma_dump::mn, or null
     int64_t rs;     // elements between two activation rows
     int64_t rows;   // rows m0 .. m0 + rows - 1 exist
+    bool int_min;   // mn receives the integer Mn_b (the operands are then the minima themselves), without the activation scale
 };
 
 // The weight operand of the Q4K / Q5K min term in its two f16 pieces (cq_min_term_groups): -dmin * min_{j/2} per
@@ -292,7 +293,7 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, 
 #pragma unroll
                         for (int i = 0; i < 16; i++) {
                             const int64_t row = (t - 1) * 32 + (i >> 2) * 8 + h * 4 + (i & 3);
-                            if (row < dl.rows) dl.mn[row * dl.rs] = m0[i] * *(const float *)(d8p + ((t - 1) * 32 + 8 * (i >> 2) + (i & 3)) * 4);
+                            if (row < dl.rows) dl.mn[row * dl.rs] = dl.int_min ? m0[i] : m0[i] * *(const float *)(d8p + ((t - 1) * 32 + 8 * (i >> 2) + (i & 3)) * 4);
                         }
                     }
                 } else {
@@ -329,7 +330,7 @@ __device__ __forceinline__ void tiles_mac(const uint8_t *cur, const LaneGeo &g, 
                     for (int i = 0; i < 16; i++) {
                         const int64_t row = (t - 1) * 32 + (i >> 2) * 8 + h * 4 + (i & 3);
                         // (stored with the activation scale, like the 128-row tiles' term)
-                        if (row < dl.rows) dl.mn[row * dl.rs] = mn[i] * *(const float *)(d8p + ((t - 1) * 32 + 8 * (i >> 2) + (i & 3)) * 4);
+                        if (row < dl.rows) dl.mn[row * dl.rs] = dl.int_min ? mn[i] : mn[i] * *(const float *)(d8p + ((t - 1) * 32 + 8 * (i >> 2) + (i & 3)) * 4);
                     }
                 }
             }
@@ -481,6 +482,13 @@ __device__ __forceinline__ void block_step(const uint8_t *__restrict__ cur, uint
     if (more) stage_issue<DT, MT>(nxt, w, a, g, m0, b + 1, wave, lane);
     if (n_ok) {
         block_unpack(wl, g, hcur, lane, bl, bh, dw, wmin);
+        if constexpr (DUMP && is_k4(DT)) {
+            if (dl.int_min) {   // verification: the minima themselves as the operand, so the MFMAs deliver the integer Mn_b
+                const uint32_t rec[4] = {hcur.rec.x, hcur.rec.y, hcur.rec.z, hcur.rec.w};
+                wmin.p1 = __builtin_bit_cast(v8h, cq_min_term_groups_int(rec, (lane >> 5) != 0, false));
+                wmin.p2 = __builtin_bit_cast(v8h, cq_min_term_groups_int(rec, (lane >> 5) != 0, true));
+            }
+        }
         if (more) stage_weights<DT>(wl, w, g, n_tile, b + 1);
         tiles_mac<DT, MT, 0, SPLIT, SHIFT, HALF, DUMP>(cur, g, bl, bh, dw, wmin, lane, out, dl);
     }
@@ -495,7 +503,7 @@ __device__ __forceinline__ void block_step(const uint8_t *__restrict__ cur, uint
 // blockIdx.x, K blocks of part blockIdx.z.
 template <int DT, int MT, bool DUMP = false>
 __device__ __forceinline__ void gemm_body(const cq_weight &w, const cq_act_view &a, int64_t m0, int64_t m,
-                                          float *__restrict__ y, int ksplit, cq_mfma_dump dump = cq_mfma_dump{nullptr, nullptr}) {
+                                          float *__restrict__ y, int ksplit, cq_mfma_dump dump = cq_mfma_dump{nullptr, nullptr, 0}) {
     typedef Tile<DT, MT> T;
     extern __shared__ __align__(16) uint8_t smem[];
     const int lane = threadIdx.x & 63;
@@ -537,10 +545,10 @@ __device__ __forceinline__ void gemm_body(const cq_weight &w, const cq_act_view 
         for (int64_t b = b0; b < b1; b++) {
             const bool more = b + 1 < b1;
             if (more) load_head(w, nc * kb + b + 1, hnxt);
-            DumpLane dl{nullptr, nullptr, 0, 0};
+            DumpLane dl{nullptr, nullptr, 0, 0, false};
             if (DUMP) {
                 const int64_t at = (m0 * w.n + nc) * kb + b;
-                dl = DumpLane{dump.i + at, dump.mn ? dump.mn + at : nullptr, w.n * kb, m - m0};
+                dl = DumpLane{dump.i + at, dump.mn ? dump.mn + at : nullptr, w.n * kb, m - m0, dump.int_min != 0};
             }
             block_step<DT, MT, decltype(trail)::value, decltype(half)::value, DUMP>(smem + ic * T::kBytes, smem + in * T::kBytes,
                                                                                     wl, w, a, g, m0, n_tile, n_ok, more, b, wave,

@@ -411,22 +411,23 @@ template <int DT> __device__ __forceinline__ RowPtr row_ptr(const cq_weight &w, 
 }
 
 template <int DT> __device__ __forceinline__ void load_unit(const RowPtr &rp, uint32_t u, UnitRaw<DT> &o) {
+    // streaming (non-temporal) loads: every weight byte is read once per launch
     if (is_k4(DT)) {
-        o.q = *(const uint4 *)(rp.p0 + u * 32u);
-        o.q2 = *(const uint4 *)(rp.p0 + u * 32u + 16u);
+        o.q = cq_ld_stream16(rp.p0 + u * 32u);
+        o.q2 = cq_ld_stream16(rp.p0 + u * 32u + 16u);
         const uint8_t *h = rp.p1 + (u >> 2) * (uint32_t)CQ_Q4K_HDR;
-        o.h.x = *(const uint32_t *)h;
-        o.h.y = *(const uint32_t *)(h + 4u + (u & 3u) * 4u);
-        if (DT == CQ_DTYPE_Q5K) o.hh = *(const uint2 *)(rp.p2 + u * 8u);
+        o.h.x = cq_ld_stream4(h);
+        o.h.y = cq_ld_stream4(h + 4u + (u & 3u) * 4u);
+        if (DT == CQ_DTYPE_Q5K) o.hh = cq_ld_stream8(rp.p2 + u * 8u);
         return;
     }
-    o.q = *(const uint4 *)(rp.p0 + u * 16u);
-    if (DT == CQ_DTYPE_Q4_0) o.d = *(const uint16_t *)(rp.p1 + u * 2u);
-    if (DT == CQ_DTYPE_Q8_0) o.d = *(const uint16_t *)(rp.p1 + (u >> 1) * 2u);
+    o.q = cq_ld_stream16(rp.p0 + u * 16u);
+    if (DT == CQ_DTYPE_Q4_0) o.d = cq_ld_stream2(rp.p1 + u * 2u);
+    if (DT == CQ_DTYPE_Q8_0) o.d = cq_ld_stream2(rp.p1 + (u >> 1) * 2u);
     if (DT == CQ_DTYPE_Q6K) {
-        o.hh = *(const uint2 *)(rp.p1 + u * 8u);
-        o.sc2 = *(const uint16_t *)(rp.p2 + u * 2u);
-        o.d = *(const uint16_t *)(rp.p3 + (u >> 3) * 2u);
+        o.hh = cq_ld_stream8(rp.p1 + u * 8u);
+        o.sc2 = cq_ld_stream2(rp.p2 + u * 2u);
+        o.d = cq_ld_stream2(rp.p3 + (u >> 3) * 2u);
     }
 }
 

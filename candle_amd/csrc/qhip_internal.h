@@ -172,6 +172,7 @@ hipError_t cq_launch_matvec_fused_multi(const cq_weight *const *ws, int count, c
 struct cq_mfma_dump {
     int32_t *i;
     float *mn;
+    int int_min;   // store the integer Mn_b = sum_j min_j * bsum32_j (exact in f32) instead of the float min term
 };
 hipError_t cq_launch_gemm_dump(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, cq_mfma_dump d, hipStream_t s);
 hipError_t cq_launch_gemm32_dump(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, cq_mfma_dump d, hipStream_t s);
@@ -253,6 +254,23 @@ __device__ __forceinline__ uint16_t cq_f2h(float f) {  // round-to-nearest-even
     __builtin_memcpy(&h, &v, 2);
     return h;
 }
+// ---- streaming loads ------------------------------------------------------------------------
+// Weight bytes are read once per launch: loads marked non-temporal (the `nt` bit of the load) do not displace what
+// the caches hold for later use, and on this part a launch that only reads runs 5-12 % faster with it
+// (9.4 MB: 3.13 -> 2.78 us, 25 MB: 5.45 -> 5.04 us, 107 MB: 19.6 -> 18.6 us per graph node).
+typedef uint32_t cq_u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t cq_u32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint4 cq_ld_stream16(const void *p) {
+    const cq_u32x4_t v = __builtin_nontemporal_load((const cq_u32x4_t *)p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint2 cq_ld_stream8(const void *p) {
+    const cq_u32x2_t v = __builtin_nontemporal_load((const cq_u32x2_t *)p);
+    return make_uint2(v.x, v.y);
+}
+__device__ __forceinline__ uint32_t cq_ld_stream4(const void *p) { return __builtin_nontemporal_load((const uint32_t *)p); }
+__device__ __forceinline__ uint16_t cq_ld_stream2(const void *p) { return __builtin_nontemporal_load((const uint16_t *)p); }
+
 // ------------------------------------------------------------------ wave reductions (DPP) ----
 template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
@@ -352,6 +370,23 @@ __device__ __forceinline__ cq_u32x4 cq_min_term_groups(uint32_t dd, const uint32
         const uint32_t u = second ? __builtin_bit_cast(uint32_t, p2) : __builtin_bit_cast(uint32_t, p1);
         out[2 * g] = __builtin_amdgcn_perm(u, u, 0x01000100u);       // sub-block 2g' twice
         out[2 * g + 1] = __builtin_amdgcn_perm(u, u, 0x03020302u);   // sub-block 2g'+1 twice
+    }
+    return out;
+}
+
+// Verification form of the operand above: the group minima themselves (first piece; the second is zero), so that the
+// same MFMAs deliver the integer sum_j bsums_j * min_{j/2} = Mn_b (at most 16 * 2048 * 63: exact in f32).
+__device__ __forceinline__ cq_u32x4 cq_min_term_groups_int(const uint32_t (&rec)[4], bool half, bool second) {
+    const cq_half2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+    cq_u32x4 out;
+#pragma unroll
+    for (int g = 0; g < 2; g++) {
+        const uint32_t rg = half ? rec[2 + g] : rec[g];
+        const uint32_t n2 = __builtin_amdgcn_perm(rg, 0u, 0x0c070c06u) | 0x64006400u;   // the two min bytes as 1024 + n
+        const cq_half2 mn = __builtin_bit_cast(cq_half2, n2) - k1024;
+        const uint32_t u = second ? 0u : __builtin_bit_cast(uint32_t, mn);
+        out[2 * g] = __builtin_amdgcn_perm(u, u, 0x01000100u);
+        out[2 * g + 1] = __builtin_amdgcn_perm(u, u, 0x03020302u);
     }
     return out;
 }

@@ -242,6 +242,12 @@ __global__ void __launch_bounds__(kThreads) skinny_kernel(cq_weight w, cq_act_vi
         float dw;
         v8h wmin;
         block_unpack(buf, lane, head, bl, bh, dw, wmin);
+        if constexpr (DUMP && is_k4(DT)) {
+            if (dump.int_min) {   // verification: the minima themselves as the operand: the MFMA delivers the integer Mn_b
+                const uint32_t rec[4] = {head.rec.x, head.rec.y, head.rec.z, head.rec.w};
+                wmin = __builtin_bit_cast(v8h, cq_min_term_groups_int(rec, (kq & 1) != 0, (kq >> 1) != 0));
+            }
+        }
 #pragma unroll
         for (int t = 0; t < NT; t++) {
             const v4f d8 = *(const v4f *)(buf + B::oD8 + (t * 16 + 4 * kq < 8u * RT ? t * 16 + 4 * kq : 0) * 4);
@@ -359,6 +365,12 @@ __device__ __forceinline__ void res_block(const uint8_t *__restrict__ wl, const 
     float dw;
     v8h wmin;
     block_unpack(wl, lane, head, bl, bh, dw, wmin);
+    if constexpr (DUMP && is_k4(DT)) {
+        if (dump.int_min) {   // verification: the minima themselves as the operand: the MFMA delivers the integer Mn_b
+            const uint32_t rec[4] = {head.rec.x, head.rec.y, head.rec.z, head.rec.w};
+            wmin = __builtin_bit_cast(v8h, cq_min_term_groups_int(rec, (kq & 1) != 0, (kq >> 1) != 0));
+        }
+    }
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         const v4f d8 = *(const v4f *)(act + R::oD8 + (t * 16 + 4 * kq < 8u * RT ? t * 16 + 4 * kq : 0) * 4);
@@ -963,7 +975,7 @@ bool cq_skinny_supported(const cq_weight *w, int act_dtype) {
 }
 
 hipError_t cq_launch_skinny(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s) {
-    return launch_any<false>(w, a, act_dtype, m, y, cq_mfma_dump{nullptr, nullptr}, s);
+    return launch_any<false>(w, a, act_dtype, m, y, cq_mfma_dump{nullptr, nullptr, 0}, s);
 }
 
 hipError_t cq_launch_skinny_dump(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, cq_mfma_dump d, hipStream_t s) {

@@ -379,6 +379,7 @@ def qmatmul_int_dots(w: QWeight, x):
 
 
 MFMA_SKINNY, MFMA_TILE = 1, 2
+MFMA_INT_MIN = 16   # added to either: the min-term contraction delivers the integer Mn_b
 
 
 def qmatmul_int_dots_mfma(w: QWeight, x, kernel: int):

@@ -72,7 +72,8 @@ enum {
                                  activations quantized by BlockQ8_1::from_float (k_quants.rs:665-691), instead of the
                                  CPU formulation's Q8K.  A dot-product kernel up to 32 rows, the matrix cores beyond; combines with
                                  CQ_FLAG_REUSE_ACT only; the grouped calls do not take it.  Its results differ from
-                                 the CPU QMatMul's by the two activation quantizers' noise (about 1e-3 relative).    */
+                                 the CPU QMatMul's by the two activation quantizers' noise (about 1e-2 relative:
+                                 rel-L2 8.7e-3 measured on M = 512, K = 4096 activations with 1 % outliers).         */
     CQ_FLAG_REUSE_ACT = 8,    /* the workspace already holds this x, quantized by an earlier cq_qmatmul call with the
                                  same m, k and activation format (q/k/v or gate/up share their input): skip the
                                  quantizer launch.  The earlier call must have gone through the workspace: more than
@@ -194,9 +195,13 @@ int cq_qmatmul_int_dots(const cq_weight *w, const float *x_dev, int64_t m, int32
  * out_i as above.  out_mn (Q4K, Q5K; else NULL) is a float: those kernels contract the min term on the f16 matrix
  * core and never hold the integer sum: -dmin * sum_j min_{j/2}*bsums_j over the sixteen sums of a block (exact in
  * f16) with -dmin*min in two f16 pieces, stored as that contraction delivers it for one block (small-batch kernels) or
- * times the activation block's scale (tile kernel).  No counterpart in the reference. */
+ * times the activation block's scale (tile kernel).  With CQ_MFMA_INT_MIN added to `kernel` the weight operand of
+ * that contraction is the group minima themselves instead of -dmin * min, and out_mn receives the integer
+ * Mn_b = sum_j min_{j/2} * bsums_j of k_quants.rs:1221-1241 (at most 16 * 2048 * 63, exact in a float): the same
+ * instructions on the same sums, checked bit for bit.  No counterpart in the reference. */
 #define CQ_MFMA_SKINNY 1
 #define CQ_MFMA_TILE 2
+#define CQ_MFMA_INT_MIN 16
 int cq_qmatmul_int_dots_mfma(const cq_weight *w, const float *x_dev, int64_t m, int kernel, int32_t *out_i_dev,
                              float *out_mn_dev, void *workspace_dev, size_t workspace_bytes, void *stream);
 

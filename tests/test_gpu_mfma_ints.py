@@ -88,6 +88,11 @@ def check_dump(qh, dt, kernel, m, k, n, seed, x_scale=1.0):
         # leaves out)
         bound = 2.0 ** -20 if tile else 2.0 ** -21
         assert np.all(np.abs(got - ref) <= bound * mag + 1e-30), float((np.abs(got - ref) / (mag + 1e-30)).max())
+        # the same launch with the minima themselves as the weight operand of that contraction: the integer Mn_b of
+        # k_quants.rs:1221-1241, bit for bit (same instructions, same sums; at most 16 * 2048 * 63: exact in f32)
+        oi2, om2 = qh.qmatmul_int_dots_mfma(qw, dev(x), kernel | qh.MFMA_INT_MIN)
+        assert np.array_equal(oi2.cpu().numpy(), wi)
+        assert np.array_equal(om2.cpu().numpy().astype(np.int64), wm.astype(np.int64))
     return x, blocks, qw
 
 
@@ -233,6 +238,13 @@ def test_tile_kernel_integers_config3(qh, dt, k, n):
         ref, mag = min_term_reference(dt, acts, len(ms), blocks, len(cols), k, with_d8=True)
         got = om[torch.from_numpy(ms).cuda()][:, torch.from_numpy(cols).cuda()].cpu().numpy().astype(np.float64)
         assert np.all(np.abs(got - ref) <= 2.0 ** -19 * mag + 1e-30)
+        # the integer Mn_b of every (row, weight row, block) of the launch against the dot-product kernels' (on the
+        # device) and, on the sampled rows, the oracle's
+        del oi, om
+        _, om2 = qh.qmatmul_int_dots_mfma(qw, xd, qh.MFMA_TILE | qh.MFMA_INT_MIN)
+        assert bool(torch.equal(om2.to(torch.int32), rm))
+        sub = om2[torch.from_numpy(ms).cuda()][:, torch.from_numpy(cols).cuda()].cpu().numpy()
+        assert np.array_equal(sub.astype(np.int64), wm.astype(np.int64))
         # whole launch: the float min term against the dot-product kernels' integer through the scales is covered by
         # the f32 comparison of the results in test_prefill_gemm_config3
 

@@ -453,10 +453,10 @@ def test_reference_goldens_through_hip(qh, goldens, seeded_inputs):
     qw = qh.QWeight.from_ggml(orc.Q4_0, orc.quantize(orc.Q4_0, rhs), n, k)
     got = qh.qmatmul(qw, dev(lhs)).cpu().numpy()
     assert np.round(got).ravel().tolist() == goldens["q4_0_matmul_neg_m3_k64_n4"]["rounded"]
-    # quantized_tests.rs:1051-1151 (seeded m=11, k=512, n=21), weights quantized on the device
+    # quantized_tests.rs:998-1151 (seeded m=11, k=512, n=21), weights quantized on the device
     g = goldens["seeded_matmul_m11_k512_n21"]
     lhs, rhs = seeded_inputs
-    for name, dt in (("q4k", orc.Q4K), ("q5k", orc.Q5K), ("q6k", orc.Q6K)):
+    for name, dt in (("q2k", orc.Q2K), ("q3k", orc.Q3K), ("q4k", orc.Q4K), ("q5k", orc.Q5K), ("q6k", orc.Q6K)):
         qw = qh.QWeight.zeros(dt, 21, 512).quantize_(dev(rhs))
         out = qh.qmatmul(qw, dev(lhs)).cpu().numpy().ravel()
         spot = [float(np.round(np.float32(1000.0) * out[i]) / np.float32(1000.0)) for i in g["flat_indices"]]

@@ -150,7 +150,7 @@ def test_dot_product_error(goldens, name):
 
 
 # ------------------------------------- G7: seeded full path m=11,k=512,n=21 ----
-@pytest.mark.parametrize("name", ["q4k", "q5k", "q6k", "q8k"])
+@pytest.mark.parametrize("name", ["q2k", "q3k", "q4k", "q5k", "q6k", "q8k"])
 def test_seeded_matmul_golden(goldens, seeded_inputs, name):
     g = goldens["seeded_matmul_m11_k512_n21"]
     lhs, rhs = seeded_inputs
@@ -526,6 +526,70 @@ def test_int_dots_and_matmul_bruteforce(name):
     # and the quantized product approximates the f32 product within quantization noise
     mm = lhs.astype(np.float64) @ rhs.astype(np.float64).T
     assert np.linalg.norm(out - mm) / np.linalg.norm(mm) < {"q3k": 0.25, "q2k": 0.45}.get(name, 0.12)   # two and three bits are noisier
+
+
+def q8_1_formula_float64(dt, x, blocks, n, k):
+    """The formula in float64 from independently unpacked blocks: every integer exact, no f32 rounding."""
+    m = x.shape[0]
+    a = np.stack([orc.quantize(orc.Q8_1, x[r]) for r in range(m)]).reshape(m, k // 32, 36)
+    d8 = a[..., :2].copy().view(np.float16)[..., 0].astype(np.float64)
+    s8 = a[..., 2:4].copy().view(np.float16)[..., 0].astype(np.float64)
+    q8 = a[..., 4:].copy().view(np.int8).astype(np.int64)                      # [m, k/32, 32]
+    kb = k // 256
+    if dt == orc.Q4K:
+        w = blocks.reshape(n, kb, 144)
+        d = w[..., 0:2].copy().view(np.float16)[..., 0].astype(np.float64)
+        dmin = w[..., 2:4].copy().view(np.float16)[..., 0].astype(np.float64)
+        sc12 = w[..., 4:16].astype(np.int64)
+        sc = np.zeros((n, kb, 8), np.int64)
+        mn = np.zeros((n, kb, 8), np.int64)
+        for j in range(8):                                                     # get_scale_min_k4, utils.rs:49-59
+            if j < 4:
+                sc[..., j] = sc12[..., j] & 63
+                mn[..., j] = sc12[..., j + 4] & 63
+            else:
+                sc[..., j] = (sc12[..., j + 4] & 0xF) | ((sc12[..., j - 4] >> 6) << 4)
+                mn[..., j] = (sc12[..., j + 4] >> 4) | ((sc12[..., j] >> 6) << 4)
+        qs = w[..., 16:].astype(np.int64).reshape(n, kb, 4, 32)
+        q = np.stack([qs & 15, qs >> 4], axis=3).reshape(n, kb, 8, 32)       # sub-blocks 2g (low), 2g + 1 (high)
+        dots = np.einsum("nbjl,mbjl->mnbj", q, q8.reshape(m, kb, 8, 32))
+        sd = (dots * sc[None] * d8.reshape(m, 1, kb, 8)).sum(-1)
+        sm = (mn[None] * s8.reshape(m, 1, kb, 8)).sum(-1)
+        return (d[None] * sd - dmin[None] * sm).sum(-1)
+    w = blocks.reshape(n, kb, 210)
+    ql = w[..., :128].astype(np.int64).reshape(n, kb, 2, 64)
+    qh = w[..., 128:192].astype(np.int64).reshape(n, kb, 2, 32)
+    scl = w[..., 192:208].copy().view(np.int8).astype(np.int64)
+    d = w[..., 208:210].copy().view(np.float16)[..., 0].astype(np.float64)
+    q = np.zeros((n, kb, 2, 128), np.int64)                                    # k_quants.rs:1716-1746
+    for half in range(2):
+        l = np.arange(32)
+        q[:, :, half, l] = (ql[:, :, half, l] & 15) | (((qh[:, :, half, l] >> 0) & 3) << 4)
+        q[:, :, half, l + 32] = (ql[:, :, half, l + 32] & 15) | (((qh[:, :, half, l] >> 2) & 3) << 4)
+        q[:, :, half, l + 64] = (ql[:, :, half, l] >> 4) | (((qh[:, :, half, l] >> 4) & 3) << 4)
+        q[:, :, half, l + 96] = (ql[:, :, half, l + 32] >> 4) | (((qh[:, :, half, l] >> 6) & 3) << 4)
+    q = (q.reshape(n, kb, 16, 16) - 32)
+    dots = np.einsum("nbjl,mbjl->mnbj", q, q8.reshape(m, kb, 16, 16))
+    d8g = np.repeat(d8.reshape(m, kb, 8), 2, axis=-1)                          # group j lies in Q8_1 block j // 2
+    return (d[None] * (dots * scl[None] * d8g[:, None]).sum(-1)).sum(-1)
+
+
+@pytest.mark.parametrize("name", ["q4k", "q6k"])
+@pytest.mark.parametrize("m,k,n", [(1, 256, 8), (3, 512, 37), (5, 4096, 16)])
+def test_q8_1_variant_exact_formula(name, m, k, n):
+    """`orc_matmul_q8_1` against the formula of candle-kernels/src/quantized.cu:2141-2166 (Q4_K) / :2258-2281 (Q6_K)
+    evaluated in float64 from independently unpacked weight blocks and Q8_1 activation blocks: every integer exact, no
+    f32 rounding.  A wrong integer, scale, sign or sub-block index anywhere moves a result by far more than f32
+    rounding does (2e-5 of the largest result)."""
+    dt = DT[name]
+    rng = np.random.default_rng(1000 * m + n)
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    x.ravel()[rng.choice(x.size, size=max(1, x.size // 100), replace=False)] = 8.0
+    blocks = orc.quantize(dt, w)
+    got = orc.matmul_q8_1(dt, x, blocks, n).astype(np.float64)
+    exact = q8_1_formula_float64(dt, x, blocks, n, k)
+    assert np.abs(got - exact).max() <= 2e-5 * np.abs(exact).max()
 
 
 @pytest.mark.parametrize("name", ["q4k", "q6k"])
