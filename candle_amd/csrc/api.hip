@@ -20,6 +20,17 @@ struct KernelTimer {
 thread_local KernelTimer g_timer;
 }  // namespace
 
+namespace {
+thread_local bool g_no_split = false;
+// Scope of one entry point: launches planned inside it never split K when the call carries CQ_FLAG_DETERMINISTIC.
+struct NoSplitScope {
+    bool prev;
+    explicit NoSplitScope(int flags) : prev(g_no_split) { g_no_split = (flags & CQ_FLAG_DETERMINISTIC) != 0; }
+    ~NoSplitScope() { g_no_split = prev; }
+};
+}  // namespace
+bool cq_no_split_k() { return g_no_split; }
+
 bool cq_timing_take(hipEvent_t *start, hipEvent_t *stop) {
     if (!g_timer.armed) return false;
     g_timer.armed = false;
@@ -463,6 +474,8 @@ static bool clear_in_quantizer_ok(const float *y, int64_t ny, const float *x, in
 
 static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int64_t m, float *y_dev, int flags,
                         void *ws, size_t ws_bytes, void *stream) {
+    const NoSplitScope no_split(flags);
+    flags &= ~CQ_FLAG_DETERMINISTIC;   // (only the tile kernels' launch plans look at it; every other kernel is deterministic as it is)
     const size_t need = cq_workspace_bytes(w, m, flags);
     int rc = check_matmul_args(w, x_dev, m, y_dev, ws, ws_bytes, need);
     if (rc || m == 0 || w->n == 0) return rc;
@@ -629,6 +642,8 @@ extern "C" int cq_qmatmul_multi(const cq_weight *const *ws, int count, int pre, 
             (pre != CQ_PRE_NONE && ranges_overlap(ys_dev[i], m * ws[i]->n, aux_dev, pre == CQ_PRE_RMS_NORM ? ws[0]->k : m * ws[0]->k)))
             return cq_set_error(CQ_ERR_INVALID, "output %d overlaps the activations: cq_qmatmul_multi does not work in place", i);
     }
+    const int det = flags & CQ_FLAG_DETERMINISTIC;
+    flags &= ~CQ_FLAG_DETERMINISTIC;
     // one activation row (or up to four of short weight rows), two or three weights: one launch over all their rows
     if (m >= 1 && m <= 4 && flags == 0 && !cq_has_min32(ws[0]->ggml_dtype) && !cq_has_min16(ws[0]->ggml_dtype) &&
         cq_matvec_fused_multi_supported(ws, count, pre, m)) {
@@ -650,7 +665,7 @@ extern "C" int cq_qmatmul_multi(const cq_weight *const *ws, int count, int pre, 
                        !(flags == 0 && pre == CQ_PRE_NONE && cq_matvec_fused_rows_supported(ws[0], m));
     for (int i = 0; i < count; i++) {
         const bool reuse = share && i > 0;
-        if (int rc = qmatmul_impl(ws[i], x_dev, reuse ? cq_no_pre() : p, m, ys_dev[i], reuse ? flags | CQ_FLAG_REUSE_ACT : flags,
+        if (int rc = qmatmul_impl(ws[i], x_dev, reuse ? cq_no_pre() : p, m, ys_dev[i], (reuse ? flags | CQ_FLAG_REUSE_ACT : flags) | det,
                                   workspace, ws_bytes, stream))
             return rc;
     }
@@ -712,6 +727,8 @@ static int grouped_impl(const cq_weight *const *experts, int n_experts, const fl
                         const int32_t *row_ids_dev, const int32_t *offsets, float *y_dev, int flags, void *ws,
                         size_t ws_bytes, void *stream) {
     if (!experts || n_experts <= 0 || !offsets) return cq_set_error(CQ_ERR_INVALID, "null argument");
+    const NoSplitScope no_split(flags);
+    flags &= ~CQ_FLAG_DETERMINISTIC;
     const cq_weight *w0 = experts[0];
     if (!w0) return cq_set_error(CQ_ERR_INVALID, "null expert");
     for (int e = 0; e < n_experts; e++) {

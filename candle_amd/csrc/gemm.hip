@@ -838,6 +838,7 @@ int num_cus() {
 // Too few workgroups for `slots` of them at once: K is split (at least four blocks per part).
 int pick_ksplit(int64_t tiles, int64_t kb, int64_t slots) {
     int ksplit = 1;
+    if (cq_no_split_k()) return 1;   // CQ_FLAG_DETERMINISTIC
     while (tiles * ksplit * 2 <= slots && kb / (ksplit * 2) >= 4 && ksplit < 16) ksplit *= 2;
     return ksplit;
 }
@@ -864,6 +865,7 @@ Plan pick_plan(const cq_weight *w, int64_t m) {
         const int64_t tiles = gx * ((m + mt * 32 - 1) / (mt * 32));
         for (int ks = 1; ks <= 16; ks *= 2) {
             if (ks > 1 && kb / ks < 4) break;
+            if (ks > 1 && cq_no_split_k()) break;   // CQ_FLAG_DETERMINISTIC
             const int64_t rounds = (tiles * ks + cus - 1) / cus;
             const double cost = (double)rounds * ((double)((kb + ks - 1) / ks) * (22.0 + 13.5 * mt) + 24.0) +
                                 (ks > 1 ? ks * atomic_pass : 0.0);

@@ -290,6 +290,7 @@ Plan pick_plan(const cq_weight *w, int64_t m) {
         const int64_t tiles = gx * ((m + mt * 32 - 1) / (mt * 32));
         for (int ks = 1; ks <= 16; ks *= 2) {
             if (ks > 1 && ks_total / ks < 2) break;
+            if (ks > 1 && cq_no_split_k()) break;   // CQ_FLAG_DETERMINISTIC
             const int64_t rounds = (tiles * ks + cus - 1) / cus;
             const double cost = (double)rounds * ((double)((ks_total + ks - 1) / ks) * (10.0 + 23.0 * mt) + 24.0) +
                                 (ks > 1 ? ks * atomic_pass : 0.0);

@@ -8,7 +8,10 @@
 //   cqp_stream_read_pol: the same through buffer loads with a chosen cache policy (the `aux` bits of
 //                        the load: 1 = sc0, 2 = nt, 16 = sc1);
 //   cqp_lds_read:        the same bytes requested as buffer loads that land in LDS (no registers per
-//                        request), each wave with a ring of `ring` one-KiB requests in flight.
+//                        request), each wave with a ring of `ring` one-KiB requests in flight;
+//   cqp_lds_read_rows:   the same with a wave owning whole rows of consecutive KiB (the decode kernels' ownership);
+//   cqp_mfma_clock:      the shader clock the part holds while every matrix pipe runs int8 MFMAs (the published
+//                        peaks assume 2.4 GHz), and the time per 32x32x32 int8 MFMA and SIMD at that clock.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -138,7 +141,44 @@ __global__ void lds_read_rows_kernel(const uint8_t *__restrict__ p, uint32_t row
     if (v == 0x12345679u) sink[0] = v;
 }
 
+// Two waves per SIMD run dependent chains of 32x32x32 int8 MFMAs on pseudo-random operands; wave 0 of workgroup 0
+// reads the shader-clock counter and the constant 100 MHz counter before and after.
+typedef int v4i_t __attribute__((ext_vector_type(4)));
+typedef int v16i_t __attribute__((ext_vector_type(16)));
+__global__ void __launch_bounds__(512) mfma_clock_kernel(int iters, uint64_t *out, int *sink) {
+    v4i_t a, b;
+    for (int i = 0; i < 4; i++) {
+        a[i] = (int)(threadIdx.x * 2654435761u + 977u * (i + 1));
+        b[i] = (int)(threadIdx.x * 40503u + 131u * (i + 7));
+    }
+    v16i_t lo = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, hi = lo;
+    const uint64_t c0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
+    for (int it = 0; it < iters; it++) {
+        asm volatile("" : "+v"(a), "+v"(b));   // not loop-invariant
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            lo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, lo, 0, 0, 0);
+            hi = __builtin_amdgcn_mfma_i32_32x32x32_i8(b, a, hi, 0, 0, 0);
+        }
+    }
+    int acc = 0;
+    for (int i = 0; i < 16; i++) acc += lo[i] ^ hi[i];
+    const uint64_t c1 = __builtin_amdgcn_s_memtime(), r1 = __builtin_amdgcn_s_memrealtime();
+    if (acc == 0x12345678) sink[0] = acc;
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        out[0] = c1 - c0;
+        out[1] = r1 - r0;
+    }
+}
+
 }  // namespace
+
+// out_dev[0] = shader-clock cycles, out_dev[1] = ticks of the constant 100 MHz counter over `iters` x 16 MFMAs per wave
+// (256 workgroups of eight waves: two per SIMD on every CU).
+extern "C" int cqp_mfma_clock(int iters, uint64_t *out_dev, int *sink_dev, void *stream) {
+    hipLaunchKernelGGL(mfma_clock_kernel, dim3(256), dim3(512), 0, (hipStream_t)stream, iters, out_dev, sink_dev);
+    return (int)hipGetLastError();
+}
 
 extern "C" int cqp_lds_read_rows(const void *buf_dev, size_t bytes, int grid, int pieces_per_row, uint32_t *sink_dev, void *stream) {
     const uint8_t *p = (const uint8_t *)buf_dev;

@@ -86,6 +86,10 @@ int cq_set_error(int code, const char *fmt, ...);
                                 __FILE__, __LINE__);                                             \
     } while (0)
 
+// CQ_FLAG_DETERMINISTIC (api.hip): true while the calling thread runs a call with the flag; the tile kernels' launchers
+// then never split K (no partial sums added atomically in arrival order).
+bool cq_no_split_k();
+
 // Kernel timing hook (api.hip): true when the calling thread armed the timer; the launch then goes
 // through CQ_LAUNCH below with the two events.  Disarms.
 bool cq_timing_take(hipEvent_t *start, hipEvent_t *stop);

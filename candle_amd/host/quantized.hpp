@@ -136,6 +136,8 @@ class QHipStorage {
         check(cq_weight_shape(w_, &n, &k), "QHipStorage::dims");
         return {n, k};
     }
+    // (state of the handle: a set-up call, not concurrent with any use of the storage; QTensor owns its storage, so no
+    // two tensors can fix different shapes on one handle)
     void set_dims(int64_t n, int64_t k) { check(cq_weight_set_shape(w_, n, k), "QHipStorage::set_dims"); }
     // cuda.rs:390-446
     Tensor dequantize(const Shape &shape, hipStream_t stream = nullptr) const {

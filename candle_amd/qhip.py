@@ -17,6 +17,7 @@ LIB_PATH = os.environ.get("CQ_LIB_PATH", os.path.join(_HERE, "lib", "libcandle_q
 Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1, Q2K, Q3K, Q4K, Q5K, Q6K, Q8K = 2, 3, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15
 FLAG_AUTO, FLAG_FORCE_MATVEC, FLAG_FORCE_GEMM, FLAG_ACT_Q8_1, FLAG_REUSE_ACT, FLAG_STAGED_ACT = 0, 1, 2, 4, 8, 16
 FLAG_FORCE_SKINNY = 32
+FLAG_DETERMINISTIC = 64   # tile kernels never split K: the same bits on every run
 PRE_NONE, PRE_RMS_NORM, PRE_SILU_MUL = 0, 1, 2
 
 EXPORTS = [

@@ -81,7 +81,15 @@ class QTensor:
         self._shape = tuple(int(s) for s in shape)
         _check_shape(self._shape, qhip.load().cq_block_size(weight.dtype))
         k = self._shape[-1]
-        weight.set_shape(int(np.prod(self._shape[:-1])) if len(self._shape) > 1 else 1, k)
+        rows = int(np.prod(self._shape[:-1])) if len(self._shape) > 1 else 1
+        # The shape is state of the storage handle (the entry points without a shape argument read it): a second
+        # QTensor over the same storage with another shape would silently re-shape the first.
+        fixed = getattr(weight, "_qtensor_dims", None)
+        if fixed is not None and fixed != (rows, k):
+            raise qhip.QHipError(f"storage is already viewed as {fixed} by another QTensor; a second view {(rows, k)} "
+                                 "goes through qhip.qmatmul_shaped, which takes the shape with the call")
+        weight.set_shape(rows, k)
+        weight._qtensor_dims = (rows, k)
 
     # ---- constructors ---------------------------------------------------------------------
     @classmethod

@@ -50,7 +50,8 @@ enum {
     CQ_DTYPE_Q5K = 13,
     CQ_DTYPE_Q6K = 14,
     CQ_DTYPE_Q8K = 15   /* the activation format of the K-quants; as a weight type (k_quants.rs:1749-1839, a type of the
-                           reference's tests rather than of checkpoints) it has one plain dot-product kernel        */
+                           reference's tests rather than of checkpoints) it has one plain dot-product kernel, which
+                           reads the weights once per activation row: m rows cost m passes over n * k bytes     */
 };
 
 /* error codes */
@@ -81,8 +82,17 @@ enum {
                                  single launch and leave the workspace alone); cq_qmatmul_multi takes care of this
                                  by itself.  No counterpart in the reference, which re-quantizes per call.            */
     CQ_FLAG_FORCE_SKINNY = 32, /* the split-K MFMA kernel for few rows whatever m is (A/B runs)                                */
-    CQ_FLAG_STAGED_ACT = 16   /* up to four rows: run the stand-alone quantizer into the workspace and a matmul kernel
+    CQ_FLAG_STAGED_ACT = 16,  /* up to four rows: run the stand-alone quantizer into the workspace and a matmul kernel
                                  (two launches, as cuda.rs:249-293 does) instead of the single fused launch           */
+    CQ_FLAG_DETERMINISTIC = 64 /* the same bits on every run, like the CPU QMatMul.  Without it one family of launches is
+                                 not: the tile kernels (more than 32 rows; grouped experts with more than 8 rows) split K
+                                 over several workgroups when the weight has few row tiles - n = 4096 at 33 .. 1024
+                                 rows, the w2 projection of an expert - and add the partial sums atomically in
+                                 arrival order, so the last bits of a result can differ between two runs (far inside
+                                 the 1e-4 bar; the reference's CUDA arm is allowed 1e-4 of drift between batch sizes,
+                                 quantized_tests.rs:203-209).  With the flag those launches never split K: each
+                                 result is one sum in a fixed order, at the price of fewer workgroups in flight.
+                                 Every other kernel is deterministic as it is.  Accepted by all matmul entry points. */
 };
 
 /* the model step a fused call computes on the way into the activation quantizer */
@@ -122,7 +132,9 @@ int cq_weight_zeros(int dev, int ggml_dtype, int64_t n, int64_t k, cq_weight **o
  * k % block_size == 0; until told otherwise it reads as [elem_count / block_size, block_size].  The shape
  * arrives with the call (cq_qmatmul_shaped, as QCudaStorage::fwd takes self_shape, cuda.rs:478-499) or is
  * fixed once with cq_weight_set_shape (QTensor::new, mod.rs:318-323), which the entry points without a
- * shape argument then use. */
+ * shape argument then use.  That shape is state of the handle: cq_weight_set_shape is a set-up call, not to run
+ * while another thread uses the handle (the matmul entry points read n and k without a lock), and two views of one
+ * storage with different shapes take cq_qmatmul_shaped / cq_workspace_bytes_shaped, which leave the handle alone. */
 int cq_weight_zeros_flat(int dev, int ggml_dtype, int64_t elem_count, cq_weight **out);
 int cq_weight_create_flat(int dev, int ggml_dtype, const void *host_ggml_blocks, size_t nbytes, cq_weight **out);
 int64_t cq_weight_elem_count(const cq_weight *w);                /* QTensor::shape().elem_count() */
@@ -177,6 +189,9 @@ int cq_qmatmul_shaped(const cq_weight *w, int64_t n, int64_t k, const float *x_d
  * code, so every GPU the library runs on holds that much until the process ends.  Calls that need more
  * (cq_workspace_bytes(w, m, flags) > CQ_STATIC_SCRATCH_BYTES) fail with CQ_ERR_WORKSPACE.  The call itself
  * allocates and frees nothing; the array's address is looked up when the first weight is created on a device.
+ * The first launch of a kernel instance on a device that needs more than 48 KiB of LDS sets that function attribute
+ * once (hipFuncSetAttribute, as in every other entry point): make one call of each shape outside stream capture
+ * before capturing.
  * All calls on one GPU share the array: calls that overlap in time on one GPU (two streams, two host threads)
  * race on it; calls in stream order do not. */
 #define CQ_STATIC_SCRATCH_BYTES (16u << 20)

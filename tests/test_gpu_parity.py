@@ -920,3 +920,42 @@ def test_weights_from_arbitrary_bytes(qh, dt, m, k, n, mode):
             continue
         assert np.isfinite(got).all()
         assert np.linalg.norm(got - ref) <= REL_L2_TOL * np.linalg.norm(ref), flags
+
+
+@pytest.mark.parametrize("dt,m", [(orc.Q4_0, 33), (orc.Q8_0, 33), (orc.Q4K, 130), (orc.Q6K, 130), (orc.Q5K, 130)])
+def test_deterministic_flag_repeats_bit_for_bit(qh, dt, m):
+    """quantized_tests.rs:181-216 (`qmm_batch`): the CPU QMatMul gives the same bits on every run.  The tile kernels split K
+    over workgroups that add their partial sums atomically when a weight has few row tiles (4096 x 4096 at these row
+    counts); with CQ_FLAG_DETERMINISTIC they do not, and twenty calls give the same bits - which also match the oracle
+    to the f32 bars on sampled rows."""
+    n = k = 4096
+    gen = torch.Generator(device="cuda").manual_seed(int(dt) * 100 + m)
+    qw = qh.QWeight.zeros(dt, n, k).quantize_(torch.randn((n, k), device="cuda", generator=gen) * 0.02)
+    x = torch.randn((m, k), device="cuda", generator=gen)
+    first = qh.qmatmul(qw, x, qh.FLAG_DETERMINISTIC)
+    for _ in range(19):
+        assert torch.equal(qh.qmatmul(qw, x, qh.FLAG_DETERMINISTIC), first)
+    blocks = qw.to_ggml().reshape(n, -1)
+    rows = np.ascontiguousarray(blocks[1000:1016]).reshape(-1)
+    xs = x[[0, m // 2, m - 1]].cpu().numpy()
+    check_f32(first[[0, m // 2, m - 1]][:, 1000:1016].cpu().numpy(), orc.matmul(dt, xs, rows, 16))
+    # the default launch of the same call agrees to rounding
+    plain = qh.qmatmul(qw, x)
+    assert float((plain - first).norm() / first.norm()) < 1e-6
+
+
+def test_deterministic_flag_grouped_experts(qh):
+    """The grouped launch of an expert's w2-shaped projection (few row tiles, long rows) splits K by default."""
+    n, k, n_e = 512, 4096, 4
+    rng = np.random.default_rng(5)
+    experts = []
+    for e in range(n_e):
+        w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+        experts.append(qh.QWeight.from_ggml(orc.Q6K, orc.quantize(orc.Q6K, w), n, k))
+    offsets = np.array([0, 12, 30, 41, 64], dtype=np.int32)
+    x = dev(rng.standard_normal((64, k)).astype(np.float32))
+    first = qh.qmatmul_grouped(experts, x, None, offsets, flags=qh.FLAG_DETERMINISTIC)
+    for _ in range(10):
+        assert torch.equal(qh.qmatmul_grouped(experts, x, None, offsets, flags=qh.FLAG_DETERMINISTIC), first)
+    plain = qh.qmatmul_grouped(experts, x, None, offsets)
+    assert float((plain - first).norm() / first.norm()) < 1e-6

@@ -90,3 +90,22 @@ def test_python_qtensor_roundtrip_and_f16():
         back = q.dequantize()
         assert back.shape == src.shape and float((back - src).abs().max()) < bound, name
         assert torch.equal(q.dequantize_f16(), back.to(torch.float16)), name   # quantized_tests.rs:229-234
+
+
+@pytest.mark.gpu
+def test_python_qtensor_second_view_of_a_storage():
+    """The [rows, k] a storage is read as is state of its handle: a second QTensor with another shape over the same
+    storage is refused (it would re-shape the first); the same shape is fine, and a differently shaped view goes
+    through the call that takes the shape with it (QCudaStorage::fwd, cuda.rs:478-499)."""
+    import torch
+    from candle_amd import qhip
+    from candle_amd.quantized import QTensor
+    src = torch.linspace(-1, 1, 8 * 512, device="cuda").reshape(8, 512)
+    q = QTensor.quantize(src, "q4k")
+    QTensor(q._w, (8, 512))
+    with pytest.raises(qhip.QHipError):
+        QTensor(q._w, (16, 256))
+    x = torch.randn((3, 256), device="cuda")
+    y = qhip.qmatmul_shaped(q._w, (16, 256), x)
+    assert tuple(y.shape) == (3, 16) and q.shape == (8, 512)
+    assert tuple(q.matmul_t(torch.randn((2, 512), device="cuda")).shape) == (2, 8)
