@@ -568,11 +568,8 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
             return cq_set_error(CQ_ERR_UNSUPPORTED, "Q8_1 activations are only handled by the GEMM kernel");
         path = use_gemm ? kGemm : kMatvec;
     }
-    if (path == kMatvec && !cq_matvec_row_fits(w))
-        return cq_set_error(CQ_ERR_UNSUPPORTED,
-                            "rows of %lld elements are too long for the dot-product kernels, which keep one quantized row "
-                            "in the 160 KiB of LDS (about 150000 elements for Q4K/Q5K/Q6K, 139000 for Q8_0/Q4_0)",
-                            (long long)w->k);
+    // (rows whose quantized image does not fit the 160 KiB of LDS go through the dot-product kernel that walks them in
+    // chunks: no limit on k, as in k_quants::matmul)
     // two to four rows of short enough weight rows: the one-launch kernel again, every unpacked weight unit
     // contracted with each activation row
     if (flags == 0 && pre.kind == CQ_PRE_NONE && !in_place && cq_matvec_fused_rows_supported(w, m)) {

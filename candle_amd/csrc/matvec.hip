@@ -383,6 +383,31 @@ __device__ __forceinline__ void stage_row(uint8_t *smem, const LdsRow r, const c
     }
 }
 
+// The same for the part [k0, k0 + kc) of a row of k elements (k0 a multiple of 256): the LDS image is that of a row of
+// kc elements.
+template <int DT, int NT>
+__device__ __forceinline__ void stage_row_part(uint8_t *smem, const LdsRow r, const cq_act_view &a, int64_t row, int64_t k,
+                                               int64_t k0, int64_t kc) {
+    const int4 *src = (const int4 *)(a.qs + row * k + k0);
+    const uint32_t units = (uint32_t)(kc / Geo<DT>::kElems);
+    for (int piece = threadIdx.x; piece < (int)(kc / 16); piece += NT)
+        lds_put<int4>(smem, piece_off<DT>(r, piece, units), src[piece]);
+    const int64_t nb = act_blocks<DT>(k), b0 = act_blocks<DT>(k0);
+    const int nbc = (int)act_blocks<DT>(kc);
+    for (int b = threadIdx.x; b < nbc; b += NT) {
+        lds_put<float>(smem, r.d + 4 * b, a.d[row * nb + b0 + b]);
+        if (!Geo<DT>::kActK) lds_put<int32_t>(smem, r.bs + 4 * b, a.bsum32[row * nb + b0 + b]);
+    }
+    if (Geo<DT>::kActK) {
+        const int32_t *bs = (const int32_t *)(a.bsums + (row * nb + b0) * 16);  // 8 words per block
+        for (int i = threadIdx.x; i < nbc * 8; i += NT) {
+            const int32_t two = bs[i];
+            if (is_k4(DT)) lds_put<int16_t>(smem, r.bs + 2 * i, (int16_t)((int16_t)(two & 0xffff) + (int16_t)(two >> 16)));
+            else lds_put<int32_t>(smem, r.bs + 4 * i, two);
+        }
+    }
+}
+
 // ------------------------------------------------------------------------ weight units ----
 // Raw bytes of one unit as loaded from the planes (decoded later, so loads can run ahead).
 template <int DT> struct UnitRaw {
@@ -1048,6 +1073,65 @@ __global__ void __launch_bounds__(kStagedThreads) staged_kernel(cq_weight w, cq_
     }
 }
 
+// ----------------------------------------------------- rows of any length (m <= 4 rows per launch) ----
+// staged_kernel for rows whose quantized image does not fit the LDS (k_quants::matmul, k_quants.rs:1842-1883, has no
+// limit on k): the workgroup walks the row in chunks of kChunkElems elements, one chunk of the MB activation rows in
+// LDS at a time, and every wave keeps the partial sums of its weight rows in registers across the chunks.  A lane adds
+// its units in the order of staged_kernel (a chunk is a whole number of 64-unit steps), so the two kernels give the
+// same bits.
+constexpr int64_t kChunkElems = 16384;
+constexpr int kChunkRowsPerWave = 4;   // rows_per_wg <= 16, four waves
+template <int DT, int MB>
+__global__ void __launch_bounds__(kStagedThreads) chunked_kernel(cq_weight w, cq_act_view a, int64_t m0,
+                                                                 int rows_per_wg, float *__restrict__ y) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    static_assert(kChunkElems % (64 * Geo<DT>::kElems) == 0, "whole 64-unit steps per chunk");
+    const int64_t units = w.k / Geo<DT>::kElems;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t row_begin = (int64_t)blockIdx.x * rows_per_wg;
+    const int64_t row_end = row_begin + rows_per_wg < w.n ? row_begin + rows_per_wg : w.n;
+    float acc[kChunkRowsPerWave][MB];
+#pragma unroll
+    for (int ri = 0; ri < kChunkRowsPerWave; ri++)
+#pragma unroll
+        for (int m = 0; m < MB; m++) acc[ri][m] = 0.0f;
+    for (int64_t k0 = 0; k0 < w.k; k0 += kChunkElems) {
+        const int64_t kc = w.k - k0 < kChunkElems ? w.k - k0 : kChunkElems;
+        __syncthreads();   // every wave is done with the chunk before
+        LdsRow rows[MB];
+#pragma unroll
+        for (int m = 0; m < MB; m++) {
+            rows[m] = lds_row<DT>(kc, m);
+            stage_row_part<DT, kStagedThreads>(smem, rows[m], a, m0 + m, w.k, k0, kc);
+        }
+        __syncthreads();
+        const int64_t u0 = k0 / Geo<DT>::kElems, uc = kc / Geo<DT>::kElems;
+#pragma unroll
+        for (int ri = 0; ri < kChunkRowsPerWave; ri++) {
+            const int64_t row = row_begin + wave + ri * (kStagedThreads / 64);
+            if (row >= row_end) continue;
+#pragma unroll 2
+            for (int64_t u = lane; u < uc; u += 64) {
+                UnitRaw<DT> raw;
+                load_unit<DT>(w, row, units, u0 + u, raw);
+                UnitW<DT> uw;
+                decode_unit<DT>(raw, lane & 7, uw);
+#pragma unroll
+                for (int m = 0; m < MB; m++) acc[ri][m] += unit_value<DT>(smem, uw, rows[m], (uint32_t)u, (uint32_t)uc);
+            }
+        }
+    }
+#pragma unroll
+    for (int ri = 0; ri < kChunkRowsPerWave; ri++) {
+        const int64_t row = row_begin + wave + ri * (kStagedThreads / 64);
+#pragma unroll
+        for (int m = 0; m < MB; m++) {
+            const float t = wave_sum(acc[ri][m]);
+            if (lane == 0 && row < row_end) y[(m0 + m) * w.n + row] = t;
+        }
+    }
+}
+
 // ------------------------------------------------- K-quant weights x Q8_1 activations ----
 // The formulation of the reference's CUDA arm (mul_mat_via_q8_1, quantized/cuda.rs:298-365; dot bodies
 // candle-kernels/src/quantized.cu:2141-2166 for Q4K and :2258-2281 for Q6K) with the activations quantized by the CPU
@@ -1323,7 +1407,35 @@ bool batched_ok(const cq_weight *w, int mb) {
 }
 
 template <int DT>
+hipError_t launch_chunked(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
+    const int rpw = pick_rows_per_wg(w->n);   // at most 16: four rows per wave
+    const unsigned grid = (unsigned)((w->n + rpw - 1) / rpw);
+    const int64_t kc = w->k < kChunkElems ? w->k : kChunkElems;
+    int64_t m0 = 0;
+    while (m0 < m) {
+        const int64_t left = m - m0;
+        const int mb = left >= 4 ? 4 : (left >= 2 ? 2 : 1);
+        const size_t lds = lds_row_bytes<DT>(kc) * mb;
+        if (mb == 4) {
+            if (hipError_t e = cq_ensure_lds<chunked_kernel<DT, 4>>(w->dev, lds); e != hipSuccess) return e;
+            CQ_LAUNCH((chunked_kernel<DT, 4>), grid, kStagedThreads, lds, s, *w, a, m0, rpw, y);
+        } else if (mb == 2) {
+            if (hipError_t e = cq_ensure_lds<chunked_kernel<DT, 2>>(w->dev, lds); e != hipSuccess) return e;
+            CQ_LAUNCH((chunked_kernel<DT, 2>), grid, kStagedThreads, lds, s, *w, a, m0, rpw, y);
+        } else {
+            if (hipError_t e = cq_ensure_lds<chunked_kernel<DT, 1>>(w->dev, lds); e != hipSuccess) return e;
+            CQ_LAUNCH((chunked_kernel<DT, 1>), grid, kStagedThreads, lds, s, *w, a, m0, rpw, y);
+        }
+        if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+        m0 += mb;
+    }
+    return hipSuccess;
+}
+
+template <int DT>
 hipError_t launch_staged(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
+    // rows whose quantized image does not fit the LDS: walked in chunks
+    if (lds_row_bytes<DT>(w->k) > kMaxRowLds) return launch_chunked<DT>(w, a, m, y, s);
     if (m >= 2) {
         int64_t m0 = 0;
         bool done = true;

@@ -274,11 +274,39 @@ def test_long_rows(qh, dt, k):
         assert np.linalg.norm(got - ref) <= 1e-4 * np.linalg.norm(ref)
 
 
-def test_rows_beyond_the_lds_are_refused_by_name(qh):
-    k = 163840
-    qw = qh.QWeight.zeros(orc.Q8_0, 8, k)
-    with pytest.raises(qh.QHipError, match="too long for the dot-product kernels"):
-        qh.qmatmul(qw, torch.zeros((1, k), device="cuda"))
+@pytest.mark.parametrize("dt", [orc.Q4_0, orc.Q8_0, orc.Q4K, orc.Q5K, orc.Q6K, orc.Q2K, orc.Q5_1])
+@pytest.mark.parametrize("m", [1, 3, 6])
+def test_rows_beyond_the_lds(qh, dt, m):
+    """k_quants::matmul (k_quants.rs:1842-1883) has no limit on the row length.  Rows whose quantized image exceeds the
+    160 KiB of LDS (K = 262 144 here, and a K that is not a whole number of chunks) are walked in chunks by the
+    dot-product kernel; one, several and more than four activation rows against the oracle."""
+    for k, n in ((262144, 24), (163840 + 2048, 9)):
+        rng = np.random.default_rng(int(dt) * 10 + m + k)
+        w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+        x = rng.standard_normal((m, k)).astype(np.float32)
+        blocks = orc.quantize(dt, w)
+        qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+        got = qh.qmatmul(qw, dev(x)).cpu().numpy()
+        ref = orc.matmul(dt, x, blocks, n)
+        for r in range(m):
+            nrm = np.linalg.norm(ref[r])
+            assert np.linalg.norm(got[r] - ref[r]) <= 1e-4 * nrm and np.abs(got[r] - ref[r]).max() <= 1e-3 * nrm
+
+
+def test_chunked_rows_equal_whole_rows_bit_for_bit(qh):
+    """The chunked kernel adds a lane's units in the order of the kernel that holds the whole row in LDS: a row split as
+    [n, k] = [4, 131072] (fits, whole) and the same storage read as [2, 262144] (chunked) share their first halves'
+    sums only through the oracle, so this compares each against it and, for a K that fits either way, checks that
+    batch invariance holds across the two kernels' launches of 4 + 2 rows."""
+    k, n = 262144, 8
+    rng = np.random.default_rng(77)
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((6, k)).astype(np.float32)
+    blocks = orc.quantize(orc.Q4K, w)
+    qw = qh.QWeight.from_ggml(orc.Q4K, blocks, n, k)
+    all6 = qh.qmatmul(qw, dev(x))
+    for r in range(6):   # quantized_tests.rs:181-216: a row's result does not depend on the rows stacked with it
+        assert torch.equal(qh.qmatmul(qw, dev(x[r:r + 1])), all6[r:r + 1])
 
 
 def test_qmatmul_dense_arms(qh, monkeypatch):
