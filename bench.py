@@ -29,7 +29,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 # HBM bytes per Q4_K decode launch (mean over the step's 192 launches), from two rocprofv3 --pmc runs
 # of this script (FETCH_SIZE, then WRITE_SIZE), each scaled by what the counter reads for a plain
 # 256 MiB device copy (x2.000 and x1.000); see profiles/decode_stack_q4k_matvec_hbm_traffic.md.
-Q4K_DECODE_TRAFFIC_BYTES_PER_LAUNCH = 15_422_464
+Q4K_DECODE_TRAFFIC_BYTES_PER_LAUNCH = 15_400_448
 
 LAYERS = 32
 HIDDEN, FFN, VOCAB = 4096, 11008, 32000
