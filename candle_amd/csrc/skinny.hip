@@ -351,26 +351,34 @@ __device__ __forceinline__ void res_issue_weights(uint8_t *__restrict__ wl, cons
     if (DT == CQ_DTYPE_Q5K && lane < 32) dma16s(pl.w5, w5_off, blk * 32u, wl + 2048);
 }
 
-// One K block of one tile: unpack the weights in `wl`, contract with the resident activation slice `act`.
+// Weight operands of one K block of one tile, unpacked into registers.
+struct ResOps {
+    v4i bl[4], bh[4];
+    float dw;
+    v8h wmin;
+};
+template <int DT, bool DUMP>
+__device__ __forceinline__ void res_unpack(const uint8_t *__restrict__ wl, int lane, const WHead<DT> &head, const cq_mfma_dump &dump,
+                                           ResOps &o) {
+    block_unpack(wl, lane, head, o.bl, o.bh, o.dw, o.wmin);
+    if constexpr (DUMP && is_k4(DT)) {
+        if (dump.int_min) {   // verification: the minima themselves as the operand: the MFMA delivers the integer Mn_b
+            const uint32_t kq = lane >> 4;
+            const uint32_t rec[4] = {head.rec.x, head.rec.y, head.rec.z, head.rec.w};
+            o.wmin = __builtin_bit_cast(v8h, cq_min_term_groups_int(rec, (kq & 1) != 0, (kq >> 1) != 0));
+        }
+    }
+}
+
+// The unpacked operands `o` contracted with the resident activation slice `act` of the same K block.
 // DUMP: the integers go to dump.i / dump.mn at `at` + row * `rs` (rows < m) instead of into `out`.
 template <int DT, int RT, int NT, bool DUMP>
-__device__ __forceinline__ void res_block(const uint8_t *__restrict__ wl, const uint8_t *__restrict__ act, int lane,
-                                          const WHead<DT> &head, const uint32_t (&a_col)[NT][2], v4f (&out)[NT],
-                                          const cq_mfma_dump &dump, int64_t at, int64_t rs, int64_t m) {
+__device__ __forceinline__ void res_mac(const uint8_t *__restrict__ act, int lane, const ResOps &o, const uint32_t (&a_col)[NT][2],
+                                        v4f (&out)[NT], const cq_mfma_dump &dump, int64_t at, int64_t rs, int64_t m) {
     typedef Res<DT, RT> R;
     constexpr bool MINS = is_k4(DT);
     constexpr int SHIFT = DT == CQ_DTYPE_Q4K ? 3 : 8;
     const uint32_t r = lane & 15, kq = lane >> 4;
-    v4i bl[4], bh[4];
-    float dw;
-    v8h wmin;
-    block_unpack(wl, lane, head, bl, bh, dw, wmin);
-    if constexpr (DUMP && is_k4(DT)) {
-        if (dump.int_min) {   // verification: the minima themselves as the operand: the MFMA delivers the integer Mn_b
-            const uint32_t rec[4] = {head.rec.x, head.rec.y, head.rec.z, head.rec.w};
-            wmin = __builtin_bit_cast(v8h, cq_min_term_groups_int(rec, (kq & 1) != 0, (kq >> 1) != 0));
-        }
-    }
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         const v4f d8 = *(const v4f *)(act + R::oD8 + (t * 16 + 4 * kq < 8u * RT ? t * 16 + 4 * kq : 0) * 4);
@@ -378,7 +386,7 @@ __device__ __forceinline__ void res_block(const uint8_t *__restrict__ wl, const 
         if (MINS) {
             const uint32_t row = t * 16 + r < 8u * RT ? t * 16 + r : 8u * RT - 1;
             const v8h ma = *(const v8h *)(act + R::oMin + row * 32 + (kq & 1) * 16);
-            mn = __builtin_amdgcn_mfma_f32_16x16x32_f16(ma, wmin, mn, 0, 0, 0);
+            mn = __builtin_amdgcn_mfma_f32_16x16x32_f16(ma, o.wmin, mn, 0, 0, 0);
             if (DUMP && dump.mn) {
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
@@ -391,8 +399,8 @@ __device__ __forceinline__ void res_block(const uint8_t *__restrict__ wl, const 
 #pragma unroll
         for (int s = 0; s < 4; s++) {
             const v4i av = *(const v4i *)(act + a_col[t][s & 1] + (s >> 1) * 1024);
-            acc_lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bl[s], acc_lo, 0, 0, 0);
-            acc_hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bh[s], acc_hi, 0, 0, 0);
+            acc_lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, o.bl[s], acc_lo, 0, 0, 0);
+            acc_hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, o.bh[s], acc_hi, 0, 0, 0);
         }
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -401,11 +409,21 @@ __device__ __forceinline__ void res_block(const uint8_t *__restrict__ wl, const 
                 const int64_t orow = t * 16 + kq * 4 + i;
                 if (orow < m) dump.i[at + orow * rs] = I;
             } else {
-                const float v = MINS ? __builtin_fmaf((float)I, dw, mn[i]) : (float)I * dw;
+                const float v = MINS ? __builtin_fmaf((float)I, o.dw, mn[i]) : (float)I * o.dw;
                 out[t][i] = __builtin_fmaf(v, d8[i], out[t][i]);
             }
         }
     }
+}
+
+// One K block of one tile: unpack the weights in `wl`, contract with the resident activation slice `act`.
+template <int DT, int RT, int NT, bool DUMP>
+__device__ __forceinline__ void res_block(const uint8_t *__restrict__ wl, const uint8_t *__restrict__ act, int lane,
+                                          const WHead<DT> &head, const uint32_t (&a_col)[NT][2], v4f (&out)[NT],
+                                          const cq_mfma_dump &dump, int64_t at, int64_t rs, int64_t m) {
+    ResOps o;
+    res_unpack<DT, DUMP>(wl, lane, head, dump, o);
+    res_mac<DT, RT, NT, DUMP>(act, lane, o, a_col, out, dump, at, rs, m);
 }
 
 // m <= 8 * RT activation rows (the workspace pads rows, so whole groups are copied); n % 16 == 0; at most
@@ -535,6 +553,164 @@ __global__ void __launch_bounds__(kWaves * 64) skinny_resident_kernel(cq_weight 
             }
         }
         par ^= 1;
+    }
+}
+
+// ------------------------------------------- resident activations, several tiles per workgroup ----
+// More weight rows than 16 x the number of CUs: every workgroup walks several 16-row tiles.  With one K block per
+// wave (k <= 256 x waves) a wave keeps its partial result of each tile in registers and the workgroup meets once per
+// round of up to four tiles, not once per tile: between two tiles of a round there is no barrier and no wait for
+// the slowest wave, so the copies of the tile after the next one (issued into the buffer the current tile has just
+// been unpacked from) really are in flight under the arithmetic.  Everything a tile needs comes through LDS copies,
+// the 20-byte block headers included: a load into registers would be tracked by the compiler, which on joining the
+// paths "copies issued" and "no tile left to copy" waits as the stricter of the two demands, i.e. for everything.
+// The waits are written out by hand instead (s_waitcnt vmcnt(copies of one tile) while a next tile is in flight).
+// The partial tiles of a round are summed in wave order as in the kernels above.  Q4K and Q5K (one header layout).
+//   LDS: activation slices as skinny_resident_kernel | per wave two slots {weights kWgt | headers 16 x 16 B, 16 x 4 B},
+//        which take the wave's partial results (1 KiB per tile) at the end of a round
+constexpr int kTilesPerRound = 4;
+template <int DT, int RT> struct ResMulti {
+    static constexpr int kWgt = Res<DT, RT>::kWgt;
+    static constexpr int oHdr = kWgt, kSlot = kWgt + 320;
+    static constexpr int kCopies = (DT == CQ_DTYPE_Q4K ? 2 : 3) + 2;   // copy instructions per tile (multi_issue)
+    static size_t bytes(int64_t kb) { return (size_t)kb * Res<DT, RT>::kActBlk + (size_t)kb * 2 * kSlot; }
+};
+
+// The copies of one tile's K block b into `slot`: weights as res_issue_weights, then the 16 rows' headers
+// (bytes 0..15 of row r at oHdr + 16 r, bytes 16..19 at oHdr + 256 + 4 r; lanes 0..15).
+template <int DT, int RT>
+__device__ __forceinline__ void multi_issue(uint8_t *__restrict__ slot, const ResPlanes &pl, __amdgpu_buffer_rsrc_t hdr, uint32_t n_tile,
+                                            uint32_t b, uint32_t kb, uint32_t wq_off, uint32_t w5_off, uint32_t hd_off, int lane) {
+    typedef ResMulti<DT, RT> M;
+    res_issue_weights<DT>(slot, pl, n_tile, b, kb, wq_off, 0, w5_off, lane);
+    const uint32_t blk = n_tile * kb + b;
+    if (lane < 16) {
+        dma16s(hdr, hd_off, blk * (uint32_t)CQ_Q4K_HDR, slot + M::oHdr);
+        // (the instruction's immediate offset moves both addresses: bytes 16.. of the header, and 16 bytes on in LDS)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(hdr, (lptr_t)(slot + M::oHdr + 256 - 16), 4, (int)hd_off, (int)(blk * (uint32_t)CQ_Q4K_HDR), 16, 0);
+    }
+}
+
+// One tile of one wave: operands out of `slot`, then (the slot is free) the copies of the tile two ahead, then the MFMAs.
+template <int DT, int RT, bool DUMP>
+__device__ __forceinline__ void multi_step(uint8_t *__restrict__ slot, const uint8_t *__restrict__ act, int lane, const ResPlanes &pl,
+                                           __amdgpu_buffer_rsrc_t hdr, bool ahead, uint32_t tile_ahead, uint32_t b, uint32_t kb32,
+                                           uint32_t wq_off, uint32_t w5_off, uint32_t hd_off, const uint32_t (&a_col)[1][2],
+                                           v4f (&out)[1], const cq_mfma_dump &dump, int64_t at, int64_t rs, int64_t m) {
+    typedef ResMulti<DT, RT> M;
+    const uint32_t r = lane & 15;
+    WHead<DT> head;
+    const uint4 h4 = *(const uint4 *)(slot + M::oHdr + r * 16u);
+    head.dd = h4.x;
+    head.rec = make_uint4(h4.y, h4.z, h4.w, *(const uint32_t *)(slot + M::oHdr + 256 + r * 4u));
+    ResOps o;
+    res_unpack<DT, DUMP>(slot, lane, head, dump, o);
+    if (ahead) {
+        __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the reads above are done with the slot
+        multi_issue<DT, RT>(slot, pl, hdr, tile_ahead * 16u, b, kb32, wq_off, w5_off, hd_off, lane);
+    }
+    res_mac<DT, RT, 1, DUMP>(act, lane, o, a_col, out, dump, at, rs, m);
+}
+
+// m <= 8 * RT <= 16 activation rows; n % 16 == 0; k / 256 <= kWaves.
+template <int DT, int RT, int kWaves, bool DUMP>
+__global__ void __launch_bounds__(kWaves * 64) skinny_resident_multi_kernel(cq_weight w, cq_act_view a, int64_t m,
+                                                                            float *__restrict__ y, cq_mfma_dump dump) {
+    typedef Res<DT, RT> R;
+    typedef ResMulti<DT, RT> M;
+    static_assert(DT == CQ_DTYPE_Q4K || DT == CQ_DTYPE_Q5K, "block headers of 20 bytes");
+    static_assert(RT <= 2, "one 16-row tile of activation rows");
+    static_assert(2 * M::kSlot >= kTilesPerRound * 1024, "a round's partial tiles fit the wave's two slots");
+    constexpr bool MINS = is_k4(DT);
+    constexpr int kAhead = 0x0F70 | M::kCopies;   // s_waitcnt vmcnt(copies of one tile)
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t r = lane & 15, kq = lane >> 4;
+    const int64_t k = w.k, kb = w.k >> 8;
+    const int64_t tiles = w.n / 16, G = gridDim.x;
+    uint8_t *wgt_base = smem + kb * R::kActBlk;
+    const bool has = wave < kb;   // this wave owns K block `wave`
+    const uint32_t b = (uint32_t)wave;
+
+    const uint32_t r8 = lane >> 3, c8 = lane & 7;
+    const uint32_t act_off = r8 * (uint32_t)k + ((c8 ^ r8) << 4);
+    const uint32_t wq_off = r8 * (uint32_t)kb * 128u + ((c8 ^ r8) << 4);
+    const uint32_t w5_off = (lane >> 1) * (uint32_t)kb * 32u + (lane & 1) * 16u;
+    const uint32_t hd_off = (uint32_t)lane * (uint32_t)kb * (uint32_t)CQ_Q4K_HDR;   // lanes 0..15: the header of row `lane`
+    uint32_t a_col[1][2];
+    {
+        const uint32_t row = r < 8u * RT ? r : 8u * RT - 1;
+#pragma unroll
+        for (uint32_t e = 0; e < 2; e++) a_col[0][e] = (row >> 3) * 2048u + (row & 7) * 128u + (((4 * e + kq) ^ (row & 7)) << 4);
+    }
+    ResPlanes pl;
+    pl.wq = wave_rsrc(w.p0);
+    pl.wh = wave_rsrc(w.p1);
+    pl.w5 = wave_rsrc(w.p2);
+    pl.aq = wave_rsrc(a.qs);
+    pl.ad = wave_rsrc(a.dT);
+    pl.am = wave_rsrc(a.bsh);
+    const __amdgpu_buffer_rsrc_t hdr = wave_rsrc(w.p1);
+    const uint32_t kb32 = (uint32_t)kb, k32 = (uint32_t)k, mstr = (uint32_t)a.m_stride;
+    uint8_t *act = smem + b * R::kActBlk;
+    uint8_t *ring = wgt_base + (size_t)b * 2 * M::kSlot;
+
+    // ---- the wave's activation slice, once
+    if (has) {
+#pragma unroll
+        for (int i = 0; i < 2 * RT; i++) {
+            const uint32_t rg = i >> 1, kh = i & 1;
+            dma16s(pl.aq, act_off, rg * 8u * k32 + b * 256u + kh * 128u, act + i * 1024);
+        }
+        if (lane < 8 * RT) dma4s(pl.ad, lane * 4u, b * mstr * 4u, act + R::oD8);
+        if (MINS && lane < 16 * RT) dma16s(pl.am, lane * 16u, b * mstr * 32u, act + R::oMin);
+    }
+    for (int64_t t0 = blockIdx.x; t0 < tiles; t0 += kTilesPerRound * G) {
+        // tiles of this round: t0, t0 + G, ... (cnt of them)
+        int cnt = (int)((tiles - t0 + G - 1) / G);
+        cnt = cnt < kTilesPerRound ? cnt : kTilesPerRound;
+        if (has) {
+            v4f o0 = {0.0f, 0.0f, 0.0f, 0.0f}, o1 = o0, o2 = o0, o3 = o0;
+            multi_issue<DT, RT>(ring, pl, hdr, (uint32_t)t0 * 16u, b, kb32, wq_off, w5_off, hd_off, lane);
+            if (cnt > 1) multi_issue<DT, RT>(ring + M::kSlot, pl, hdr, (uint32_t)(t0 + G) * 16u, b, kb32, wq_off, w5_off, hd_off, lane);
+#pragma nounroll
+            for (int i = 0; i < cnt; i++) {
+                // everything but the copies of the next tile has landed
+                if (i + 1 < cnt) __builtin_amdgcn_s_waitcnt(kAhead);
+                else __builtin_amdgcn_s_waitcnt(0x0F70);
+                const int64_t tile = t0 + i * G;
+                v4f acc[1] = {{0.0f, 0.0f, 0.0f, 0.0f}};
+                multi_step<DT, RT, DUMP>(ring + (i & 1) * M::kSlot, act, lane, pl, hdr, i + 2 < cnt, (uint32_t)(tile + 2 * G), b, kb32,
+                                         wq_off, w5_off, hd_off, a_col, acc, dump, (tile * 16 + r) * kb + b, w.n * kb, m);
+                // (i is wave-uniform: real branches, four moves, instead of sixteen selects - the empty statements keep them)
+                if (i == 0) { o0 = acc[0]; asm volatile(""); }
+                else if (i == 1) { o1 = acc[0]; asm volatile(""); }
+                else if (i == 2) { o2 = acc[0]; asm volatile(""); }
+                else { o3 = acc[0]; asm volatile(""); }
+            }
+            // ---- the round's partial tiles into the wave's slots (every copy into them has landed and been unpacked)
+            *(v4f *)(ring + lane * 16) = o0;
+            *(v4f *)(ring + 1024 + lane * 16) = o1;
+            *(v4f *)(ring + 2048 + lane * 16) = o2;
+            *(v4f *)(ring + 3072 + lane * 16) = o3;
+        }
+        __syncthreads();
+        if (wave < cnt && !DUMP) {   // wave i sums tile i of the round, in wave order
+            v4f s = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+            const int64_t nw = kb < kWaves ? kb : kWaves;   // waves that own a block
+            for (int64_t o = 0; o < nw; o++) {
+                const v4f p = *(const v4f *)(wgt_base + (size_t)o * 2 * M::kSlot + wave * 1024 + lane * 16);
+                s += p;
+            }
+            const int64_t col = (t0 + wave * G) * 16 + r;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int64_t row = kq * 4 + i;
+                if (row < m) y[row * w.n + col] = s[i];
+            }
+        }
+        if (t0 + kTilesPerRound * G < tiles) __syncthreads();   // the sums have been read: the slots take the next round's copies
     }
 }
 
@@ -915,6 +1091,13 @@ hipError_t launch_res_inst(const cq_weight *w, cq_act_view a, int64_t m, float *
     CQ_LAUNCH((skinny_resident_kernel<DT, RT, NW, NBUF, DUMP>), grid, NW * 64, lds, s, *w, a, m, y, d);
     return hipGetLastError();
 }
+template <int DT, int RT, int NW, bool DUMP>
+hipError_t launch_multi_inst(const cq_weight *w, cq_act_view a, int64_t m, float *y, size_t lds, unsigned grid, cq_mfma_dump d,
+                             hipStream_t s) {
+    if (hipError_t e = cq_ensure_lds<skinny_resident_multi_kernel<DT, RT, NW, DUMP>>(w->dev, lds); e != hipSuccess) return e;
+    CQ_LAUNCH((skinny_resident_multi_kernel<DT, RT, NW, DUMP>), grid, NW * 64, lds, s, *w, a, m, y, d);
+    return hipGetLastError();
+}
 template <int DT, int RT, bool DUMP>
 bool launch_res_rt(const cq_weight *w, cq_act_view a, int64_t m, float *y, cq_mfma_dump d, hipStream_t s, hipError_t *err) {
     const int64_t kb = w->k >> 8, tiles = w->n / 16;
@@ -929,7 +1112,22 @@ bool launch_res_rt(const cq_weight *w, cq_act_view a, int64_t m, float *y, cq_mf
     // Measured (Q4K, 16 rows, matmul kernel alone): 4096 x 4096, one tile per workgroup, 5.95 us against 6.5 us for the
     // kernel that copies activations per block; 11008 x 4096, two or three tiles per workgroup, 12.7 against 12.5 us
     // (also with the next tile's weights copied ahead into a second buffer): taken where every workgroup has one tile.
-    if (tiles > grid) return false;
+    if (tiles > grid) {
+        // several tiles per workgroup: the kernel that meets once per round of tiles, where a wave has one K block
+        if constexpr (RT <= 2 && (DT == CQ_DTYPE_Q4K || DT == CQ_DTYPE_Q5K)) {
+            const size_t two = ResMulti<DT, RT>::bytes(kb);
+            // Measured (Q4K, whole calls in us, the kernel that copies activations per block -> this one): 16 rows 11008 x 4096
+            // 13.6 -> 12.6, 14336 x 4096 15.9 -> 14.3, 32000 x 4096 28.3 -> 24.1; 8 rows 11.7 -> 12.2, 14.1 -> 13.6, 24.1 -> 23.6:
+            // with up to 8 rows five of the other kernel's workgroups share a CU and hide each other's waits.
+            // K = 2048 (eight waves): 16 rows 8192 x 2048 10.0 -> 10.2; left with the other kernel.
+            const bool pays = RT == 2 || tiles > 3 * (int64_t)cus;
+            if (pays && sixteen && kb <= 16 && two <= (size_t)kMaxLds) {
+                *err = launch_multi_inst<DT, RT, 16, DUMP>(w, a, m, y, two, grid, d, s);
+                return true;
+            }
+        }
+        return false;
+    }
     const size_t one = Res<DT, RT>::bytes(kb, 1);
     if (one <= (size_t)kMaxLds) {
         *err = sixteen ? launch_res_inst<DT, RT, 16, 1, DUMP>(w, a, m, y, one, grid, d, s)

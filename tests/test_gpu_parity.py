@@ -265,6 +265,22 @@ def test_small_batch_matches_oracle(qh, dt, m, k, n):
     check_f32(got, orc.matmul(dt, x, blocks, n))
 
 
+@pytest.mark.parametrize("dt,m,n", [(orc.Q4K, 9, 11008), (orc.Q4K, 16, 14336), (orc.Q4K, 13, 16 * 1100), (orc.Q4K, 8, 16 * 800),
+                                     (orc.Q4K, 16, 16 * 1025), (orc.Q5K, 5, 16 * 800), (orc.Q5K, 16, 11008), (orc.Q6K, 16, 11008)])
+def test_small_batch_many_tiles_match_oracle(qh, dt, m, n):
+    """5-16 rows against more 16-row weight tiles than compute units at K = 4096: two to five tiles per workgroup
+    (rounds of four with one meeting each, a second round of a single tile), and the cases next to them that the
+    per-block kernel takes."""
+    w, x = make_inputs(3 * dt + m + n, m, 4096, n, outliers=True)
+    blocks = orc.quantize(dt, w)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, 4096)
+    got = qh.qmatmul(qw, dev(x)).cpu().numpy()
+    check_f32(got, orc.matmul(dt, x, blocks, n))
+    # run-to-run: the partial tiles are summed in wave order
+    again = qh.qmatmul(qw, dev(x)).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
+
+
 @pytest.mark.parametrize("dt", WEIGHT_DTYPES)
 @pytest.mark.parametrize("m,k,n", [(3, 512, 37), (5, 1024, 64), (7, 2048, 9), (9, 256, 130), (12, 11008, 24),
                                    (2, 256, 8), (8, 14336, 16), (70, 512, 48), (133, 256, 32)])
