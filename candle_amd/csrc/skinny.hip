@@ -1007,6 +1007,192 @@ __global__ void __launch_bounds__(kWaves * 64) skinny_blk32_resident_kernel(cq_w
     }
 }
 
+// ------------------------------------- Q8_0 / Q4_0: resident activations, several tiles per workgroup ----
+// The counterpart of skinny_resident_multi_kernel for the 32-element block types: one K group of 256 elements per wave
+// (k <= 256 x waves), rounds of up to four 16-row tiles with one meeting per round, the weight scales through an LDS
+// copy like the weights.  Q8_0 tiles are 4 KiB per wave and the LDS has room for one slot each: a tile's operands
+// are read into registers first and the next tile's copies go out right behind them, under the MFMAs and the
+// scaling.  Q4_0 (2 KiB) has two slots and keeps the tile after the next in flight.
+//   LDS: activation groups as skinny_blk32_resident_kernel | per wave kSlots x {weights kWgt | scales 16 rows x 16 B};
+//        the slots take the wave's partial results (1 KiB per tile) at the end of a round
+template <int DT, int RT> struct ResQ8Multi {
+    typedef ResQ8<DT, RT> R;
+    static constexpr int kSlots = R::Q4 ? 2 : 1;
+    static constexpr int oSc = R::kWgt, kSlot = R::kWgt + 256;
+    static constexpr int kCopies = (R::Q4 ? 2 : 4) + 1;   // copy instructions per tile (blk32_multi_issue)
+    static size_t bytes(int64_t kg) { return (size_t)kg * R::kActGrp + (size_t)kg * kSlots * kSlot; }
+};
+
+template <int DT, int RT>
+__device__ __forceinline__ void blk32_multi_issue(uint8_t *__restrict__ slot, const cq_weight &w, int64_t n_tile, int64_t g, uint32_t row_off,
+                                                  uint32_t q4_off, uint32_t ws_off, int lane) {
+    typedef ResQ8Multi<DT, RT> M;
+    const int64_t k = w.k, kb = w.k >> 5;
+    if (M::R::Q4) {
+#pragma unroll
+        for (int rg = 0; rg < 2; rg++) dma16(w.p0 + (n_tile + rg * 8) * (k >> 1) + g * 128, q4_off, slot + rg * 1024);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int rg = i >> 1, kh = i & 1;
+            dma16(w.p0 + (n_tile + rg * 8) * k + g * 256 + kh * 128, row_off, slot + i * 1024);
+        }
+    }
+    if (lane < 16) dma16(w.p1 + (n_tile * kb + g * 8) * 2, ws_off, slot + M::oSc);   // eight f16 scales of row `lane`
+}
+
+// One tile of one wave: operands out of `slot` into registers, the copies of a tile ahead into the free slot, MFMAs.
+template <int DT, int RT, bool DUMP>
+__device__ __forceinline__ void blk32_multi_step(uint8_t *__restrict__ slot, const uint8_t *__restrict__ act, int lane, const cq_weight &w,
+                                                 bool ahead, int64_t tile_ahead, int64_t g, uint32_t row_off, uint32_t q4_off,
+                                                 uint32_t ws_off, uint32_t w4_col, uint32_t w4_shift, const uint32_t (&w_col)[4],
+                                                 const uint32_t (&a_col)[4], v4f &out, const cq_mfma_dump &dump, int64_t at, int64_t rs,
+                                                 int64_t m) {
+    typedef ResQ8Multi<DT, RT> M;
+    typedef ResQ8<DT, RT> R;
+    constexpr bool Q4 = R::Q4;
+    const uint32_t r = lane & 15, kq = lane >> 4;
+    const uint4 dwv = *(const uint4 *)(slot + M::oSc + r * 16u);
+    long wv[8];
+#pragma unroll
+    for (int b = 0; b < 8; b++) {
+        if (Q4) {
+            const uint2 raw = *(const uint2 *)(slot + w4_col + (((uint32_t)b ^ (r & 7)) << 4));
+            const uint32_t lo = (raw.x >> w4_shift) & 0x0F0F0F0Fu, hi = (raw.y >> w4_shift) & 0x0F0F0F0Fu;
+            wv[b] = (long)(((uint64_t)hi << 32) | lo);
+        } else {
+            wv[b] = *(const long *)(slot + w_col[b & 3] + (b >> 2) * 1024);
+        }
+    }
+    if (ahead) {
+        __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the reads above are done with the slot
+        blk32_multi_issue<DT, RT>(slot, w, tile_ahead * 16, g, row_off, q4_off, ws_off, lane);
+    }
+    const uint32_t dww[4] = {dwv.x, dwv.y, dwv.z, dwv.w};
+#pragma unroll
+    for (int b = 0; b < 8; b++) {
+        const float dw = cq_h2f((uint16_t)(dww[b >> 1] >> (16 * (b & 1))));
+        const long av = *(const long *)(act + a_col[b & 3] + (b >> 2) * 1024);
+        const v4i acc = __builtin_amdgcn_mfma_i32_16x16x32_i8(av, wv[b], (v4i){0, 0, 0, 0}, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            // scales of result row 4kq + i (rows past the held groups: the last one, not stored)
+            const uint32_t srow_i = 4 * kq + i < 8u * RT ? 4 * kq + i : 8u * RT - 1;
+            const float da = *(const float *)(act + R::oD + srow_i * 32 + b * 4);
+            const int I = Q4 ? acc[i] - 8 * *(const int32_t *)(act + R::oBs + srow_i * 32 + b * 4) : acc[i];
+            if (DUMP) {
+                const int64_t orow = kq * 4 + i;
+                if (orow < m) dump.i[at + orow * rs + b] = I;
+            } else {
+                out[i] = __builtin_fmaf((float)I * dw, da, out[i]);
+            }
+        }
+    }
+}
+
+// m <= 8 * RT <= 16 rows; n % 16 == 0; k / 256 <= kWaves.
+template <int DT, int RT, int kWaves, bool DUMP>
+__global__ void __launch_bounds__(kWaves * 64) skinny_blk32_multi_kernel(cq_weight w, cq_act_view a, int64_t m,
+                                                                         float *__restrict__ y, cq_mfma_dump dump) {
+    typedef ResQ8<DT, RT> R;
+    typedef ResQ8Multi<DT, RT> M;
+    constexpr bool Q4 = R::Q4;
+    static_assert(RT <= 2, "one 16-row tile of activation rows");
+    static_assert(M::kSlots * M::kSlot >= kTilesPerRound * 1024, "a round's partial tiles fit the wave's slots");
+    constexpr int kAhead = 0x0F70 | M::kCopies;   // s_waitcnt vmcnt(copies of one tile)
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t r = lane & 15, kq = lane >> 4;
+    const int64_t k = w.k, kg = w.k >> 8, kb = w.k >> 5;
+    const int64_t tiles = w.n / 16, G = gridDim.x;
+    uint8_t *wgt_base = smem + kg * R::kActGrp;
+    const bool has = wave < kg;   // this wave owns K group `wave`
+    const int64_t g = wave;
+
+    const uint32_t r8 = lane >> 3, c8 = lane & 7;
+    const uint32_t row_off = r8 * (uint32_t)k + ((c8 ^ r8) << 4);
+    const uint32_t q4_off = r8 * (uint32_t)(k >> 1) + ((c8 ^ r8) << 4);
+    const uint32_t ws_off = (uint32_t)lane * (uint32_t)kb * 2u;   // lanes 0..15: the scales of row `lane`
+    const int64_t srow = (int64_t)(lane >> 1) < m ? (lane >> 1) : m - 1;
+    const uint32_t sc_off = (uint32_t)(srow * kb * 4) + (lane & 1) * 16u;
+    const uint32_t w4_col = (r >> 3) * 1024u + (r & 7) * 128u + (kq & 1) * 8u, w4_shift = 4 * (kq >> 1);
+    uint32_t w_col[4], a_col[4];
+    {
+        const uint32_t row = r < 8u * RT ? r : 8u * RT - 1;
+#pragma unroll
+        for (uint32_t c = 0; c < 4; c++) {
+            w_col[c] = (r >> 3) * 2048u + (r & 7) * 128u + (((2 * c + (kq >> 1)) ^ (r & 7)) << 4) + (kq & 1) * 8u;
+            a_col[c] = (row >> 3) * 2048u + (row & 7) * 128u + (((2 * c + (kq >> 1)) ^ (row & 7)) << 4) + (kq & 1) * 8u;
+        }
+    }
+    uint8_t *act = smem + g * R::kActGrp;
+    uint8_t *ring = wgt_base + (size_t)g * M::kSlots * M::kSlot;
+
+    // ---- the wave's activation group, once
+    if (has) {
+#pragma unroll
+        for (int i = 0; i < 2 * RT; i++) {
+            const int rg = i >> 1, kh = i & 1;
+            dma16(a.qs + (int64_t)(rg * 8) * k + g * 256 + kh * 128, row_off, act + i * 1024);
+        }
+        if (lane < 16 * RT) dma16((const uint8_t *)(a.d + g * 8), sc_off, act + R::oD);
+        if (Q4 && lane < 16 * RT) dma16((const uint8_t *)(a.bsum32 + g * 8), sc_off, act + R::oBs);
+    }
+    for (int64_t t0 = blockIdx.x; t0 < tiles; t0 += kTilesPerRound * G) {
+        int cnt = (int)((tiles - t0 + G - 1) / G);
+        cnt = cnt < kTilesPerRound ? cnt : kTilesPerRound;
+        if (has) {
+            v4f o0 = {0.0f, 0.0f, 0.0f, 0.0f}, o1 = o0, o2 = o0, o3 = o0;
+            blk32_multi_issue<DT, RT>(ring, w, t0 * 16, g, row_off, q4_off, ws_off, lane);
+            if (M::kSlots == 2 && cnt > 1) blk32_multi_issue<DT, RT>(ring + M::kSlot, w, (t0 + G) * 16, g, row_off, q4_off, ws_off, lane);
+#pragma nounroll
+            for (int i = 0; i < cnt; i++) {
+                // everything but the copies of a tile in flight ahead has landed
+                if (M::kSlots == 2 && i + 1 < cnt) __builtin_amdgcn_s_waitcnt(kAhead);
+                else __builtin_amdgcn_s_waitcnt(0x0F70);
+                const int64_t tile = t0 + i * G;
+                v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+                blk32_multi_step<DT, RT, DUMP>(ring + (M::kSlots == 2 ? (i & 1) * M::kSlot : 0), act, lane, w, i + M::kSlots < cnt,
+                                               tile + M::kSlots * G, g, row_off, q4_off, ws_off, w4_col, w4_shift, w_col, a_col, acc, dump,
+                                               (tile * 16 + r) * kb + g * 8, w.n * kb, m);
+                if (i == 0) { o0 = acc; asm volatile(""); }
+                else if (i == 1) { o1 = acc; asm volatile(""); }
+                else if (i == 2) { o2 = acc; asm volatile(""); }
+                else { o3 = acc; asm volatile(""); }
+            }
+            *(v4f *)(ring + lane * 16) = o0;
+            *(v4f *)(ring + 1024 + lane * 16) = o1;
+            *(v4f *)(ring + 2048 + lane * 16) = o2;
+            *(v4f *)(ring + 3072 + lane * 16) = o3;
+        }
+        __syncthreads();
+        if (wave < cnt && !DUMP) {   // wave i sums tile i of the round, in wave order
+            v4f s = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+            const int64_t nw = kg < kWaves ? kg : kWaves;   // waves that own a group
+            for (int64_t o = 0; o < nw; o++) {
+                const v4f p = *(const v4f *)(wgt_base + (size_t)o * M::kSlots * M::kSlot + wave * 1024 + lane * 16);
+                s += p;
+            }
+            const int64_t col = (t0 + wave * G) * 16 + r;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int64_t row = kq * 4 + i;
+                if (row < m) y[row * w.n + col] = s[i];
+            }
+        }
+        if (t0 + kTilesPerRound * G < tiles) __syncthreads();   // the sums have been read: the slots take the next round's copies
+    }
+}
+
+template <int DT, int RT, int NW, bool DUMP>
+hipError_t launch_blk32_multi_inst(const cq_weight *w, cq_act_view a, int64_t m, float *y, size_t lds, unsigned grid, cq_mfma_dump d,
+                                   hipStream_t s) {
+    if (hipError_t e = cq_ensure_lds<skinny_blk32_multi_kernel<DT, RT, NW, DUMP>>(w->dev, lds); e != hipSuccess) return e;
+    CQ_LAUNCH((skinny_blk32_multi_kernel<DT, RT, NW, DUMP>), grid, NW * 64, lds, s, *w, a, m, y, d);
+    return hipGetLastError();
+}
+
 template <int DT, int RT, int NW, bool DUMP>
 hipError_t launch_blk32_res_inst(const cq_weight *w, cq_act_view a, int64_t m, float *y, size_t lds, cq_mfma_dump d, hipStream_t s) {
     if (hipError_t e = cq_ensure_lds<skinny_blk32_resident_kernel<DT, RT, NW, DUMP>>(w->dev, lds); e != hipSuccess) return e;
@@ -1020,8 +1206,18 @@ bool launch_blk32_res_rt(const cq_weight *w, cq_act_view a, int64_t m, float *y,
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     if (cus <= 0) cus = 256;
-    if (tiles > cus) return false;
     const bool sixteen = kg > 8;
+    if (tiles > cus) {
+        // several tiles per workgroup: rounds of tiles with one meeting each, where a wave has one K group
+        if constexpr (RT <= 2) {
+            const size_t lm = ResQ8Multi<DT, RT>::bytes(kg);
+            if (sixteen && kg <= 16 && lm <= (size_t)kMaxLds && (uint64_t)w->n * (uint64_t)w->k < (1ull << 32)) {
+                *err = launch_blk32_multi_inst<DT, RT, 16, DUMP>(w, a, m, y, lm, (unsigned)cus, d, s);
+                return true;
+            }
+        }
+        return false;
+    }
     if (kg > (sixteen ? 16 : 8) * kMaxBpw) return false;
     const size_t lds = ResQ8<DT, RT>::bytes(kg);
     if (lds > (size_t)kMaxLds) return false;

@@ -111,11 +111,13 @@ def test_skinny_kernel_integers_many_tiles(qh, dt):
 
 
 @pytest.mark.parametrize("dt,m,n", [(orc.Q4K, 16, 16 * 300), (orc.Q4K, 11, 16 * 700), (orc.Q4K, 16, 16 * 1100),
-                                     (orc.Q4K, 7, 16 * 800), (orc.Q5K, 8, 16 * 800), (orc.Q5K, 16, 16 * 300)])
+                                     (orc.Q4K, 7, 16 * 800), (orc.Q5K, 8, 16 * 800), (orc.Q5K, 16, 16 * 300),
+                                     (orc.Q8_0, 16, 16 * 300), (orc.Q8_0, 5, 16 * 1100), (orc.Q4_0, 16, 16 * 700),
+                                     (orc.Q4_0, 8, 16 * 1030)])
 def test_skinny_kernel_integers_rounds_of_tiles(qh, dt, m, n):
     """K = 4096 and more 16-row tiles than compute units: a workgroup walks its tiles in rounds of up to four with one
-    meeting per round (Q4K / Q5K where the slots fit the LDS; the other cases take the per-block kernel): one tile
-    more for some workgroups than for others, two rounds, a round of one."""
+    meeting per round (Q4K / Q5K / Q8_0 / Q4_0 where the slots fit the LDS; the other cases take the per-block kernel):
+    one tile more for some workgroups than for others, two rounds, a round of one."""
     check_dump(qh, dt, qh.MFMA_SKINNY, m, 4096, n, 5 * dt + m + n)
 
 

@@ -266,7 +266,9 @@ def test_small_batch_matches_oracle(qh, dt, m, k, n):
 
 
 @pytest.mark.parametrize("dt,m,n", [(orc.Q4K, 9, 11008), (orc.Q4K, 16, 14336), (orc.Q4K, 13, 16 * 1100), (orc.Q4K, 8, 16 * 800),
-                                     (orc.Q4K, 16, 16 * 1025), (orc.Q5K, 5, 16 * 800), (orc.Q5K, 16, 11008), (orc.Q6K, 16, 11008)])
+                                     (orc.Q4K, 16, 16 * 1025), (orc.Q5K, 5, 16 * 800), (orc.Q5K, 16, 11008), (orc.Q6K, 16, 11008),
+                                     (orc.Q8_0, 16, 11008), (orc.Q8_0, 6, 16 * 1100), (orc.Q8_0, 12, 16 * 1025), (orc.Q4_0, 16, 11008),
+                                     (orc.Q4_0, 7, 16 * 1100), (orc.Q4_0, 9, 16 * 1025), (orc.Q5_0, 16, 11008), (orc.Q4_1, 11, 11008)])
 def test_small_batch_many_tiles_match_oracle(qh, dt, m, n):
     """5-16 rows against more 16-row weight tiles than compute units at K = 4096: two to five tiles per workgroup
     (rounds of four with one meeting each, a second round of a single tile), and the cases next to them that the
