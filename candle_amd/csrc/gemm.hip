@@ -63,6 +63,12 @@ template <int DT, int MT> struct Tile {
     static constexpr int kBytes = oMin + kMin;                                  // one activation stage (three of them)
     static constexpr int oWgt = 3 * kBytes;                                     // weights: one buffer per wave
     static constexpr int kTotal = oWgt + kWaves * kWgtWave;
+    // two buffers per wave (WBUF == 2): each also takes the 32 rows' block headers (bytes 0..15 at kWgtWave + 16 r,
+    // bytes 16..19 at kWgtWave + 512 + 4 r)
+    // ... and a fourth activation stage: the copies of block b+2 are issued while block b is contracted
+    static constexpr int oHdr = kWgtWave, kSlot2 = kWgtWave + 640;
+    static constexpr int oWgt2 = 4 * kBytes;
+    static constexpr int kTotal2 = oWgt2 + kWaves * 2 * kSlot2;
 };
 
 // both 16-bit halves of `a` times `b` (a splat: the packed instruction takes one half of its operand twice)
@@ -88,6 +94,10 @@ __device__ __forceinline__ void dma16(const void *base, uint32_t off, uint8_t *l
 __device__ __forceinline__ void dma4(const void *base, uint32_t off, uint8_t *lds) {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(wave_rsrc(base), (lptr_t)lds, 4, (int)off, 0, 0, 0);
 }
+// the same 16 bytes further on in both memories (the instruction's immediate offset moves both addresses)
+__device__ __forceinline__ void dma4_at16(const void *base, uint32_t off, uint8_t *lds) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(wave_rsrc(base), (lptr_t)lds, 4, (int)off, 0, 16, 0);
+}
 
 // Per-lane constants of the copies and of the operand reads.
 // Q4K / Q5K min term: tiles of up to 64 rows keep it in an accumulator of its own until the integers are scaled; the
@@ -99,6 +109,7 @@ struct LaneGeo {
     uint32_t wq_off;    // the same over the weights' 128-byte plane: (l/8)*kb*128 + ...
     uint32_t wh_off;    // Q6K qh plane, 16 rows x 64 B: (l/4)*kb*64 + ((l%4) ^ ((l/8)%4))*16
     uint32_t w5_off;    // Q5K fifth-bit plane, 32 rows x 32 B: (l/2)*kb*32 + (l%2)*16
+    uint32_t hd_off;    // Q4K / Q5K header plane, the 20 bytes of row l%32: (l%32)*kb*20
     uint32_t col[4];    // operand read: byte offset of chunk 2j+h of row l%32 inside a [4][8][8] x 16 B image
     uint32_t qh_col[4]; // Q6K: byte offset of the 8 bytes of unit 2x+h of row l%32 inside the qh image
 };
@@ -112,6 +123,7 @@ __device__ __forceinline__ LaneGeo lane_geo(int lane, int64_t k) {
     const uint32_t r16 = lane >> 2, c4 = lane & 3;
     g.wh_off = r16 * kb * 64u + ((c4 ^ ((r16 >> 1) & 3)) << 4);
     g.w5_off = (uint32_t)(lane >> 1) * kb * 32u + (uint32_t)(lane & 1) * 16u;
+    g.hd_off = (uint32_t)(lane & 31) * kb * (uint32_t)CQ_Q4K_HDR;
     const uint32_t r = lane & 31, h = lane >> 5;
 #pragma unroll
     for (uint32_t j = 0; j < 4; j++) {
@@ -164,6 +176,44 @@ __device__ __forceinline__ void stage_weights(uint8_t *wl, const cq_weight &w, c
         if (DT == CQ_DTYPE_Q5K) dma16(w.p2 + (n_tile * kb + b) * 32, g.w5_off, wl + 4096);
     }
 }
+// s_waitcnt vmcnt(n) lgkmcnt(0) for a wave-uniform n <= 15 (the instruction takes the count as an immediate).
+__device__ __forceinline__ void wait_all_but(int n) {
+    switch (n) {
+    case 0: __builtin_amdgcn_s_waitcnt(0x0070); break;
+    case 1: __builtin_amdgcn_s_waitcnt(0x0071); break;
+    case 2: __builtin_amdgcn_s_waitcnt(0x0072); break;
+    case 3: __builtin_amdgcn_s_waitcnt(0x0073); break;
+    case 4: __builtin_amdgcn_s_waitcnt(0x0074); break;
+    case 5: __builtin_amdgcn_s_waitcnt(0x0075); break;
+    case 6: __builtin_amdgcn_s_waitcnt(0x0076); break;
+    case 7: __builtin_amdgcn_s_waitcnt(0x0077); break;
+    case 8: __builtin_amdgcn_s_waitcnt(0x0078); break;
+    case 9: __builtin_amdgcn_s_waitcnt(0x0079); break;
+    case 10: __builtin_amdgcn_s_waitcnt(0x007A); break;
+    case 11: __builtin_amdgcn_s_waitcnt(0x007B); break;
+    case 12: __builtin_amdgcn_s_waitcnt(0x007C); break;
+    default: __builtin_amdgcn_s_waitcnt(0x0070); break;
+    }
+}
+// Copy instructions one wave issues in stage_issue.
+template <int DT, int MT> __device__ __forceinline__ int stage_copies(int wave) {
+    return MT * 8 / kWaves + (wave < (MT * 32 + 63) / 64 ? 1 : 0) + (is_k4(DT) && wave >= 4 && wave < 4 + MT ? 1 : 0);
+}
+// Copy instructions of stage_weights_hdr (the count of its s_waitcnt).
+template <int DT> constexpr int weight_copies_hdr() { return 4 + (DT == CQ_DTYPE_Q5K ? 1 : 0) + 2; }
+// The same plus the 32 rows' block headers behind the weights (Q4K / Q5K; lanes 0..31).
+template <int DT, int MT>
+__device__ __forceinline__ void stage_weights_hdr(uint8_t *wl, const cq_weight &w, const LaneGeo &g, int64_t n_tile, int64_t b,
+                                                  int lane) {
+    typedef Tile<DT, MT> T;
+    stage_weights<DT>(wl, w, g, n_tile, b);
+    const int64_t kb = w.k >> 8;
+    if (lane < 32) {
+        const uint8_t *h = w.p1 + (n_tile * kb + b) * CQ_Q4K_HDR;
+        dma16(h, g.hd_off, wl + T::oHdr);
+        dma4_at16(h, g.hd_off, wl + T::oHdr + 512 - 16);
+    }
+}
 
 // The small per-block weight fields, loaded straight into registers one block ahead.
 template <int DT> struct WHead;
@@ -179,6 +229,14 @@ __device__ __forceinline__ void load_head(const cq_weight &w, int64_t blk, WHead
     r.sc = *(const uint4 *)(w.p2 + blk * 16);
     r.d = ((const uint16_t *)w.p3)[blk];
 }
+// The header of row l%32 out of the copy stage_weights_hdr made.
+__device__ __forceinline__ void head_from_lds(const uint8_t *hd, int lane, WHead<CQ_DTYPE_Q4K> &r) {
+    const uint32_t row = lane & 31;
+    const uint4 v = *(const uint4 *)(hd + row * 16u);
+    r.dd = v.x;
+    r.rec = make_uint4(v.y, v.z, v.w, *(const uint32_t *)(hd + 512 + row * 4u));
+}
+__device__ __forceinline__ void head_from_lds(const uint8_t *, int, WHead<CQ_DTYPE_Q6K> &) {}   // (not used: Q6K keeps one buffer)
 
 // Verification build (DUMP): where a lane's integers of the current block go, and how many of the tile rows exist.
 struct DumpLane {
@@ -469,18 +527,27 @@ __device__ __forceinline__ void block_unpack(const uint8_t *wl, const LaneGeo &g
 // which is refilled for block b+1 as soon as they are in registers.  The LDS regions are distinct
 // (`__restrict__`): without that knowledge the compiler makes every LDS read wait for all copies in
 // flight, which would serialise the pipeline.
-template <int DT, int MT, bool TRAIL, bool HALF, bool DUMP>
+// `more`: the block whose copies this step issues exists (b+1; b+2 when WBUF == 2).
+// WBUF == 2 (a launch whose weights come cold from HBM, a few activation rows per weight row: a block takes less time
+// than a copy): everything is copied two blocks ahead.  Two weight buffers per wave - the buffer block b has just been
+// unpacked from takes block b+2 - and four activation stages; the copies of block b+2 stay in flight across the barrier
+// (the waits are written out: everything but those copies).  The block headers then come through the same copies -
+// a load into registers would be tracked by the compiler, which on joining the paths "copies issued" / "no block left"
+// waits as the stricter of the two demands, i.e. for the copies just issued.
+template <int DT, int MT, bool TRAIL, bool HALF, bool DUMP, int WBUF>
 __device__ __forceinline__ void block_step(const uint8_t *__restrict__ cur, uint8_t *__restrict__ nxt,
                                            uint8_t *__restrict__ wl, const cq_weight &w, const cq_act_view &a,
                                            const LaneGeo &g, int64_t m0, int64_t n_tile, bool n_ok, bool more, int64_t b,
-                                           int wave, int lane, const WHead<DT> &hcur, v16f (&out)[MT], const DumpLane &dl) {
+                                           int wave, int lane, const WHead<DT> &hreg, v16f (&out)[MT], const DumpLane &dl) {
     constexpr int SHIFT = DT == CQ_DTYPE_Q4K ? 3 : 8;
     constexpr int SPLIT = TRAIL ? MT / 2 : MT;   // tiles [SPLIT, MT) follow the barrier
     v4i bl[8], bh[8];
     float dw = 0.0f;
     MinW wmin = {};
-    if (more) stage_issue<DT, MT>(nxt, w, a, g, m0, b + 1, wave, lane);
+    if (more) stage_issue<DT, MT>(nxt, w, a, g, m0, b + (WBUF == 2 ? 2 : 1), wave, lane);
     if (n_ok) {
+        WHead<DT> hcur = hreg;
+        if (WBUF == 2) head_from_lds(wl + Tile<DT, MT>::oHdr, lane, hcur);
         block_unpack(wl, g, hcur, lane, bl, bh, dw, wmin);
         if constexpr (DUMP && is_k4(DT)) {
             if (dl.int_min) {   // verification: the minima themselves as the operand, so the MFMAs deliver the integer Mn_b
@@ -489,11 +556,28 @@ __device__ __forceinline__ void block_step(const uint8_t *__restrict__ cur, uint
                 wmin.p2 = __builtin_bit_cast(v8h, cq_min_term_groups_int(rec, (lane >> 5) != 0, true));
             }
         }
-        if (more) stage_weights<DT>(wl, w, g, n_tile, b + 1);
+        if (WBUF == 2) {
+            if (more) {
+                __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the reads above are done with the buffer
+                stage_weights_hdr<DT, MT>(wl, w, g, n_tile, b + 2, lane);
+            }
+        } else if (more) {
+            stage_weights<DT>(wl, w, g, n_tile, b + 1);
+        }
         tiles_mac<DT, MT, 0, SPLIT, SHIFT, HALF, DUMP>(cur, g, bl, bh, dw, wmin, lane, out, dl);
     }
-    __builtin_amdgcn_s_waitcnt(0);   // the next stage and the wave's next weights have landed in LDS
-    __syncthreads();
+    if (WBUF == 2) {
+        // the next stage and the weights of block b+1 have landed; the copies of block b+2 may still be in flight
+        // (the empty statements keep the compiler from moving LDS reads and copies across the barrier, which by itself
+        // orders nothing for it)
+        wait_all_but(more ? stage_copies<DT, MT>(wave) + (n_ok ? weight_copies_hdr<DT>() : 0) : 0);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    } else {
+        __builtin_amdgcn_s_waitcnt(0);   // the next stage and the wave's next weights have landed in LDS
+        __syncthreads();
+    }
     if (TRAIL && n_ok) tiles_mac<DT, MT, SPLIT, MT, SHIFT, HALF, DUMP>(cur, g, bl, bh, dw, wmin, lane, out, dl);
 }
 
@@ -501,9 +585,10 @@ __device__ __forceinline__ void block_step(const uint8_t *__restrict__ cur, uint
 // Requires n % 32 == 0 and an activation workspace with padded rows (cq_act_view::m_stride).
 // One workgroup: activation rows [m0, m0 + 32*MT) (stored up to row m - 1) x the 256 weight rows of
 // blockIdx.x, K blocks of part blockIdx.z.
-template <int DT, int MT, bool DUMP = false>
+template <int DT, int MT, bool DUMP = false, int WBUF = 1>
 __device__ __forceinline__ void gemm_body(const cq_weight &w, const cq_act_view &a, int64_t m0, int64_t m,
                                           float *__restrict__ y, int ksplit, cq_mfma_dump dump = cq_mfma_dump{nullptr, nullptr, 0}) {
+    static_assert(WBUF == 1 || DT == CQ_DTYPE_Q4K || DT == CQ_DTYPE_Q5K, "block headers of 20 bytes");
     typedef Tile<DT, MT> T;
     extern __shared__ __align__(16) uint8_t smem[];
     const int lane = threadIdx.x & 63;
@@ -524,35 +609,50 @@ __device__ __forceinline__ void gemm_body(const cq_weight &w, const cq_act_view 
 #pragma unroll
         for (int i = 0; i < 16; i++) out[t][i] = 0.0f;
 
-    WHead<DT> hcur, hnxt;
-    uint8_t *wl = smem + T::oWgt + wave * T::kWgtWave;
+    WHead<DT> hcur = {}, hnxt = {};
+    uint8_t *wl = WBUF == 2 ? smem + T::oWgt2 + wave * 2 * T::kSlot2 : smem + T::oWgt + wave * T::kWgtWave;
     stage_issue<DT, MT>(smem, w, a, g, m0, b0, wave, lane);
-    if (n_ok) stage_weights<DT>(wl, w, g, n_tile, b0);
-    load_head(w, nc * kb + b0, hcur);
-    hnxt = hcur;
+    if (WBUF == 2) {
+        if (b0 + 1 < b1) stage_issue<DT, MT>(smem + T::kBytes, w, a, g, m0, b0 + 1, wave, lane);
+        if (n_ok) {
+            stage_weights_hdr<DT, MT>(wl, w, g, n_tile, b0, lane);
+            if (b0 + 1 < b1) stage_weights_hdr<DT, MT>(wl + T::kSlot2, w, g, n_tile, b0 + 1, lane);
+        }
+    } else {
+        if (n_ok) stage_weights<DT>(wl, w, g, n_tile, b0);
+        load_head(w, nc * kb + b0, hcur);
+        hnxt = hcur;
+    }
     __builtin_amdgcn_s_waitcnt(0);   // the LDS copies above (and everything else outstanding)
     __syncthreads();
 
-    // Stage of block b: (b - b0) % 3.  Both loops pass the same number of barriers.
-    int ic = 0, in = 1, ifree = 2;
+    // Stage of block b: (b - b0) % 3 (% 4 when WBUF == 2); `in` is the stage this step's copies go to.  Both loops pass
+    // the same number of barriers.
+    int ic = 0, in = WBUF == 2 ? 2 : 1, ifree = WBUF == 2 ? 3 : 2, imid = 1;
     auto rotate = [&]() {
         const int t = ic;
-        ic = in;
+        if (WBUF == 2) {
+            ic = imid;
+            imid = in;
+        } else {
+            ic = in;
+        }
         in = ifree;
         ifree = t;
     };
     auto run = [&](auto trail, auto half) {
         for (int64_t b = b0; b < b1; b++) {
-            const bool more = b + 1 < b1;
-            if (more) load_head(w, nc * kb + b + 1, hnxt);
+            const bool more = b + (WBUF == 2 ? 2 : 1) < b1;
+            if (WBUF == 1 && more) load_head(w, nc * kb + b + 1, hnxt);
             DumpLane dl{nullptr, nullptr, 0, 0, false};
             if (DUMP) {
                 const int64_t at = (m0 * w.n + nc) * kb + b;
                 dl = DumpLane{dump.i + at, dump.mn ? dump.mn + at : nullptr, w.n * kb, m - m0, dump.int_min != 0};
             }
-            block_step<DT, MT, decltype(trail)::value, decltype(half)::value, DUMP>(smem + ic * T::kBytes, smem + in * T::kBytes,
-                                                                                    wl, w, a, g, m0, n_tile, n_ok, more, b, wave,
-                                                                                    lane, hcur, out, dl);
+            uint8_t *wb = WBUF == 2 ? wl + ((b - b0) & 1) * T::kSlot2 : wl;   // the buffer that holds block b
+            block_step<DT, MT, decltype(trail)::value, decltype(half)::value, DUMP, WBUF>(smem + ic * T::kBytes, smem + in * T::kBytes,
+                                                                                          wb, w, a, g, m0, n_tile, n_ok, more, b,
+                                                                                          wave, lane, hcur, out, dl);
             hcur = hnxt;
             rotate();
         }
@@ -608,12 +708,14 @@ struct GroupArgs {
     int8_t expert[kMaxGroupTiles];
 };
 
+// Expert weights are read once per launch, cold: the types whose headers can come through the copies take two buffers.
+template <int DT> constexpr int grouped_wbuf() { return DT == CQ_DTYPE_Q4K || DT == CQ_DTYPE_Q5K ? 2 : 1; }
 template <int DT>
 __global__ void __launch_bounds__(kThreads) gemm_grouped_kernel(GroupArgs ga, cq_act_view a, float *__restrict__ y,
                                                                 int ksplit) {
     const int tile = blockIdx.y;
     const cq_weight w = ga.w[ga.expert[tile]];
-    gemm_body<DT, 1>(w, a, ga.row0[tile], ga.row_end[tile], y, ksplit);
+    gemm_body<DT, 1, false, grouped_wbuf<DT>()>(w, a, ga.row0[tile], ga.row_end[tile], y, ksplit);
 }
 
 // ------------------------------------------------ K-quant weights x Q8_1 activations (tile kernel) ----
@@ -935,7 +1037,7 @@ hipError_t launch_grouped(const cq_weight *const *experts, int n_experts, const 
     }
     if (ntiles == 0) return hipSuccess;
     const cq_weight *w = experts[0];
-    const size_t lds = Tile<DT, 1>::kTotal;
+    const size_t lds = grouped_wbuf<DT>() == 2 ? Tile<DT, 1>::kTotal2 : Tile<DT, 1>::kTotal;
     if (hipError_t e = cq_ensure_lds<gemm_grouped_kernel<DT>>(w->dev, lds); e != hipSuccess) return e;
     const int64_t gx = n_tiles(w);
     const int ksplit = pick_ksplit(gx * ntiles, w->k >> 8, 2 * num_cus());   // two single-tile workgroups per CU
