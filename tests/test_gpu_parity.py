@@ -273,9 +273,20 @@ def test_small_batch_many_tiles_match_oracle(qh, dt, m, n):
     """5-16 rows against more 16-row weight tiles than compute units at K = 4096: two to five tiles per workgroup
     (rounds of four with one meeting each, a second round of a single tile), and the cases next to them that the
     per-block kernel takes."""
-    w, x = make_inputs(3 * dt + m + n, m, 4096, n, outliers=True)
+    check_many_tiles(qh, dt, m, 4096, n)
+
+
+@pytest.mark.parametrize("dt,m,k,n", [(orc.Q4K, 16, 2560, 16 * 300), (orc.Q8_0, 9, 3840, 16 * 520), (orc.Q4_0, 16, 2304, 16 * 1030),
+                                       (orc.Q4K, 12, 3328, 16 * 1100)])
+def test_small_batch_many_tiles_fewer_k_blocks_than_waves(qh, dt, m, k, n):
+    """The same with 9-15 K blocks: some of the sixteen waves own no block and only meet the others."""
+    check_many_tiles(qh, dt, m, k, n)
+
+
+def check_many_tiles(qh, dt, m, k, n):
+    w, x = make_inputs(3 * dt + m + n + k, m, k, n, outliers=True)
     blocks = orc.quantize(dt, w)
-    qw = qh.QWeight.from_ggml(dt, blocks, n, 4096)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
     got = qh.qmatmul(qw, dev(x)).cpu().numpy()
     check_f32(got, orc.matmul(dt, x, blocks, n))
     # run-to-run: the partial tiles are summed in wave order
