@@ -572,6 +572,35 @@ def test_moe_ffn_matches_oracle(qh, tokens, starve):
     assert np.linalg.norm(ys - want) / np.linalg.norm(want) < 5e-3
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3, 4, 5, 6])
+def test_grouped_random_shapes_match_oracle(qh, seed):
+    """The grouped launch over random expert slices (empty ones, more than one 32-row tile, a single row), 1-9 K blocks
+    (fewer blocks than the copies run ahead, odd counts, K split over workgroups or not) and weight row counts that
+    leave waves of the last workgroup without rows: every slice against the oracle's matmul with its expert."""
+    rng = np.random.default_rng(100 + seed)
+    dt = [orc.Q4K, orc.Q5K, orc.Q6K][seed % 3]
+    k = 256 * int(rng.integers(1, 10))
+    n = 32 * int(rng.integers(1, 14))
+    n_e = int(rng.integers(1, 7))
+    rows = [int(rng.choice([0, 1, 5, 16, 17, 31, 32, 33, 45])) for _ in range(n_e)]
+    offsets = np.concatenate([[0], np.cumsum(rows)]).astype(np.int32)
+    total = int(offsets[-1])
+    if total == 0:
+        rows[0] = 7
+        offsets = np.concatenate([[0], np.cumsum(rows)]).astype(np.int32)
+        total = int(offsets[-1])
+    blocks = [orc.quantize(dt, (rng.standard_normal((n, k)) * 0.03).astype(np.float32)) for _ in range(n_e)]
+    experts = [qh.QWeight.from_ggml(dt, b, n, k) for b in blocks]
+    tokens = 19
+    x = rng.standard_normal((tokens, k)).astype(np.float32)
+    rid = rng.integers(0, tokens, size=total).astype(np.int32)
+    y = qh.qmatmul_grouped(experts, dev(x), torch.from_numpy(rid).cuda(), offsets).cpu().numpy()
+    for e in range(n_e):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        if lo < hi:
+            check_f32(y[lo:hi], orc.matmul(dt, x[rid[lo:hi]], blocks[e], n))
+
+
 @pytest.mark.parametrize("tokens,total,hidden", [(5, 9, 6), (7, 200, 8), (64, 128, 4096), (3, 70, 1028), (4, 0, 16)])
 def test_moe_scatter_add_order_and_shapes(qh, tokens, total, hidden):
     """ys[row_ids[p]] += weights[p] * y[p] for p in increasing order (cpu_backend/mod.rs:619-653): both
