@@ -698,6 +698,124 @@ __global__ void __launch_bounds__(kThreads) gemm_dump_kernel(cq_weight w, cq_act
     gemm_body<DT, MT, true>(w, a, (int64_t)blockIdx.y * (MT * 32), m, nullptr, ksplit, dump);
 }
 
+// ------------------------------------------------------ few weight rows, long K: K halved inside the workgroup ----
+// With few 256-row column tiles (n = 4096: sixteen) the launches above fill the machine either with 32-row tiles, which
+// unpack every weight block once per 32 activation rows, or by splitting K over workgroups, whose parts are added to
+// the output atomically (about 1.1 TB/s, and the order of the sum is not fixed).  Here a workgroup covers 128 weight
+// rows x 32*MT activation rows and halves K between its waves: waves 0..3 (one per SIMD) take the first half of the K
+// blocks for their 32 weight rows, waves 4..7 the second half for the same rows - a SIMD's two waves are again half a
+// step apart in what they do, the leading and trailing roles of gemm_body - and the two partial tiles meet in LDS at
+// the end, first half + second half: twice the workgroups at the same tile height, no atomics, a fixed order.
+// Stage layout: two activation parts per stage (the block of each half), Tile::kBytes each.
+template <int DT, int MT> struct TileKH {
+    typedef Tile<DT, MT> T;
+    static constexpr int kStage = 2 * T::kBytes;
+    static constexpr int oWgt = 3 * kStage;
+    static constexpr int kTotal = oWgt + kWaves * T::kWgtWave;
+    static_assert(MT * 16 * 256 * (kWaves / 2) <= oWgt, "the partial tiles of the second half fit the stages");
+};
+
+template <int DT, int MT, bool TRAIL>
+__device__ __forceinline__ void block_step_kh(const uint8_t *__restrict__ cur, uint8_t *__restrict__ nxt, uint8_t *__restrict__ wl,
+                                              const cq_weight &w, const cq_act_view &a, const LaneGeo &g, int64_t m0, int64_t n_tile,
+                                              bool work, int64_t next0, int64_t next1, int64_t mine_next, int wave, int lane,
+                                              const WHead<DT> &hcur, v16f (&out)[MT]) {
+    typedef Tile<DT, MT> T;
+    constexpr int SHIFT = DT == CQ_DTYPE_Q4K ? 3 : 8;
+    constexpr int SPLIT = TRAIL ? MT / 2 : MT;   // tiles [SPLIT, MT) follow the barrier
+    const DumpLane dl{nullptr, nullptr, 0, 0, false};
+    v4i bl[8], bh[8];
+    float dw = 0.0f;
+    MinW wmin = {};
+    if (next0 >= 0) stage_issue<DT, MT>(nxt, w, a, g, m0, next0, wave, lane);
+    if (next1 >= 0) stage_issue<DT, MT>(nxt + T::kBytes, w, a, g, m0, next1, wave, lane);
+    if (work) {
+        block_unpack(wl, g, hcur, lane, bl, bh, dw, wmin);
+        if (mine_next >= 0) stage_weights<DT>(wl, w, g, n_tile, mine_next);
+        tiles_mac<DT, MT, 0, SPLIT, SHIFT, false, false>(cur, g, bl, bh, dw, wmin, lane, out, dl);
+    }
+    __builtin_amdgcn_s_waitcnt(0);   // the next stage and the wave's next weights have landed in LDS
+    __syncthreads();
+    if (TRAIL && work) tiles_mac<DT, MT, SPLIT, MT, SHIFT, false, false>(cur, g, bl, bh, dw, wmin, lane, out, dl);
+}
+
+// Requires n % 32 == 0.  One workgroup: activation rows [m0, m0 + 32*MT) x the 128 weight rows of blockIdx.x, all K.
+template <int DT, int MT>
+__global__ void __launch_bounds__(kThreads) gemm_kh_kernel(cq_weight w, cq_act_view a, int64_t m, float *__restrict__ y) {
+    typedef Tile<DT, MT> T;
+    typedef TileKH<DT, MT> TK;
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int64_t m0 = (int64_t)blockIdx.y * (MT * 32);
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int colw = wave & 3, half = wave >> 2;
+    const int h = lane >> 5, col = lane & 31;
+    const int64_t kb = w.k >> 8;
+    const int64_t n_tile = ((int64_t)blockIdx.x * (kWaves / 2) + colw) * 32;
+    const bool n_ok = n_tile < w.n;
+    const int64_t n = n_tile + col;
+    const int64_t nc = n_ok ? n : 0;
+    const int64_t nh = (kb + 1) / 2;                        // steps; the first half has nh blocks, the second kb - nh
+    const int64_t first = half ? nh : 0, count = half ? kb - nh : nh;
+    const LaneGeo g = lane_geo(lane, w.k);
+
+    v16f out[MT];
+#pragma unroll
+    for (int t = 0; t < MT; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) out[t][i] = 0.0f;
+
+    WHead<DT> hcur = {}, hnxt = {};
+    uint8_t *wl = smem + TK::oWgt + wave * T::kWgtWave;
+    stage_issue<DT, MT>(smem, w, a, g, m0, 0, wave, lane);
+    if (kb - nh > 0) stage_issue<DT, MT>(smem + T::kBytes, w, a, g, m0, nh, wave, lane);
+    if (n_ok && count > 0) {
+        stage_weights<DT>(wl, w, g, n_tile, first);
+        load_head(w, nc * kb + first, hcur);
+    }
+    hnxt = hcur;
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+
+    int ic = 0, in = 1, ifree = 2;
+    for (int64_t it = 0; it < nh; it++) {
+        const bool work = n_ok && it < count;
+        const int64_t next0 = it + 1 < nh ? it + 1 : -1, next1 = it + 1 < kb - nh ? nh + it + 1 : -1;
+        const int64_t mine_next = it + 1 < count ? first + it + 1 : -1;
+        if (n_ok && mine_next >= 0) load_head(w, nc * kb + mine_next, hnxt);
+        const uint8_t *cur = smem + ic * TK::kStage + half * T::kBytes;
+        uint8_t *nxt = smem + in * TK::kStage;
+        if (half == 0) block_step_kh<DT, MT, false>(cur, nxt, wl, w, a, g, m0, n_tile, work, next0, next1, mine_next, wave, lane, hcur, out);
+        else block_step_kh<DT, MT, true>(cur, nxt, wl, w, a, g, m0, n_tile, work, next0, next1, mine_next, wave, lane, hcur, out);
+        hcur = hnxt;
+        const int t = ic;
+        ic = in;
+        in = ifree;
+        ifree = t;
+    }
+
+    // ---- first half + second half through LDS (the stages are free: every wave is past its last read)
+    __syncthreads();
+    float *part = (float *)smem + (size_t)colw * (MT * 16 * 64);
+    if (half == 1) {
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) part[(t * 16 + i) * 64 + lane] = out[t][i];
+    }
+    __syncthreads();
+    if (half == 0 && n_ok) {
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int64_t row = m0 + t * 32 + (i >> 2) * 8 + h * 4 + (i & 3);
+                if (row < m) y[row * w.n + n] = out[t][i] + part[(t * 16 + i) * 64 + lane];
+            }
+        }
+    }
+}
+
 // Grouped (mixture-of-experts) variant: one launch for every expert.  blockIdx.y walks a table of
 // 32-row tiles of the expert-sorted activation rows; each tile names its expert's weights.
 constexpr int kMaxGroupExperts = 16, kMaxGroupTiles = 96;
@@ -955,9 +1073,12 @@ int64_t n_tiles(const cq_weight *w) { return (w->n + kWaves * 32 - 1) / (kWaves 
 // 64 tiles of 128 rows split four ways and 42 us as 256 tiles of 32 rows.
 struct Plan {
     int mt, ksplit;
+    int kh = 1;   // 2: gemm_kh_kernel (K halved inside the workgroup, 128 weight rows per workgroup)
 };
 Plan pick_plan(const cq_weight *w, int64_t m) {
     const int64_t gx = n_tiles(w), kb = w->k >> 8, cus = num_cus();
+    // unpacking one K block of a wave's 32 rows: 152 vector instructions for Q4K, about 370 for Q6K
+    const double unpack = w->dtype == CQ_DTYPE_Q4K ? 22.0 : w->dtype == CQ_DTYPE_Q5K ? 32.0 : 50.0;
     const double atomic_pass = (double)m * (double)w->n * 4.0 / 1.1e6 * 16.0;   // bytes / (1.1e6 bytes per us) in units
     Plan best{1, 1};
     double best_cost = 0.0;
@@ -969,13 +1090,26 @@ Plan pick_plan(const cq_weight *w, int64_t m) {
             if (ks > 1 && kb / ks < 4) break;
             if (ks > 1 && cq_no_split_k()) break;   // CQ_FLAG_DETERMINISTIC
             const int64_t rounds = (tiles * ks + cus - 1) / cus;
-            const double cost = (double)rounds * ((double)((kb + ks - 1) / ks) * (22.0 + 13.5 * mt) + 24.0) +
+            const double cost = (double)rounds * ((double)((kb + ks - 1) / ks) * (unpack + 13.5 * mt) + 24.0) +
                                 (ks > 1 ? ks * atomic_pass : 0.0);
             if (first || cost < best_cost) {
                 best = Plan{mt, ks};
                 best_cost = cost;
                 first = false;
             }
+        }
+    }
+    // K halved inside the workgroup: twice the column tiles, half the blocks per wave, 8 units for the meeting at the end
+    const int64_t gx128 = (w->n + 127) / 128;
+    for (int mt = 2; mt >= 1; mt >>= 1) {
+        if (mt > 1 && m <= 16 * mt) continue;
+        if (kb < 2) break;
+        const int64_t tiles = gx128 * ((m + mt * 32 - 1) / (mt * 32));
+        const int64_t rounds = (tiles + cus - 1) / cus;
+        const double cost = (double)rounds * ((double)((kb + 1) / 2) * (unpack + 13.5 * mt) + 24.0 + 8.0);
+        if (cost < best_cost) {
+            best = Plan{mt, 1, 2};
+            best_cost = cost;
         }
     }
     return best;
@@ -995,9 +1129,19 @@ hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, int
     return hipGetLastError();
 }
 
+template <int DT, int MT>
+hipError_t launch_kh(const cq_weight *w, cq_act_view a, int64_t m, float *y, hipStream_t s) {
+    const size_t lds = TileKH<DT, MT>::kTotal;
+    if (hipError_t e = cq_ensure_lds<gemm_kh_kernel<DT, MT>>(w->dev, lds); e != hipSuccess) return e;
+    dim3 grid((unsigned)((w->n + 127) / 128), (unsigned)((m + MT * 32 - 1) / (MT * 32)), 1);
+    CQ_LAUNCH((gemm_kh_kernel<DT, MT>), grid, kThreads, lds, s, *w, a, m, y);
+    return hipGetLastError();
+}
+
 template <int DT>
 hipError_t launch_dt(const cq_weight *w, cq_act_view a, int64_t m, float *y, bool y_cleared, hipStream_t s) {
     const Plan p = pick_plan(w, m);
+    if (p.kh == 2) return p.mt == 1 ? launch_kh<DT, 1>(w, a, m, y, s) : launch_kh<DT, 2>(w, a, m, y, s);
     if (p.mt == 1) return launch_mt<DT, 1>(w, a, m, y, p.ksplit, y_cleared, s);
     if (p.mt == 2) return launch_mt<DT, 2>(w, a, m, y, p.ksplit, y_cleared, s);
     return launch_mt<DT, 4>(w, a, m, y, p.ksplit, y_cleared, s);

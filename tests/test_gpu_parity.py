@@ -521,6 +521,24 @@ def test_forward_shape_and_errors(qh):
     assert tuple(qh.qmatmul(qw, torch.zeros((0, 256), device="cuda")).shape) == (0, 8)
 
 
+@pytest.mark.parametrize("dt", [orc.Q4K, orc.Q5K, orc.Q6K])
+@pytest.mark.parametrize("m,k,n", [(300, 256 * 7, 1056), (512, 4096, 4096), (130, 256 * 3, 160), (65, 256 * 2, 128),
+                                   (200, 256 * 9, 2048 + 96), (96, 256 * 16, 512)])
+def test_prefill_few_weight_rows_long_k(qh, dt, m, k, n):
+    """Few column tiles and a long K: the launches that halve K between the waves of a workgroup (odd block counts:
+    unequal halves; 2 and 3 blocks; weight row counts that leave waves of the last workgroup without rows; ragged
+    activation rows) - against the oracle, and bit for bit the same on a second call."""
+    w, x = make_inputs(17 * dt + m + k + n, m, k, n, outliers=True)
+    blocks = orc.quantize(dt, w)
+    qw = qh.QWeight.from_ggml(dt, blocks, n, k)
+    got = qh.qmatmul(qw, dev(x)).cpu().numpy()
+    check_f32(got, orc.matmul(dt, x, blocks, n))
+    again = qh.qmatmul(qw, dev(x), qh.FLAG_DETERMINISTIC).cpu().numpy()
+    check_f32(again, got)
+    third = qh.qmatmul(qw, dev(x), qh.FLAG_DETERMINISTIC).cpu().numpy()
+    assert np.array_equal(again.view(np.uint32), third.view(np.uint32))
+
+
 # ------------------------------------------------------------------------- MoE ----
 @pytest.mark.parametrize("tokens,starve", [(24, False), (64, True)])
 def test_moe_ffn_matches_oracle(qh, tokens, starve):
