@@ -535,23 +535,29 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
     // Which kernel takes the rows.  Decided before the quantizer runs, because the quantizer clears the
     // output of a launch that splits K on its way.
     enum { kSkinny, kGemm32, kGemm, kMatvec } path;
-    // Few rows: split K over the waves instead of tiling rows.  Measured faster than the dot-product
-    // kernels from 2 rows on and than the tile kernel up to 32 rows (up to 64 rows when n is small
-    // and the tile kernel cannot fill the machine).
-    // (the 32-element-block types from 4 rows (Q8_0) or 5 rows (Q4_0) on: below that the batched
-    // dot-product kernel is as fast or faster, it has no per-block scaling of MFMA results to do)
+    // Few rows: split K over the waves instead of tiling rows.  Measured (weights from HBM, 4096..32000 weight rows,
+    // k 4096..14336) faster than the dot-product kernels from 2 rows on and than the tile kernels
+    //   up to 16 rows everywhere; up to 24 rows below 24576 weight rows; up to 32 rows below 12288 weight rows;
+    //   up to 64 rows where n is small and k short, so that the tile kernel cannot fill the machine.
+    // (the 32-element-block types from 4 rows (Q8_0) or 5 rows (Q4_0) on: below that the one-launch dot-product
+    // kernel is as fast or faster, it has no per-block scaling of MFMA results to do - where it takes the rows)
+    const bool rows_fused = flags == 0 && pre.kind == CQ_PRE_NONE && !in_place && cq_matvec_fused_rows_supported(w, m);
     const int64_t skinny_from = w->dtype == CQ_DTYPE_Q8_0 ? 4 : w->dtype == CQ_DTYPE_Q4_0 ? 5 : 2;
     const bool has_tile_kernel = cq_gemm_supported(w, m, act);
+    const bool has_tile32 = m > 16 && cq_gemm32_supported(w, act);
+    const bool skinny_rows = m <= 16 || (m <= 24 && w->n < 24576) || (m <= 32 && w->n < 12288) ||
+                             (m <= 64 && w->n < 8192 && w->k <= 6144);
     if (flags & CQ_FLAG_FORCE_SKINNY) {
         if (!cq_skinny_supported(w, act))
             return cq_set_error(CQ_ERR_UNSUPPORTED, "no split-K MFMA kernel for dtype %d with activation dtype %d and n = %lld",
                                 w->dtype, act, (long long)w->n);
         path = kSkinny;
-    } else if (!(flags & CQ_FLAG_FORCE_MATVEC) && m > 32 && cq_gemm32_supported(w, act)) {
-        // Q8_0 / Q4_0 beyond 32 rows: their own tile kernel (whole 256-element K steps, n a multiple of 32)
+    } else if (!(flags & CQ_FLAG_FORCE_MATVEC) && has_tile32) {
+        // Q8_0 / Q4_0 beyond 16 rows: their own tile kernel (whole 256-element K steps, n a multiple of 32), measured
+        // ahead of the split-K kernel from 17 rows on at every shape
         path = kGemm32;
-    } else if (!(flags & (CQ_FLAG_FORCE_GEMM | CQ_FLAG_FORCE_MATVEC)) && m >= skinny_from && cq_skinny_supported(w, act) &&
-               (m <= 32 || (m <= 64 && w->n < 8192) || !has_tile_kernel)) {
+    } else if (!(flags & (CQ_FLAG_FORCE_GEMM | CQ_FLAG_FORCE_MATVEC)) && (m >= skinny_from || (m >= 2 && !rows_fused)) &&
+               cq_skinny_supported(w, act) && (skinny_rows || !has_tile_kernel)) {
         // (shapes the tile kernels do not take: the split-K kernel, 32 rows per pass over the weights, stays
         // ahead of the dot-product kernel, 8 rows per pass, at every row count)
         path = kSkinny;
@@ -572,7 +578,7 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
     // chunks: no limit on k, as in k_quants::matmul)
     // two to four rows of short enough weight rows: the one-launch kernel again, every unpacked weight unit
     // contracted with each activation row
-    if (flags == 0 && pre.kind == CQ_PRE_NONE && !in_place && cq_matvec_fused_rows_supported(w, m)) {
+    if (rows_fused) {
         CQ_HIP_CHECK(cq_launch_matvec_fused_rows(w, x_dev, m, y_dev, s));
         return CQ_OK;
     }
@@ -697,7 +703,7 @@ extern "C" int cq_qmatmul_int_dots_mfma(const cq_weight *w, const float *x_dev, 
     kernel &= ~CQ_MFMA_INT_MIN;
     bool ok = false;
     if (kernel == CQ_MFMA_SKINNY) ok = cq_skinny_supported(w, act);
-    else if (kernel == CQ_MFMA_TILE) ok = kquant ? cq_gemm_supported(w, m, act) : m > 32 && cq_gemm32_supported(w, act);   // as cq_qmatmul
+    else if (kernel == CQ_MFMA_TILE) ok = kquant ? cq_gemm_supported(w, m, act) : m > 16 && cq_gemm32_supported(w, act);   // as cq_qmatmul
     else return cq_set_error(CQ_ERR_INVALID, "kernel must be CQ_MFMA_SKINNY or CQ_MFMA_TILE (plus CQ_MFMA_INT_MIN)");
     if (!ok) return cq_set_error(CQ_ERR_UNSUPPORTED, "that kernel does not take this weight (dtype %d, %lld x %lld) with %lld rows", w->dtype,
                                  (long long)w->n, (long long)w->k, (long long)m);

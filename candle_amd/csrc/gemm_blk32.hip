@@ -342,7 +342,7 @@ hipError_t cq_launch_gemm32(const cq_weight *w, cq_act_view a, int act_dtype, in
                             hipStream_t s) {
     if (!cq_gemm32_supported(w, act_dtype)) return hipErrorNotSupported;
     if (m == 0) return hipSuccess;
-    if (a.m_stride < (m + 127) / 128 * 128) return hipErrorInvalidValue;   // rows the last tile may read
+    if (a.m_stride < (m <= 32 ? 32 : (m + 127) / 128 * 128)) return hipErrorInvalidValue;   // rows the last tile may read
     const cq_mfma_dump none{nullptr, nullptr};
     if (w->dtype == CQ_DTYPE_Q8_0) return launch_dt<CQ_DTYPE_Q8_0, false>(w, a, m, y, y_cleared, none, s);
     return launch_dt<CQ_DTYPE_Q4_0, false>(w, a, m, y, y_cleared, none, s);
@@ -351,7 +351,7 @@ hipError_t cq_launch_gemm32(const cq_weight *w, cq_act_view a, int act_dtype, in
 hipError_t cq_launch_gemm32_dump(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, cq_mfma_dump d, hipStream_t s) {
     if (!cq_gemm32_supported(w, act_dtype)) return hipErrorNotSupported;
     if (m == 0) return hipSuccess;
-    if (a.m_stride < (m + 127) / 128 * 128) return hipErrorInvalidValue;
+    if (a.m_stride < (m <= 32 ? 32 : (m + 127) / 128 * 128)) return hipErrorInvalidValue;
     if (w->dtype == CQ_DTYPE_Q8_0) return launch_dt<CQ_DTYPE_Q8_0, true>(w, a, m, nullptr, true, d, s);
     return launch_dt<CQ_DTYPE_Q4_0, true>(w, a, m, nullptr, true, d, s);
 }

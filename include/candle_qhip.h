@@ -85,7 +85,7 @@ enum {
     CQ_FLAG_STAGED_ACT = 16,  /* up to four rows: run the stand-alone quantizer into the workspace and a matmul kernel
                                  (two launches, as cuda.rs:249-293 does) instead of the single fused launch           */
     CQ_FLAG_DETERMINISTIC = 64 /* the same bits on every run, like the CPU QMatMul.  Without it one family of launches is
-                                 not: the tile kernels (more than 32 rows; grouped experts with more than 8 rows) split K
+                                 not: the tile kernels (17 rows and more; grouped experts with more than 8 rows) split K
                                  over several workgroups when the weight has few row tiles - n = 4096 at 33 .. 1024
                                  rows, the w2 projection of an expert - and add the partial sums atomically in
                                  arrival order, so the last bits of a result can differ between two runs (far inside
@@ -204,9 +204,9 @@ int cq_qmatmul_int_dots(const cq_weight *w, const float *x_dev, int64_t m, int32
                         void *stream);
 
 /* The same integers out of the matrix-core kernels (the verification above runs the dot-product kernels): `kernel`
- * picks the small-batch kernel (CQ_MFMA_SKINNY: the launch cq_qmatmul makes for 2..32 rows, whatever m is here) or
+ * picks the small-batch kernel (CQ_MFMA_SKINNY: the launch cq_qmatmul makes for few rows, whatever m is here) or
  * the tile kernel of the prefill path (CQ_MFMA_TILE, with the tile height and K split cq_qmatmul picks for m;
- * Q8_0 and Q4_0 weights: more than 32 rows, as in cq_qmatmul).
+ * Q8_0 and Q4_0 weights: more than 16 rows, as in cq_qmatmul).
  * out_i as above.  out_mn (Q4K, Q5K; else NULL) is a float: those kernels contract the min term on the f16 matrix
  * core and never hold the integer sum: -dmin * sum_j min_{j/2}*bsums_j over the sixteen sums of a block (exact in
  * f16) with -dmin*min in two f16 pieces, stored as that contraction delivers it for one block (small-batch kernels) or

@@ -122,11 +122,12 @@ def test_skinny_kernel_integers_rounds_of_tiles(qh, dt, m, n):
 
 
 @pytest.mark.parametrize("dt", KQ + B32)
-@pytest.mark.parametrize("m,k,n", [(9, 256, 32), (33, 512, 96), (64, 1024, 160), (130, 768, 288), (129, 2048, 416)])
+@pytest.mark.parametrize("m,k,n", [(9, 256, 32), (17, 1024, 352), (32, 512, 64), (33, 512, 96), (64, 1024, 160), (130, 768, 288),
+                                   (129, 2048, 416)])
 def test_tile_kernel_integers(qh, dt, m, k, n):
     """The prefill tile kernels on ragged shapes: tile heights of 32, 64 and 128 rows, with and without K split."""
-    if dt in B32 and m <= 32:
-        pytest.skip("the Q8_0 / Q4_0 tile kernel is taken above 32 rows only")
+    if dt in B32 and m <= 16:
+        pytest.skip("the Q8_0 / Q4_0 tile kernel is taken above 16 rows only")
     check_dump(qh, dt, qh.MFMA_TILE, m, k, n, 13 * dt + m + k + n)
 
 

@@ -337,9 +337,12 @@ def test_skinny_q8_0_matches_oracle(qh, dt, m, k, n):
     got = qh.qmatmul(qw, dev(x), qh.FLAG_FORCE_SKINNY)
     check_f32(got.cpu().numpy(), orc.matmul(dt, x, blocks, n))
     assert torch.equal(got, qh.qmatmul(qw, dev(x), qh.FLAG_FORCE_SKINNY))
-    # from five rows on this kernel is the default choice; it agrees with the dot-product one
-    if m >= 5:
+    # from five to sixteen rows this kernel is the default choice (beyond, where n is no multiple of 32 and the tile
+    # kernel does not take the weight); it agrees with the dot-product one
+    if m >= 5 and (m <= 16 or n % 32):
         assert torch.equal(got, qh.qmatmul(qw, dev(x)))
+    else:
+        check_f32(got.cpu().numpy(), qh.qmatmul(qw, dev(x)).cpu().numpy())
     check_f32(got.cpu().numpy(), qh.qmatmul(qw, dev(x), qh.FLAG_FORCE_MATVEC).cpu().numpy())
 
 
@@ -539,6 +542,37 @@ def test_prefill_few_weight_rows_long_k(qh, dt, m, k, n):
     assert np.array_equal(again.view(np.uint32), third.view(np.uint32))
 
 
+@pytest.mark.parametrize("dt,m,k,n", [(orc.Q4K, 17, 4096, 24576), (orc.Q4K, 24, 4096, 24544), (orc.Q6K, 32, 4096, 12288),
+                                       (orc.Q5K, 25, 4096, 12256), (orc.Q4K, 48, 8192, 4096), (orc.Q6K, 64, 6144, 4096),
+                                       (orc.Q8_0, 17, 4096, 12288), (orc.Q4_0, 32, 4096, 12288), (orc.Q8_0, 24, 2048, 24576),
+                                       (orc.Q4_0, 21, 4096, 12256), (orc.Q8_0, 3, 11008, 4096), (orc.Q4_0, 4, 11008, 512),
+                                       (orc.Q8_0, 2, 256 * 400, 64)])
+def test_kernel_choice_at_its_row_count_limits(qh, dt, m, k, n):
+    """Shapes either side of the limits at which a call goes to the split-K kernel, a tile kernel or a dot-product
+    kernel (17-32 rows against many weight rows; 33-64 rows against few weight rows with a long K; 2-4 rows of
+    Q8_0 / Q4_0 whose weight rows are too long for the one-launch kernel): the call's own choice against 40 sampled
+    weight rows of the oracle and against every kernel that can be forced on the same shape."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(7 * dt + m + n)
+    w = torch.randn((n, k), generator=gen, device="cuda", dtype=torch.float32) * 0.02
+    x = torch.randn((m, k), generator=gen, device="cuda", dtype=torch.float32)
+    qw = qh.QWeight.zeros(dt, n, k).quantize_(w)
+    got = qh.qmatmul(qw, x)
+    rows = np.random.default_rng(n + m).choice(n, 40, replace=False)
+    blocks = qw.to_ggml().reshape(n, -1)
+    want = orc.matmul(dt, x.cpu().numpy(), np.ascontiguousarray(blocks[rows]).ravel(), len(rows))
+    check_f32(got.cpu().numpy()[:, rows], want)
+    forced = 0
+    for flag in (qh.FLAG_FORCE_SKINNY, qh.FLAG_FORCE_GEMM, qh.FLAG_FORCE_MATVEC):
+        try:
+            other = qh.qmatmul(qw, x, flag)
+        except qh.QHipError:
+            continue   # that kernel does not take the shape
+        forced += 1
+        assert torch.allclose(got, other, rtol=3e-5, atol=3e-5), flag
+    assert forced >= 2
+
+
 # ------------------------------------------------------------------------- MoE ----
 @pytest.mark.parametrize("tokens,starve", [(24, False), (64, True)])
 def test_moe_ffn_matches_oracle(qh, tokens, starve):
@@ -697,10 +731,10 @@ def test_moe_config4_full_size(qh):
 
 # ------------------------------------- tile kernel of the 32-element-block types (Q8_0, Q4_0) ----
 @pytest.mark.parametrize("dt", [orc.Q8_0, orc.Q4_0])
-@pytest.mark.parametrize("m,k,n", [(33, 256, 32), (64, 512, 64), (70, 1024, 96), (130, 768, 288), (200, 2048, 32),
-                                   (129, 4096, 64)])
+@pytest.mark.parametrize("m,k,n", [(17, 512, 32), (32, 4096, 96), (33, 256, 32), (64, 512, 64), (70, 1024, 96), (130, 768, 288),
+                                   (200, 2048, 32), (129, 4096, 64)])
 def test_gemm_blk32_matches_oracle(qh, dt, m, k, n):
-    """More than 32 rows of Q8_0 / Q4_0 weights go to their own int8-MFMA tile kernel (one MFMA result per
+    """More than 16 rows of Q8_0 / Q4_0 weights go to their own int8-MFMA tile kernel (one MFMA result per
     32-element block, scaled by the two block scales): ragged row counts, one and several K steps,
     split K (few workgroups), against the oracle and against the split-K kernel on the same workspace."""
     w, x = make_inputs(3 * dt + m + k, m, k, n, outliers=True)
