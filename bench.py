@@ -788,7 +788,7 @@ def main() -> int:
 
         def moe_ffn():
             h1 = qhip.qmatmul_grouped(w1, xs, rid_d, offs, workspace=moe_ws)
-            h3 = qhip.qmatmul_grouped(w3, xs, rid_d, offs, workspace=moe_ws)
+            h3 = qhip.qmatmul_grouped(w3, xs, rid_d, offs, flags=qhip.FLAG_REUSE_ACT, workspace=moe_ws)   # the rows quantized for w1
             y_ = qhip.qmatmul_grouped(w2, h1, None, offs, workspace=moe_ws, pre=qhip.PRE_SILU_MUL, aux=h3)
             return qhip.moe_scatter_add(y_, rid_d, wts_d, tokens)
 

@@ -750,6 +750,11 @@ static int grouped_impl(const cq_weight *const *experts, int n_experts, const fl
     if (cq_has_min32(w0->ggml_dtype) || cq_has_min16(w0->ggml_dtype) || w0->dtype == CQ_DTYPE_Q8K)
         return cq_set_error(CQ_ERR_UNSUPPORTED, "grouped matmul does not take Q4_1 / Q5_1 / Q2K / Q8K experts (no grouped launch for them)");
     if ((rc = check_pre(pre))) return rc;
+    // (the same routed rows against a second set of experts, w1 and w3 of quantized_llama.rs:60-61: the workspace of the
+    // first grouped call holds them)
+    const bool reuse = (flags & CQ_FLAG_REUSE_ACT) != 0;
+    if (reuse && pre.kind != CQ_PRE_NONE)
+        return cq_set_error(CQ_ERR_INVALID, "a fused step and a reused workspace exclude each other");
     CQ_HIP_CHECK(hipSetDevice(w0->dev));
     hipStream_t s = (hipStream_t)stream;
     cq_act_view v;
@@ -762,10 +767,10 @@ static int grouped_impl(const cq_weight *const *experts, int n_experts, const fl
     // gather + quantize every routed row once (clearing the output on the way if the grouped launch splits K;
     // with row ids the extent of x is not known here, so nothing is cleared then)
     cq_clear clear = cq_no_clear();
-    if (grouped && !row_ids_dev && cq_gemm_grouped_splits_k(experts, n_experts, offsets) &&
+    if (!reuse && grouped && !row_ids_dev && cq_gemm_grouped_splits_k(experts, n_experts, offsets) &&
         clear_in_quantizer_ok(y_dev, total * w0->n, x_dev, total * w0->k, pre))
         clear = cq_clear{y_dev, total * w0->n};
-    CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, row_ids_dev, total, w0->k, pre, v, clear, s));
+    if (!reuse) CQ_HIP_CHECK(cq_launch_quantize_act_ws(act, x_dev, row_ids_dev, total, w0->k, pre, v, clear, s));
     if (grouped) {
         CQ_HIP_CHECK(cq_launch_gemm_grouped(experts, n_experts, offsets, v, y_dev, clear.p != nullptr, s));
         return CQ_OK;

@@ -80,7 +80,10 @@ enum {
                                  quantizer launch.  The earlier call must have gone through the workspace: more than
                                  four rows, or CQ_FLAG_STAGED_ACT (calls of up to four rows may quantize inside their
                                  single launch and leave the workspace alone); cq_qmatmul_multi takes care of this
-                                 by itself.  No counterpart in the reference, which re-quantizes per call.            */
+                                 by itself.  cq_qmatmul_grouped takes it too: the routed rows of the previous grouped
+                                 call (same x, row ids, offsets, k and activation format) against another set of
+                                 experts, w1 and w3 of an expert FFN.  No counterpart in the reference, which
+                                 re-quantizes per call.                                                              */
     CQ_FLAG_FORCE_SKINNY = 32, /* the split-K MFMA kernel for few rows whatever m is (A/B runs)                                */
     CQ_FLAG_STAGED_ACT = 16,  /* up to four rows: run the stand-alone quantizer into the workspace and a matmul kernel
                                  (two launches, as cuda.rs:249-293 does) instead of the single fused launch           */

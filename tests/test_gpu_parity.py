@@ -599,6 +599,8 @@ def test_moe_ffn_matches_oracle(qh, tokens, starve):
     x_d, rid_d, wt_d = dev(xs), dev(row_ids), dev(weights)
     h1 = qh.qmatmul_grouped(q1, x_d, rid_d, offsets)
     h3 = qh.qmatmul_grouped(q3, x_d, rid_d, offsets)
+    # w3 on the rows the workspace already holds (quantized for w1 / w3 just now): no second quantizer launch
+    assert torch.allclose(h3, qh.qmatmul_grouped(q3, x_d, rid_d, offsets, flags=qh.FLAG_REUSE_ACT), rtol=1e-5, atol=1e-5)
     h = qh.silu_mul(h1, h3)
     y = qh.qmatmul_grouped(q2, h, None, offsets)
     ys = qh.moe_scatter_add(y, rid_d, wt_d, tokens).cpu().numpy()
@@ -697,6 +699,9 @@ def test_moe_config4_full_size(qh):
     x_d, rid_d, wt_d = dev(xs), dev(row_ids), dev(weights)
     h1 = qh.qmatmul_grouped(q1, x_d, rid_d, offsets)
     h3 = qh.qmatmul_grouped(q3, x_d, rid_d, offsets)
+    assert torch.equal(h3, qh.qmatmul_grouped(q3, x_d, rid_d, offsets, flags=qh.FLAG_REUSE_ACT))   # (no K split at 14336 rows)
+    with pytest.raises(qh.QHipError, match="exclude each other"):
+        qh.qmatmul_grouped(q2, h1, None, offsets, flags=qh.FLAG_REUSE_ACT, pre=qh.PRE_SILU_MUL, aux=h3)
     h = qh.silu_mul(h1, h3)
     y = qh.qmatmul_grouped(q2, h, None, offsets)
     y_fused = qh.qmatmul_grouped(q2, h1, None, offsets, pre=qh.PRE_SILU_MUL, aux=h3)
