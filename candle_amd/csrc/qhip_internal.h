@@ -198,7 +198,7 @@ bool cq_gemm32_supported(const cq_weight *w, int act_dtype);
 hipError_t cq_launch_gemm32(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, bool y_cleared,
                             hipStream_t s);
 bool cq_gemm32_splits_k(const cq_weight *w, int64_t m);
-// skinny.hip: 2..32 activation rows on the int8 MFMA, K split over the waves of a workgroup
+// skinny.hip: a few activation rows (32 per pass) on the int8 MFMA, K split over the waves of a workgroup
 bool cq_skinny_supported(const cq_weight *w, int act_dtype);
 hipError_t cq_launch_skinny(const cq_weight *w, cq_act_view a, int act_dtype, int64_t m, float *y, hipStream_t s);
 // moe.hip

@@ -1,4 +1,5 @@
-// Skinny matmul on int8 MFMA for 2..32 activation rows: y[m, n] = x[m, k] . W[n, k]^T with K-quant
+// Skinny matmul on int8 MFMA for a few activation rows (32 per pass over the weights; cq_qmatmul sends it 2..16 rows,
+// more where the weight has few rows): y[m, n] = x[m, k] . W[n, k]^T with K-quant
 // weights and Q8K activations (Q8_0 weights with Q8_0 activations: second kernel below) (k_quants.rs:1842-1883 with vec_dot :1171-1250 for Q4K, :1585-1641
 // for Q6K) - the small-batch decode and the per-expert shapes of a mixture-of-experts layer, where
 // the weights are still read once and the job stays bound by HBM.  The arithmetic is that of the
