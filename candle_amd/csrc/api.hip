@@ -537,7 +537,7 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
     enum { kSkinny, kGemm32, kGemm, kMatvec } path;
     // Few rows: split K over the waves instead of tiling rows.  Measured (weights from HBM, 4096..32000 weight rows,
     // k 4096..14336) faster than the dot-product kernels from 2 rows on and than the tile kernels
-    //   up to 16 rows everywhere; up to 24 rows below 24576 weight rows; up to 32 rows below 12288 weight rows;
+    //   up to 16 rows everywhere; up to 24 rows below 14336 weight rows; up to 32 rows below 12288 weight rows;
     //   up to 64 rows where n is small and k short, so that the tile kernel cannot fill the machine.
     // (the 32-element-block types from 4 rows (Q8_0) or 5 rows (Q4_0) on: below that the one-launch dot-product
     // kernel is as fast or faster, it has no per-block scaling of MFMA results to do - where it takes the rows)
@@ -545,7 +545,7 @@ static int qmatmul_impl(const cq_weight *w, const float *x_dev, cq_pre pre, int6
     const int64_t skinny_from = w->dtype == CQ_DTYPE_Q8_0 ? 4 : w->dtype == CQ_DTYPE_Q4_0 ? 5 : 2;
     const bool has_tile_kernel = cq_gemm_supported(w, m, act);
     const bool has_tile32 = m > 16 && cq_gemm32_supported(w, act);
-    const bool skinny_rows = m <= 16 || (m <= 24 && w->n < 24576) || (m <= 32 && w->n < 12288) ||
+    const bool skinny_rows = m <= 16 || (m <= 24 && w->n < 14336) || (m <= 32 && w->n < 12288) ||
                              (m <= 64 && w->n < 8192 && w->k <= 6144);
     if (flags & CQ_FLAG_FORCE_SKINNY) {
         if (!cq_skinny_supported(w, act))

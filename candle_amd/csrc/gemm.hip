@@ -704,6 +704,15 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(cq_weight w, cq_act_view
     gemm_body<DT, MT>(w, a, (int64_t)blockIdx.y * (MT * 32), m, y, ksplit);
 }
 
+// Up to 32 activation rows (one row tile): every weight byte is read once by the launch, cold - the form of the grouped
+// expert launches (copies marked non-temporal; Q4K / Q5K: everything two blocks ahead).
+template <int DT> constexpr int once_wbuf() { return DT == CQ_DTYPE_Q4K || DT == CQ_DTYPE_Q5K ? 2 : 1; }
+template <int DT>
+__global__ void __launch_bounds__(kThreads) gemm_once_kernel(cq_weight w, cq_act_view a, int64_t m, float *__restrict__ y,
+                                                             int ksplit) {
+    gemm_body<DT, 1, false, once_wbuf<DT>(), true>(w, a, 0, m, y, ksplit);
+}
+
 // The same launch with the block integers stored instead of the result (verification).
 template <int DT, int MT>
 __global__ void __launch_bounds__(kThreads) gemm_dump_kernel(cq_weight w, cq_act_view a, int64_t m, int ksplit,
@@ -1141,6 +1150,14 @@ hipError_t launch_mt(const cq_weight *w, cq_act_view a, int64_t m, float *y, int
         if (e != hipSuccess) return e;
     }
     dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)ksplit);
+    if constexpr (MT == 1) {
+        if (gy == 1) {
+            const size_t lds1 = once_wbuf<DT>() == 2 ? Tile<DT, 1>::kTotal2 : Tile<DT, 1>::kTotal;
+            if (hipError_t e = cq_ensure_lds<gemm_once_kernel<DT>>(w->dev, lds1); e != hipSuccess) return e;
+            CQ_LAUNCH((gemm_once_kernel<DT>), grid, kThreads, lds1, s, *w, a, m, y, ksplit);
+            return hipGetLastError();
+        }
+    }
     CQ_LAUNCH((gemm_kernel<DT, MT>), grid, kThreads, lds, s, *w, a, m, y, ksplit);
     return hipGetLastError();
 }

@@ -542,7 +542,7 @@ def test_prefill_few_weight_rows_long_k(qh, dt, m, k, n):
     assert np.array_equal(again.view(np.uint32), third.view(np.uint32))
 
 
-@pytest.mark.parametrize("dt,m,k,n", [(orc.Q4K, 17, 4096, 24576), (orc.Q4K, 24, 4096, 24544), (orc.Q6K, 32, 4096, 12288),
+@pytest.mark.parametrize("dt,m,k,n", [(orc.Q4K, 17, 4096, 14336), (orc.Q4K, 24, 4096, 14304), (orc.Q6K, 32, 4096, 12288),
                                        (orc.Q5K, 25, 4096, 12256), (orc.Q4K, 48, 8192, 4096), (orc.Q6K, 64, 6144, 4096),
                                        (orc.Q8_0, 17, 4096, 12288), (orc.Q4_0, 32, 4096, 12288), (orc.Q8_0, 24, 2048, 24576),
                                        (orc.Q4_0, 21, 4096, 12256), (orc.Q8_0, 3, 11008, 4096), (orc.Q4_0, 4, 11008, 512),
