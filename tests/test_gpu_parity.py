@@ -545,7 +545,7 @@ def test_prefill_few_weight_rows_long_k(qh, dt, m, k, n):
 @pytest.mark.parametrize("dt,m,k,n", [(orc.Q4K, 17, 4096, 14336), (orc.Q4K, 24, 4096, 14304), (orc.Q6K, 32, 4096, 12288),
                                        (orc.Q5K, 25, 4096, 12256), (orc.Q4K, 48, 8192, 4096), (orc.Q6K, 64, 6144, 4096),
                                        (orc.Q8_0, 17, 4096, 12288), (orc.Q4_0, 32, 4096, 12288), (orc.Q8_0, 24, 2048, 24576),
-                                       (orc.Q4_0, 21, 4096, 12256), (orc.Q8_0, 3, 11008, 4096), (orc.Q4_0, 4, 11008, 512),
+                                       (orc.Q4_0, 21, 4096, 12256), (orc.Q4_0, 29, 4096, 20480), (orc.Q8_0, 3, 11008, 4096), (orc.Q4_0, 4, 11008, 512),
                                        (orc.Q8_0, 2, 256 * 400, 64)])
 def test_kernel_choice_at_its_row_count_limits(qh, dt, m, k, n):
     """Shapes either side of the limits at which a call goes to the split-K kernel, a tile kernel or a dot-product
